@@ -1,0 +1,112 @@
+/*
+ * Native entry points of libmf_hip_dataplane.so beyond the drop-in surface of
+ * mf_xcopy_api.h: the raw batch enqueue the benchmark times, runtime services
+ * a host program needs to own GPU memory and streams without touching HIP
+ * itself, and read-only views of the host logic (planner, address registry,
+ * direction algebra) for tests.  Plain C types only; a stream or event is an
+ * opaque void*.  Functions returning int32_t give 0 or a negative BM_* code
+ * unless stated; the mfrt_* services return 0 or a positive HIP error number.
+ *
+ * None of these has a counterpart in the reference's public headers; where
+ * one stands in for reference-internal code the comment says which.
+ */
+#ifndef MF_HIP_DATAPLANE_H
+#define MF_HIP_DATAPLANE_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ---- which memory a copy touches (selects the kernel's cache policy) ---- */
+#define MF_ROUTE_HBM 0
+#define MF_ROUTE_TO_HOST 1
+#define MF_ROUTE_FROM_HOST 2
+
+/* Enqueue `n` independent copies dst[i][0..len[i]) = src[i][0..len[i]) as one
+ * fused launch on `stream` (NULL: the calling thread's stream).  This is the
+ * body of HostDataOpSDMA::BatchCopyG2G
+ * (src/hybm/csrc/data_operation/host/hybm_data_op_sdma.cpp:545-595) without
+ * the pool range checks of the entry layer: every address must be
+ * device-accessible.  Does not wait. */
+int32_t mf_xcopy_batch(const uint64_t *src, const uint64_t *dst, const uint64_t *len, uint32_t n, int32_t route,
+                       void *stream);
+
+/* Same for a {src,dst,len} triple table that already lives in device memory. */
+int32_t mf_xcopy_device_table(const void *triples, uint32_t n, int32_t route, void *stream);
+
+/* Launch-shape knobs.  units: 16-byte units per workgroup chunk (0 = choose
+ * per batch); wgPerCu / wgPerCuLink: resident workgroups per CU for HBM and
+ * host-link routes (0 = keep). */
+int32_t mf_xcopy_tune(uint32_t units, uint32_t wgPerCu, uint32_t wgPerCuLink);
+uint32_t mf_xcopy_choose_units(uint64_t totalBytes, uint32_t cuCount, int32_t route);
+uint64_t mf_xcopy_launch_count(void);
+
+/* Host-only view of the work decomposition: writes, for every chunk of the
+ * normalised batch, up to three byte ranges {srcAddr, dstAddr, bytes, chunk}
+ * (head, 16-byte body, tail) into out[4*i..].  Returns the number of ranges,
+ * or -(needed) when capacity (in ranges) is too small.  inlineForm receives 1
+ * when the batch fits the kernel-argument form. */
+int64_t mf_xcopy_describe_plan(const uint64_t *src, const uint64_t *dst, const uint64_t *len, uint32_t n,
+                               uint32_t units, uint64_t *out, uint64_t capacity, int32_t *inlineForm);
+
+/* ---- runtime services (thin layer over HIP) ------------------------------ */
+int mfrt_init(int device);
+void mfrt_shutdown(void);
+int mfrt_is_initialised(void);
+int mfrt_device_id(void);
+int mfrt_current_device(void);
+int mfrt_bind_thread(void);
+uint32_t mfrt_cu_count(void);
+const char *mfrt_error_string(int err);
+void *mfrt_alloc_device(uint64_t bytes);
+int mfrt_free_device(void *p);
+void *mfrt_alloc_host(uint64_t bytes);
+int mfrt_free_host(void *p);
+int mfrt_pointer_kind(const void *p);
+void *mfrt_stream_create(void);
+int mfrt_stream_destroy(void *stream);
+int mfrt_stream_sync(void *stream);
+int mfrt_device_sync(void);
+void *mfrt_event_create(void);
+int mfrt_event_destroy(void *event);
+int mfrt_event_record(void *event, void *stream);
+int mfrt_event_sync(void *event);
+int mfrt_event_done(void *event);
+float mfrt_event_elapsed_ms(void *start, void *stop);
+int mfrt_memcpy(void *dst, const void *src, uint64_t bytes);
+int mfrt_memset(void *dst, int value, uint64_t bytes);
+
+/* ---- address registry view (HybmVaManager counterpart,
+ *      src/hybm/csrc/mm/hybm_va_manager.h:175-264) -------------------------- */
+void mf_va_clear(void);
+int32_t mf_va_add(uint64_t gva, uint64_t size, int32_t memType, uint64_t lva, uint32_t localRank);
+int32_t mf_va_add_external(uint64_t gva, uint64_t size, int32_t memType, uint64_t lva, uint32_t localRank,
+                           uint32_t importedRank);
+void mf_va_remove(uint64_t va);
+uint64_t mf_va_gva_of_lva(uint64_t lva);
+uint64_t mf_va_lva_of_gva(uint64_t gva);
+int32_t mf_va_is_gva(uint64_t va);
+int32_t mf_va_is_known(uint64_t va);
+int32_t mf_va_mem_type(uint64_t va);
+int64_t mf_va_rank(uint64_t gva);                    /* -1 when not found */
+int32_t mf_va_infer_direction(uint64_t srcVa, uint64_t dstVa);
+uint64_t mf_va_reserve(uint32_t localRank, uint64_t size, int32_t memType);
+void mf_va_unreserve(uint64_t start);
+uint64_t mf_va_range_count(void);
+uint64_t mf_va_reserved_count(void);
+
+/* ---- direction algebra and window arithmetic views ------------------------ */
+int32_t mf_dir_compose(int32_t srcPool, int32_t srcDevice, int32_t dstPool, int32_t dstDevice);
+int32_t mf_dir_translate_smem(int32_t copyType, int32_t srcPoolType, int32_t dstPoolType);
+int32_t mf_dir_checks(int32_t direction);            /* bit 0: source checked, bit 1: destination checked */
+int32_t mf_gva_contains(uint64_t base, uint64_t stride, uint64_t rankCount, uint64_t addr, uint64_t size);
+uint32_t mf_gva_rank(uint64_t base, uint64_t stride, uint64_t rankCount, uint64_t rankSpace, uint64_t addr);
+uint64_t mf_gva_mask48(uint64_t addr);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* MF_HIP_DATAPLANE_H */

@@ -1,0 +1,90 @@
+// The two symbols of libmf_hybm_copy_extend.so (declared in
+// include/mf_hip_copy_extend.h).  They take over from the AscendC launchers at
+// src/hybm/csrc/copy_extend/hybm_copy_kernel.cpp:80-83,121-124, so the
+// reference's own HostDataOpSDMA can drive the HIP kernels through its
+// COPY_EXTEND_FLAG path without a source change.
+#include <stdint.h>
+
+#include <vector>
+
+#include "../../../include/mf_hip_copy_extend.h"
+#include "../../../include/mf_xcopy_types.h"
+#include "../rt/mf_rt.h"
+#include "mf_log.h"
+#include "xcopy_engine.h"
+
+using namespace mf;
+
+namespace {
+
+// The host program selected its GPU long before it loaded the plugin; adopt it.
+bool EngineReady()
+{
+    XcopyEngine &engine = XcopyEngine::Instance();
+    if (engine.Started()) {
+        return true;
+    }
+    int dev = mfrt_current_device();
+    if (dev < 0) {
+        MF_ERROR("copy plugin: no current GPU");
+        return false;
+    }
+    return engine.Start(dev) == BM_OK;
+}
+
+int RouteFor(const void *src, const void *dst)
+{
+    if (mfrt_pointer_kind(dst) == MFRT_PTR_PINNED_HOST) {
+        return MFRT_ROUTE_TO_HOST;
+    }
+    if (mfrt_pointer_kind(src) == MFRT_PTR_PINNED_HOST) {
+        return MFRT_ROUTE_FROM_HOST;
+    }
+    return MFRT_ROUTE_HBM;
+}
+
+}  // namespace
+
+extern "C" __attribute__((visibility("default"))) void hybm_copy_extend(void *src, void *dst, uint64_t len,
+                                                                          uint32_t dim, void *stream)
+{
+    (void)dim;
+    if (src == nullptr || dst == nullptr || len == 0 || !EngineReady()) {
+        return;
+    }
+    const uint64_t s = reinterpret_cast<uint64_t>(src);
+    const uint64_t d = reinterpret_cast<uint64_t>(dst);
+    // NULL stream means the null stream to this ABI, which the engine cannot tell from "pick one":
+    // the reference never passes NULL here (hybm_data_op_sdma.cpp:420), so the thread stream is fine.
+    (void)XcopyEngine::Instance().Submit(&s, &d, &len, 1, RouteFor(src, dst), stream, nullptr, 0);
+}
+
+extern "C" __attribute__((visibility("default"))) void hybm_batch_copy_extend(void *param, uint32_t count, void *mask,
+                                                                                uint32_t dim, void *stream)
+{
+    if (param == nullptr || !EngineReady()) {
+        return;
+    }
+    XcopyEngine &engine = XcopyEngine::Instance();
+    if (mfrt_pointer_kind(param) != MFRT_PTR_DEVICE) {
+        // Host-visible table (what the reference passes: a pinned, device-mapped parameter slot).
+        // It is consumed right here, so the caller may recycle it the moment the mask flips.
+        const uint64_t *t = static_cast<const uint64_t *>(param);
+        thread_local std::vector<uint64_t> s;
+        thread_local std::vector<uint64_t> d;
+        thread_local std::vector<uint64_t> l;
+        s.resize(count);
+        d.resize(count);
+        l.resize(count);
+        for (uint32_t i = 0; i < count; ++i) {
+            s[i] = t[3ull * i];
+            d[i] = t[3ull * i + 1];
+            l[i] = t[3ull * i + 2];
+        }
+        const int route = count == 0 ? MFRT_ROUTE_HBM
+                                     : RouteFor(reinterpret_cast<const void *>(s[0]), reinterpret_cast<const void *>(d[0]));
+        (void)engine.Submit(s.data(), d.data(), l.data(), count, route, stream, mask, dim);
+        return;
+    }
+    (void)engine.SubmitDeviceTable(param, count, MFRT_ROUTE_HBM, stream, mask, dim);
+}

@@ -1,0 +1,249 @@
+// Native C entry points declared in include/mf_hip_dataplane.h.
+#include <vector>
+
+#include "../../../include/mf_hip_dataplane.h"
+#include "../../../include/mf_xcopy_types.h"
+#include "copy_direction.h"
+#include "gva_layout.h"
+#include "mf_log.h"
+#include "va_manager.h"
+#include "xcopy_engine.h"
+
+using namespace mf;
+
+#define MF_EXPORT extern "C" __attribute__((visibility("default")))
+
+MF_EXPORT int32_t mf_xcopy_batch(const uint64_t *src, const uint64_t *dst, const uint64_t *len, uint32_t n,
+                                 int32_t route, void *stream)
+{
+    if ((n != 0 && (src == nullptr || dst == nullptr || len == nullptr)) || route < 0 || route > MF_ROUTE_FROM_HOST) {
+        MF_FAIL(BM_INVALID_PARAM, "mf_xcopy_batch: null array or unknown route " << route);
+    }
+    return XcopyEngine::Instance().Submit(src, dst, len, n, route, stream, nullptr, 0);
+}
+
+MF_EXPORT int32_t mf_xcopy_device_table(const void *triples, uint32_t n, int32_t route, void *stream)
+{
+    if ((n != 0 && triples == nullptr) || route < 0 || route > MF_ROUTE_FROM_HOST) {
+        MF_FAIL(BM_INVALID_PARAM, "mf_xcopy_device_table: null table or unknown route " << route);
+    }
+    return XcopyEngine::Instance().SubmitDeviceTable(triples, n, route, stream, nullptr, 0);
+}
+
+MF_EXPORT int32_t mf_xcopy_tune(uint32_t units, uint32_t wgPerCu, uint32_t wgPerCuLink)
+{
+    XcopyTuning &t = XcopyEngine::Instance().Tuning();
+    t.unitsOverride = units;
+    if (wgPerCu != 0) {
+        t.wgPerCu = wgPerCu;
+    }
+    if (wgPerCuLink != 0) {
+        t.wgPerCuLink = wgPerCuLink;
+    }
+    return BM_OK;
+}
+
+MF_EXPORT uint32_t mf_xcopy_choose_units(uint64_t totalBytes, uint32_t cuCount, int32_t route)
+{
+    return ChooseUnits(totalBytes, cuCount, route, XcopyEngine::Instance().Tuning());
+}
+
+MF_EXPORT uint64_t mf_xcopy_launch_count(void)
+{
+    return XcopyEngine::Instance().LaunchCount();
+}
+
+MF_EXPORT int64_t mf_xcopy_describe_plan(const uint64_t *src, const uint64_t *dst, const uint64_t *len, uint32_t n,
+                                         uint32_t units, uint64_t *out, uint64_t capacity, int32_t *inlineForm)
+{
+    if (units == 0 || units % kXcopyThreads != 0) {
+        return 0;
+    }
+    SegList segs;
+    NormalizeSegments(src, dst, len, n, 1ull << 30, segs);
+    InlinePlan plan;
+    const bool fits = BuildInlinePlan(segs, units, plan);
+    if (inlineForm != nullptr) {
+        *inlineForm = fits ? 1 : 0;
+    }
+    std::vector<uint64_t> triples(3ull * segs.Size() + 3);
+    std::vector<uint32_t> first(segs.Size() + 1);
+    const uint64_t nchunk = BuildTablePlan(segs, units, triples.data(), first.data());
+    uint64_t count = 0;
+    auto emit = [&](uint64_t s, uint64_t d, uint64_t bytes, uint64_t chunk) {
+        if (bytes == 0) {
+            return;
+        }
+        if (count < capacity && out != nullptr) {
+            out[4 * count] = s;
+            out[4 * count + 1] = d;
+            out[4 * count + 2] = bytes;
+            out[4 * count + 3] = chunk;
+        }
+        ++count;
+    };
+    // Walk chunk ids exactly as the kernels do: locate the owner by prefix, then cut by geometry.
+    uint32_t seg = 0;
+    for (uint64_t c = 0; c < nchunk; ++c) {
+        while (seg + 1 <= segs.Size() && first[seg + 1] <= c) {
+            ++seg;
+        }
+        if (fits) {
+            // the inline lookup must agree with the table prefix
+            uint32_t hi = 0;
+            for (uint32_t i = 1; i < kInlineCoarse; ++i) {
+                hi += plan.coarse[i] <= c ? 1u : 0u;
+            }
+            uint32_t s2 = hi * kInlineFan;
+            const uint32_t base = s2;
+            for (uint32_t j = 1; j < kInlineFan; ++j) {
+                s2 += plan.first[base + j] <= c ? 1u : 0u;
+            }
+            if (s2 != seg) {
+                return -1;
+            }
+        }
+        const uint64_t s = segs.src[seg];
+        const uint64_t d = segs.dst[seg];
+        const uint64_t l = segs.len[seg];
+        const SegGeom g = SegmentGeometry(d, l);
+        const uint64_t k = c - first[seg];
+        const uint64_t u0 = k * units;
+        const uint64_t left = g.body > u0 ? g.body - u0 : 0;
+        const uint64_t nunits = left < units ? left : units;
+        if (k == 0) {
+            emit(s, d, g.head, c);
+        }
+        emit(s + g.head + u0 * kUnitBytes, d + g.head + u0 * kUnitBytes, nunits * kUnitBytes, c);
+        if (u0 + units >= g.body) {
+            const uint64_t off = g.head + g.body * kUnitBytes;
+            emit(s + off, d + off, g.tail, c);
+        }
+    }
+    if (count > capacity) {
+        return -static_cast<int64_t>(count);
+    }
+    return static_cast<int64_t>(count);
+}
+
+/* ---- address registry view ------------------------------------------------ */
+MF_EXPORT void mf_va_clear(void)
+{
+    VaManager::Global().Clear();
+}
+
+MF_EXPORT int32_t mf_va_add(uint64_t gva, uint64_t size, int32_t memType, uint64_t lva, uint32_t localRank)
+{
+    return VaManager::Global().AddOwn(gva, size, static_cast<hybm_mem_type>(memType), lva, localRank);
+}
+
+MF_EXPORT int32_t mf_va_add_external(uint64_t gva, uint64_t size, int32_t memType, uint64_t lva, uint32_t localRank,
+                                     uint32_t importedRank)
+{
+    return VaManager::Global().AddExternal(gva, size, static_cast<hybm_mem_type>(memType), lva, localRank, importedRank);
+}
+
+MF_EXPORT void mf_va_remove(uint64_t va)
+{
+    VaManager::Global().Remove(va);
+}
+
+MF_EXPORT uint64_t mf_va_gva_of_lva(uint64_t lva)
+{
+    return VaManager::Global().GvaOfLva(lva);
+}
+
+MF_EXPORT uint64_t mf_va_lva_of_gva(uint64_t gva)
+{
+    return VaManager::Global().LvaOfGva(gva);
+}
+
+MF_EXPORT int32_t mf_va_is_gva(uint64_t va)
+{
+    return VaManager::Global().IsGva(va) ? 1 : 0;
+}
+
+MF_EXPORT int32_t mf_va_is_known(uint64_t va)
+{
+    return VaManager::Global().IsKnown(va) ? 1 : 0;
+}
+
+MF_EXPORT int32_t mf_va_mem_type(uint64_t va)
+{
+    return static_cast<int32_t>(VaManager::Global().MemTypeOf(va));
+}
+
+MF_EXPORT int64_t mf_va_rank(uint64_t gva)
+{
+    uint32_t rank = 0;
+    return VaManager::Global().RankOf(gva, rank) ? static_cast<int64_t>(rank) : -1;
+}
+
+MF_EXPORT int32_t mf_va_infer_direction(uint64_t srcVa, uint64_t dstVa)
+{
+    return static_cast<int32_t>(VaManager::Global().InferDirection(srcVa, dstVa));
+}
+
+MF_EXPORT uint64_t mf_va_reserve(uint32_t localRank, uint64_t size, int32_t memType)
+{
+    return VaManager::Global().Reserve(localRank, size, static_cast<hybm_mem_type>(memType)).start;
+}
+
+MF_EXPORT void mf_va_unreserve(uint64_t start)
+{
+    VaManager::Global().Unreserve(start);
+}
+
+MF_EXPORT uint64_t mf_va_range_count(void)
+{
+    return VaManager::Global().RangeCount();
+}
+
+MF_EXPORT uint64_t mf_va_reserved_count(void)
+{
+    return VaManager::Global().ReservedCount();
+}
+
+/* ---- direction algebra and window arithmetic views -------------------------- */
+MF_EXPORT int32_t mf_dir_compose(int32_t srcPool, int32_t srcDevice, int32_t dstPool, int32_t dstDevice)
+{
+    return static_cast<int32_t>(
+        ComposeDirection(Endpoint{srcPool != 0, srcDevice != 0}, Endpoint{dstPool != 0, dstDevice != 0}));
+}
+
+MF_EXPORT int32_t mf_dir_translate_smem(int32_t copyType, int32_t srcPoolType, int32_t dstPoolType)
+{
+    return static_cast<int32_t>(TranslateSmemCopy(static_cast<smem_bm_copy_type>(copyType),
+                                                  static_cast<smem_bm_mem_type>(srcPoolType),
+                                                  static_cast<smem_bm_mem_type>(dstPoolType)));
+}
+
+MF_EXPORT int32_t mf_dir_checks(int32_t direction)
+{
+    const auto d = static_cast<hybm_data_copy_direction>(direction);
+    return (MustCheckSource(d) ? 1 : 0) | (MustCheckDestination(d) ? 2 : 0);
+}
+
+MF_EXPORT int32_t mf_gva_contains(uint64_t base, uint64_t stride, uint64_t rankCount, uint64_t addr, uint64_t size)
+{
+    GvaWindow w;
+    w.base = base;
+    w.stride = stride;
+    w.rankCount = rankCount;
+    return w.Contains(addr, size) ? 1 : 0;
+}
+
+MF_EXPORT uint32_t mf_gva_rank(uint64_t base, uint64_t stride, uint64_t rankCount, uint64_t rankSpace, uint64_t addr)
+{
+    GvaWindow w;
+    w.base = base;
+    w.stride = stride;
+    w.rankCount = rankCount;
+    w.rankSpace = rankSpace;
+    return w.RankBySpace(addr);
+}
+
+MF_EXPORT uint64_t mf_gva_mask48(uint64_t addr)
+{
+    return Mask48(addr);
+}

@@ -1,0 +1,239 @@
+#include "hip_data_op.h"
+
+#include <cstring>
+#include <vector>
+
+#include "../rt/mf_rt.h"
+#include "copy_direction.h"
+#include "mf_log.h"
+#include "xcopy_engine.h"
+
+namespace mf {
+namespace {
+
+constexpr uint64_t kBounceBytes = 32ull << 20;
+
+// Pinned staging area for caller memory the GPU cannot address (ordinary
+// pageable host memory).  The reference allocates and frees a device buffer
+// per segment for these directions
+// (src/hybm/csrc/data_operation/host/hybm_data_op_sdma.cpp:171-221); here one
+// pinned area per thread is filled by the CPU and scattered by one launch.
+struct Bounce {
+    void *base = nullptr;
+    ~Bounce()
+    {
+        if (base != nullptr && mfrt_is_initialised() != 0) {
+            (void)mfrt_free_host(base);
+        }
+    }
+    uint8_t *Get()
+    {
+        if (base == nullptr) {
+            base = mfrt_alloc_host(kBounceBytes);
+        }
+        return static_cast<uint8_t *>(base);
+    }
+};
+thread_local Bounce t_bounce;
+
+struct Piece {
+    uint64_t src;
+    uint64_t dst;
+    uint64_t len;
+};
+
+bool AnyPageable(void *const *ptrs, uint32_t n)
+{
+    for (uint32_t i = 0; i < n; ++i) {
+        if (mfrt_pointer_kind(ptrs[i]) == MFRT_PTR_PAGEABLE) {
+            return true;
+        }
+    }
+    return false;
+}
+
+int RouteOf(bool srcOnHost, bool dstOnHost)
+{
+    if (dstOnHost) {
+        return MFRT_ROUTE_TO_HOST;
+    }
+    return srcOnHost ? MFRT_ROUTE_FROM_HOST : MFRT_ROUTE_HBM;
+}
+
+}  // namespace
+
+HipDataOp::Result HipDataOp::Initialize() noexcept
+{
+    if (inited_) {
+        return BM_OK;
+    }
+    if (!XcopyEngine::Instance().Started()) {
+        MF_FAIL(BM_NOT_INITIALIZED, "GPU copy engine is not running; call hybm_init first");
+    }
+    inited_ = true;
+    return BM_OK;
+}
+
+void HipDataOp::UnInitialize() noexcept
+{
+    inited_ = false;
+}
+
+HipDataOp::Result HipDataOp::Wait(int32_t) noexcept
+{
+    if (!inited_) {
+        return BM_NOT_INITIALIZED;
+    }
+    return XcopyEngine::Instance().DrainThread();
+}
+
+void HipDataOp::CleanUp() noexcept
+{
+    (void)XcopyEngine::Instance().DrainThread();
+}
+
+HipDataOp::Result HipDataOp::DataCopy(hybm_copy_params &params, hybm_data_copy_direction direction,
+                                      const ExtOptions &options) noexcept
+{
+    void *src = params.src;
+    void *dst = params.dest;
+    uint64_t len = params.dataSize;
+    return Run(&src, &dst, &len, 1, direction, options, (options.flags & ASYNC_COPY_FLAG) != 0);
+}
+
+HipDataOp::Result HipDataOp::DataCopyAsync(hybm_copy_params &params, hybm_data_copy_direction direction,
+                                           const ExtOptions &options) noexcept
+{
+    void *src = params.src;
+    void *dst = params.dest;
+    uint64_t len = params.dataSize;
+    return Run(&src, &dst, &len, 1, direction, options, true);
+}
+
+HipDataOp::Result HipDataOp::BatchDataCopy(hybm_batch_copy_params &params, hybm_data_copy_direction direction,
+                                           const ExtOptions &options) noexcept
+{
+    return Run(params.sources, params.destinations, params.dataSizes, params.batchSize, direction, options,
+               (options.flags & ASYNC_COPY_FLAG) != 0);
+}
+
+HipDataOp::Result HipDataOp::Run(void *const *src, void *const *dst, const uint64_t *len, uint32_t n,
+                                 hybm_data_copy_direction direction, const ExtOptions &options, bool async) noexcept
+{
+    if (!inited_) {
+        return BM_NOT_INITIALIZED;
+    }
+    if (!DirectionValid(direction)) {
+        MF_FAIL(BM_INVALID_PARAM, "copy direction " << direction << " is not executable");
+    }
+    XcopyEngine &engine = XcopyEngine::Instance();
+    const Endpoint se = SourceOf(direction);
+    const Endpoint de = DestinationOf(direction);
+    const bool srcOnHost = !se.device;
+    const bool dstOnHost = !de.device;
+    // Only caller-private host memory can be invisible to the GPU; pool memory is pinned by construction.
+    const bool srcPageable = !se.pool && srcOnHost && AnyPageable(src, n);
+    const bool dstPageable = !de.pool && dstOnHost && AnyPageable(dst, n);
+    void *stream = options.stream != nullptr ? options.stream : engine.ThreadStream();
+    if (stream == nullptr) {
+        MF_FAIL(BM_ERROR, "no stream available for the copy");
+    }
+
+    if (!srcPageable && !dstPageable) {
+        static_assert(sizeof(void *) == sizeof(uint64_t), "64-bit addresses expected");
+        int ret = engine.Submit(reinterpret_cast<const uint64_t *>(src), reinterpret_cast<const uint64_t *>(dst), len, n,
+                                RouteOf(srcOnHost, dstOnHost), stream, nullptr, 0);
+        if (ret != BM_OK) {
+            return ret;
+        }
+        if (!async) {
+            int err = mfrt_stream_sync(stream);
+            if (err != 0) {
+                MF_FAIL(BM_ERROR, "copy failed on the GPU: " << mfrt_error_string(err));
+            }
+        }
+        return BM_OK;
+    }
+
+    // Host DRAM to host DRAM with a pageable side: both buffers are only a CPU
+    // store away from each other, no accelerator is involved.
+    if (srcOnHost && dstOnHost) {
+        int err = mfrt_stream_sync(stream);  // keep order with copies queued earlier
+        if (err != 0) {
+            MF_FAIL(BM_ERROR, "stream wait failed: " << mfrt_error_string(err));
+        }
+        for (uint32_t i = 0; i < n; ++i) {
+            std::memmove(dst[i], src[i], len[i]);
+        }
+        return BM_OK;
+    }
+
+    uint8_t *bounce = t_bounce.Get();
+    if (bounce == nullptr) {
+        MF_FAIL(BM_MALLOC_FAILED, "pinned staging allocation failed");
+    }
+    // Cut the batch into pieces that fit the staging area, then move it round by round.
+    std::vector<Piece> pieces;
+    pieces.reserve(n);
+    for (uint32_t i = 0; i < n; ++i) {
+        uint64_t s = reinterpret_cast<uint64_t>(src[i]);
+        uint64_t d = reinterpret_cast<uint64_t>(dst[i]);
+        uint64_t left = len[i];
+        while (left > 0) {
+            const uint64_t take = left > kBounceBytes ? kBounceBytes : left;
+            pieces.push_back(Piece{s, d, take});
+            s += take;
+            d += take;
+            left -= take;
+        }
+    }
+    std::vector<uint64_t> a;
+    std::vector<uint64_t> b;
+    std::vector<uint64_t> l;
+    size_t at = 0;
+    while (at < pieces.size()) {
+        a.clear();
+        b.clear();
+        l.clear();
+        uint64_t used = 0;
+        size_t end = at;
+        while (end < pieces.size()) {
+            const uint64_t padded = (pieces[end].len + 63) & ~63ull;  // keep staged pieces 64-byte aligned
+            if (used + padded > kBounceBytes) {
+                break;
+            }
+            const uint64_t slot = reinterpret_cast<uint64_t>(bounce) + used;
+            if (srcPageable) {
+                std::memcpy(reinterpret_cast<void *>(slot), reinterpret_cast<const void *>(pieces[end].src),
+                            pieces[end].len);
+                a.push_back(slot);
+                b.push_back(pieces[end].dst);
+            } else {
+                a.push_back(pieces[end].src);
+                b.push_back(slot);
+            }
+            l.push_back(pieces[end].len);
+            used += padded;
+            ++end;
+        }
+        const int route = srcPageable ? MFRT_ROUTE_FROM_HOST : MFRT_ROUTE_TO_HOST;
+        int ret = engine.Submit(a.data(), b.data(), l.data(), static_cast<uint32_t>(l.size()), route, stream, nullptr, 0);
+        if (ret != BM_OK) {
+            return ret;
+        }
+        int err = mfrt_stream_sync(stream);  // the staging area is reused next round
+        if (err != 0) {
+            MF_FAIL(BM_ERROR, "copy failed on the GPU: " << mfrt_error_string(err));
+        }
+        if (dstPageable) {
+            for (size_t i = at; i < end; ++i) {
+                std::memcpy(reinterpret_cast<void *>(pieces[i].dst), reinterpret_cast<const void *>(b[i - at]),
+                            pieces[i].len);
+            }
+        }
+        at = end;
+    }
+    return BM_OK;
+}
+
+}  // namespace mf

@@ -1,0 +1,369 @@
+#include "mem_entity.h"
+
+#include "../rt/mf_rt.h"
+#include "mf_log.h"
+#include "va_manager.h"
+
+namespace mf {
+
+using ock::mf::ExtOptions;
+
+MemEntity::MemEntity(uint16_t id, const hybm_options &options) : id_(id), options_(options) {}
+
+MemEntity::~MemEntity()
+{
+    UnInitialize();
+}
+
+int MemEntity::Initialize(OperatorFactory factory)
+{
+    if (initialized_) {
+        return BM_OK;
+    }
+    if (options_.bmType != HYBM_TYPE_AI_CORE_INITIATE) {
+        dataOperator_ = std::make_shared<ComposeDataOp>(options_, std::move(factory));
+        int ret = dataOperator_->Initialize();
+        if (ret != BM_OK) {
+            dataOperator_ = nullptr;
+            MF_FAIL(ret, "copy engine set-up failed: " << ret);
+        }
+    }
+    initialized_ = true;
+    return BM_OK;
+}
+
+void MemEntity::UnInitialize()
+{
+    if (!initialized_) {
+        return;
+    }
+    if (dataOperator_ != nullptr) {
+        dataOperator_->CleanUp();
+        dataOperator_->UnInitialize();
+        dataOperator_ = nullptr;
+    }
+    (void)UnreserveSpace();
+    initialized_ = false;
+}
+
+int MemEntity::ReserveSpace()
+{
+    if (!initialized_) {
+        return BM_NOT_INITIALIZED;
+    }
+    if (reserved_) {
+        return BM_OK;
+    }
+    if (mfrt_bind_thread() != 0) {
+        MF_FAIL(BM_ERROR, "no GPU bound; call hybm_init first");
+    }
+    // A world of one: the whole window is this rank's, so it is allocated in
+    // one piece now and the address it lands on becomes the window base.
+    if ((options_.memType & HYBM_MEM_TYPE_DEVICE) != 0 && options_.deviceVASpace > 0) {
+        void *p = mfrt_alloc_device(options_.deviceVASpace);
+        if (p == nullptr) {
+            MF_FAIL(BM_MALLOC_FAILED, "HBM pool allocation of " << options_.deviceVASpace << " bytes failed");
+        }
+        device_.base = reinterpret_cast<uint64_t>(p);
+        device_.stride = options_.maxHBMSize;
+        device_.rankCount = options_.rankCount;
+        device_.rankSpace = options_.maxHBMSize;
+        deviceBacked_ = options_.deviceVASpace;
+    }
+    if ((options_.memType & HYBM_MEM_TYPE_HOST) != 0 && options_.hostVASpace > 0) {
+        void *p = mfrt_alloc_host(options_.hostVASpace);
+        if (p == nullptr) {
+            if (device_.base != 0) {
+                (void)mfrt_free_device(reinterpret_cast<void *>(device_.base));
+                device_ = GvaWindow{};
+                deviceBacked_ = 0;
+            }
+            MF_FAIL(BM_MALLOC_FAILED, "pinned DRAM pool allocation of " << options_.hostVASpace << " bytes failed");
+        }
+        host_.base = reinterpret_cast<uint64_t>(p);
+        host_.stride = options_.maxDRAMSize;
+        host_.rankCount = options_.rankCount;
+        host_.rankSpace = options_.maxDRAMSize;
+        hostBacked_ = options_.hostVASpace;
+    }
+    if (dataOperator_ != nullptr) {
+        if (device_.base != 0) {
+            dataOperator_->UpdateGvaSpace(HYBM_MEM_TYPE_DEVICE, device_.base, device_.stride, device_.rankCount);
+        }
+        if (host_.base != 0) {
+            dataOperator_->UpdateGvaSpace(HYBM_MEM_TYPE_HOST, host_.base, host_.stride, host_.rankCount);
+        }
+    }
+    reserved_ = true;
+    return BM_OK;
+}
+
+int MemEntity::UnreserveSpace()
+{
+    if (!reserved_) {
+        return BM_OK;
+    }
+    if (dataOperator_ != nullptr) {
+        dataOperator_->CleanUp();  // nothing may still be reading the pools
+    }
+    if (deviceSlice_ != nullptr) {
+        VaManager::Global().Remove(deviceSlice_->va);
+        deviceSlice_ = nullptr;
+    }
+    if (hostSlice_ != nullptr) {
+        VaManager::Global().Remove(hostSlice_->va);
+        hostSlice_ = nullptr;
+    }
+    if (device_.base != 0) {
+        (void)mfrt_device_sync();
+        (void)mfrt_free_device(reinterpret_cast<void *>(device_.base));
+    }
+    if (host_.base != 0) {
+        (void)mfrt_free_host(reinterpret_cast<void *>(host_.base));
+    }
+    device_ = GvaWindow{};
+    host_ = GvaWindow{};
+    deviceBacked_ = 0;
+    hostBacked_ = 0;
+    reserved_ = false;
+    return BM_OK;
+}
+
+void *MemEntity::WindowBase(hybm_mem_type t) const
+{
+    if (t == HYBM_MEM_TYPE_DEVICE) {
+        return reinterpret_cast<void *>(device_.base);
+    }
+    if (t == HYBM_MEM_TYPE_HOST) {
+        return reinterpret_cast<void *>(host_.base);
+    }
+    return nullptr;
+}
+
+LocalSlice *MemEntity::AllocLocal(hybm_mem_type t, uint64_t size)
+{
+    if (!initialized_ || !reserved_) {
+        MF_ERROR("local allocation before the address space was reserved");
+        return nullptr;
+    }
+    if (size == 0 || size % kLargePage != 0) {
+        MF_ERROR("local allocation size " << size << " is not a positive multiple of 2 MiB");
+        return nullptr;
+    }
+    const bool device = t == HYBM_MEM_TYPE_DEVICE;
+    if (!device && t != HYBM_MEM_TYPE_HOST) {
+        MF_ERROR("local allocation with memory type " << t);
+        return nullptr;
+    }
+    const GvaWindow &w = device ? device_ : host_;
+    std::unique_ptr<LocalSlice> &slot = device ? deviceSlice_ : hostSlice_;
+    const uint64_t backed = device ? deviceBacked_ : hostBacked_;
+    if (w.base == 0 || slot != nullptr || size > backed) {
+        MF_ERROR("local allocation of " << size << " bytes does not fit the reserved window of " << backed);
+        return nullptr;
+    }
+    const uint64_t va = w.PtrOfRank(options_.rankId);
+    if (VaManager::Global().AddOwn(va, size, t, va, options_.rankId) != BM_OK) {
+        return nullptr;
+    }
+    slot.reset(new LocalSlice{t, va, size});
+    return slot.get();
+}
+
+int MemEntity::FreeLocal(LocalSlice *slice)
+{
+    for (std::unique_ptr<LocalSlice> *slot : {&deviceSlice_, &hostSlice_}) {
+        if (slot->get() == slice && slice != nullptr) {
+            VaManager::Global().Remove(slice->va);
+            slot->reset();
+            return BM_OK;
+        }
+    }
+    return BM_INVALID_PARAM;
+}
+
+bool MemEntity::CheckAddressInEntity(const void *ptr, uint64_t length) const
+{
+    if (!initialized_) {
+        return false;
+    }
+    const uint64_t a = reinterpret_cast<uint64_t>(ptr);
+    // Window test as in the reference, narrowed to the bytes that are real
+    // memory: an address in the unbacked remainder of a window would fault
+    // the GPU instead of failing a remote transfer.
+    if (device_.Contains(a, length)) {
+        return a + length <= device_.base + deviceBacked_ || options_.rankCount > 1;
+    }
+    if (host_.Contains(a, length)) {
+        return a + length <= host_.base + hostBacked_ || options_.rankCount > 1;
+    }
+    return false;
+}
+
+void MemEntity::LocateAddrAndRank(void *&src, void *&dest, uint64_t length, std::pair<uint32_t, uint32_t> &ranks) const
+{
+    auto owner = [&](uint64_t a) -> uint32_t {
+        bool inside = false;
+        uint32_t r = host_.RankByStride(a, length, options_.rankId, inside);
+        if (inside) {
+            return r;
+        }
+        return device_.RankByStride(a, length, options_.rankId, inside);
+    };
+    ranks.first = owner(reinterpret_cast<uint64_t>(src));
+    src = reinterpret_cast<void *>(Mask48(reinterpret_cast<uint64_t>(src)));
+    ranks.second = owner(reinterpret_cast<uint64_t>(dest));
+    dest = reinterpret_cast<void *>(Mask48(reinterpret_cast<uint64_t>(dest)));
+}
+
+int MemEntity::CopyData(hybm_copy_params &params, hybm_data_copy_direction direction, void *stream, uint32_t flags)
+{
+    if (!initialized_) {
+        return BM_NOT_INITIALIZED;
+    }
+    if (dataOperator_ == nullptr) {
+        MF_FAIL(BM_ERROR, "this pool has no host copy engine");
+    }
+    if (mfrt_bind_thread() != 0) {
+        return BM_ERROR;
+    }
+    std::pair<uint32_t, uint32_t> ranks;
+    LocateAddrAndRank(params.src, params.dest, params.dataSize, ranks);
+    ExtOptions options{};
+    options.flags = flags;
+    options.stream = stream;
+    options.srcRankId = ranks.first;
+    options.destRankId = ranks.second;
+    return dataOperator_->DataCopy(params, direction, options);
+}
+
+int MemEntity::BatchCopyData(hybm_batch_copy_params &params, hybm_data_copy_direction direction, void *stream,
+                             uint32_t flags)
+{
+    if (!initialized_) {
+        return BM_NOT_INITIALIZED;
+    }
+    if (dataOperator_ == nullptr) {
+        MF_FAIL(BM_ERROR, "this pool has no host copy engine");
+    }
+    if (mfrt_bind_thread() != 0) {
+        return BM_ERROR;
+    }
+    ExtOptions options{};
+    options.stream = stream;
+    options.flags = flags;
+    options.srcRankId = options_.rankId;
+    options.destRankId = options_.rankId;
+    if (options_.rankCount > 1) {
+        for (uint32_t i = 0; i < params.batchSize; ++i) {
+            std::pair<uint32_t, uint32_t> ranks;
+            LocateAddrAndRank(params.sources[i], params.destinations[i], params.dataSizes[i], ranks);
+            options.groupMap[ranks].push_back(i);
+        }
+    } else {
+        // One rank: every element belongs to the pair (rank, rank).  The
+        // addresses are still normalised in place as callers may rely on it.
+        for (uint32_t i = 0; i < params.batchSize; ++i) {
+            params.sources[i] = reinterpret_cast<void *>(Mask48(reinterpret_cast<uint64_t>(params.sources[i])));
+            params.destinations[i] =
+                reinterpret_cast<void *>(Mask48(reinterpret_cast<uint64_t>(params.destinations[i])));
+        }
+    }
+    return dataOperator_->BatchDataCopy(params, direction, options);
+}
+
+int MemEntity::Wait()
+{
+    if (!initialized_) {
+        return BM_NOT_INITIALIZED;
+    }
+    if (dataOperator_ == nullptr) {
+        return BM_ERROR;
+    }
+    return dataOperator_->Wait(0);
+}
+
+EntityRegistry &EntityRegistry::Instance()
+{
+    static EntityRegistry registry;
+    return registry;
+}
+
+void EntityRegistry::SetFactory(OperatorFactory factory)
+{
+    std::lock_guard<std::mutex> guard(lock_);
+    factory_ = std::move(factory);
+}
+
+std::shared_ptr<MemEntity> EntityRegistry::Create(uint16_t id, const hybm_options &options, int &result)
+{
+    std::lock_guard<std::mutex> guard(lock_);
+    if (byId_.count(id) != 0) {
+        result = BM_ERROR;
+        MF_ERROR("pool id " << id << " already exists");
+        return nullptr;
+    }
+    auto entity = std::make_shared<MemEntity>(id, options);
+    result = entity->Initialize(factory_);
+    if (result != BM_OK) {
+        return nullptr;
+    }
+    byId_[id] = entity;
+    byPtr_[entity.get()] = id;
+    return entity;
+}
+
+std::shared_ptr<MemEntity> EntityRegistry::FindById(uint16_t id)
+{
+    std::lock_guard<std::mutex> guard(lock_);
+    auto it = byId_.find(id);
+    return it == byId_.end() ? nullptr : it->second;
+}
+
+std::shared_ptr<MemEntity> EntityRegistry::FindByPtr(const void *handle)
+{
+    std::lock_guard<std::mutex> guard(lock_);
+    auto it = byPtr_.find(handle);
+    if (it == byPtr_.end()) {
+        return nullptr;
+    }
+    auto e = byId_.find(it->second);
+    return e == byId_.end() ? nullptr : e->second;
+}
+
+bool EntityRegistry::Remove(const void *handle)
+{
+    std::shared_ptr<MemEntity> victim;
+    {
+        std::lock_guard<std::mutex> guard(lock_);
+        auto it = byPtr_.find(handle);
+        if (it == byPtr_.end()) {
+            return false;
+        }
+        auto e = byId_.find(it->second);
+        if (e != byId_.end()) {
+            victim = e->second;
+            byId_.erase(e);
+        }
+        byPtr_.erase(it);
+    }
+    if (victim != nullptr) {
+        victim->UnInitialize();
+    }
+    return true;
+}
+
+void EntityRegistry::Clear()
+{
+    std::map<uint16_t, std::shared_ptr<MemEntity>> victims;
+    {
+        std::lock_guard<std::mutex> guard(lock_);
+        victims.swap(byId_);
+        byPtr_.clear();
+    }
+    for (auto &kv : victims) {
+        kv.second->UnInitialize();
+    }
+}
+
+}  // namespace mf

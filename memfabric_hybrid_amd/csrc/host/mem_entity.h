@@ -1,0 +1,92 @@
+// One pooled-memory object of this process: its two address windows (HBM and
+// pinned host DRAM), the local slices that back them, and the copy engine.
+// Single-rank counterpart of MemEntityDefault
+// (src/hybm/csrc/entity/hybm_entity_default.cpp:737-827,995-1017,1141-1157) and
+// of the handle registry in src/hybm/csrc/entity/hybm_entity_factory.cpp:27-54.
+#ifndef MF_MEM_ENTITY_H
+#define MF_MEM_ENTITY_H
+
+#include <map>
+#include <memory>
+#include <mutex>
+#include <utility>
+
+#include "compose_data_op.h"
+#include "gva_layout.h"
+
+namespace mf {
+
+constexpr uint64_t kLargePage = 2ull << 20;     // local allocations are multiples of this
+constexpr uint32_t kEntityIdMax = 510;
+
+struct LocalSlice {
+    hybm_mem_type memType;
+    uint64_t va;
+    uint64_t size;
+};
+
+class MemEntity {
+public:
+    MemEntity(uint16_t id, const hybm_options &options);
+    ~MemEntity();
+
+    int Initialize(OperatorFactory factory);
+    void UnInitialize();
+
+    int ReserveSpace();
+    int UnreserveSpace();
+    void *WindowBase(hybm_mem_type t) const;
+    LocalSlice *AllocLocal(hybm_mem_type t, uint64_t size);
+    int FreeLocal(LocalSlice *slice);
+
+    bool CheckAddressInEntity(const void *ptr, uint64_t length) const;
+    void LocateAddrAndRank(void *&src, void *&dest, uint64_t length, std::pair<uint32_t, uint32_t> &ranks) const;
+
+    int CopyData(hybm_copy_params &params, hybm_data_copy_direction direction, void *stream, uint32_t flags);
+    int BatchCopyData(hybm_batch_copy_params &params, hybm_data_copy_direction direction, void *stream, uint32_t flags);
+    int Wait();
+
+    const hybm_options &Options() const
+    {
+        return options_;
+    }
+    uint16_t Id() const
+    {
+        return id_;
+    }
+
+private:
+    uint16_t id_;
+    hybm_options options_;
+    bool initialized_ = false;
+    bool reserved_ = false;
+    GvaWindow device_;          // stride = maxHBMSize
+    GvaWindow host_;            // stride = maxDRAMSize
+    uint64_t deviceBacked_ = 0; // bytes of the local device window that are real memory
+    uint64_t hostBacked_ = 0;
+    std::unique_ptr<LocalSlice> deviceSlice_;
+    std::unique_ptr<LocalSlice> hostSlice_;
+    std::shared_ptr<ComposeDataOp> dataOperator_;
+};
+
+class EntityRegistry {
+public:
+    static EntityRegistry &Instance();
+    std::shared_ptr<MemEntity> Create(uint16_t id, const hybm_options &options, int &result);
+    std::shared_ptr<MemEntity> FindById(uint16_t id);
+    std::shared_ptr<MemEntity> FindByPtr(const void *handle);
+    bool Remove(const void *handle);
+    void Clear();
+    // Test hook: engines used by entities created afterwards.
+    void SetFactory(OperatorFactory factory);
+
+private:
+    std::mutex lock_;
+    std::map<uint16_t, std::shared_ptr<MemEntity>> byId_;
+    std::map<const void *, uint16_t> byPtr_;
+    OperatorFactory factory_ = OperatorFactory::Default();
+};
+
+}  // namespace mf
+
+#endif  // MF_MEM_ENTITY_H

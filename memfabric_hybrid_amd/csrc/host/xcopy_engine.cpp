@@ -1,0 +1,441 @@
+#include "xcopy_engine.h"
+
+#include <atomic>
+#include <cstring>
+
+#include "../../../include/mf_xcopy_types.h"
+#include "../rt/mf_rt.h"
+#include "mf_log.h"
+
+namespace mf {
+namespace {
+
+constexpr uint32_t kCounters = 4096;          // completion counters shared by launches that carry a mask
+constexpr uint32_t kSlots = 4;                // table staging slots per thread
+constexpr uint64_t kInlinePiece = 1ull << 30; // cut for segments the 32-bit inline length cannot hold
+
+std::atomic<uint32_t> g_counterCursor{0};
+std::atomic<uint64_t> g_launches{0};
+
+// One descriptor table in flight: host fills `host`, a copy kernel moves it to
+// `dev`, the table kernel reads `dev`.  `event` marks the point on the stream
+// after which `host` may be rewritten.
+struct StagingSlot {
+    void *host = nullptr;
+    void *dev = nullptr;
+    uint64_t capacity = 0;
+    void *event = nullptr;
+    bool pending = false;
+};
+
+struct ThreadCtx {
+    void *stream = nullptr;
+    StagingSlot slots[kSlots];
+    uint32_t cursor = 0;
+    SegList segs;
+    ~ThreadCtx()
+    {
+        Release();
+    }
+    void Release()
+    {
+        if (mfrt_is_initialised() == 0) {
+            return;  // runtime already gone at process exit: nothing to hand back
+        }
+        for (auto &slot : slots) {
+            if (slot.event != nullptr) {
+                if (slot.pending) {
+                    (void)mfrt_event_sync(slot.event);
+                }
+                (void)mfrt_event_destroy(slot.event);
+            }
+            if (slot.host != nullptr) {
+                (void)mfrt_free_host(slot.host);
+            }
+            if (slot.dev != nullptr) {
+                (void)mfrt_free_device(slot.dev);
+            }
+            slot = StagingSlot{};
+        }
+        if (stream != nullptr) {
+            (void)mfrt_stream_sync(stream);
+            (void)mfrt_stream_destroy(stream);
+            stream = nullptr;
+        }
+    }
+};
+
+thread_local ThreadCtx t_ctx;
+
+uint64_t RoundUp(uint64_t v, uint64_t to)
+{
+    return (v + to - 1) / to * to;
+}
+
+int AcquireSlot(ThreadCtx &ctx, uint64_t bytes, StagingSlot *&out)
+{
+    StagingSlot &slot = ctx.slots[ctx.cursor];
+    ctx.cursor = (ctx.cursor + 1) % kSlots;
+    if (slot.pending) {
+        int err = mfrt_event_sync(slot.event);
+        if (err != 0) {
+            MF_FAIL(BM_ERROR, "staging slot wait failed: " << mfrt_error_string(err));
+        }
+        slot.pending = false;
+    }
+    if (slot.capacity < bytes) {
+        if (slot.host != nullptr) {
+            (void)mfrt_free_host(slot.host);
+            slot.host = nullptr;
+        }
+        if (slot.dev != nullptr) {
+            (void)mfrt_free_device(slot.dev);
+            slot.dev = nullptr;
+        }
+        const uint64_t cap = RoundUp(bytes < 65536 ? 65536 : bytes, 65536);
+        slot.host = mfrt_alloc_host(cap);
+        slot.dev = mfrt_alloc_device(cap);
+        if (slot.host == nullptr || slot.dev == nullptr) {
+            slot.capacity = 0;
+            MF_FAIL(BM_MALLOC_FAILED, "descriptor staging allocation of " << cap << " bytes failed");
+        }
+        slot.capacity = cap;
+    }
+    if (slot.event == nullptr) {
+        slot.event = mfrt_event_create();
+        if (slot.event == nullptr) {
+            MF_FAIL(BM_ERROR, "event creation failed");
+        }
+    }
+    out = &slot;
+    return BM_OK;
+}
+
+uint32_t GridFor(uint64_t nchunk, uint32_t cuCount, int route, const XcopyTuning &tuning)
+{
+    const uint32_t perCu = route == MFRT_ROUTE_HBM ? tuning.wgPerCu : tuning.wgPerCuLink;
+    uint64_t cap = static_cast<uint64_t>(cuCount == 0 ? 256 : cuCount) * (perCu == 0 ? 1 : perCu);
+    uint64_t grid = nchunk < cap ? nchunk : cap;
+    return grid == 0 ? 1u : static_cast<uint32_t>(grid);
+}
+
+}  // namespace
+
+void NormalizeSegments(const uint64_t *src, const uint64_t *dst, const uint64_t *len, uint32_t n, uint64_t pieceLimit,
+                       SegList &out)
+{
+    out.Clear();
+    uint64_t curSrc = 0;
+    uint64_t curDst = 0;
+    uint64_t curLen = 0;
+    auto flush = [&]() {
+        while (curLen > 0) {
+            uint64_t piece = (pieceLimit != 0 && curLen > pieceLimit) ? pieceLimit : curLen;
+            out.src.push_back(curSrc);
+            out.dst.push_back(curDst);
+            out.len.push_back(piece);
+            out.totalBytes += piece;
+            curSrc += piece;
+            curDst += piece;
+            curLen -= piece;
+        }
+    };
+    for (uint32_t i = 0; i < n; ++i) {
+        if (len[i] == 0) {
+            continue;
+        }
+        if (curLen > 0 && curSrc + curLen == src[i] && curDst + curLen == dst[i]) {
+            curLen += len[i];
+            continue;
+        }
+        flush();
+        curSrc = src[i];
+        curDst = dst[i];
+        curLen = len[i];
+    }
+    flush();
+}
+
+uint32_t ChooseUnits(uint64_t totalBytes, uint32_t cuCount, int route, const XcopyTuning &tuning)
+{
+    if (tuning.unitsOverride != 0) {
+        return static_cast<uint32_t>(RoundUp(tuning.unitsOverride, kXcopyThreads));
+    }
+    const uint32_t perCu = route == MFRT_ROUTE_HBM ? tuning.wgPerCu : tuning.wgPerCuLink;
+    const uint64_t groups = static_cast<uint64_t>(cuCount == 0 ? 256 : cuCount) * (perCu == 0 ? 1 : perCu);
+    uint64_t units = RoundUp(totalBytes / kUnitBytes / groups + 1, kXcopyThreads);
+    if (units < tuning.minUnits) {
+        units = tuning.minUnits;
+    }
+    if (units > tuning.maxUnits) {
+        units = tuning.maxUnits;
+    }
+    return static_cast<uint32_t>(units);
+}
+
+bool BuildInlinePlan(const SegList &segs, uint32_t units, InlinePlan &plan)
+{
+    const uint32_t n = segs.Size();
+    if (n > kInlineSegs) {
+        return false;
+    }
+    uint64_t run = 0;
+    for (uint32_t i = 0; i < n; ++i) {
+        if (segs.len[i] > 0xFFFFFFFFull) {
+            return false;
+        }
+        plan.src[i] = segs.src[i];
+        plan.dst[i] = segs.dst[i];
+        plan.len[i] = static_cast<uint32_t>(segs.len[i]);
+        plan.first[i] = static_cast<uint32_t>(run);
+        run += SegmentChunks(segs.dst[i], segs.len[i], units);
+        if (run >= kNoChunk) {
+            return false;
+        }
+    }
+    for (uint32_t i = n; i < kInlineSegs; ++i) {
+        plan.src[i] = 0;
+        plan.dst[i] = 0;
+        plan.len[i] = 0;
+        plan.first[i] = kNoChunk;
+    }
+    for (uint32_t i = 0; i < kInlineCoarse; ++i) {
+        plan.coarse[i] = plan.first[i * kInlineFan];
+    }
+    plan.nchunk = static_cast<uint32_t>(run);
+    plan.units = units;
+    return true;
+}
+
+uint64_t BuildTablePlan(const SegList &segs, uint32_t units, uint64_t *triples, uint32_t *first)
+{
+    const uint32_t n = segs.Size();
+    uint64_t run = 0;
+    for (uint32_t i = 0; i < n; ++i) {
+        triples[3 * i] = segs.src[i];
+        triples[3 * i + 1] = segs.dst[i];
+        triples[3 * i + 2] = segs.len[i];
+        first[i] = static_cast<uint32_t>(run);
+        run += SegmentChunks(segs.dst[i], segs.len[i], units);
+    }
+    first[n] = static_cast<uint32_t>(run);
+    return run;
+}
+
+XcopyEngine &XcopyEngine::Instance()
+{
+    static XcopyEngine engine;
+    return engine;
+}
+
+int XcopyEngine::Start(int device)
+{
+    int err = mfrt_init(device);
+    if (err != 0) {
+        MF_FAIL(BM_ERROR, "GPU runtime start on device " << device << " failed: " << mfrt_error_string(err));
+    }
+    if (started_) {
+        return BM_OK;
+    }
+    counters_ = mfrt_alloc_device(kCounters * sizeof(uint32_t));
+    if (counters_ == nullptr) {
+        MF_FAIL(BM_MALLOC_FAILED, "completion counter allocation failed");
+    }
+    err = mfrt_memset(counters_, 0, kCounters * sizeof(uint32_t));
+    if (err != 0) {
+        (void)mfrt_free_device(counters_);
+        counters_ = nullptr;
+        MF_FAIL(BM_ERROR, "completion counter clear failed: " << mfrt_error_string(err));
+    }
+    started_ = true;
+    return BM_OK;
+}
+
+void XcopyEngine::Stop()
+{
+    if (!started_) {
+        return;
+    }
+    t_ctx.Release();
+    (void)mfrt_device_sync();
+    if (counters_ != nullptr) {
+        (void)mfrt_free_device(counters_);
+        counters_ = nullptr;
+    }
+    started_ = false;
+    mfrt_shutdown();
+}
+
+bool XcopyEngine::Started() const
+{
+    return started_;
+}
+
+void *XcopyEngine::NextCounter()
+{
+    const uint32_t idx = g_counterCursor.fetch_add(1, std::memory_order_relaxed) % kCounters;
+    return static_cast<uint32_t *>(counters_) + idx;
+}
+
+void *XcopyEngine::ThreadStream()
+{
+    if (t_ctx.stream == nullptr) {
+        if (mfrt_bind_thread() != 0) {
+            return nullptr;
+        }
+        t_ctx.stream = mfrt_stream_create();
+    }
+    return t_ctx.stream;
+}
+
+int XcopyEngine::DrainThread()
+{
+    if (!started_) {
+        return BM_NOT_INITIALIZED;
+    }
+    if (t_ctx.stream == nullptr) {
+        return BM_OK;
+    }
+    int err = mfrt_stream_sync(t_ctx.stream);
+    if (err != 0) {
+        MF_FAIL(BM_ERROR, "stream wait failed: " << mfrt_error_string(err));
+    }
+    return BM_OK;
+}
+
+uint64_t XcopyEngine::LaunchCount() const
+{
+    return g_launches.load();
+}
+
+int XcopyEngine::Submit(const uint64_t *src, const uint64_t *dst, const uint64_t *len, uint32_t n, int route,
+                        void *stream, void *mask, uint32_t maskValue)
+{
+    if (!started_) {
+        MF_FAIL(BM_NOT_INITIALIZED, "xcopy engine not started");
+    }
+    if (mfrt_bind_thread() != 0) {
+        MF_FAIL(BM_ERROR, "cannot make the GPU current on this thread");
+    }
+    if (stream == nullptr) {
+        stream = ThreadStream();
+        if (stream == nullptr) {
+            MF_FAIL(BM_ERROR, "cannot create the thread's stream");
+        }
+    }
+    ThreadCtx &ctx = t_ctx;
+    NormalizeSegments(src, dst, len, n, kInlinePiece, ctx.segs);
+    const uint32_t cu = mfrt_cu_count();
+    const uint32_t units = ChooseUnits(ctx.segs.totalBytes, cu, route, tuning_);
+    void *counter = mask != nullptr ? NextCounter() : nullptr;
+
+    InlinePlan plan;
+    if (BuildInlinePlan(ctx.segs, units, plan)) {
+        const uint32_t grid = GridFor(plan.nchunk, cu, route, tuning_);
+        int err = mfk_xcopy_inline(&plan, route, grid, mask, maskValue, counter, stream);
+        if (err != 0) {
+            MF_FAIL(BM_ERROR, "xcopy launch failed: " << mfrt_error_string(err));
+        }
+        g_launches.fetch_add(1, std::memory_order_relaxed);
+        return BM_OK;
+    }
+
+    // Table form: stage {triples, prefix} through a pinned slot into HBM, then search it there.
+    const uint32_t count = ctx.segs.Size();
+    const uint64_t tripleBytes = 24ull * count;
+    const uint64_t tableBytes = RoundUp(tripleBytes + 4ull * (count + 1), kUnitBytes);
+    StagingSlot *slot = nullptr;
+    int ret = AcquireSlot(ctx, tableBytes, slot);
+    if (ret != BM_OK) {
+        return ret;
+    }
+    uint64_t *triples = static_cast<uint64_t *>(slot->host);
+    uint32_t *first = reinterpret_cast<uint32_t *>(static_cast<uint8_t *>(slot->host) + tripleBytes);
+    const uint64_t nchunk = BuildTablePlan(ctx.segs, units, triples, first);
+    if (nchunk >= kNoChunk) {
+        MF_FAIL(BM_INVALID_PARAM, "batch too large for one launch: " << nchunk << " chunks");
+    }
+
+    SegList stage;
+    const uint64_t hostAddr = reinterpret_cast<uint64_t>(slot->host);
+    const uint64_t devAddr = reinterpret_cast<uint64_t>(slot->dev);
+    NormalizeSegments(&hostAddr, &devAddr, &tableBytes, 1, 0, stage);
+    InlinePlan stagePlan;
+    const uint32_t stageUnits = kXcopyThreads;
+    (void)BuildInlinePlan(stage, stageUnits, stagePlan);
+    int err = mfk_xcopy_inline(&stagePlan, MFRT_ROUTE_FROM_HOST, stagePlan.nchunk, nullptr, 0, nullptr, stream);
+    if (err != 0) {
+        MF_FAIL(BM_ERROR, "descriptor staging launch failed: " << mfrt_error_string(err));
+    }
+    const uint32_t grid = GridFor(nchunk, cu, route, tuning_);
+    const uint8_t *devBase = static_cast<const uint8_t *>(slot->dev);
+    err = mfk_xcopy_table(devBase, devBase + tripleBytes, nullptr, count, static_cast<uint32_t>(nchunk), units, route,
+                          grid, mask, maskValue, counter, stream);
+    if (err != 0) {
+        MF_FAIL(BM_ERROR, "xcopy table launch failed: " << mfrt_error_string(err));
+    }
+    // Both halves of the slot are free again once the table kernel has run.
+    err = mfrt_event_record(slot->event, stream);
+    if (err != 0) {
+        MF_FAIL(BM_ERROR, "event record failed: " << mfrt_error_string(err));
+    }
+    slot->pending = true;
+    g_launches.fetch_add(2, std::memory_order_relaxed);
+    return BM_OK;
+}
+
+int XcopyEngine::SubmitDeviceTable(const void *triples, uint32_t n, int route, void *stream, void *mask,
+                                   uint32_t maskValue)
+{
+    if (!started_) {
+        MF_FAIL(BM_NOT_INITIALIZED, "xcopy engine not started");
+    }
+    if (mfrt_bind_thread() != 0) {
+        MF_FAIL(BM_ERROR, "cannot make the GPU current on this thread");
+    }
+    if (stream == nullptr) {
+        stream = ThreadStream();
+        if (stream == nullptr) {
+            MF_FAIL(BM_ERROR, "cannot create the thread's stream");
+        }
+    }
+    void *counter = mask != nullptr ? NextCounter() : nullptr;
+    if (n == 0) {
+        InlinePlan empty;
+        SegList none;
+        (void)BuildInlinePlan(none, kXcopyThreads, empty);
+        int err = mfk_xcopy_inline(&empty, route, 1, mask, maskValue, counter, stream);
+        return err == 0 ? BM_OK : BM_ERROR;
+    }
+    // The prefix is computed on the GPU; its slot is only ever touched by kernels of this stream.
+    ThreadCtx &ctx = t_ctx;
+    StagingSlot *slot = nullptr;
+    const uint64_t prefixBytes = RoundUp(4ull * (n + 2), kUnitBytes);
+    int ret = AcquireSlot(ctx, prefixBytes, slot);
+    if (ret != BM_OK) {
+        return ret;
+    }
+    const uint32_t units = tuning_.unitsOverride != 0 ? static_cast<uint32_t>(RoundUp(tuning_.unitsOverride, kXcopyThreads))
+                                                      : 4 * kXcopyThreads;
+    uint32_t *first = static_cast<uint32_t *>(slot->dev);
+    uint32_t *nchunkDev = first + n + 1;
+    int err = mfk_xcopy_plan(triples, n, units, first, nchunkDev, stream);
+    if (err != 0) {
+        MF_FAIL(BM_ERROR, "xcopy plan launch failed: " << mfrt_error_string(err));
+    }
+    const uint32_t cu = mfrt_cu_count();
+    const uint32_t grid = GridFor(~0ull, cu, route, tuning_);
+    err = mfk_xcopy_table(triples, first, nchunkDev, n, 0, units, route, grid, mask, maskValue, counter, stream);
+    if (err != 0) {
+        MF_FAIL(BM_ERROR, "xcopy table launch failed: " << mfrt_error_string(err));
+    }
+    err = mfrt_event_record(slot->event, stream);
+    if (err != 0) {
+        MF_FAIL(BM_ERROR, "event record failed: " << mfrt_error_string(err));
+    }
+    slot->pending = true;
+    g_launches.fetch_add(2, std::memory_order_relaxed);
+    return BM_OK;
+}
+
+}  // namespace mf

@@ -1,0 +1,99 @@
+// Host planner and submission engine of the xcopy kernels (plain C++, no HIP
+// types).  It turns a caller's segment list into one fused kernel launch on a
+// stream: the job HostDataOpSDMA::BatchCopyG2G / BatchCopyExtend do with one
+// SDMA descriptor per segment or a 32-block plugin launch
+// (src/hybm/csrc/data_operation/host/hybm_data_op_sdma.cpp:504-595).
+#ifndef MF_XCOPY_ENGINE_H
+#define MF_XCOPY_ENGINE_H
+
+#include <stdint.h>
+
+#include <vector>
+
+#include "../kernels/xcopy_plan.h"
+
+namespace mf {
+
+// Segment list after normalisation: empty segments dropped, neighbours that
+// continue each other on both sides merged (the reference merges the same
+// way before building descriptors, hybm_data_op_sdma.cpp:571-574).
+struct SegList {
+    std::vector<uint64_t> src;
+    std::vector<uint64_t> dst;
+    std::vector<uint64_t> len;
+    uint64_t totalBytes = 0;
+    void Clear()
+    {
+        src.clear();
+        dst.clear();
+        len.clear();
+        totalBytes = 0;
+    }
+    uint32_t Size() const
+    {
+        return static_cast<uint32_t>(src.size());
+    }
+};
+
+// pieceLimit: segments longer than this are cut into pieces of at most that
+// many bytes (the inline plan stores 32-bit lengths); 0 = never cut.
+void NormalizeSegments(const uint64_t *src, const uint64_t *dst, const uint64_t *len, uint32_t n, uint64_t pieceLimit,
+                       SegList &out);
+
+struct XcopyTuning {
+    uint32_t unitsOverride = 0;  // 16-byte units per chunk, 0 = choose from batch size
+    uint32_t wgPerCu = 8;        // resident workgroups per CU for HBM routes
+    uint32_t wgPerCuLink = 2;    // the same for routes bound by the host link
+    uint32_t minUnits = kXcopyThreads;
+    uint32_t maxUnits = 16 * kXcopyThreads;
+};
+
+uint32_t ChooseUnits(uint64_t totalBytes, uint32_t cuCount, int route, const XcopyTuning &tuning);
+
+// Returns false when the list does not fit the inline form.
+bool BuildInlinePlan(const SegList &segs, uint32_t units, InlinePlan &plan);
+
+// triples: 3 * segs.Size() words, first: segs.Size() + 1 words.  Returns total chunks.
+uint64_t BuildTablePlan(const SegList &segs, uint32_t units, uint64_t *triples, uint32_t *first);
+
+class XcopyEngine {
+public:
+    static XcopyEngine &Instance();
+
+    int Start(int device);          // BM_* code
+    void Stop();
+    bool Started() const;
+
+    XcopyTuning &Tuning()
+    {
+        return tuning_;
+    }
+
+    // The calling thread's own stream (created on first use).
+    void *ThreadStream();
+    // Wait for everything this thread enqueued on its own stream.
+    int DrainThread();
+
+    // Enqueue one batch.  Addresses must be device-accessible.  stream may be
+    // NULL (thread stream).  mask/maskValue: plugin completion word or NULL.
+    // Returns 0 or a negative BM_* code; never waits for the copy itself.
+    int Submit(const uint64_t *src, const uint64_t *dst, const uint64_t *len, uint32_t n, int route, void *stream,
+               void *mask, uint32_t maskValue);
+
+    // Same for a triple table that lives in device memory the host cannot read.
+    int SubmitDeviceTable(const void *triples, uint32_t n, int route, void *stream, void *mask, uint32_t maskValue);
+
+    uint64_t LaunchCount() const;
+
+private:
+    XcopyEngine() = default;
+    void *NextCounter();
+
+    XcopyTuning tuning_;
+    void *counters_ = nullptr;   // device uint32[kCounters], all zero between launches
+    bool started_ = false;
+};
+
+}  // namespace mf
+
+#endif  // MF_XCOPY_ENGINE_H

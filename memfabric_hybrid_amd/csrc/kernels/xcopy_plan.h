@@ -1,0 +1,94 @@
+// Work decomposition shared by the host planner and the xcopy kernels.
+//
+// A batch is a list of segments {src, dst, len} (the reference's uint64
+// triples, src/hybm/csrc/data_operation/host/hybm_data_op_sdma.cpp:520-528).
+// Each segment is cut into "chunks", the unit one workgroup copies in one
+// loop iteration, so that work is proportional to bytes and not to segment
+// count (the reference's kernel gives every core count/32 whole segments,
+// src/hybm/csrc/copy_extend/hybm_copy_kernel.cpp:102-104).
+//
+// Geometry of one segment (all derived from dst, len and the chunk size):
+//   head  = bytes until dst reaches a 16-byte boundary (capped at len)
+//   body  = the following floor((len-head)/16) 16-byte units; stores are aligned
+//   tail  = the remaining (len-head) % 16 bytes
+//   chunk k covers body units [k*U, min((k+1)*U, body)); chunk 0 also copies
+//   the head, the last chunk also copies the tail.  A segment of len > 0 has
+//   max(1, ceil(body/U)) chunks, a segment of len 0 has none.
+//
+// This header is plain C++ (no HIP types) so the host planner and its CPU
+// tests can include it.
+#ifndef MF_XCOPY_PLAN_H
+#define MF_XCOPY_PLAN_H
+
+#include <stdint.h>
+
+namespace mf {
+
+constexpr uint32_t kXcopyThreads = 256;       // lanes per workgroup (4 wave64)
+constexpr uint32_t kUnitBytes = 16;           // one 128-bit access
+constexpr uint32_t kInlineSegs = 128;         // segments that fit in the kernel-argument block
+constexpr uint32_t kInlineFan = 8;            // second-level fan-out of the two-level lookup
+constexpr uint32_t kInlineCoarse = kInlineSegs / kInlineFan;  // 16 first-level keys
+constexpr uint32_t kNoChunk = 0xFFFFFFFFu;    // sentinel prefix for unused slots
+
+#if defined(__HIPCC__) || defined(__CUDACC__)
+#define MF_HD __host__ __device__
+#else
+#define MF_HD
+#endif
+
+struct SegGeom {
+    uint32_t head;     // 0..15
+    uint32_t tail;     // 0..15
+    uint64_t body;     // 16-byte units
+};
+
+MF_HD inline SegGeom SegmentGeometry(uint64_t dst, uint64_t len)
+{
+    SegGeom g;
+    uint64_t h = (0 - dst) & (kUnitBytes - 1);
+    if (h > len) {
+        h = len;
+    }
+    g.head = static_cast<uint32_t>(h);
+    g.body = (len - h) / kUnitBytes;
+    g.tail = static_cast<uint32_t>((len - h) % kUnitBytes);
+    return g;
+}
+
+// Chunks of a segment for `units` 16-byte units per chunk.
+MF_HD inline uint64_t SegmentChunks(uint64_t dst, uint64_t len, uint32_t units)
+{
+    if (len == 0) {
+        return 0;
+    }
+    SegGeom g = SegmentGeometry(dst, len);
+    uint64_t n = (g.body + units - 1) / units;
+    return n == 0 ? 1 : n;
+}
+
+// Everything a launch of up to kInlineSegs segments needs, passed by value in
+// the kernel-argument block (3144 bytes of the 4096 available): no table
+// upload, no extra dependent memory round trip before the first data load.
+struct InlinePlan {
+    uint64_t src[kInlineSegs];
+    uint64_t dst[kInlineSegs];
+    uint32_t len[kInlineSegs];          // inline path carries segments < 4 GiB only
+    uint32_t first[kInlineSegs];        // exclusive prefix of chunk counts, kNoChunk past the end
+    uint32_t coarse[kInlineCoarse];     // first[kInlineFan * i]
+    uint32_t nchunk;
+    uint32_t units;                     // 16-byte units per chunk, multiple of kXcopyThreads
+};
+
+// A table-driven launch: triples and prefix live in device memory.
+struct TablePlan {
+    const uint64_t *triples;            // {src,dst,len} * nseg
+    const uint32_t *first;              // nseg + 1 entries, first[nseg] == nchunk
+    uint32_t nseg;
+    uint32_t nchunk;
+    uint32_t units;
+};
+
+}  // namespace mf
+
+#endif  // MF_XCOPY_PLAN_H

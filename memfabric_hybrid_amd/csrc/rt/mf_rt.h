@@ -1,0 +1,75 @@
+// Thin C layer over HIP.  Host C++ above this line never sees a HIP type:
+// streams, events and device pointers travel as void*, sizes as integers.
+// mfrt_* = runtime services, mfk_* = kernel launchers (enqueue only).
+// Every int return is 0 on success or the hipError_t value.
+#ifndef MF_RT_H
+#define MF_RT_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* The plugin library keeps the runtime layer private so that it can share a
+ * process with the data-plane library. */
+#ifndef MF_RT_HIDDEN
+#pragma GCC visibility push(default)
+#endif
+
+#define MFRT_ROUTE_HBM 0        /* source and destination in HBM            */
+#define MFRT_ROUTE_TO_HOST 1    /* destination in pinned, mapped host DRAM  */
+#define MFRT_ROUTE_FROM_HOST 2  /* source in pinned, mapped host DRAM       */
+
+#define MFRT_PTR_PAGEABLE 0     /* ordinary host memory the GPU cannot address */
+#define MFRT_PTR_DEVICE 1
+#define MFRT_PTR_PINNED_HOST 2
+
+/* ---- runtime ------------------------------------------------------------ */
+int mfrt_init(int device);
+int mfrt_current_device(void);          /* device current on the calling thread, -1 on error */
+int mfrt_bind_thread(void);             /* make the initialised device current on this thread */
+void mfrt_shutdown(void);
+int mfrt_is_initialised(void);
+int mfrt_device_id(void);
+uint32_t mfrt_cu_count(void);
+const char *mfrt_error_string(int err);
+
+void *mfrt_alloc_device(uint64_t bytes);
+int mfrt_free_device(void *p);
+void *mfrt_alloc_host(uint64_t bytes);  /* pinned + device-mapped + portable */
+int mfrt_free_host(void *p);
+int mfrt_pointer_kind(const void *p);
+
+void *mfrt_stream_create(void);
+int mfrt_stream_destroy(void *stream);
+int mfrt_stream_sync(void *stream);
+int mfrt_device_sync(void);
+
+void *mfrt_event_create(void);
+int mfrt_event_destroy(void *event);
+int mfrt_event_record(void *event, void *stream);
+int mfrt_event_sync(void *event);
+int mfrt_event_done(void *event);       /* 1 finished, 0 pending, <0 error */
+float mfrt_event_elapsed_ms(void *start, void *stop);
+
+int mfrt_memcpy(void *dst, const void *src, uint64_t bytes);  /* blocking hipMemcpy, direction inferred */
+int mfrt_memset(void *dst, int value, uint64_t bytes);
+
+/* ---- xcopy launchers (kernels/xcopy.hip) --------------------------------- */
+int mfk_xcopy_inline(const void *inlinePlan, int route, uint32_t grid, void *mask, uint32_t maskValue, void *counter,
+                     void *stream);
+int mfk_xcopy_table(const void *triples, const void *first, const void *nchunkDev, uint32_t nseg, uint32_t nchunk,
+                    uint32_t units, int route, uint32_t grid, void *mask, uint32_t maskValue, void *counter,
+                    void *stream);
+int mfk_xcopy_plan(const void *triples, uint32_t nseg, uint32_t units, void *first, void *nchunk, void *stream);
+
+#ifndef MF_RT_HIDDEN
+#pragma GCC visibility pop
+#endif
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* MF_RT_H */

@@ -1,0 +1,245 @@
+// HIP side of the thin runtime layer declared in mf_rt.h.
+// On MI355X this replaces the reference's whole stream engine
+// (src/hybm/csrc/ts_engine/hybm_stream.cpp:213-242,358-389: hand-built SQEs,
+// one driver call per descriptor, usleep polling) and its dlopen shims for
+// the vendor runtime (src/hybm/csrc/under_api/dl_acl_api.cpp:73-101): a HIP
+// stream is the submission queue, an event is the completion record.
+#include <hip/hip_runtime.h>
+
+#include <atomic>
+#include <mutex>
+
+#include "mf_rt.h"
+
+namespace {
+
+std::mutex g_lock;
+std::atomic<int> g_device{-1};
+uint32_t g_cuCount = 0;
+
+inline int Code(hipError_t e)
+{
+    return static_cast<int>(e);
+}
+
+}  // namespace
+
+extern "C" int mfrt_init(int device)
+{
+    std::lock_guard<std::mutex> guard(g_lock);
+    if (g_device.load() >= 0) {
+        return g_device.load() == device ? 0 : Code(hipErrorInvalidDevice);
+    }
+    int count = 0;
+    hipError_t err = hipGetDeviceCount(&count);
+    if (err != hipSuccess) {
+        return Code(err);
+    }
+    if (device < 0 || device >= count) {
+        return Code(hipErrorInvalidDevice);
+    }
+    err = hipSetDevice(device);
+    if (err != hipSuccess) {
+        return Code(err);
+    }
+    hipDeviceProp_t prop;
+    err = hipGetDeviceProperties(&prop, device);
+    if (err != hipSuccess) {
+        return Code(err);
+    }
+    g_cuCount = static_cast<uint32_t>(prop.multiProcessorCount);
+    g_device.store(device);
+    return 0;
+}
+
+extern "C" int mfrt_current_device(void)
+{
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess) {
+        (void)hipGetLastError();
+        return -1;
+    }
+    return dev;
+}
+
+extern "C" int mfrt_bind_thread(void)
+{
+    const int dev = g_device.load();
+    if (dev < 0) {
+        return Code(hipErrorNotInitialized);
+    }
+    thread_local int bound = -1;
+    if (bound == dev) {
+        return 0;
+    }
+    hipError_t err = hipSetDevice(dev);
+    if (err == hipSuccess) {
+        bound = dev;
+    }
+    return Code(err);
+}
+
+extern "C" void mfrt_shutdown(void)
+{
+    std::lock_guard<std::mutex> guard(g_lock);
+    if (g_device.load() >= 0) {
+        (void)hipDeviceSynchronize();
+        g_device.store(-1);
+    }
+}
+
+extern "C" int mfrt_is_initialised(void)
+{
+    return g_device.load() >= 0 ? 1 : 0;
+}
+
+extern "C" int mfrt_device_id(void)
+{
+    return g_device.load();
+}
+
+extern "C" uint32_t mfrt_cu_count(void)
+{
+    return g_cuCount;
+}
+
+extern "C" const char *mfrt_error_string(int err)
+{
+    return hipGetErrorString(static_cast<hipError_t>(err));
+}
+
+extern "C" void *mfrt_alloc_device(uint64_t bytes)
+{
+    void *p = nullptr;
+    if (hipMalloc(&p, bytes) != hipSuccess) {
+        (void)hipGetLastError();
+        return nullptr;
+    }
+    return p;
+}
+
+extern "C" int mfrt_free_device(void *p)
+{
+    return Code(hipFree(p));
+}
+
+extern "C" void *mfrt_alloc_host(uint64_t bytes)
+{
+    void *p = nullptr;
+    if (hipHostMalloc(&p, bytes, hipHostMallocMapped | hipHostMallocPortable) != hipSuccess) {
+        (void)hipGetLastError();
+        return nullptr;
+    }
+    return p;
+}
+
+extern "C" int mfrt_free_host(void *p)
+{
+    return Code(hipHostFree(p));
+}
+
+extern "C" int mfrt_pointer_kind(const void *p)
+{
+    hipPointerAttribute_t attr;
+    if (hipPointerGetAttributes(&attr, p) != hipSuccess) {
+        (void)hipGetLastError();  // unknown to the runtime: plain pageable memory
+        return MFRT_PTR_PAGEABLE;
+    }
+    switch (attr.type) {
+        case hipMemoryTypeDevice:
+            return MFRT_PTR_DEVICE;
+        case hipMemoryTypeHost:
+            return MFRT_PTR_PINNED_HOST;
+        case hipMemoryTypeManaged:
+            return MFRT_PTR_DEVICE;
+        default:
+            return MFRT_PTR_PAGEABLE;
+    }
+}
+
+extern "C" void *mfrt_stream_create(void)
+{
+    hipStream_t s = nullptr;
+    if (hipStreamCreateWithFlags(&s, hipStreamNonBlocking) != hipSuccess) {
+        (void)hipGetLastError();
+        return nullptr;
+    }
+    return s;
+}
+
+extern "C" int mfrt_stream_destroy(void *stream)
+{
+    return Code(hipStreamDestroy(static_cast<hipStream_t>(stream)));
+}
+
+extern "C" int mfrt_stream_sync(void *stream)
+{
+    return Code(hipStreamSynchronize(static_cast<hipStream_t>(stream)));
+}
+
+extern "C" int mfrt_device_sync(void)
+{
+    return Code(hipDeviceSynchronize());
+}
+
+extern "C" void *mfrt_event_create(void)
+{
+    hipEvent_t e = nullptr;
+    if (hipEventCreate(&e) != hipSuccess) {
+        (void)hipGetLastError();
+        return nullptr;
+    }
+    return e;
+}
+
+extern "C" int mfrt_event_destroy(void *event)
+{
+    return Code(hipEventDestroy(static_cast<hipEvent_t>(event)));
+}
+
+extern "C" int mfrt_event_record(void *event, void *stream)
+{
+    return Code(hipEventRecord(static_cast<hipEvent_t>(event), static_cast<hipStream_t>(stream)));
+}
+
+extern "C" int mfrt_event_sync(void *event)
+{
+    return Code(hipEventSynchronize(static_cast<hipEvent_t>(event)));
+}
+
+extern "C" int mfrt_event_done(void *event)
+{
+    hipError_t err = hipEventQuery(static_cast<hipEvent_t>(event));
+    if (err == hipSuccess) {
+        return 1;
+    }
+    if (err == hipErrorNotReady) {
+        (void)hipGetLastError();
+        return 0;
+    }
+    return -Code(err);
+}
+
+extern "C" float mfrt_event_elapsed_ms(void *start, void *stop)
+{
+    float ms = -1.0f;
+    if (hipEventElapsedTime(&ms, static_cast<hipEvent_t>(start), static_cast<hipEvent_t>(stop)) != hipSuccess) {
+        (void)hipGetLastError();
+        return -1.0f;
+    }
+    return ms;
+}
+
+extern "C" int mfrt_memcpy(void *dst, const void *src, uint64_t bytes)
+{
+    return Code(hipMemcpy(dst, src, bytes, hipMemcpyDefault));
+}
+
+extern "C" int mfrt_memset(void *dst, int value, uint64_t bytes)
+{
+    hipError_t err = hipMemset(dst, value, bytes);
+    if (err != hipSuccess) {
+        return Code(err);
+    }
+    return Code(hipDeviceSynchronize());
+}

@@ -1,0 +1,353 @@
+"""Pins of oracle/mf_oracle.c: each restated function is checked against
+something that does not share its code (reference-built library, known
+answers, closed forms, brute force) before any test trusts it as the checker."""
+
+import ctypes
+import json
+import os
+
+import numpy as np
+import pytest
+
+from tests import oracle_lib
+from tests.oracle_lib import np_ptr, ptr_array, u64_array
+
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+
+
+# ---- data pattern ------------------------------------------------------------
+def test_lcg_pattern_known_answers(oracle):
+    gold = json.load(open(os.path.join(GOLDEN, "lcg_pattern.json")))
+    for rank, words in gold["ranks"].items():
+        buf = np.zeros(gold["words"], dtype=np.int32)
+        oracle.orc_lcg_fill(np_ptr(buf), int(rank), buf.nbytes)
+        assert buf.tolist() == words
+    for rank, total in gold["sum_4096"].items():
+        buf = np.zeros(4096, dtype=np.int32)
+        oracle.orc_lcg_fill(np_ptr(buf), int(rank), buf.nbytes)
+        assert int(buf.astype(np.int64).sum()) == total
+
+
+def test_lcg_ignores_trailing_bytes_and_null(oracle):
+    buf = np.full(5, 0x55555555, dtype=np.int32)
+    oracle.orc_lcg_fill(np_ptr(buf), 0, 4 * 4 + 3)  # 19 bytes -> 4 whole words
+    assert buf[4] == 0x55555555 and buf[0] == -17
+    oracle.orc_lcg_fill(None, 0, 64)
+    other = buf.copy()
+    other[2] += 1
+    assert oracle.orc_lcg_mismatch(np_ptr(buf), np_ptr(other), 16) == 1
+    assert oracle.orc_lcg_mismatch(None, np_ptr(other), 16) == 0
+
+
+# ---- copies --------------------------------------------------------------------
+def test_copy_is_memcpy_with_bound_check(oracle):
+    rng = np.random.default_rng(1)
+    src = rng.integers(0, 256, 4099, dtype=np.uint8)
+    for count, off in [(0, 0), (1, 3), (257, 5), (4099, 0), (1000, 1)]:
+        dst = np.full(4200, 0xAB, dtype=np.uint8)
+        assert oracle.orc_copy(np_ptr(dst) + off, count, np_ptr(src), count) == 0
+        assert np.array_equal(dst[off:off + count], src[:count])
+        assert np.all(dst[:off] == 0xAB) and np.all(dst[off + count:] == 0xAB)
+    dst = np.zeros(8, dtype=np.uint8)
+    assert oracle.orc_copy(np_ptr(dst), 4, np_ptr(src), 5) == -2
+    assert np.all(dst == 0)
+
+
+def test_copy_matches_reference_memcpy(oracle, ref):
+    rng = np.random.default_rng(2)
+    src = rng.integers(0, 256, 70000, dtype=np.uint8)
+    for count in (0, 1, 15, 16, 17, 4096, 65537):
+        a = np.full(70016, 1, dtype=np.uint8)
+        b = np.full(70016, 1, dtype=np.uint8)
+        assert oracle.orc_copy(np_ptr(a) + 7, count, np_ptr(src) + 3, count) == 0
+        assert ref.ref_memcpy(np_ptr(b) + 7, count, np_ptr(src) + 3, count, 0) == 0
+        assert np.array_equal(a, b)
+    a = np.zeros(16, dtype=np.uint8)
+    assert ref.ref_memcpy(np_ptr(a), 4, np_ptr(src), 5, 0) == oracle.orc_copy(np_ptr(a), 4, np_ptr(src), 5) == -2
+    # any kind other than host-to-host is refused by the reference's CPU branch
+    assert ref.ref_memcpy(np_ptr(a), 4, np_ptr(src), 4, 1) == -2
+
+
+def _random_batch(rng, n, pool):
+    lens = rng.integers(0, 5000, n)
+    lens[rng.integers(0, n, 3)] = 0
+    dst_off = np.cumsum(np.concatenate([[0], lens[:-1] + rng.integers(0, 64, n - 1)]))
+    src_off = rng.integers(0, pool - 5000, n)
+    return src_off, dst_off, lens
+
+
+def test_batch_copy_equals_numpy_and_reference(oracle):
+    rng = np.random.default_rng(3)
+    pool = 1 << 20
+    src = rng.integers(0, 256, pool, dtype=np.uint8)
+    n = 200
+    src_off, dst_off, lens = _random_batch(rng, n, pool)
+    expect = np.full(pool, 7, dtype=np.uint8)
+    for s, d, l in zip(src_off, dst_off, lens):
+        expect[d:d + l] = src[s:s + l]
+    outs = []
+    fns = [oracle.orc_batch_copy, oracle.orc_batch_copy_fast]
+    if oracle_lib.reference() is not None:
+        fns.append(oracle_lib.reference().ref_batch_copy)
+    for fn in fns:
+        dst = np.full(pool, 7, dtype=np.uint8)
+        srcs = ptr_array([np_ptr(src) + int(s) for s in src_off])
+        dsts = ptr_array([np_ptr(dst) + int(d) for d in dst_off])
+        assert fn(dsts, srcs, u64_array(lens), n) == 0
+        outs.append(dst)
+    for dst in outs:
+        assert np.array_equal(dst, expect)
+
+
+def test_copy_2d_equals_numpy(oracle):
+    rng = np.random.default_rng(4)
+    src = rng.integers(0, 256, (37, 160), dtype=np.uint8)
+    dst = np.zeros((37, 300), dtype=np.uint8)
+    oracle.orc_copy_2d(np_ptr(dst) + 11, 300, np_ptr(src) + 5, 160, 90, 37)
+    expect = np.zeros((37, 300), dtype=np.uint8)
+    expect[:, 11:101] = src[:, 5:95]
+    assert np.array_equal(dst, expect)
+
+
+# ---- tables ---------------------------------------------------------------------
+def _endpoint(smem_type):
+    # LOCAL_DEVICE 0, LOCAL_HOST 1, DEVICE 2, HOST 3 -> (in pool, on device)
+    return smem_type >= 2, smem_type in (0, 2)
+
+
+def test_direct_map_has_the_product_structure(oracle):
+    """Independent derivation: directions enumerate {L,G}x{H,D} on both sides in a fixed order."""
+    names = {(False, False): "LH", (False, True): "LD", (True, False): "GH", (True, True): "GD"}
+    order = ["LH2GH", "LH2GD", "LD2GH", "LD2GD", "GH2GH", "GH2GD", "GH2LH", "GH2LD", "GD2GH", "GD2GD", "GD2LH",
+             "GD2LD"]
+    for s in range(5):
+        for d in range(5):
+            got = oracle.orc_direct_map(s, d)
+            if s == 4 or d == 4 or (s < 2 and d < 2):
+                assert got == 13
+            else:
+                assert got == order.index(names[_endpoint(s)] + "2" + names[_endpoint(d)])
+    assert oracle.orc_direct_map(5, 0) == 13 and oracle.orc_direct_map(0, -1) == 13
+
+
+def test_infer_table_equals_direct_map_under_category_renaming(oracle):
+    # categories GLOBAL_DEVICE 0, GLOBAL_HOST 1, LOCAL_DEVICE 2, LOCAL_HOST 3 <-> smem types 2, 3, 0, 1
+    to_smem = {0: 2, 1: 3, 2: 0, 3: 1}
+    for s in range(4):
+        for d in range(4):
+            assert oracle.orc_infer_table(s, d) == oracle.orc_direct_map(to_smem[s], to_smem[d])
+
+
+def test_check_map_means_pool_side(oracle):
+    for direction in range(12):
+        name = ["LH2GH", "LH2GD", "LD2GH", "LD2GD", "GH2GH", "GH2GD", "GH2LH", "GH2LD", "GD2GH", "GD2GD", "GD2LH",
+                "GD2LD"][direction]
+        src, dst = name.split("2")
+        assert oracle.orc_check_map(direction, 1) == (1 if src[0] == "G" else 0)
+        assert oracle.orc_check_map(direction, 2) == (1 if dst[0] == "G" else 0)
+    assert oracle.orc_check_map(12, 1) == 0
+
+
+def test_trans_direction_overrides(oracle):
+    GD2GD, LD2GD, GD2LD, GD2LH, LH2GD, LH2GH, GH2LH, BUTT = 9, 3, 11, 10, 1, 0, 6, 13
+    DEVICE, HOST, OUT = 2, 3, 4
+    assert oracle.orc_trans_direction(8, DEVICE, DEVICE) == GD2GD
+    assert oracle.orc_trans_direction(0, OUT, DEVICE) == LD2GD      # L2G forces a local-device source
+    assert oracle.orc_trans_direction(1, DEVICE, OUT) == GD2LD      # G2L forces a local-device destination
+    assert oracle.orc_trans_direction(2, DEVICE, OUT) == GD2LH      # G2H
+    assert oracle.orc_trans_direction(3, OUT, DEVICE) == LH2GD      # H2G
+    assert oracle.orc_trans_direction(7, OUT, HOST) == LH2GH        # H2GH
+    assert oracle.orc_trans_direction(6, HOST, OUT) == GH2LH        # GH2H
+    # L2GH and GH2L do not override anything: a side outside the pool stays unclassifiable
+    assert oracle.orc_trans_direction(4, OUT, HOST) == BUTT
+    assert oracle.orc_trans_direction(5, HOST, OUT) == BUTT
+    assert oracle.orc_trans_direction(8, OUT, DEVICE) == BUTT
+
+
+# ---- window arithmetic -------------------------------------------------------------
+def test_gva_window_brute_force(oracle):
+    base, per, ranks = 0x1000, 0x100, 4
+    end = base + per * ranks
+    for addr in range(base - 3, end + 4):
+        for size in (0, 1, 2, 0x100, 0x400):
+            expect = 1 if (addr >= base and addr + size <= end) else 0
+            assert oracle.orc_gva_contains(base, per, ranks, addr, size) == expect
+        expect_rank = (addr - base) // 0x100 if base <= addr and addr + 1 <= end else 0xFFFFFFFF
+        assert oracle.orc_gva_rank(base, per, ranks, 0x100, addr) == expect_rank
+    assert oracle.orc_gva_contains(0, per, ranks, 0x1000, 1) == 0
+    assert oracle.orc_gva_ptr_of_rank(base, per, 3) == base + 0x300
+    # rank divisor and window stride are independent inputs
+    assert oracle.orc_gva_rank(base, 0x100, 4, 0x80, base + 0x17f) == 2
+    assert oracle.orc_operator_rank(base + 0x3ff, base, 0x100, 4) == 3
+    assert oracle.orc_operator_rank(base + 0x400, base, 0x100, 4) == 0xFFFFFFFF
+    assert oracle.orc_operator_rank(base - 1, base, 0x100, 4) == 0xFFFFFFFF
+
+
+def test_mask48(oracle):
+    for a in (0, 1, 0xFFFF_FFFF_FFFF, 0x1_0000_0000_0000, 0xABCD_1234_5678_9ABC, 2**64 - 1):
+        assert oracle.orc_mask48(a) == a % (1 << 48)
+        if oracle_lib.reference() is not None:
+            assert oracle_lib.reference().ref_mask48(a) == a % (1 << 48)
+
+
+# ---- descriptor merge --------------------------------------------------------------------
+def test_coalesce_preserves_bytes(oracle):
+    rng = np.random.default_rng(5)
+    pool = 1 << 16
+    src = rng.integers(0, 256, pool, dtype=np.uint8)
+    # build runs of adjacent segments separated by gaps
+    s_off, d_off, lens = [], [], []
+    s, d = 0, 100
+    for _ in range(60):
+        l = int(rng.integers(0, 300))
+        if rng.random() < 0.4:
+            s += int(rng.integers(1, 50))
+            d += int(rng.integers(1, 50))
+        s_off.append(s)
+        d_off.append(d)
+        lens.append(l)
+        s += l
+        d += l
+    n = len(lens)
+    out = (ctypes.c_uint64 * (3 * n))()
+    k = oracle.orc_coalesce(u64_array(s_off), u64_array(d_off), u64_array(lens), n, out)
+    assert 0 < k < n
+    a = np.zeros(pool, dtype=np.uint8)
+    b = np.zeros(pool, dtype=np.uint8)
+    for so, do, l in zip(s_off, d_off, lens):
+        a[do:do + l] = src[so:so + l]
+    for i in range(k):
+        so, do, l = out[3 * i], out[3 * i + 1], out[3 * i + 2]
+        b[do:do + l] = src[so:so + l]
+    assert np.array_equal(a, b)
+    assert sum(out[3 * i + 2] for i in range(k)) == sum(lens)
+
+
+# ---- the reference kernels' partition, for the record ------------------------------------------
+def test_reference_kernel_partition_properties(oracle):
+    b, e = ctypes.c_uint64(), ctypes.c_uint64()
+    for length in (1, 127, 128, 129, 4096, 131072, 1 << 30):
+        covered = 0
+        for idx in range(32):
+            oracle.orc_ref_kernel_single_range(length, idx, 32, ctypes.byref(b), ctypes.byref(e))
+            if b.value < length:
+                assert b.value == covered and b.value % 128 == 0
+                covered = e.value
+        assert covered == length
+    # short copies: trailing blocks start beyond the end (begin > end), the wrap the HIP kernels avoid
+    oracle.orc_ref_kernel_single_range(128, 5, 32, ctypes.byref(b), ctypes.byref(e))
+    assert b.value > e.value
+    bb, ee = ctypes.c_uint32(), ctypes.c_uint32()
+    seen = []
+    for idx in range(32):
+        oracle.orc_ref_kernel_batch_range(122, idx, 32, ctypes.byref(bb), ctypes.byref(ee))
+        seen.extend(range(bb.value, ee.value))
+    assert seen == list(range(122))
+    oracle.orc_ref_kernel_batch_range(122, 0, 32, ctypes.byref(bb), ctypes.byref(ee))
+    assert ee.value - bb.value == 4  # whole segments per block whatever their length
+
+
+# ---- MoE specification ------------------------------------------------------------------------
+def _route(oracle, logits, k):
+    t, e = logits.shape
+    topk = np.zeros((t, k), dtype=np.int32)
+    w = np.zeros((t, k), dtype=np.float32)
+    oracle.orc_moe_route(np_ptr(logits), t, e, k, np_ptr(topk), np_ptr(w))
+    return topk, w
+
+
+def test_route_is_topk_with_softmax(oracle):
+    rng = np.random.default_rng(6)
+    logits = rng.standard_normal((50, 32), dtype=np.float32)
+    logits[3, 5] = logits[3, 9] = 10.0  # a tie: the lower expert id comes first
+    topk, w = _route(oracle, logits, 4)
+    order = np.argsort(-logits, axis=1, kind="stable")[:, :4]
+    assert np.array_equal(topk, order)
+    assert topk[3, 0] == 5 and topk[3, 1] == 9
+    sel = np.take_along_axis(logits, order, axis=1).astype(np.float64)
+    soft = np.exp(sel - sel.max(axis=1, keepdims=True))
+    soft /= soft.sum(axis=1, keepdims=True)
+    assert np.allclose(w, soft, rtol=1e-5, atol=1e-7)
+
+
+def test_dispatch_is_a_stable_counting_sort(oracle):
+    rng = np.random.default_rng(7)
+    T, H, K, E = 300, 24, 4, 16
+    x = rng.integers(0, 65536, (T, H), dtype=np.uint16)
+    topk = np.stack([rng.choice(E, K, replace=False) for _ in range(T)]).astype(np.int32)
+    topk[topk == 11] = 12  # leave one expert empty (duplicates within a token are legal for the sort)
+    out = np.zeros((T * K, H), dtype=np.uint16)
+    counts = np.zeros(E, dtype=np.int32)
+    offsets = np.zeros(E, dtype=np.int32)
+    row_of = np.zeros(T * K, dtype=np.int32)
+    src_of = np.zeros(T * K, dtype=np.int32)
+    assert oracle.orc_moe_dispatch(np_ptr(x), np_ptr(topk), T, H, K, E, np_ptr(out), np_ptr(counts), np_ptr(offsets),
+                                   np_ptr(row_of), np_ptr(src_of)) == 0
+    flat = topk.reshape(-1)
+    assert counts.sum() == T * K and counts[11] == 0
+    assert np.array_equal(counts, np.bincount(flat, minlength=E))
+    assert np.array_equal(offsets, np.concatenate([[0], np.cumsum(counts)[:-1]]))
+    assert sorted(row_of.tolist()) == list(range(T * K))          # a bijection
+    order = np.argsort(flat, kind="stable")                         # textbook stable sort by expert
+    assert np.array_equal(src_of, order)
+    assert np.array_equal(row_of[order], np.arange(T * K))
+    assert np.array_equal(out, x[order // K])
+    bad = topk.copy()
+    bad[0, 0] = E
+    assert oracle.orc_moe_dispatch(np_ptr(x), np_ptr(bad), T, H, K, E, np_ptr(out), np_ptr(counts), np_ptr(offsets),
+                                   np_ptr(row_of), np_ptr(src_of)) == -2
+
+
+def test_combine_special_cases_and_fp64_check(oracle):
+    from memfabric_hybrid_amd.workloads import bf16_words_to_f32, f32_to_bf16_words
+    rng = np.random.default_rng(8)
+    T, H, K = 40, 64, 8
+    rows = f32_to_bf16_words(rng.standard_normal((T * K, H), dtype=np.float32))
+    row_of = rng.permutation(T * K).astype(np.int32)
+    # one-hot weights return the selected row exactly
+    w = np.zeros((T, K), dtype=np.float32)
+    pick = rng.integers(0, K, T)
+    w[np.arange(T), pick] = 1.0
+    y = np.zeros((T, H), dtype=np.uint16)
+    oracle.orc_moe_combine(np_ptr(rows), np_ptr(row_of), np_ptr(w), T, H, K, np_ptr(y))
+    assert np.array_equal(y, rows[row_of.reshape(T, K)[np.arange(T), pick]])
+    # w = 1/8 on eight copies of one row is exact (power-of-two scaling, exact partial sums)
+    same = np.repeat(rows[:T], K, axis=0)
+    ident = np.arange(T * K, dtype=np.int32)
+    w8 = np.full((T, K), 0.125, dtype=np.float32)
+    oracle.orc_moe_combine(np_ptr(same), np_ptr(ident), np_ptr(w8), T, H, K, np_ptr(y))
+    assert np.array_equal(y, rows[:T])
+    # general weights: agree with an fp64 evaluation to bf16 resolution
+    w = rng.random((T, K), dtype=np.float32)
+    oracle.orc_moe_combine(np_ptr(rows), np_ptr(row_of), np_ptr(w), T, H, K, np_ptr(y))
+    vals = bf16_words_to_f32(rows).astype(np.float64)[row_of.reshape(T, K)]      # T, K, H
+    exact = (vals * w.astype(np.float64)[:, :, None]).sum(axis=1)
+    got = bf16_words_to_f32(y).astype(np.float64)
+    assert np.all(np.abs(got - exact) <= np.abs(exact) * 2 ** -8 + 1e-6)
+
+
+def test_bf16_rounding_is_nearest_even(oracle):
+    # combine of a single row with weight 1 exposes the final rounding: feed fp32 sums through K=2
+    from memfabric_hybrid_amd.workloads import f32_to_bf16_words
+    cases = np.array([1.0, 1.00390625, 1.01171875, -2.5, 3.0e38, 1e-40], dtype=np.float32)
+    # numpy restatement used for workload synthesis agrees with the known roundings
+    words = f32_to_bf16_words(cases)
+    assert words[0] == 0x3F80
+    assert words[1] == 0x3F80      # 1 + 2^-8 is a tie -> even (0x3F80)
+    assert words[2] == 0x3F82      # 1 + 3*2^-8 is a tie -> even (0x3F82)
+
+
+def test_fill_random_is_reproducible_and_seed_sensitive(oracle):
+    a = np.zeros(1003, dtype=np.uint8)
+    b = np.zeros(1003, dtype=np.uint8)
+    c = np.zeros(1003, dtype=np.uint8)
+    oracle.orc_fill_random(np_ptr(a), a.nbytes, 0xC1)
+    oracle.orc_fill_random(np_ptr(b), b.nbytes, 0xC1)
+    oracle.orc_fill_random(np_ptr(c), c.nbytes, 0xC2)
+    assert np.array_equal(a, b) and not np.array_equal(a, c)
+    # splitmix64, first output for seed 0 (published test vector)
+    z = np.zeros(8, dtype=np.uint8)
+    oracle.orc_fill_random(np_ptr(z), 8, 0)
+    assert int.from_bytes(z.tobytes(), "little") == 0xE220A8397B1DCDAF
+    hist = np.bincount(a, minlength=256)
+    assert hist.max() < 20
