@@ -36,6 +36,11 @@ int32_t mf_xcopy_batch(const uint64_t *src, const uint64_t *dst, const uint64_t 
 /* Same for a {src,dst,len} triple table that already lives in device memory. */
 int32_t mf_xcopy_device_table(const void *triples, uint32_t n, int32_t route, void *stream);
 
+/* The stream copies of the calling thread run on when the caller passes none
+ * (the per-thread stream of the reference's HybmStreamManager,
+ * src/hybm/csrc/ts_engine/hybm_stream_manager.cpp:73-90).  NULL before init. */
+void *mf_xcopy_thread_stream(void);
+
 /* Launch-shape knobs.  units: 16-byte units per workgroup chunk (0 = choose
  * per batch); wgPerCu / wgPerCuLink: resident workgroups per CU for HBM and
  * host-link routes (0 = keep). */

@@ -30,6 +30,12 @@ MF_EXPORT int32_t mf_xcopy_device_table(const void *triples, uint32_t n, int32_t
     return XcopyEngine::Instance().SubmitDeviceTable(triples, n, route, stream, nullptr, 0);
 }
 
+MF_EXPORT void *mf_xcopy_thread_stream(void)
+{
+    XcopyEngine &engine = XcopyEngine::Instance();
+    return engine.Started() ? engine.ThreadStream() : nullptr;
+}
+
 MF_EXPORT int32_t mf_xcopy_tune(uint32_t units, uint32_t wgPerCu, uint32_t wgPerCuLink)
 {
     XcopyTuning &t = XcopyEngine::Instance().Tuning();

@@ -166,6 +166,7 @@ _SIGNATURES = {
     # mf_hip_dataplane.h
     "mf_xcopy_batch": (i32, [u64p, u64p, u64p, u32, i32, vp]),
     "mf_xcopy_device_table": (i32, [vp, u32, i32, vp]),
+    "mf_xcopy_thread_stream": (vp, []),
     "mf_xcopy_tune": (i32, [u32, u32, u32]),
     "mf_xcopy_choose_units": (u32, [u64, u32, i32]),
     "mf_xcopy_launch_count": (u64, []),
