@@ -23,6 +23,8 @@ extern "C" {
 #define MF_ROUTE_HBM 0
 #define MF_ROUTE_TO_HOST 1
 #define MF_ROUTE_FROM_HOST 2
+#define MF_ROUTE_HBM_CACHED 3  /* HBM to HBM through the caches, for data that is re-read soon */
+#define MF_ROUTE_HBM_THROUGH 4 /* HBM to HBM, destination written through while the copy runs */
 
 /* Enqueue `n` independent copies dst[i][0..len[i]) = src[i][0..len[i]) as one
  * fused launch on `stream` (NULL: the calling thread's stream).  This is the

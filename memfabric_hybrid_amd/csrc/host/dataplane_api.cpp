@@ -16,7 +16,7 @@ using namespace mf;
 MF_EXPORT int32_t mf_xcopy_batch(const uint64_t *src, const uint64_t *dst, const uint64_t *len, uint32_t n,
                                  int32_t route, void *stream)
 {
-    if ((n != 0 && (src == nullptr || dst == nullptr || len == nullptr)) || route < 0 || route > MF_ROUTE_FROM_HOST) {
+    if ((n != 0 && (src == nullptr || dst == nullptr || len == nullptr)) || route < 0 || route > MF_ROUTE_HBM_THROUGH) {
         MF_FAIL(BM_INVALID_PARAM, "mf_xcopy_batch: null array or unknown route " << route);
     }
     return XcopyEngine::Instance().Submit(src, dst, len, n, route, stream, nullptr, 0);
@@ -24,7 +24,7 @@ MF_EXPORT int32_t mf_xcopy_batch(const uint64_t *src, const uint64_t *dst, const
 
 MF_EXPORT int32_t mf_xcopy_device_table(const void *triples, uint32_t n, int32_t route, void *stream)
 {
-    if ((n != 0 && triples == nullptr) || route < 0 || route > MF_ROUTE_FROM_HOST) {
+    if ((n != 0 && triples == nullptr) || route < 0 || route > MF_ROUTE_HBM_THROUGH) {
         MF_FAIL(BM_INVALID_PARAM, "mf_xcopy_device_table: null table or unknown route " << route);
     }
     return XcopyEngine::Instance().SubmitDeviceTable(triples, n, route, stream, nullptr, 0);
@@ -95,17 +95,12 @@ MF_EXPORT int64_t mf_xcopy_describe_plan(const uint64_t *src, const uint64_t *ds
             ++seg;
         }
         if (fits) {
-            // the inline lookup must agree with the table prefix
-            uint32_t hi = 0;
-            for (uint32_t i = 1; i < kInlineCoarse; ++i) {
-                hi += plan.coarse[i] <= c ? 1u : 0u;
+            // the inline lookup (count of rows whose prefix is <= c, minus one) must agree with the table prefix
+            uint32_t below = 0;
+            for (uint32_t i = 0; i < kInlineSegs; ++i) {
+                below += plan.first[i] <= c ? 1u : 0u;
             }
-            uint32_t s2 = hi * kInlineFan;
-            const uint32_t base = s2;
-            for (uint32_t j = 1; j < kInlineFan; ++j) {
-                s2 += plan.first[base + j] <= c ? 1u : 0u;
-            }
-            if (s2 != seg) {
+            if (below - 1 != seg) {
                 return -1;
             }
         }

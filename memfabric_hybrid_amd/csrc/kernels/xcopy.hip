@@ -6,14 +6,17 @@
 // segments per block, one 64 KiB staging tile, load and store serialised).
 // Here a workgroup owns a chunk of bytes, not a segment; data goes
 // register-to-register with four 128-bit loads in flight per lane, and
-// the descriptor lookup costs two scalar loads from the kernel-argument
-// block for batches of up to 128 segments.
+// the descriptor lookup costs one memory round trip (the table comes out of
+// the kernel-argument block into registers, two rows per lane) for batches
+// of up to 128 segments.
 //
 // Bound: HBM bandwidth (2 bytes of traffic per payload byte) for device to
 // device, the host link (1 byte per payload byte) when one side is pinned
 // host memory.  No LDS, no MFMA: nothing here is reused or contracted.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+
+#include <type_traits>
 
 #include "xcopy_plan.h"
 #include "../rt/mf_rt.h"
@@ -30,28 +33,40 @@ typedef MF_GLOBAL u32x4 *GDstUnit;
 typedef const MF_GLOBAL uint8_t *GSrcByte;
 typedef MF_GLOBAL uint8_t *GDstByte;
 
-// kRoute selects cache policy only; addressing is identical.
-//   MFRT_ROUTE_HBM        both sides in HBM: streaming loads and stores
-//   MFRT_ROUTE_TO_HOST    destination is pinned host DRAM: write-combining friendly nontemporal stores
-//   MFRT_ROUTE_FROM_HOST  source is pinned host DRAM: plain stores into HBM
-template <int kRoute>
+// Cache policy of one launch.  Addressing is the same for all of them.
+//   HBM to HBM          streaming loads and streaming stores (nothing is reused)
+//   to pinned host      plain loads, nontemporal stores (full-line writes for the host link)
+//   from pinned host    streaming loads, plain stores into HBM
+enum StoreMode : int { kStorePlain = 0, kStoreStream = 1, kStoreThrough = 2 };
+
+struct Policy {
+    bool ntLoad;
+    int store;
+};
+
+template <bool kNtLoad>
 __device__ __forceinline__ u32x4 LoadUnit(uint64_t addr)
 {
     GSrcUnit p = reinterpret_cast<GSrcUnit>(addr);
-    if (kRoute == MFRT_ROUTE_TO_HOST) {
-        return *p;
+    if (kNtLoad) {
+        return __builtin_nontemporal_load(p);
     }
-    return __builtin_nontemporal_load(p);
+    return *p;
 }
 
-template <int kRoute>
+// kStoreStream: nontemporal hint, the line may still linger dirty in L2 until the end of the kernel.
+// kStoreThrough: nontemporal and written through at system scope, so that the write-back of the
+// destination overlaps the copy instead of trailing it.
+template <int kStore>
 __device__ __forceinline__ void StoreUnit(uint64_t addr, u32x4 v)
 {
     GDstUnit p = reinterpret_cast<GDstUnit>(addr);
-    if (kRoute == MFRT_ROUTE_FROM_HOST) {
-        *p = v;
-    } else {
+    if (kStore == kStoreThrough) {
+        asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1 nt" : : "v"(p), "v"(v) : "memory");
+    } else if (kStore == kStoreStream) {
         __builtin_nontemporal_store(v, p);
+    } else {
+        *p = v;
     }
 }
 
@@ -64,7 +79,7 @@ constexpr uint32_t kDepth = 4;                          // 128-bit loads in flig
 constexpr uint32_t kTile = kDepth * kXcopyThreads;      // units one workgroup moves per step
 
 // Copy chunk k of one segment.  All arguments are wave-uniform.
-template <int kRoute>
+template <bool kNtLoad, int kStore>
 __device__ __forceinline__ void CopyChunk(uint64_t src, uint64_t dst, uint64_t len, uint64_t k, uint32_t units)
 {
     const SegGeom g = SegmentGeometry(dst, len);
@@ -80,11 +95,11 @@ __device__ __forceinline__ void CopyChunk(uint64_t src, uint64_t dst, uint64_t l
         u32x4 v[kDepth];
 #pragma unroll
         for (uint32_t j = 0; j < kDepth; ++j) {
-            v[j] = LoadUnit<kRoute>(s + static_cast<uint64_t>(i + j * kXcopyThreads + tid) * kUnitBytes);
+            v[j] = LoadUnit<kNtLoad>(s + static_cast<uint64_t>(i + j * kXcopyThreads + tid) * kUnitBytes);
         }
 #pragma unroll
         for (uint32_t j = 0; j < kDepth; ++j) {
-            StoreUnit<kRoute>(d + static_cast<uint64_t>(i + j * kXcopyThreads + tid) * kUnitBytes, v[j]);
+            StoreUnit<kStore>(d + static_cast<uint64_t>(i + j * kXcopyThreads + tid) * kUnitBytes, v[j]);
         }
     }
     if (i < n) {
@@ -93,14 +108,14 @@ __device__ __forceinline__ void CopyChunk(uint64_t src, uint64_t dst, uint64_t l
         for (uint32_t j = 0; j < kDepth; ++j) {
             const uint32_t u = i + j * kXcopyThreads + tid;
             if (u < n) {
-                v[j] = LoadUnit<kRoute>(s + static_cast<uint64_t>(u) * kUnitBytes);
+                v[j] = LoadUnit<kNtLoad>(s + static_cast<uint64_t>(u) * kUnitBytes);
             }
         }
 #pragma unroll
         for (uint32_t j = 0; j < kDepth; ++j) {
             const uint32_t u = i + j * kXcopyThreads + tid;
             if (u < n) {
-                StoreUnit<kRoute>(d + static_cast<uint64_t>(u) * kUnitBytes, v[j]);
+                StoreUnit<kStore>(d + static_cast<uint64_t>(u) * kUnitBytes, v[j]);
             }
         }
     }
@@ -129,31 +144,74 @@ __device__ __forceinline__ void SignalDone(uint64_t *mask, uint32_t value, uint3
     }
 }
 
-template <int kRoute>
+__device__ __forceinline__ uint64_t ReadLane64(uint64_t v, uint32_t lane)
+{
+    const uint32_t lo = __builtin_amdgcn_readlane(static_cast<uint32_t>(v), lane);
+    const uint32_t hi = __builtin_amdgcn_readlane(static_cast<uint32_t>(v >> 32), lane);
+    return (static_cast<uint64_t>(hi) << 32) | lo;
+}
+
+// The plan sits in the kernel-argument block.  Every lane fetches "its" two
+// table rows (rows lane and lane + 64) with loads that depend on nothing but
+// the lane id, so the whole table is in registers after ONE memory round
+// trip; the owner of a chunk is then found with two ballots and read out of
+// the owning lane.  (A scalar search would chain three dependent loads, each
+// a full L2 round trip, before the first byte of payload is requested.)
+template <bool kNtLoad, int kStore>
 __global__ __launch_bounds__(kXcopyThreads) void XcopyInlineKernel(const InlinePlan p, uint64_t *mask, uint32_t maskValue,
                                                                    uint32_t *counter)
 {
-    for (uint32_t c = blockIdx.x; c < p.nchunk; c += gridDim.x) {
-        // Two-level lookup of the segment that owns chunk c: largest s with first[s] <= c.
-        uint32_t hi = 0;
-#pragma unroll
-        for (uint32_t i = 1; i < kInlineCoarse; ++i) {
-            hi += (p.coarse[i] <= c) ? 1u : 0u;
+    const uint32_t lane = threadIdx.x & 63u;
+    const uint32_t f0 = p.first[lane];
+    const uint32_t f1 = p.first[lane + 64];
+    const uint64_t s0 = p.src[lane];
+    const uint64_t s1 = p.src[lane + 64];
+    const uint64_t d0 = p.dst[lane];
+    const uint64_t d1 = p.dst[lane + 64];
+    const uint32_t l0 = p.len[lane];
+    const uint32_t l1 = p.len[lane + 64];
+    const uint32_t nchunk = p.nchunk;
+    const uint32_t units = p.units;
+    // The host launches at most nchunk workgroups (and never this kernel for an empty plan), so
+    // the first chunk needs no bound check and the table loads above are not held behind one.
+    uint32_t c = blockIdx.x;
+    do {
+        // rows are ordered by prefix: the owner is the last row whose prefix is <= c
+        const uint32_t below = __popcll(__ballot(f0 <= c)) + __popcll(__ballot(f1 <= c));
+        const uint32_t s = below - 1;
+        const uint32_t row = s & 63u;
+        uint64_t src;
+        uint64_t dst;
+        uint32_t len;
+        uint32_t first;
+        if (s < 64) {
+            src = ReadLane64(s0, row);
+            dst = ReadLane64(d0, row);
+            len = __builtin_amdgcn_readlane(l0, row);
+            first = __builtin_amdgcn_readlane(f0, row);
+        } else {
+            src = ReadLane64(s1, row);
+            dst = ReadLane64(d1, row);
+            len = __builtin_amdgcn_readlane(l1, row);
+            first = __builtin_amdgcn_readlane(f1, row);
         }
-        const uint32_t base = hi * kInlineFan;
-        uint32_t s = base;
-#pragma unroll
-        for (uint32_t j = 1; j < kInlineFan; ++j) {
-            s += (p.first[base + j] <= c) ? 1u : 0u;
-        }
-        CopyChunk<kRoute>(p.src[s], p.dst[s], p.len[s], c - p.first[s], p.units);
-    }
+        CopyChunk<kNtLoad, kStore>(src, dst, len, c - first, units);
+        c += gridDim.x;
+    } while (c < nchunk);
     if (mask != nullptr) {
         SignalDone(mask, maskValue, counter);
     }
 }
 
-template <int kRoute>
+// An empty batch that still owes its caller a completion word.
+__global__ void XcopySignalKernel(uint64_t *mask, uint32_t maskValue)
+{
+    if (threadIdx.x == 0 && blockIdx.x == 0) {
+        __hip_atomic_store(mask, static_cast<uint64_t>(maskValue), __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+    }
+}
+
+template <bool kNtLoad, int kStore>
 __global__ __launch_bounds__(kXcopyThreads) void XcopyTableKernel(const uint64_t *__restrict__ triples,
                                                                   const uint32_t *__restrict__ first,
                                                                   const uint32_t *__restrict__ nchunkDev, uint32_t nseg,
@@ -174,7 +232,7 @@ __global__ __launch_bounds__(kXcopyThreads) void XcopyTableKernel(const uint64_t
             }
         }
         const uint64_t *t = triples + 3ull * lo;
-        CopyChunk<kRoute>(t[0], t[1], t[2], c - first[lo], units);
+        CopyChunk<kNtLoad, kStore>(t[0], t[1], t[2], c - first[lo], units);
     }
     if (mask != nullptr) {
         SignalDone(mask, maskValue, counter);
@@ -217,21 +275,59 @@ __global__ __launch_bounds__(kPlanThreads) void XcopyPlanKernel(const uint64_t *
     }
 }
 
-template <int kRoute>
+Policy PolicyOf(int route)
+{
+    switch (route) {
+        case MFRT_ROUTE_TO_HOST:
+            return Policy{false, kStoreStream};
+        case MFRT_ROUTE_FROM_HOST:
+            return Policy{true, kStorePlain};
+        case MFRT_ROUTE_HBM_CACHED:
+            return Policy{false, kStorePlain};
+        case MFRT_ROUTE_HBM_THROUGH:
+            return Policy{true, kStoreThrough};
+        default:
+            return Policy{true, kStoreStream};
+    }
+}
+
+// Runs `launch` with the template instance matching a run-time policy.
+template <class Launch>
+int WithPolicy(const Policy &policy, Launch launch)
+{
+    if (policy.ntLoad) {
+        switch (policy.store) {
+            case kStoreThrough:
+                return launch(std::true_type{}, std::integral_constant<int, kStoreThrough>{});
+            case kStoreStream:
+                return launch(std::true_type{}, std::integral_constant<int, kStoreStream>{});
+            default:
+                return launch(std::true_type{}, std::integral_constant<int, kStorePlain>{});
+        }
+    }
+    switch (policy.store) {
+        case kStoreStream:
+            return launch(std::false_type{}, std::integral_constant<int, kStoreStream>{});
+        default:
+            return launch(std::false_type{}, std::integral_constant<int, kStorePlain>{});
+    }
+}
+
+template <bool kNtLoad, int kStore>
 int LaunchInline(const InlinePlan &plan, uint32_t grid, uint64_t *mask, uint32_t maskValue, uint32_t *counter,
                  hipStream_t stream)
 {
-    hipLaunchKernelGGL(XcopyInlineKernel<kRoute>, dim3(grid), dim3(kXcopyThreads), 0, stream, plan, mask, maskValue,
-                       counter);
+    hipLaunchKernelGGL((XcopyInlineKernel<kNtLoad, kStore>), dim3(grid), dim3(kXcopyThreads), 0, stream, plan, mask,
+                       maskValue, counter);
     return static_cast<int>(hipGetLastError());
 }
 
-template <int kRoute>
+template <bool kNtLoad, int kStore>
 int LaunchTable(const TablePlan &plan, const uint32_t *nchunkDev, uint32_t grid, uint64_t *mask, uint32_t maskValue,
                 uint32_t *counter, hipStream_t stream)
 {
-    hipLaunchKernelGGL(XcopyTableKernel<kRoute>, dim3(grid), dim3(kXcopyThreads), 0, stream, plan.triples, plan.first,
-                       nchunkDev, plan.nseg, plan.nchunk, plan.units, mask, maskValue, counter);
+    hipLaunchKernelGGL((XcopyTableKernel<kNtLoad, kStore>), dim3(grid), dim3(kXcopyThreads), 0, stream, plan.triples,
+                       plan.first, nchunkDev, plan.nseg, plan.nchunk, plan.units, mask, maskValue, counter);
     return static_cast<int>(hipGetLastError());
 }
 
@@ -242,25 +338,23 @@ extern "C" int mfk_xcopy_inline(const void *inlinePlan, int route, uint32_t grid
                                 void *counter, void *stream)
 {
     const mf::InlinePlan &plan = *static_cast<const mf::InlinePlan *>(inlinePlan);
-    if (plan.nchunk == 0 && mask == nullptr) {
+    if (plan.nchunk == 0) {
+        if (mask != nullptr) {
+            hipLaunchKernelGGL(mf::XcopySignalKernel, dim3(1), dim3(64), 0, static_cast<hipStream_t>(stream),
+                               static_cast<uint64_t *>(mask), maskValue);
+            return static_cast<int>(hipGetLastError());
+        }
         return 0;
     }
-    if (grid == 0) {
-        grid = 1;
+    if (grid == 0 || grid > plan.nchunk) {
+        grid = plan.nchunk;
     }
     uint64_t *m = static_cast<uint64_t *>(mask);
     uint32_t *c = static_cast<uint32_t *>(counter);
     hipStream_t s = static_cast<hipStream_t>(stream);
-    switch (route) {
-        case MFRT_ROUTE_HBM:
-            return mf::LaunchInline<MFRT_ROUTE_HBM>(plan, grid, m, maskValue, c, s);
-        case MFRT_ROUTE_TO_HOST:
-            return mf::LaunchInline<MFRT_ROUTE_TO_HOST>(plan, grid, m, maskValue, c, s);
-        case MFRT_ROUTE_FROM_HOST:
-            return mf::LaunchInline<MFRT_ROUTE_FROM_HOST>(plan, grid, m, maskValue, c, s);
-        default:
-            return -1;
-    }
+    return mf::WithPolicy(mf::PolicyOf(route), [&](auto ntLoad, auto store) {
+        return mf::LaunchInline<decltype(ntLoad)::value, decltype(store)::value>(plan, grid, m, maskValue, c, s);
+    });
 }
 
 extern "C" int mfk_xcopy_table(const void *triples, const void *first, const void *nchunkDev, uint32_t nseg,
@@ -275,16 +369,9 @@ extern "C" int mfk_xcopy_table(const void *triples, const void *first, const voi
     uint64_t *m = static_cast<uint64_t *>(mask);
     uint32_t *c = static_cast<uint32_t *>(counter);
     hipStream_t s = static_cast<hipStream_t>(stream);
-    switch (route) {
-        case MFRT_ROUTE_HBM:
-            return mf::LaunchTable<MFRT_ROUTE_HBM>(plan, nd, grid, m, maskValue, c, s);
-        case MFRT_ROUTE_TO_HOST:
-            return mf::LaunchTable<MFRT_ROUTE_TO_HOST>(plan, nd, grid, m, maskValue, c, s);
-        case MFRT_ROUTE_FROM_HOST:
-            return mf::LaunchTable<MFRT_ROUTE_FROM_HOST>(plan, nd, grid, m, maskValue, c, s);
-        default:
-            return -1;
-    }
+    return mf::WithPolicy(mf::PolicyOf(route), [&](auto ntLoad, auto store) {
+        return mf::LaunchTable<decltype(ntLoad)::value, decltype(store)::value>(plan, nd, grid, m, maskValue, c, s);
+    });
 }
 
 extern "C" int mfk_xcopy_plan(const void *triples, uint32_t nseg, uint32_t units, void *first, void *nchunk,

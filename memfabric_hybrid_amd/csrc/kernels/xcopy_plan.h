@@ -26,9 +26,7 @@ namespace mf {
 
 constexpr uint32_t kXcopyThreads = 256;       // lanes per workgroup (4 wave64)
 constexpr uint32_t kUnitBytes = 16;           // one 128-bit access
-constexpr uint32_t kInlineSegs = 128;         // segments that fit in the kernel-argument block
-constexpr uint32_t kInlineFan = 8;            // second-level fan-out of the two-level lookup
-constexpr uint32_t kInlineCoarse = kInlineSegs / kInlineFan;  // 16 first-level keys
+constexpr uint32_t kInlineSegs = 128;         // segments that fit in the kernel-argument block: 2 table rows per lane of a wave64
 constexpr uint32_t kNoChunk = 0xFFFFFFFFu;    // sentinel prefix for unused slots
 
 #if defined(__HIPCC__) || defined(__CUDACC__)
@@ -68,14 +66,13 @@ MF_HD inline uint64_t SegmentChunks(uint64_t dst, uint64_t len, uint32_t units)
 }
 
 // Everything a launch of up to kInlineSegs segments needs, passed by value in
-// the kernel-argument block (3144 bytes of the 4096 available): no table
+// the kernel-argument block (3080 bytes of the 4096 available): no table
 // upload, no extra dependent memory round trip before the first data load.
 struct InlinePlan {
     uint64_t src[kInlineSegs];
     uint64_t dst[kInlineSegs];
     uint32_t len[kInlineSegs];          // inline path carries segments < 4 GiB only
     uint32_t first[kInlineSegs];        // exclusive prefix of chunk counts, kNoChunk past the end
-    uint32_t coarse[kInlineCoarse];     // first[kInlineFan * i]
     uint32_t nchunk;
     uint32_t units;                     // 16-byte units per chunk, multiple of kXcopyThreads
 };

@@ -20,6 +20,8 @@ extern "C" {
 #define MFRT_ROUTE_HBM 0        /* source and destination in HBM            */
 #define MFRT_ROUTE_TO_HOST 1    /* destination in pinned, mapped host DRAM  */
 #define MFRT_ROUTE_FROM_HOST 2  /* source in pinned, mapped host DRAM       */
+#define MFRT_ROUTE_HBM_CACHED 3 /* HBM to HBM through the caches (data that is re-read soon) */
+#define MFRT_ROUTE_HBM_THROUGH 4 /* HBM to HBM, destination written through as it is produced */
 
 #define MFRT_PTR_PAGEABLE 0     /* ordinary host memory the GPU cannot address */
 #define MFRT_PTR_DEVICE 1

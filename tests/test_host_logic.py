@@ -156,11 +156,11 @@ def test_plan_splits_segments_the_inline_form_cannot_hold(lib):
 
 
 def test_choose_units_policy(lib):
-    # small batches use the smallest chunk so that every CU gets work; big copies use the largest
+    # latency-bound batches use the smallest chunk, the bulk 16 KiB, multi-GiB copies the largest
     assert lib.mf_xcopy_choose_units(64 * 1024, 256, native.ROUTE_HBM) == 256
-    assert lib.mf_xcopy_choose_units(1 << 30, 256, native.ROUTE_HBM) == 4096
-    mid = lib.mf_xcopy_choose_units(workloads.KV_PAYLOAD, 256, native.ROUTE_HBM)
-    assert mid % 256 == 0 and 256 <= mid <= 1024
+    assert lib.mf_xcopy_choose_units(workloads.KV_PAYLOAD, 256, native.ROUTE_HBM) == 1024
+    assert lib.mf_xcopy_choose_units(1 << 30, 256, native.ROUTE_HBM) == 1024
+    assert lib.mf_xcopy_choose_units(2 << 30, 256, native.ROUTE_HBM) == 4096
 
 
 # ---- error contracts that need no GPU (test/ut/testcase/smem/smem_bm_test.cpp:59-201 of the reference) ----
