@@ -58,6 +58,31 @@ uint64_t mf_xcopy_launch_count(void);
 int64_t mf_xcopy_describe_plan(const uint64_t *src, const uint64_t *dst, const uint64_t *len, uint32_t n,
                                uint32_t units, uint64_t *out, uint64_t capacity, int32_t *inlineForm);
 
+/* ---- local MoE dispatch / combine over pooled memory ------------------------
+ * No reference implementation exists; the specification is the stable counting
+ * sort / fixed-order fp32 FMA chain stated in oracle/mf_oracle.c.  All buffers
+ * are device memory; x, out, rows, y hold 16-bit (bf16) elements, 16-byte
+ * aligned, hidden a multiple of 8; topK <= 16, experts <= 512.
+ *
+ * dispatch: x[tokens][hidden], topk[tokens][topK] expert ids ->
+ *   counts[experts], offsets[experts] (exclusive scan of counts),
+ *   rowOf[tokens*topK] (destination row of entry t*topK+k, -1 for an id outside
+ *   [0, experts)), srcOf[tokens*topK] (inverse, may be NULL),
+ *   out[tokens*topK][hidden] expert-contiguous (x and out may both be NULL to
+ *   compute the permutation only).
+ * workspace: mf_moe_workspace_bytes() bytes of device memory, no initialisation
+ *   needed; after the stream has drained its first uint32 is 1 if any expert id
+ *   was out of range.  Enqueues on `stream` (NULL: thread stream), does not wait. */
+uint64_t mf_moe_workspace_bytes(uint32_t tokens, uint32_t topK, uint32_t experts);
+int32_t mf_moe_dispatch(const void *x, const int32_t *topk, uint32_t tokens, uint32_t hidden, uint32_t topK,
+                        uint32_t experts, void *out, int32_t *counts, int32_t *offsets, int32_t *rowOf, int32_t *srcOf,
+                        void *workspace, uint64_t workspaceBytes, void *stream);
+/* combine: y[t][h] = bf16(sum_k weights[t][k] * rows[rowOf[t*topK+k]][h]), fp32
+ * fused multiply-add in slot order k = 0..topK-1 starting from 0, one final
+ * round-to-nearest-even; entries with rowOf < 0 contribute nothing. */
+int32_t mf_moe_combine(const void *rows, const int32_t *rowOf, const float *weights, uint32_t tokens, uint32_t hidden,
+                       uint32_t topK, void *y, void *stream);
+
 /* ---- runtime services (thin layer over HIP) ------------------------------ */
 int mfrt_init(int device);
 void mfrt_shutdown(void);

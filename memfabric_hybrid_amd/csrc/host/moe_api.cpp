@@ -1,0 +1,91 @@
+// Native C entry points of the local MoE dispatch / combine (declared in
+// include/mf_hip_dataplane.h).
+#include "../../../include/mf_hip_dataplane.h"
+#include "../../../include/mf_xcopy_types.h"
+#include "../rt/mf_rt.h"
+#include "mf_log.h"
+#include "xcopy_engine.h"
+
+using namespace mf;
+
+#define MF_EXPORT extern "C" __attribute__((visibility("default")))
+
+namespace {
+
+int Prepare(void *&stream)
+{
+    XcopyEngine &engine = XcopyEngine::Instance();
+    if (!engine.Started()) {
+        MF_FAIL(BM_NOT_INITIALIZED, "GPU data plane is not running; call hybm_init first");
+    }
+    if (mfrt_bind_thread() != 0) {
+        MF_FAIL(BM_ERROR, "cannot make the GPU current on this thread");
+    }
+    if (stream == nullptr) {
+        stream = engine.ThreadStream();
+        if (stream == nullptr) {
+            MF_FAIL(BM_ERROR, "cannot create the thread's stream");
+        }
+    }
+    return BM_OK;
+}
+
+}  // namespace
+
+MF_EXPORT uint64_t mf_moe_workspace_bytes(uint32_t tokens, uint32_t topK, uint32_t experts)
+{
+    return mfk_moe_workspace_bytes(tokens, topK, experts);
+}
+
+MF_EXPORT int32_t mf_moe_dispatch(const void *x, const int32_t *topk, uint32_t tokens, uint32_t hidden, uint32_t topK,
+                                  uint32_t experts, void *out, int32_t *counts, int32_t *offsets, int32_t *rowOf,
+                                  int32_t *srcOf, void *workspace, uint64_t workspaceBytes, void *stream)
+{
+    if (topk == nullptr || counts == nullptr || offsets == nullptr || rowOf == nullptr || workspace == nullptr ||
+        tokens == 0 || topK == 0 || experts == 0 || (x == nullptr) != (out == nullptr)) {
+        MF_FAIL(BM_INVALID_PARAM, "mf_moe_dispatch: null argument or empty problem");
+    }
+    if (topK > 16 || experts > 512 || (out != nullptr && (hidden == 0 || hidden % 8 != 0))) {
+        MF_FAIL(BM_INVALID_PARAM, "mf_moe_dispatch: needs topK <= 16, experts <= 512 and hidden a multiple of 8, got "
+                                      << topK << ", " << experts << ", " << hidden);
+    }
+    if ((reinterpret_cast<uint64_t>(x) | reinterpret_cast<uint64_t>(out)) % 16 != 0) {
+        MF_FAIL(BM_INVALID_PARAM, "mf_moe_dispatch: token buffers must be 16-byte aligned");
+    }
+    if (workspaceBytes < mfk_moe_workspace_bytes(tokens, topK, experts)) {
+        MF_FAIL(BM_INVALID_PARAM, "mf_moe_dispatch: workspace of " << workspaceBytes << " bytes is too small");
+    }
+    int ret = Prepare(stream);
+    if (ret != BM_OK) {
+        return ret;
+    }
+    int err = mfk_moe_dispatch(x, topk, tokens, hidden, topK, experts, out, counts, offsets, rowOf, srcOf, workspace,
+                               stream);
+    if (err != 0) {
+        MF_FAIL(BM_ERROR, "mf_moe_dispatch: launch failed: " << (err > 0 ? mfrt_error_string(err) : "bad shape"));
+    }
+    return BM_OK;
+}
+
+MF_EXPORT int32_t mf_moe_combine(const void *rows, const int32_t *rowOf, const float *weights, uint32_t tokens,
+                                 uint32_t hidden, uint32_t topK, void *y, void *stream)
+{
+    if (rows == nullptr || rowOf == nullptr || weights == nullptr || y == nullptr || tokens == 0 || topK == 0) {
+        MF_FAIL(BM_INVALID_PARAM, "mf_moe_combine: null argument or empty problem");
+    }
+    if (topK > 16 || hidden == 0 || hidden % 8 != 0) {
+        MF_FAIL(BM_INVALID_PARAM, "mf_moe_combine: needs topK <= 16 and hidden a multiple of 8");
+    }
+    if ((reinterpret_cast<uint64_t>(rows) | reinterpret_cast<uint64_t>(y)) % 16 != 0) {
+        MF_FAIL(BM_INVALID_PARAM, "mf_moe_combine: row buffers must be 16-byte aligned");
+    }
+    int ret = Prepare(stream);
+    if (ret != BM_OK) {
+        return ret;
+    }
+    int err = mfk_moe_combine(rows, rowOf, weights, tokens, hidden, topK, y, stream);
+    if (err != 0) {
+        MF_FAIL(BM_ERROR, "mf_moe_combine: launch failed: " << (err > 0 ? mfrt_error_string(err) : "bad shape"));
+    }
+    return BM_OK;
+}

@@ -1,0 +1,387 @@
+// Local MoE token dispatch / combine for gfx950.
+//
+// The reference has no counterpart (its only device code is the copy plugin,
+// src/hybm/csrc/copy_extend/hybm_copy_kernel.cpp); the arithmetic these kernels
+// are held to is the specification in the test oracle:
+//   dispatch  entry i = t*K + k goes to row offsets[e] + #{j < i : topk[j] == e}
+//             (a stable counting sort of the flat (t,k) order by expert id)
+//   combine   y[t][h] = bf16_rne(fma(w[t][K-1], v[K-1], ... fma(w[t][0], v[0], 0)))
+//
+// Three launches for dispatch, one for combine:
+//   MoeHistKernel    per-block expert histograms (wave ballots + LDS)
+//   MoeRankKernel    cross-block scan, stable rank of every entry -> rowOf/srcOf, counts, offsets
+//   MoePermuteKernel one workgroup per token: the row is read once into registers and
+//                    stored to its K destination rows (HBM bound: H*2*(1+K) bytes per token)
+//   MoeCombineKernel one workgroup per token: K rows gathered, fp32 FMA chain in slot
+//                    order, one rounding to bf16 (HBM bound: H*2*(K+1) bytes per token)
+// Ranks come from ballots and prefix sums, never from atomics on a shared
+// cursor, so the permutation is the same on every run and equals the CPU sort.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../rt/mf_rt.h"
+
+namespace mf {
+namespace {
+
+constexpr uint32_t kRankThreads = 256;                 // 4 waves
+constexpr uint32_t kRankRounds = 4;                    // entries per lane
+constexpr uint32_t kRankBlock = kRankThreads * kRankRounds;  // 1024 entries per workgroup
+constexpr uint32_t kRankSlices = kRankBlock / 64;      // 16 wave-sized slices, in entry order
+constexpr uint32_t kMaxExperts = 512;
+constexpr uint32_t kRowThreads = 256;
+constexpr uint32_t kMaxTopK = 16;
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+#define MF_GLOBAL __attribute__((address_space(1)))
+
+// Lanes of the wave whose expert id equals mine (among lanes with valid == true).
+__device__ __forceinline__ uint64_t PeersOf(uint32_t expert, bool valid, uint32_t bits)
+{
+    uint64_t peers = __ballot(valid);
+    for (uint32_t b = 0; b < bits; ++b) {
+        const bool bit = (expert >> b) & 1u;
+        const uint64_t vote = __ballot(bit);
+        peers &= bit ? vote : ~vote;
+    }
+    return peers;
+}
+
+__device__ __forceinline__ uint32_t BitsFor(uint32_t experts)
+{
+    return 32u - __builtin_clz(experts > 1 ? experts - 1 : 1u);
+}
+
+// Slice s of a block holds entries [block*1024 + s*64, +64), lane = offset in the slice.
+// Wave w of the workgroup handles slices w, w+4, w+8, w+12.
+// hist[s][e] = number of entries of slice s routed to expert e.
+__device__ __forceinline__ void SliceHistograms(const int32_t *__restrict__ topk, uint32_t total, uint32_t experts,
+                                                uint32_t blockBase, uint32_t *hist /* [kRankSlices][experts] in LDS */,
+                                                uint32_t *myExpert, uint32_t *myRank, uint32_t *bad)
+{
+    const uint32_t lane = threadIdx.x & 63u;
+    const uint32_t wave = threadIdx.x >> 6;
+    const uint32_t bits = BitsFor(experts);
+    for (uint32_t i = threadIdx.x; i < kRankSlices * experts; i += kRankThreads) {
+        hist[i] = 0;
+    }
+    __syncthreads();
+#pragma unroll
+    for (uint32_t r = 0; r < kRankRounds; ++r) {
+        const uint32_t slice = wave + r * (kRankThreads / 64);
+        const uint32_t idx = blockBase + slice * 64 + lane;
+        int32_t e = -1;
+        if (idx < total) {
+            e = topk[idx];
+        }
+        const bool valid = e >= 0 && static_cast<uint32_t>(e) < experts;
+        if (idx < total && !valid) {
+            *bad = 1;
+        }
+        const uint64_t peers = PeersOf(static_cast<uint32_t>(e), valid, bits);
+        const uint64_t below = peers & ((1ull << lane) - 1ull);
+        myExpert[r] = valid ? static_cast<uint32_t>(e) : 0xFFFFFFFFu;
+        myRank[r] = __popcll(below);
+        if (valid && below == 0) {  // first lane of each group publishes the group's size
+            hist[slice * experts + static_cast<uint32_t>(e)] = __popcll(peers);
+        }
+    }
+    __syncthreads();
+}
+
+__global__ __launch_bounds__(kRankThreads) void MoeHistKernel(const int32_t *__restrict__ topk, uint32_t total,
+                                                              uint32_t experts, uint32_t *__restrict__ blockHist,
+                                                              uint32_t *__restrict__ blockBad)
+{
+    extern __shared__ uint32_t hist[];
+    uint32_t e[kRankRounds];
+    uint32_t r[kRankRounds];
+    uint32_t bad = 0;
+    SliceHistograms(topk, total, experts, blockIdx.x * kRankBlock, hist, e, r, &bad);
+    for (uint32_t x = threadIdx.x; x < experts; x += kRankThreads) {
+        uint32_t sum = 0;
+        for (uint32_t s = 0; s < kRankSlices; ++s) {
+            sum += hist[s * experts + x];
+        }
+        blockHist[static_cast<uint64_t>(blockIdx.x) * experts + x] = sum;
+    }
+    // every block reports, so the flags need no clearing between calls
+    const uint32_t anyBad = __syncthreads_or(static_cast<int>(bad)) != 0 ? 1u : 0u;
+    if (threadIdx.x == 0) {
+        blockBad[blockIdx.x] = anyBad;
+    }
+}
+
+__global__ __launch_bounds__(kRankThreads) void MoeRankKernel(const int32_t *__restrict__ topk, uint32_t total,
+                                                              uint32_t experts, const uint32_t *__restrict__ blockHist,
+                                                              int32_t *__restrict__ counts, int32_t *__restrict__ offsets,
+                                                              int32_t *__restrict__ rowOf, int32_t *__restrict__ srcOf,
+                                                              const uint32_t *__restrict__ blockBad,
+                                                              uint32_t *__restrict__ status)
+{
+    extern __shared__ uint32_t lds[];
+    uint32_t *hist = lds;                                 // [kRankSlices][experts]
+    uint32_t *base = lds + kRankSlices * experts;         // [experts] first row of this block's entries per expert
+    uint32_t *scan = base + experts;                      // [kRankThreads] scratch of the block scan
+    uint32_t myExpert[kRankRounds];
+    uint32_t myRank[kRankRounds];
+    uint32_t bad = 0;
+    SliceHistograms(topk, total, experts, blockIdx.x * kRankBlock, hist, myExpert, myRank, &bad);
+
+    if (blockIdx.x == 0 && threadIdx.x == 0) {
+        uint32_t any = 0;
+        for (uint32_t blk = 0; blk < gridDim.x; ++blk) {
+            any |= blockBad[blk];
+        }
+        status[0] = any;  // 1: some expert id was outside [0, experts); those entries got row -1
+    }
+    // totals and "entries of earlier blocks" per expert
+    uint32_t tot[kMaxExperts / kRankThreads];
+    uint32_t before[kMaxExperts / kRankThreads];
+    uint32_t mine = 0;
+#pragma unroll
+    for (uint32_t j = 0; j < kMaxExperts / kRankThreads; ++j) {
+        // thread t owns the contiguous experts t*per .. t*per+per-1 so that a scan over threads is a scan over experts
+        tot[j] = 0;
+        before[j] = 0;
+    }
+    const uint32_t per = (experts + kRankThreads - 1) / kRankThreads;  // 1 or 2
+    for (uint32_t j = 0; j < per; ++j) {
+        const uint32_t x = threadIdx.x * per + j;
+        if (x < experts) {
+            uint32_t t = 0;
+            uint32_t b = 0;
+            for (uint32_t blk = 0; blk < gridDim.x; ++blk) {
+                const uint32_t v = blockHist[static_cast<uint64_t>(blk) * experts + x];
+                t += v;
+                b += blk < blockIdx.x ? v : 0u;
+            }
+            tot[j] = t;
+            before[j] = b;
+            mine += t;
+        }
+    }
+    // exclusive scan of `mine` over the 256 threads
+    scan[threadIdx.x] = mine;
+    __syncthreads();
+    for (uint32_t step = 1; step < kRankThreads; step <<= 1) {
+        const uint32_t add = threadIdx.x >= step ? scan[threadIdx.x - step] : 0u;
+        __syncthreads();
+        scan[threadIdx.x] += add;
+        __syncthreads();
+    }
+    uint32_t run = scan[threadIdx.x] - mine;
+    for (uint32_t j = 0; j < per; ++j) {
+        const uint32_t x = threadIdx.x * per + j;
+        if (x < experts) {
+            if (blockIdx.x == 0) {
+                counts[x] = static_cast<int32_t>(tot[j]);
+                offsets[x] = static_cast<int32_t>(run);
+            }
+            base[x] = run + before[j];
+            run += tot[j];
+        }
+    }
+    __syncthreads();
+    // turn slice histograms into exclusive prefixes over the slices of this block
+    for (uint32_t x = threadIdx.x; x < experts; x += kRankThreads) {
+        uint32_t acc = base[x];
+        for (uint32_t s = 0; s < kRankSlices; ++s) {
+            const uint32_t v = hist[s * experts + x];
+            hist[s * experts + x] = acc;
+            acc += v;
+        }
+    }
+    __syncthreads();
+    const uint32_t lane = threadIdx.x & 63u;
+    const uint32_t wave = threadIdx.x >> 6;
+#pragma unroll
+    for (uint32_t r = 0; r < kRankRounds; ++r) {
+        const uint32_t slice = wave + r * (kRankThreads / 64);
+        const uint32_t idx = blockIdx.x * kRankBlock + slice * 64 + lane;
+        if (idx < total) {
+            int32_t row = -1;
+            if (myExpert[r] != 0xFFFFFFFFu) {
+                row = static_cast<int32_t>(hist[slice * experts + myExpert[r]] + myRank[r]);
+                if (srcOf != nullptr) {
+                    srcOf[row] = static_cast<int32_t>(idx);
+                }
+            }
+            rowOf[idx] = row;
+        }
+    }
+}
+
+// One workgroup per token.  unitsPerRow = H*2/16.
+__global__ __launch_bounds__(kRowThreads) void MoePermuteKernel(const u32x4 *__restrict__ x,
+                                                                const int32_t *__restrict__ rowOf, uint32_t topK,
+                                                                uint32_t unitsPerRow, u32x4 *__restrict__ out)
+{
+    const uint32_t token = blockIdx.x;
+    const MF_GLOBAL u32x4 *src = reinterpret_cast<const MF_GLOBAL u32x4 *>(reinterpret_cast<uint64_t>(x)) + static_cast<uint64_t>(token) * unitsPerRow;
+    int32_t rows[kMaxTopK];
+#pragma unroll
+    for (uint32_t k = 0; k < kMaxTopK; ++k) {
+        rows[k] = k < topK ? rowOf[static_cast<uint64_t>(token) * topK + k] : -1;
+    }
+    for (uint32_t u0 = 0; u0 < unitsPerRow; u0 += 4 * kRowThreads) {
+        u32x4 v[4];
+#pragma unroll
+        for (uint32_t j = 0; j < 4; ++j) {
+            const uint32_t u = u0 + j * kRowThreads + threadIdx.x;
+            if (u < unitsPerRow) {
+                v[j] = __builtin_nontemporal_load(src + u);
+            }
+        }
+#pragma unroll
+        for (uint32_t k = 0; k < kMaxTopK; ++k) {
+            if (k < topK && rows[k] >= 0) {
+                MF_GLOBAL u32x4 *dst =
+                    reinterpret_cast<MF_GLOBAL u32x4 *>(reinterpret_cast<uint64_t>(out)) + static_cast<uint64_t>(rows[k]) * unitsPerRow;
+#pragma unroll
+                for (uint32_t j = 0; j < 4; ++j) {
+                    const uint32_t u = u0 + j * kRowThreads + threadIdx.x;
+                    if (u < unitsPerRow) {
+                        __builtin_nontemporal_store(v[j], dst + u);
+                    }
+                }
+            }
+        }
+    }
+}
+
+__device__ __forceinline__ float Bf16Lo(uint32_t w)
+{
+    return __uint_as_float(w << 16);
+}
+
+__device__ __forceinline__ float Bf16Hi(uint32_t w)
+{
+    return __uint_as_float(w & 0xFFFF0000u);
+}
+
+// round to nearest even; NaN stays a quiet NaN
+__device__ __forceinline__ uint32_t ToBf16(float f)
+{
+    const uint32_t w = __float_as_uint(f);
+    if ((w & 0x7FFFFFFFu) > 0x7F800000u) {
+        return (w >> 16) | 0x0040u;
+    }
+    return (w + 0x7FFFu + ((w >> 16) & 1u)) >> 16;
+}
+
+template <uint32_t kTopK>
+__global__ __launch_bounds__(kRowThreads) void MoeCombineKernel(const u32x4 *__restrict__ rowsIn,
+                                                                const int32_t *__restrict__ rowOf,
+                                                                const float *__restrict__ weights, uint32_t topK,
+                                                                uint32_t unitsPerRow, u32x4 *__restrict__ y)
+{
+    const uint32_t token = blockIdx.x;
+    const uint32_t nk = kTopK != 0 ? kTopK : topK;
+    constexpr uint32_t kSlots = kTopK != 0 ? kTopK : kMaxTopK;
+    uint64_t rowBase[kSlots];
+    float w[kSlots];
+#pragma unroll
+    for (uint32_t k = 0; k < kSlots; ++k) {
+        if (k < nk) {
+            const int32_t row = rowOf[static_cast<uint64_t>(token) * nk + k];
+            rowBase[k] = static_cast<uint64_t>(row < 0 ? 0 : row) * unitsPerRow;
+            w[k] = row < 0 ? 0.0f : weights[static_cast<uint64_t>(token) * nk + k];
+        } else {
+            rowBase[k] = 0;
+            w[k] = 0.0f;
+        }
+    }
+    const MF_GLOBAL u32x4 *in = reinterpret_cast<const MF_GLOBAL u32x4 *>(reinterpret_cast<uint64_t>(rowsIn));
+    MF_GLOBAL u32x4 *dst = reinterpret_cast<MF_GLOBAL u32x4 *>(reinterpret_cast<uint64_t>(y)) + static_cast<uint64_t>(token) * unitsPerRow;
+    for (uint32_t u = threadIdx.x; u < unitsPerRow; u += kRowThreads) {
+        u32x4 v[kSlots];
+#pragma unroll
+        for (uint32_t k = 0; k < kSlots; ++k) {
+            if (k < nk) {
+                v[k] = __builtin_nontemporal_load(in + rowBase[k] + u);
+            }
+        }
+        float acc[8];
+#pragma unroll
+        for (uint32_t i = 0; i < 8; ++i) {
+            acc[i] = 0.0f;
+        }
+#pragma unroll
+        for (uint32_t k = 0; k < kSlots; ++k) {
+            if (k < nk) {
+#pragma unroll
+                for (uint32_t i = 0; i < 4; ++i) {
+                    acc[2 * i] = __builtin_fmaf(w[k], Bf16Lo(v[k][i]), acc[2 * i]);
+                    acc[2 * i + 1] = __builtin_fmaf(w[k], Bf16Hi(v[k][i]), acc[2 * i + 1]);
+                }
+            }
+        }
+        u32x4 o;
+#pragma unroll
+        for (uint32_t i = 0; i < 4; ++i) {
+            o[i] = ToBf16(acc[2 * i]) | (ToBf16(acc[2 * i + 1]) << 16);
+        }
+        __builtin_nontemporal_store(o, dst + u);
+    }
+}
+
+}  // namespace
+}  // namespace mf
+
+extern "C" uint64_t mfk_moe_workspace_bytes(uint32_t tokens, uint32_t topK, uint32_t experts)
+{
+    const uint64_t total = static_cast<uint64_t>(tokens) * topK;
+    const uint64_t blocks = (total + mf::kRankBlock - 1) / mf::kRankBlock;
+    return 256 + blocks * sizeof(uint32_t) + blocks * experts * sizeof(uint32_t);
+}
+
+extern "C" int mfk_moe_dispatch(const void *x, const void *topk, uint32_t tokens, uint32_t hidden, uint32_t topK,
+                                uint32_t experts, void *out, void *counts, void *offsets, void *rowOf, void *srcOf,
+                                void *workspace, void *stream)
+{
+    using namespace mf;
+    const uint64_t total64 = static_cast<uint64_t>(tokens) * topK;
+    if (total64 == 0 || total64 > 0x7FFFFFFFull || experts == 0 || experts > kMaxExperts || topK > kMaxTopK ||
+        (static_cast<uint64_t>(hidden) * 2) % 16 != 0) {
+        return -1;
+    }
+    const uint32_t total = static_cast<uint32_t>(total64);
+    const uint32_t blocks = (total + kRankBlock - 1) / kRankBlock;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    uint32_t *status = static_cast<uint32_t *>(workspace);
+    uint32_t *blockBad = status + 64;
+    uint32_t *blockHist = blockBad + blocks;
+    const size_t histLds = static_cast<size_t>(kRankSlices) * experts * sizeof(uint32_t);
+    const size_t rankLds = histLds + (experts + kRankThreads) * sizeof(uint32_t);
+    hipLaunchKernelGGL(MoeHistKernel, dim3(blocks), dim3(kRankThreads), histLds, s, static_cast<const int32_t *>(topk),
+                       total, experts, blockHist, blockBad);
+    hipLaunchKernelGGL(MoeRankKernel, dim3(blocks), dim3(kRankThreads), rankLds, s, static_cast<const int32_t *>(topk),
+                       total, experts, blockHist, static_cast<int32_t *>(counts), static_cast<int32_t *>(offsets),
+                       static_cast<int32_t *>(rowOf), static_cast<int32_t *>(srcOf), blockBad, status);
+    if (x != nullptr && out != nullptr && hidden != 0) {
+        hipLaunchKernelGGL(MoePermuteKernel, dim3(tokens), dim3(kRowThreads), 0, s, static_cast<const u32x4 *>(x),
+                           static_cast<const int32_t *>(rowOf), topK, hidden / 8, static_cast<u32x4 *>(out));
+    }
+    return static_cast<int>(hipGetLastError());
+}
+
+extern "C" int mfk_moe_combine(const void *rows, const void *rowOf, const void *weights, uint32_t tokens,
+                               uint32_t hidden, uint32_t topK, void *y, void *stream)
+{
+    using namespace mf;
+    if (tokens == 0 || topK == 0 || topK > kMaxTopK || hidden == 0 || (static_cast<uint64_t>(hidden) * 2) % 16 != 0) {
+        return -1;
+    }
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const u32x4 *in = static_cast<const u32x4 *>(rows);
+    const int32_t *ro = static_cast<const int32_t *>(rowOf);
+    const float *w = static_cast<const float *>(weights);
+    u32x4 *o = static_cast<u32x4 *>(y);
+    if (topK == 8) {
+        hipLaunchKernelGGL(MoeCombineKernel<8>, dim3(tokens), dim3(kRowThreads), 0, s, in, ro, w, topK, hidden / 8, o);
+    } else {
+        hipLaunchKernelGGL(MoeCombineKernel<0>, dim3(tokens), dim3(kRowThreads), 0, s, in, ro, w, topK, hidden / 8, o);
+    }
+    return static_cast<int>(hipGetLastError());
+}

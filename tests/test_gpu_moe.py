@@ -1,0 +1,213 @@
+"""GPU parity of the local MoE dispatch / combine against the CPU specification in
+oracle/mf_oracle.c.  Dispatch is integer/byte work: bit-exact.  Combine is floating point: the
+stated tolerance is 1e-2 relative (bf16); because both sides use the same fp32 FMA chain and one
+final rounding, the test additionally demands bit-equality, which is the stronger statement."""
+
+import ctypes
+
+import numpy as np
+import pytest
+
+from memfabric_hybrid_amd import native, workloads
+from tests import gpu_util
+from tests.oracle_lib import np_ptr
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def gpu(lib):
+    assert lib.hybm_init(0, 0) == 0, native.last_error()
+    yield lib
+    lib.hybm_uninit()
+
+
+def _dev(gpu, array):
+    a = np.ascontiguousarray(array)
+    buf = gpu_util.DeviceBuffer(gpu, max(a.nbytes, 16))
+    if a.nbytes:
+        buf.upload(a.view(np.uint8).reshape(-1))
+    return buf
+
+
+def _fetch(buf, dtype, shape):
+    n = int(np.prod(shape)) * np.dtype(dtype).itemsize
+    return buf.download(0, n).view(dtype).reshape(shape)
+
+
+def _oracle_dispatch(oracle, x, topk, E):
+    T, H = x.shape
+    K = topk.shape[1]
+    out = np.zeros((T * K, H), dtype=np.uint16)
+    counts = np.zeros(E, dtype=np.int32)
+    offsets = np.zeros(E, dtype=np.int32)
+    row_of = np.zeros(T * K, dtype=np.int32)
+    src_of = np.zeros(T * K, dtype=np.int32)
+    ret = oracle.orc_moe_dispatch(np_ptr(x), np_ptr(topk), T, H, K, E, np_ptr(out), np_ptr(counts), np_ptr(offsets),
+                                  np_ptr(row_of), np_ptr(src_of))
+    assert ret == 0
+    return out, counts, offsets, row_of, src_of
+
+
+def _gpu_dispatch(gpu, x, topk, E, with_rows=True):
+    T, H = x.shape
+    K = topk.shape[1]
+    ws_bytes = gpu.mf_moe_workspace_bytes(T, K, E)
+    bufs = {
+        "x": _dev(gpu, x), "topk": _dev(gpu, topk), "out": gpu_util.DeviceBuffer(gpu, max(T * K * H * 2, 16)),
+        "counts": gpu_util.DeviceBuffer(gpu, E * 4), "offsets": gpu_util.DeviceBuffer(gpu, E * 4),
+        "row_of": gpu_util.DeviceBuffer(gpu, T * K * 4), "src_of": gpu_util.DeviceBuffer(gpu, T * K * 4),
+        "ws": gpu_util.DeviceBuffer(gpu, ws_bytes),
+    }
+    bufs["ws"].fill(0xFF)  # the workspace needs no initialisation
+    bufs["src_of"].fill(0xFF)
+    ret = gpu.mf_moe_dispatch(bufs["x"].ptr if with_rows else None, bufs["topk"].ptr, T, H, K, E,
+                              bufs["out"].ptr if with_rows else None, bufs["counts"].ptr, bufs["offsets"].ptr,
+                              bufs["row_of"].ptr, bufs["src_of"].ptr, bufs["ws"].ptr, ws_bytes, None)
+    assert ret == 0, native.last_error()
+    assert gpu.mfrt_device_sync() == 0
+    return bufs
+
+
+def _free(bufs):
+    for b in bufs.values():
+        b.free()
+
+
+def _inputs(oracle, seed, T, H, K, E):
+    x, logits = workloads.moe_inputs(seed, T, H, E, K)
+    topk = np.zeros((T, K), dtype=np.int32)
+    w = np.zeros((T, K), dtype=np.float32)
+    oracle.orc_moe_route(np_ptr(logits), T, E, K, np_ptr(topk), np_ptr(w))
+    return x, topk, w
+
+
+@pytest.mark.parametrize("T,H,K,E", [
+    (1, 8, 1, 1), (7, 64, 2, 4), (300, 64, 4, 16), (1000, 520, 8, 256), (129, 1024, 8, 300),
+    (2050, 72, 16, 512), (4096, 2048, 8, 256), (511, 16384, 3, 37),
+])
+def test_dispatch_and_combine_match_the_specification(gpu, oracle, T, H, K, E):
+    K = min(K, E)
+    x, topk, w = _inputs(oracle, 0xC4 + T, T, H, K, E)
+    exp_out, exp_counts, exp_offsets, exp_row, exp_src = _oracle_dispatch(oracle, x, topk, E)
+    bufs = _gpu_dispatch(gpu, x, topk, E)
+    try:
+        assert np.array_equal(_fetch(bufs["counts"], np.int32, (E,)), exp_counts)
+        assert np.array_equal(_fetch(bufs["offsets"], np.int32, (E,)), exp_offsets)
+        assert np.array_equal(_fetch(bufs["row_of"], np.int32, (T * K,)), exp_row)
+        assert np.array_equal(_fetch(bufs["src_of"], np.int32, (T * K,)), exp_src)
+        assert np.array_equal(_fetch(bufs["out"], np.uint16, (T * K, H)), exp_out)
+        assert _fetch(bufs["ws"], np.uint32, (1,))[0] == 0
+
+        wdev = _dev(gpu, w)
+        y = gpu_util.DeviceBuffer(gpu, T * H * 2)
+        assert gpu.mf_moe_combine(bufs["out"].ptr, bufs["row_of"].ptr, wdev.ptr, T, H, K, y.ptr, None) == 0
+        assert gpu.mfrt_device_sync() == 0
+        got = _fetch(y, np.uint16, (T, H))
+        exp_y = np.zeros((T, H), dtype=np.uint16)
+        oracle.orc_moe_combine(np_ptr(exp_out), np_ptr(exp_row), np_ptr(w), T, H, K, np_ptr(exp_y))
+        gf = workloads.bf16_words_to_f32(got).astype(np.float64)
+        ef = workloads.bf16_words_to_f32(exp_y).astype(np.float64)
+        assert np.all(np.abs(gf - ef) <= 1e-2 * np.abs(ef) + 1e-6)   # the stated tolerance
+        assert np.array_equal(got, exp_y)                             # and in fact bit-equal
+        wdev.free()
+        y.free()
+    finally:
+        _free(bufs)
+
+
+def test_skewed_routing_with_empty_and_hot_experts(gpu, oracle):
+    rng = np.random.default_rng(3)
+    T, H, K, E = 3000, 128, 8, 256
+    x, _ = workloads.moe_inputs(3, T, H, E, K)
+    topk = rng.integers(0, 5, (T, K)).astype(np.int32)       # everything lands on 5 experts, duplicates included
+    topk[::7, 0] = 255
+    exp_out, exp_counts, exp_offsets, exp_row, exp_src = _oracle_dispatch(oracle, x, topk, E)
+    bufs = _gpu_dispatch(gpu, x, topk, E)
+    try:
+        assert np.array_equal(_fetch(bufs["counts"], np.int32, (E,)), exp_counts)
+        assert np.array_equal(_fetch(bufs["row_of"], np.int32, (T * K,)), exp_row)
+        assert np.array_equal(_fetch(bufs["out"], np.uint16, (T * K, H)), exp_out)
+    finally:
+        _free(bufs)
+
+
+def test_out_of_range_expert_ids_are_flagged_not_followed(gpu, oracle):
+    T, H, K, E = 500, 64, 4, 32
+    x, topk, _ = _inputs(oracle, 9, T, H, K, E)
+    bad = topk.copy()
+    bad[10, 1] = E
+    bad[499, 3] = -3
+    bufs = _gpu_dispatch(gpu, x, bad, E)
+    try:
+        assert _fetch(bufs["ws"], np.uint32, (1,))[0] == 1
+        row_of = _fetch(bufs["row_of"], np.int32, (T * K,))
+        assert row_of[10 * K + 1] == -1 and row_of[499 * K + 3] == -1
+        good = np.delete(np.arange(T * K), [10 * K + 1, 499 * K + 3])
+        assert sorted(row_of[good].tolist()) == list(range(T * K - 2))
+        assert _fetch(bufs["counts"], np.int32, (E,)).sum() == T * K - 2
+    finally:
+        _free(bufs)
+    # the same call with valid ids clears the flag again without any reset by the caller
+    bufs = _gpu_dispatch(gpu, x, topk, E)
+    try:
+        assert _fetch(bufs["ws"], np.uint32, (1,))[0] == 0
+    finally:
+        _free(bufs)
+
+
+def test_argument_errors(gpu):
+    p = ctypes.c_void_p(0x1000)
+    assert gpu.mf_moe_dispatch(p, None, 4, 8, 2, 4, p, p, p, p, None, p, 1 << 20, None) == native.BM_INVALID_PARAM
+    assert gpu.mf_moe_dispatch(p, p, 4, 12, 2, 4, p, p, p, p, None, p, 1 << 20, None) == native.BM_INVALID_PARAM
+    assert gpu.mf_moe_dispatch(p, p, 4, 8, 17, 4, p, p, p, p, None, p, 1 << 20, None) == native.BM_INVALID_PARAM
+    assert gpu.mf_moe_dispatch(p, p, 4, 8, 2, 513, p, p, p, p, None, p, 1 << 20, None) == native.BM_INVALID_PARAM
+    assert gpu.mf_moe_dispatch(p, p, 4, 8, 2, 4, p, p, p, p, None, p, 8, None) == native.BM_INVALID_PARAM
+    assert gpu.mf_moe_combine(p, p, None, 4, 8, 2, p, None) == native.BM_INVALID_PARAM
+    assert gpu.mf_moe_combine(p, p, p, 4, 9, 2, p, None) == native.BM_INVALID_PARAM
+
+
+def test_full_size_local_share(gpu, oracle):
+    """8192 tokens x 7168 bf16, 256 experts, top-8: whole outputs against the oracle, plus the
+    size-independent properties (bijection, counts, one-hot combine returns the token)."""
+    T, H, K, E = 8192, 7168, 8, 256
+    x, topk, w = _inputs(oracle, 0xC4, T, H, K, E)
+    exp_out, exp_counts, exp_offsets, exp_row, exp_src = _oracle_dispatch(oracle, x, topk, E)
+    bufs = _gpu_dispatch(gpu, x, topk, E)
+    try:
+        row_of = _fetch(bufs["row_of"], np.int32, (T * K,))
+        counts = _fetch(bufs["counts"], np.int32, (E,))
+        assert counts.sum() == T * K
+        assert np.array_equal(np.sort(row_of), np.arange(T * K))
+        assert np.array_equal(counts, exp_counts)
+        assert np.array_equal(_fetch(bufs["offsets"], np.int32, (E,)), exp_offsets)
+        assert np.array_equal(row_of, exp_row)
+        assert np.array_equal(_fetch(bufs["src_of"], np.int32, (T * K,)), exp_src)
+        got_out = _fetch(bufs["out"], np.uint16, (T * K, H))
+        assert np.array_equal(got_out, exp_out)
+        del got_out
+
+        wdev = _dev(gpu, w)
+        y = gpu_util.DeviceBuffer(gpu, T * H * 2)
+        assert gpu.mf_moe_combine(bufs["out"].ptr, bufs["row_of"].ptr, wdev.ptr, T, H, K, y.ptr, None) == 0
+        assert gpu.mfrt_device_sync() == 0
+        got = _fetch(y, np.uint16, (T, H))
+        exp_y = np.zeros((T, H), dtype=np.uint16)
+        oracle.orc_moe_combine(np_ptr(exp_out), np_ptr(exp_row), np_ptr(w), T, H, K, np_ptr(exp_y))
+        gf = workloads.bf16_words_to_f32(got)
+        ef = workloads.bf16_words_to_f32(exp_y)
+        assert np.all(np.abs(gf - ef) <= 1e-2 * np.abs(ef) + 1e-6)
+        assert np.array_equal(got, exp_y)
+        # one-hot weights: combine(dispatch(x)) == x
+        onehot = np.zeros((T, K), dtype=np.float32)
+        onehot[:, 5] = 1.0
+        wdev.upload(onehot.view(np.uint8).reshape(-1))
+        assert gpu.mf_moe_combine(bufs["out"].ptr, bufs["row_of"].ptr, wdev.ptr, T, H, K, y.ptr, None) == 0
+        assert gpu.mfrt_device_sync() == 0
+        back = _fetch(y, np.uint16, (T, H))
+        # the chain starts from +0, so a -0.0 input comes back as +0.0 (as it does in the oracle)
+        assert np.array_equal(np.where(back == 0x8000, 0, back), np.where(x == 0x8000, 0, x))
+        wdev.free()
+        y.free()
+    finally:
+        _free(bufs)
