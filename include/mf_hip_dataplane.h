@@ -43,6 +43,21 @@ int32_t mf_xcopy_device_table(const void *triples, uint32_t n, int32_t route, vo
  * src/hybm/csrc/ts_engine/hybm_stream_manager.cpp:73-90).  NULL before init. */
 void *mf_xcopy_thread_stream(void);
 
+/* Batched strided 2-D copy: for each descriptor, `height` rows of `width` bytes,
+ * consecutive rows `spitch` / `dpitch` bytes apart (cudaMemcpy2D-style geometry;
+ * the reference loads aclrtMemcpy2d at src/hybm/csrc/under_api/dl_acl_api.cpp:87-88
+ * but never calls it).  Rectangles of one call must not overlap each other's
+ * destinations.  Enqueues on `stream` (NULL: thread stream), does not wait. */
+typedef struct {
+    uint64_t src;
+    uint64_t dst;
+    uint64_t width;
+    uint64_t height;
+    uint64_t spitch;
+    uint64_t dpitch;
+} mf_copy2d_desc;
+int32_t mf_xcopy_2d_batch(const mf_copy2d_desc *descs, uint32_t n, int32_t route, void *stream);
+
 /* Launch-shape knobs.  units: 16-byte units per workgroup chunk (0 = choose
  * per batch); wgPerCu / wgPerCuLink: resident workgroups per CU for HBM and
  * host-link routes (0 = keep). */

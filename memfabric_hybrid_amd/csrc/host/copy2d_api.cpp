@@ -1,0 +1,123 @@
+// Native C entry point of the batched strided 2-D copy (declared in
+// include/mf_hip_dataplane.h).  Rectangles whose addresses, pitches and width
+// are all multiples of 16 go to the 2-D kernel; anything else is expanded into
+// one segment per row and takes the ordinary batch path.
+#include <vector>
+
+#include "../../../include/mf_hip_dataplane.h"
+#include "../../../include/mf_xcopy_types.h"
+#include "../kernels/copy2d_plan.h"
+#include "../rt/mf_rt.h"
+#include "mf_log.h"
+#include "xcopy_engine.h"
+
+using namespace mf;
+
+#define MF_EXPORT extern "C" __attribute__((visibility("default")))
+
+namespace {
+
+constexpr uint32_t kChunkBytes = 16384;
+
+bool Aligned16(const mf_copy2d_desc &d)
+{
+    return ((d.src | d.dst | d.width | d.spitch | d.dpitch) & 15u) == 0 && d.width / 16 <= 0xFFFFu &&
+           d.spitch / 16 <= 0xFFFFFFFFull && d.dpitch / 16 <= 0xFFFFFFFFull && d.height <= 0xFFFFFFFFull;
+}
+
+}  // namespace
+
+MF_EXPORT int32_t mf_xcopy_2d_batch(const mf_copy2d_desc *descs, uint32_t n, int32_t route, void *stream)
+{
+    if ((n != 0 && descs == nullptr) || route < 0 || route > MF_ROUTE_HBM_THROUGH) {
+        MF_FAIL(BM_INVALID_PARAM, "mf_xcopy_2d_batch: null descriptors or unknown route");
+    }
+    XcopyEngine &engine = XcopyEngine::Instance();
+    if (!engine.Started()) {
+        MF_FAIL(BM_NOT_INITIALIZED, "GPU data plane is not running; call hybm_init first");
+    }
+    if (mfrt_bind_thread() != 0) {
+        MF_FAIL(BM_ERROR, "cannot make the GPU current on this thread");
+    }
+    if (stream == nullptr) {
+        stream = engine.ThreadStream();
+    }
+    for (uint32_t i = 0; i < n; ++i) {
+        if (descs[i].width > descs[i].spitch && descs[i].height > 1) {
+            MF_FAIL(BM_INVALID_PARAM, "rectangle " << i << ": width exceeds the source pitch");
+        }
+        if (descs[i].width > descs[i].dpitch && descs[i].height > 1) {
+            MF_FAIL(BM_INVALID_PARAM, "rectangle " << i << ": width exceeds the destination pitch");
+        }
+    }
+    const uint32_t cu = mfrt_cu_count() == 0 ? 256 : mfrt_cu_count();
+    std::vector<uint64_t> rs;
+    std::vector<uint64_t> rd;
+    std::vector<uint64_t> rl;
+    RectPlan plan;
+    uint32_t used = 0;
+    uint64_t run = 0;
+    auto flush = [&]() -> int {
+        if (used == 0) {
+            return 0;
+        }
+        for (uint32_t i = used; i < kRectInline; ++i) {
+            plan.src[i] = plan.dst[i] = 0;
+            plan.spitchUnits[i] = plan.dpitchUnits[i] = plan.widthUnits[i] = plan.height[i] = 0;
+            plan.rowsPerChunk[i] = 1;
+            plan.magic[i] = 0;
+            plan.first[i] = 0xFFFFFFFFu;
+        }
+        plan.nchunk = static_cast<uint32_t>(run);
+        const uint64_t cap = static_cast<uint64_t>(cu) * engine.Tuning().wgPerCu;
+        int err = mfk_copy2d(&plan, static_cast<uint32_t>(run < cap ? run : cap), stream);
+        used = 0;
+        run = 0;
+        return err;
+    };
+    for (uint32_t i = 0; i < n; ++i) {
+        const mf_copy2d_desc &d = descs[i];
+        if (d.width == 0 || d.height == 0) {
+            continue;
+        }
+        if (!Aligned16(d)) {
+            for (uint64_t r = 0; r < d.height; ++r) {
+                rs.push_back(d.src + r * d.spitch);
+                rd.push_back(d.dst + r * d.dpitch);
+                rl.push_back(d.width);
+            }
+            continue;
+        }
+        const uint32_t wu = static_cast<uint32_t>(d.width / 16);
+        uint32_t rpc = kChunkBytes / static_cast<uint32_t>(d.width);
+        if (rpc == 0) {
+            rpc = 1;
+        }
+        const uint64_t chunks = (d.height + rpc - 1) / rpc;
+        if (run + chunks >= 0xFFFFFFFFull || used == kRectInline) {
+            int err = flush();
+            if (err != 0) {
+                MF_FAIL(BM_ERROR, "2-D copy launch failed: " << mfrt_error_string(err));
+            }
+        }
+        plan.src[used] = d.src;
+        plan.dst[used] = d.dst;
+        plan.spitchUnits[used] = static_cast<uint32_t>(d.spitch / 16);
+        plan.dpitchUnits[used] = static_cast<uint32_t>(d.dpitch / 16);
+        plan.widthUnits[used] = wu;
+        plan.height[used] = static_cast<uint32_t>(d.height);
+        plan.rowsPerChunk[used] = rpc;
+        plan.magic[used] = wu == 1 ? 0u : static_cast<uint32_t>((1ull << 32) / wu) + 1u;
+        plan.first[used] = static_cast<uint32_t>(run);
+        run += chunks;
+        ++used;
+    }
+    int err = flush();
+    if (err != 0) {
+        MF_FAIL(BM_ERROR, "2-D copy launch failed: " << mfrt_error_string(err));
+    }
+    if (!rs.empty()) {
+        return engine.Submit(rs.data(), rd.data(), rl.data(), static_cast<uint32_t>(rs.size()), route, stream, nullptr, 0);
+    }
+    return BM_OK;
+}

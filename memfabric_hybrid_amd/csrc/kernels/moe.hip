@@ -103,7 +103,7 @@ __global__ __launch_bounds__(kRankThreads) void MoeHistKernel(const int32_t *__r
         for (uint32_t s = 0; s < kRankSlices; ++s) {
             sum += hist[s * experts + x];
         }
-        blockHist[static_cast<uint64_t>(blockIdx.x) * experts + x] = sum;
+        blockHist[static_cast<uint64_t>(x) * gridDim.x + blockIdx.x] = sum;  // [expert][block]
     }
     // every block reports, so the flags need no clearing between calls
     const uint32_t anyBad = __syncthreads_or(static_cast<int>(bad)) != 0 ? 1u : 0u;
@@ -149,10 +149,13 @@ __global__ __launch_bounds__(kRankThreads) void MoeRankKernel(const int32_t *__r
     for (uint32_t j = 0; j < per; ++j) {
         const uint32_t x = threadIdx.x * per + j;
         if (x < experts) {
+            // one contiguous row of the [expert][block] table per expert: independent, coalescable loads
+            const uint32_t *rowHist = blockHist + static_cast<uint64_t>(x) * gridDim.x;
             uint32_t t = 0;
             uint32_t b = 0;
+#pragma unroll 16
             for (uint32_t blk = 0; blk < gridDim.x; ++blk) {
-                const uint32_t v = blockHist[static_cast<uint64_t>(blk) * experts + x];
+                const uint32_t v = rowHist[blk];
                 t += v;
                 b += blk < blockIdx.x ? v : 0u;
             }
@@ -212,23 +215,38 @@ __global__ __launch_bounds__(kRankThreads) void MoeRankKernel(const int32_t *__r
     }
 }
 
-// One workgroup per token.  unitsPerRow = H*2/16.
-__global__ __launch_bounds__(kRowThreads) void MoePermuteKernel(const u32x4 *__restrict__ x,
-                                                                const int32_t *__restrict__ rowOf, uint32_t topK,
-                                                                uint32_t unitsPerRow, u32x4 *__restrict__ out)
+template <int kMode>
+__device__ __forceinline__ void RowStore(MF_GLOBAL u32x4 *p, u32x4 v)
+{
+    if (kMode == 2) {
+        asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1 nt" : : "v"(p), "v"(v) : "memory");
+    } else if (kMode == 1) {
+        __builtin_nontemporal_store(v, p);
+    } else {
+        *p = v;
+    }
+}
+
+// One workgroup per token.  unitsPerRow = H*2/16.  Each lane keeps up to kHold 128-bit pieces of
+// the token's row in registers and stores them to the token's K destination rows.
+template <uint32_t kThreads, uint32_t kHold, int kMode>
+__global__ __launch_bounds__(kThreads) void MoePermuteKernel(const u32x4 *__restrict__ x,
+                                                             const int32_t *__restrict__ rowOf, uint32_t topK,
+                                                             uint32_t unitsPerRow, u32x4 *__restrict__ out)
 {
     const uint32_t token = blockIdx.x;
-    const MF_GLOBAL u32x4 *src = reinterpret_cast<const MF_GLOBAL u32x4 *>(reinterpret_cast<uint64_t>(x)) + static_cast<uint64_t>(token) * unitsPerRow;
+    const MF_GLOBAL u32x4 *src = reinterpret_cast<const MF_GLOBAL u32x4 *>(reinterpret_cast<uint64_t>(x)) +
+                                 static_cast<uint64_t>(token) * unitsPerRow;
     int32_t rows[kMaxTopK];
 #pragma unroll
     for (uint32_t k = 0; k < kMaxTopK; ++k) {
         rows[k] = k < topK ? rowOf[static_cast<uint64_t>(token) * topK + k] : -1;
     }
-    for (uint32_t u0 = 0; u0 < unitsPerRow; u0 += 4 * kRowThreads) {
-        u32x4 v[4];
+    for (uint32_t u0 = 0; u0 < unitsPerRow; u0 += kHold * kThreads) {
+        u32x4 v[kHold];
 #pragma unroll
-        for (uint32_t j = 0; j < 4; ++j) {
-            const uint32_t u = u0 + j * kRowThreads + threadIdx.x;
+        for (uint32_t j = 0; j < kHold; ++j) {
+            const uint32_t u = u0 + j * kThreads + threadIdx.x;
             if (u < unitsPerRow) {
                 v[j] = __builtin_nontemporal_load(src + u);
             }
@@ -236,13 +254,13 @@ __global__ __launch_bounds__(kRowThreads) void MoePermuteKernel(const u32x4 *__r
 #pragma unroll
         for (uint32_t k = 0; k < kMaxTopK; ++k) {
             if (k < topK && rows[k] >= 0) {
-                MF_GLOBAL u32x4 *dst =
-                    reinterpret_cast<MF_GLOBAL u32x4 *>(reinterpret_cast<uint64_t>(out)) + static_cast<uint64_t>(rows[k]) * unitsPerRow;
+                MF_GLOBAL u32x4 *dst = reinterpret_cast<MF_GLOBAL u32x4 *>(reinterpret_cast<uint64_t>(out)) +
+                                       static_cast<uint64_t>(rows[k]) * unitsPerRow;
 #pragma unroll
-                for (uint32_t j = 0; j < 4; ++j) {
-                    const uint32_t u = u0 + j * kRowThreads + threadIdx.x;
+                for (uint32_t j = 0; j < kHold; ++j) {
+                    const uint32_t u = u0 + j * kThreads + threadIdx.x;
                     if (u < unitsPerRow) {
-                        __builtin_nontemporal_store(v[j], dst + u);
+                        RowStore<kMode>(dst + u, v[j]);
                     }
                 }
             }
@@ -329,6 +347,12 @@ __global__ __launch_bounds__(kRowThreads) void MoeCombineKernel(const u32x4 *__r
 }  // namespace
 }  // namespace mf
 
+static int g_permuteVariant = -1;  // -1: choose from the row width
+extern "C" void mfk_moe_tune(int permuteVariant)
+{
+    g_permuteVariant = permuteVariant;
+}
+
 extern "C" uint64_t mfk_moe_workspace_bytes(uint32_t tokens, uint32_t topK, uint32_t experts)
 {
     const uint64_t total = static_cast<uint64_t>(tokens) * topK;
@@ -360,8 +384,18 @@ extern "C" int mfk_moe_dispatch(const void *x, const void *topk, uint32_t tokens
                        total, experts, blockHist, static_cast<int32_t *>(counts), static_cast<int32_t *>(offsets),
                        static_cast<int32_t *>(rowOf), static_cast<int32_t *>(srcOf), blockBad, status);
     if (x != nullptr && out != nullptr && hidden != 0) {
-        hipLaunchKernelGGL(MoePermuteKernel, dim3(tokens), dim3(kRowThreads), 0, s, static_cast<const u32x4 *>(x),
-                           static_cast<const int32_t *>(rowOf), topK, hidden / 8, static_cast<u32x4 *>(out));
+        const u32x4 *xi = static_cast<const u32x4 *>(x);
+        const int32_t *ro = static_cast<const int32_t *>(rowOf);
+        u32x4 *oo = static_cast<u32x4 *>(out);
+        const uint32_t upr = hidden / 8;
+        // One wave per token holding the whole row (14 pieces per lane covers 7168 elements)
+        // measured best for wide rows; narrow rows use four waves with fewer pieces each.
+        const int variant = g_permuteVariant >= 0 ? g_permuteVariant : (upr >= 512 ? 1 : 0);
+        if (variant == 1) {
+            hipLaunchKernelGGL((MoePermuteKernel<64, 14, 1>), dim3(tokens), dim3(64), 0, s, xi, ro, topK, upr, oo);
+        } else {
+            hipLaunchKernelGGL((MoePermuteKernel<256, 4, 1>), dim3(tokens), dim3(256), 0, s, xi, ro, topK, upr, oo);
+        }
     }
     return static_cast<int>(hipGetLastError());
 }

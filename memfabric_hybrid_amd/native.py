@@ -104,6 +104,10 @@ class BatchCopyParams(ctypes.Structure):
                 ("dataSizes", u64p), ("batchSize", u32)]
 
 
+class Copy2dDesc(ctypes.Structure):
+    _fields_ = [("src", u64), ("dst", u64), ("width", u64), ("height", u64), ("spitch", u64), ("dpitch", u64)]
+
+
 class HybmCopyParams(ctypes.Structure):
     _fields_ = [("src", vp), ("dest", vp), ("dataSize", u64)]
 
@@ -166,6 +170,7 @@ _SIGNATURES = {
     # mf_hip_dataplane.h
     "mf_xcopy_batch": (i32, [u64p, u64p, u64p, u32, i32, vp]),
     "mf_xcopy_device_table": (i32, [vp, u32, i32, vp]),
+    "mf_xcopy_2d_batch": (i32, [vp, u32, i32, vp]),
     "mf_xcopy_thread_stream": (vp, []),
     "mf_xcopy_tune": (i32, [u32, u32, u32]),
     "mf_xcopy_choose_units": (u32, [u64, u32, i32]),

@@ -130,17 +130,110 @@ def bf16_words_to_f32(w):
     return (w.astype(np.uint32) << np.uint32(16)).view(np.float32)
 
 
-# ---- 7B decoder reshard, TP=8 storage -> TP=4 layout -------------------------
+# ---- decoder weight reshard, TP=8 storage -> TP=4 layout ---------------------------
+# Row-major [out, in] bf16 tensors per layer.  Column-parallel tensors (q, gate, up) are split on
+# `out`; k and v (4 KV heads) are split per head, each head held by two of the eight ranks;
+# row-parallel tensors (o, down) are split on `in`.
 RESHARD_LAYERS = 28
 RESHARD_HIDDEN = 3584
 RESHARD_FFN = 18944
-RESHARD_KV_OUT = 512  # 4 KV heads x 128
+RESHARD_KV_HEADS = 4
+RESHARD_HEAD_DIM = 128
+ELEM = 2
 
 
-def reshard_tensors():
-    """(name, rows(out), cols(in), kind) of one layer; kind 'col' splits rows, 'row' splits columns."""
-    h, f, kv = RESHARD_HIDDEN, RESHARD_FFN, RESHARD_KV_OUT
-    return [
-        ("q", h, h, "col"), ("k", kv, h, "col_kv"), ("v", kv, h, "col_kv"), ("o", h, h, "row"),
-        ("gate", f, h, "col"), ("up", f, h, "col"), ("down", h, f, "row"),
-    ]
+def reshard_tensors(hidden=RESHARD_HIDDEN, ffn=RESHARD_FFN, kv_heads=RESHARD_KV_HEADS, head_dim=RESHARD_HEAD_DIM):
+    """(name, out rows, in cols, kind) of one layer."""
+    kv = kv_heads * head_dim
+    return [("q", hidden, hidden, "col"), ("k", kv, hidden, "kv"), ("v", kv, hidden, "kv"),
+            ("o", hidden, hidden, "row"), ("gate", ffn, hidden, "col"), ("up", ffn, hidden, "col"),
+            ("down", hidden, ffn, "row")]
+
+
+def tp8_shard_shape(out, cols, kind):
+    if kind == "col":
+        return out // 8, cols
+    if kind == "kv":
+        return out // 4, cols          # one KV head per rank, every head on two ranks
+    return out, cols // 8
+
+
+def tp4_shard_shape(out, cols, kind):
+    if kind in ("col", "kv"):
+        return out // 4, cols
+    return out, cols // 4
+
+
+def reshard_layout(tensors, layers):
+    """Byte offsets of every (layer, tensor, shard) in the TP8 source pool and the TP4 destination
+    pool, plus the pool sizes.  Shards of a tensor are stored one after another in rank order."""
+    src, dst = {}, {}
+    s_off = d_off = 0
+    for layer in range(layers):
+        for name, out, cols, kind in tensors:
+            r8, c8 = tp8_shard_shape(out, cols, kind)
+            for r in range(8):
+                src[(layer, name, r)] = s_off
+                s_off += r8 * c8 * ELEM
+            r4, c4 = tp4_shard_shape(out, cols, kind)
+            for r in range(4):
+                dst[(layer, name, r)] = d_off
+                d_off += r4 * c4 * ELEM
+    return src, dst, s_off, d_off
+
+
+def reshard_plan(tensors, layers, src_base, dst_base):
+    """The re-layout as copy descriptors: (segments, rectangles).
+
+    segments: list of (src, dst, bytes) contiguous copies (column-parallel merges; KV duplicates
+    are simply not read).  rectangles: list of (src, dst, width, height, spitch, dpitch) strided
+    copies (row-parallel merges: two old column blocks side by side in each new shard)."""
+    src, dst, _, _ = reshard_layout(tensors, layers)
+    segments, rects = [], []
+    for layer in range(layers):
+        for name, out, cols, kind in tensors:
+            r8, c8 = tp8_shard_shape(out, cols, kind)
+            shard_bytes = r8 * c8 * ELEM
+            for new in range(4):
+                d = dst_base + dst[(layer, name, new)]
+                if kind == "col":
+                    for half in range(2):
+                        segments.append((src_base + src[(layer, name, 2 * new + half)], d + half * shard_bytes,
+                                         shard_bytes))
+                elif kind == "kv":
+                    segments.append((src_base + src[(layer, name, 2 * new)], d, shard_bytes))
+                else:
+                    width = c8 * ELEM
+                    for half in range(2):
+                        rects.append((src_base + src[(layer, name, 2 * new + half)], d + half * width, width, out,
+                                      width, 2 * width))
+    return segments, rects
+
+
+def reshard_reference(tensors, layers, full):
+    """TP8 storage and the expected TP4 storage cut directly out of the full tensors
+    full[(layer, name)] (uint16 arrays [out, in]); independent of the descriptors above."""
+    src, dst, s_bytes, d_bytes = reshard_layout(tensors, layers)
+    s_pool = np.zeros(s_bytes // ELEM, dtype=np.uint16)
+    d_pool = np.zeros(d_bytes // ELEM, dtype=np.uint16)
+    for layer in range(layers):
+        for name, out, cols, kind in tensors:
+            w = full[(layer, name)]
+            for r in range(8):
+                if kind == "col":
+                    part = w[r * (out // 8):(r + 1) * (out // 8), :]
+                elif kind == "kv":
+                    head = r // 2
+                    part = w[head * (out // 4):(head + 1) * (out // 4), :]
+                else:
+                    part = w[:, r * (cols // 8):(r + 1) * (cols // 8)]
+                o = src[(layer, name, r)] // ELEM
+                s_pool[o:o + part.size] = part.reshape(-1)
+            for r in range(4):
+                if kind in ("col", "kv"):
+                    part = w[r * (out // 4):(r + 1) * (out // 4), :]
+                else:
+                    part = w[:, r * (cols // 4):(r + 1) * (cols // 4)]
+                o = dst[(layer, name, r)] // ELEM
+                d_pool[o:o + part.size] = part.reshape(-1)
+    return s_pool, d_pool
