@@ -1,12 +1,15 @@
 #!/usr/bin/env python3
-"""Benchmark of the 122-segment KV-block batch copy (device to device inside a 4 GiB HBM pool)
-through smem_bm_copy_batch, plus the CPU baseline and the roofline of the copy kernel.
+"""Benchmark of the MemFabric xcopy hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--extras]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-extras] [--no-cpu]
 
-A step is one batch: 61 x (128 KiB + 16 KiB) = 8 994 816 payload bytes, i.e. 17 989 632 bytes
-of HBM traffic (read + write).  Steps rotate over 64 different segment tables so that the
-touched set (about 1.1 GiB) does not fit the 256 MiB last-level cache.  Prints one JSON line.
+Headline (value / roofline): the 122-segment KV-block batch copy, device to device inside a
+4 GiB HBM pool, through smem_bm_copy_batch on one stream.  A step is one batch:
+61 x (128 KiB + 16 KiB) = 8 994 816 payload bytes = 17 989 632 bytes of HBM traffic.  Steps
+rotate over 64 segment tables so that the touched set (~1.1 GiB) exceeds the 256 MiB
+last-level cache.  `extras` holds the other workload shapes (host link, large copies, paged
+gather, MoE dispatch/combine, weight reshard), concurrency and the yardstick kernels.
+Prints ONE JSON line.
 """
 
 import argparse
@@ -14,6 +17,7 @@ import ctypes
 import json
 import os
 import sys
+import threading
 import time
 
 import numpy as np
@@ -29,6 +33,7 @@ HBM_PEAK_GBPS = 8000.0
 LINK_PEAK_GBPS = 64.0
 POOL_BYTES = 4 << 30
 TABLES = 64
+MIB = 1 << 20
 
 
 class Batch:
@@ -36,19 +41,42 @@ class Batch:
 
     def __init__(self, src, dst, lens):
         self.n = len(lens)
-        self.srcs = native.ptr_array(src.tolist())
-        self.dsts = native.ptr_array(dst.tolist())
-        self.lens = native.u64_array(lens.tolist())
+        self.srcs = native.ptr_array(np.asarray(src).tolist())
+        self.dsts = native.ptr_array(np.asarray(dst).tolist())
+        self.lens = native.u64_array(np.asarray(lens).tolist())
         self.params = native.BatchCopyParams(self.srcs, self.dsts, self.lens, self.n)
         self.ref = ctypes.byref(self.params)
-        self.payload = int(lens.sum())
+        self.payload = int(np.asarray(lens).sum())
+
+
+class Timer:
+    """HIP events on the stream the kernels are launched on."""
+
+    def __init__(self, lib):
+        self.lib = lib
+        self.stream = lib.mf_xcopy_thread_stream()
+        self.e0 = lib.mfrt_event_create()
+        self.e1 = lib.mfrt_event_create()
+
+    def run(self, fn, reps, warm=2):
+        lib = self.lib
+        for _ in range(warm):
+            fn()
+        assert lib.mfrt_stream_sync(self.stream) == 0
+        t0 = time.perf_counter()
+        lib.mfrt_event_record(self.e0, self.stream)
+        for _ in range(reps):
+            fn()
+        lib.mfrt_event_record(self.e1, self.stream)
+        assert lib.mfrt_stream_sync(self.stream) == 0
+        wall = time.perf_counter() - t0
+        return lib.mfrt_event_elapsed_ms(self.e0, self.e1) * 1e3 / reps, wall * 1e6 / reps  # us, us
 
 
 def fill_device_pool(lib, dev, nbytes, seed):
-    """Uniform random bytes: a 64 MiB block generated on the host, uploaded and re-uploaded with a
-    different XOR mask per block so that no two blocks are equal."""
+    """Uniform random bytes: a 64 MiB host block, re-uploaded with a different XOR mask per block."""
     rng = np.random.default_rng(seed)
-    block = rng.integers(0, 256, 64 << 20, dtype=np.uint8)
+    block = rng.integers(0, 256, 64 * MIB, dtype=np.uint8)
     for i in range(nbytes // len(block)):
         chunk = block ^ np.uint8((i * 37 + 11) & 0xFF)
         err = lib.mfrt_memcpy(dev + i * len(block), chunk.ctypes.data, len(block))
@@ -56,7 +84,7 @@ def fill_device_pool(lib, dev, nbytes, seed):
 
 
 def timed_steps(lib, handle, batches, copy_type, steps, warmup, flags):
-    """K async batch copies between two events on the launch stream; returns (wall s, event ms)."""
+    """K batch copies between two events on the launch stream; returns (wall s, event ms)."""
     stream = lib.mf_xcopy_thread_stream()
     start, stop = lib.mfrt_event_create(), lib.mfrt_event_create()
     call = lib.smem_bm_copy_batch
@@ -82,6 +110,47 @@ def timed_steps(lib, handle, batches, copy_type, steps, warmup, flags):
     return wall, ms
 
 
+def threaded_steps(lib, handle, batches, copy_type, steps, threads):
+    """The same batches submitted by `threads` host threads, each on its own stream (the
+    reference gives every calling thread its own stream as well); wall-clock time."""
+    barrier = threading.Barrier(threads + 1)
+    errors = []
+
+    def worker(tid):
+        try:
+            lib.mfrt_bind_thread()
+            nb = len(batches)
+            for i in range(50):
+                lib.smem_bm_copy_batch(handle, batches[(tid * 7 + i) % nb].ref, copy_type, native.ASYNC_COPY_FLAG)
+            lib.smem_bm_wait(handle)
+            barrier.wait()
+            for i in range(tid, steps, threads):
+                if lib.smem_bm_copy_batch(handle, batches[i % nb].ref, copy_type, native.ASYNC_COPY_FLAG) != 0:
+                    raise RuntimeError(native.last_error())
+            if lib.smem_bm_wait(handle) != 0:
+                raise RuntimeError(native.last_error())
+        except Exception as exc:  # noqa: BLE001
+            errors.append(exc)
+            try:
+                barrier.abort()
+            except Exception:  # noqa: BLE001
+                pass
+
+    # the library rewrites the address arrays in place with the same (already normalised) values,
+    # so sharing one set of tables between the threads is harmless
+    pool = [threading.Thread(target=worker, args=(t,)) for t in range(threads)]
+    for t in pool:
+        t.start()
+    barrier.wait()
+    t0 = time.perf_counter()
+    for t in pool:
+        t.join()
+    wall = time.perf_counter() - t0
+    if errors:
+        raise errors[0]
+    return wall
+
+
 def cpu_baseline(tables, budget_s=12.0):
     """The reference's CPU copy path (single thread, one memcpy per segment, host pool to host
     pool) on the same segment tables: the reference's own DlHybridApi::Memcpy when oracle/_ref was
@@ -90,13 +159,13 @@ def cpu_baseline(tables, budget_s=12.0):
     ref = oracle_lib.reference()
     fn = ref.ref_batch_copy if ref is not None else oracle_lib.oracle().orc_batch_copy_fast
     kind = "reference" if ref is not None else "port"
-    pool = 1 << 30  # host pools of 1 GiB each; the tables are folded into them
+    pool = 1 << 30  # host pools of 1 GiB each; the 4 GiB offsets are folded into them
     src_pool = np.random.default_rng(1).integers(0, 256, pool, dtype=np.uint8)
     dst_pool = np.zeros(pool, dtype=np.uint8)
     prepared = []
     for src, dst, lens in tables:
-        s = oracle_lib.ptr_array((src_pool.ctypes.data + (src % np.uint64(pool - (1 << 20)))).tolist())
-        d = oracle_lib.ptr_array((dst_pool.ctypes.data + (dst % np.uint64(pool - (1 << 20)))).tolist())
+        s = oracle_lib.ptr_array((src_pool.ctypes.data + (src % np.uint64(pool - MIB))).tolist())
+        d = oracle_lib.ptr_array((dst_pool.ctypes.data + (dst % np.uint64(pool - MIB))).tolist())
         prepared.append((d, s, oracle_lib.u64_array(lens.tolist()), len(lens), int(lens.sum())))
     for d, s, l, n, _ in prepared[:8]:
         fn(d, s, l, n)
@@ -107,16 +176,211 @@ def cpu_baseline(tables, budget_s=12.0):
             done_bytes += payload
             batches += 1
         elapsed = time.perf_counter() - t0
-        if elapsed > budget_s or batches >= 64 * 40:
+        if elapsed > budget_s or batches >= 64 * 400:
             break
     return {
         "value": done_bytes / elapsed / GB,
-        "unit": "GB/s payload",
+        "unit": "GB/s",
         "cores": 1,
         "kind": kind,
-        "sample": f"{batches} batches of the same 122-segment tables, host pool to host pool, "
-                  f"{elapsed:.1f} s, single thread, nproc={os.cpu_count()}",
+        "sample": f"{batches} batches of the same 122-segment tables (8994816 B each), host pool to host pool, "
+                  f"{elapsed:.1f} s, single thread as the reference runs it; host has {os.cpu_count()} cores",
     }
+
+
+def read_traffic():
+    """HBM bytes per launch of the headline kernel, from the committed counter summary (rocprofv3
+    --pmc FETCH_SIZE / WRITE_SIZE scaled by the plain copy kernel); None when it is absent."""
+    path = os.path.join(ROOT, "profiles", "xcopy_inline_kv122_counters.txt")
+    try:
+        for line in open(path):
+            if line.startswith("traffic_bytes_per_launch"):
+                return float(line.split("=")[1].split()[0])
+    except OSError:
+        pass
+    return None
+
+
+def frac(gbps, peak):
+    return round(gbps / peak, 4)
+
+
+def extras_block(lib, pool, dev, batches, tables, steps):
+    out = {}
+    timer = Timer(lib)
+    g2g = int(bm.BmCopyType.G2G)
+    payload = batches[0].payload
+    handle = pool.handle
+
+    # ---- yardsticks: what this GPU sustains for flat streaming kernels --------------------------------
+    half = POOL_BYTES // 2
+    sink = lib.mfrt_alloc_device(256)
+    yard = {}
+    for kind, name, factor in ((0, "copy", 2), (1, "fill", 1), (2, "read", 1)):
+        dst = sink if kind == 2 else dev + half
+        us, _ = timer.run(lambda k=kind, d=dst: lib.mf_probe_hbm(k, d, dev, 1 << 30, None), 10)
+        yard[name + "_GBps"] = round(factor * (1 << 30) / us / 1e3, 1)
+    lib.mfrt_free_device(sink)
+    out["hbm_yardstick_1GiB"] = yard
+    copy_ceiling = yard["copy_GBps"]
+
+    # ---- KV batch: synchronous calls, concurrency ---------------------------------------------------------
+    k = max(200, steps // 10)
+    w, _ = timed_steps(lib, handle, batches, g2g, k, 50, 0)
+    out["kv122_d2d_sync_call_us"] = round(w * 1e6 / k, 2)
+    conc = {}
+    for threads in (2, 4, 8):
+        wall = threaded_steps(lib, handle, batches, g2g, steps, threads)
+        hbm = 2 * payload * steps / wall / GB
+        conc[f"threads_{threads}"] = {"us_per_batch": round(wall * 1e6 / steps, 2), "hbm_GBps": round(hbm, 1),
+                                      "frac_of_hbm_peak": frac(hbm, HBM_PEAK_GBPS)}
+    out["kv122_d2d_concurrent_streams"] = conc
+
+    # ---- KV batch over the host link ------------------------------------------------------------------------
+    host = pool.peer_rank_ptr(0, bm.BmMemType.HOST)
+    split = [workloads.kv_batch(0xD1 + b, POOL_BYTES, same_pool=False) for b in range(16)]
+    for name, bs in (("kv122_h2d", [Batch(host + s, dev + d, l) for s, d, l in split]),
+                     ("kv122_d2h", [Batch(dev + s, host + d, l) for s, d, l in split])):
+        kk = max(100, steps // 20)
+        _, ms = timed_steps(lib, handle, bs, g2g, kk, 10, native.ASYNC_COPY_FLAG)
+        gbps = payload * kk / (ms * 1e-3) / GB
+        out[name] = {"GBps": round(gbps, 2), "frac_of_link_peak": frac(gbps, LINK_PEAK_GBPS),
+                     "us_per_batch": round(ms * 1e3 / kk, 1)}
+    for name, (d, s) in (("dma_h2d_1GiB", (dev, host)), ("dma_d2h_1GiB", (host, dev))):
+        us, _ = timer.run(lambda d=d, s=s: lib.mfrt_memcpy_async(d, s, 1 << 30, timer.stream), 3, warm=1)
+        out[name + "_GBps"] = round((1 << 30) / us / 1e3, 2)   # the runtime's DMA engines, for comparison
+
+    # ---- large single copies through smem_bm_copy --------------------------------------------------------------
+    big = {}
+    for size_name, nbytes in (("1GiB", 1 << 30), ("2GiB", 2 << 30)):
+        for dname, (s, d, peak, factor) in (("d2d", (dev, dev + half, HBM_PEAK_GBPS, 2)),
+                                            ("h2d", (host, dev, LINK_PEAK_GBPS, 1)),
+                                            ("d2h", (dev, host, LINK_PEAK_GBPS, 1))):
+            params = native.SmemCopyParams(s, d, nbytes)
+            us, _ = timer.run(lambda p=params: lib.smem_bm_copy(handle, ctypes.byref(p), g2g, native.ASYNC_COPY_FLAG),
+                              10 if dname == "d2d" else 2, warm=1)
+            gbps = factor * nbytes / us / 1e3
+            big[f"{dname}_{size_name}"] = {"GBps": round(gbps, 1), "frac_of_peak": frac(gbps, peak), "us": round(us, 1)}
+    out["single_copy"] = big
+    return out, copy_ceiling
+
+
+def extras_paged(lib):
+    """Paged KV gather/scatter: 4096 distinct 32 KiB pages out of a 40 GiB pool."""
+    page, count = 32768, 4096
+    pool_bytes = 40 << 30
+    pool = lib.mfrt_alloc_device(pool_bytes)
+    buf = lib.mfrt_alloc_device(count * page * 4)
+    if not pool or not buf:
+        return {"error": "allocation failed"}
+    timer = Timer(lib)
+    sets = []
+    for b in range(4):
+        ids = workloads.page_ids(0xC3 + b, pool_bytes // page, count)
+        flat = buf + b * count * page + np.arange(count, dtype=np.uint64) * page
+        sets.append((native.u64_array((pool + ids * page).tolist()), native.u64_array(flat.tolist()),
+                     native.u64_array([page] * count)))
+    i = [0]
+
+    def gather():
+        s, d, l = sets[i[0] % 4]
+        i[0] += 1
+        assert lib.mf_xcopy_batch(s, d, l, count, native.ROUTE_HBM, None) == 0
+
+    def scatter():
+        s, d, l = sets[i[0] % 4]
+        i[0] += 1
+        assert lib.mf_xcopy_batch(d, s, l, count, native.ROUTE_HBM, None) == 0
+
+    res = {}
+    for name, fn in (("gather", gather), ("scatter", scatter)):
+        us, _ = timer.run(fn, 40, warm=4)
+        hbm = 2 * count * page / us / 1e3
+        res[name] = {"us": round(us, 1), "hbm_GBps": round(hbm, 1), "frac_of_hbm_peak": frac(hbm, HBM_PEAK_GBPS)}
+    res["shape"] = "4096 x 32 KiB pages, 40 GiB pool, one K-or-V plane of one layer per call (134 217 728 B)"
+    lib.mfrt_device_sync()
+    lib.mfrt_free_device(buf)
+    lib.mfrt_free_device(pool)
+    return res
+
+
+def extras_moe(lib):
+    from tests import oracle_lib
+    oracle = oracle_lib.oracle()
+    T, H, K, E = 8192, 7168, 8, 256
+    x, logits = workloads.moe_inputs(0xC4, T, H, E, K)
+    topk = np.zeros((T, K), dtype=np.int32)
+    w = np.zeros((T, K), dtype=np.float32)
+    oracle.orc_moe_route(logits.ctypes.data, T, E, K, topk.ctypes.data, w.ctypes.data)  # input synthesis only
+
+    def dev_of(a):
+        p = lib.mfrt_alloc_device(a.nbytes)
+        assert lib.mfrt_memcpy(p, a.ctypes.data, a.nbytes) == 0
+        return p
+
+    dx, dt, dw = dev_of(x), dev_of(topk), dev_of(w)
+    out = lib.mfrt_alloc_device(T * K * H * 2)
+    y = lib.mfrt_alloc_device(T * H * 2)
+    counts, offs = lib.mfrt_alloc_device(E * 4), lib.mfrt_alloc_device(E * 4)
+    row, src = lib.mfrt_alloc_device(T * K * 4), lib.mfrt_alloc_device(T * K * 4)
+    wsb = lib.mf_moe_workspace_bytes(T, K, E)
+    ws = lib.mfrt_alloc_device(wsb)
+    timer = Timer(lib)
+
+    def dispatch():
+        assert lib.mf_moe_dispatch(dx, dt, T, H, K, E, out, counts, offs, row, src, ws, wsb, None) == 0
+
+    def combine():
+        assert lib.mf_moe_combine(out, row, dw, T, H, K, y, None) == 0
+
+    d_us, _ = timer.run(dispatch, 30, warm=3)
+    c_us, _ = timer.run(combine, 30, warm=3)
+    d_bytes = T * H * 2 + T * K * H * 2 + T * K * 4
+    c_bytes = T * K * H * 2 + T * K * 4 + T * K * 4 + T * H * 2
+    res = {
+        "shape": "8192 tokens x 7168 bf16, 256 experts, top-8 (local share)",
+        "dispatch": {"us": round(d_us, 1), "algorithmic_bytes": d_bytes, "hbm_GBps": round(d_bytes / d_us / 1e3, 1),
+                     "frac_of_hbm_peak": frac(d_bytes / d_us / 1e3, HBM_PEAK_GBPS)},
+        "combine": {"us": round(c_us, 1), "algorithmic_bytes": c_bytes, "hbm_GBps": round(c_bytes / c_us / 1e3, 1),
+                    "frac_of_hbm_peak": frac(c_bytes / c_us / 1e3, HBM_PEAK_GBPS)},
+    }
+    both = (d_bytes + c_bytes) / (d_us + c_us) / 1e3
+    res["dispatch_plus_combine"] = {"hbm_GBps": round(both, 1), "frac_of_hbm_peak": frac(both, HBM_PEAK_GBPS)}
+    lib.mfrt_device_sync()
+    for p in (dx, dt, dw, out, y, counts, offs, row, src, ws):
+        lib.mfrt_free_device(p)
+    return res
+
+
+def extras_reshard(lib):
+    tensors = workloads.reshard_tensors()
+    layers = workloads.RESHARD_LAYERS
+    _, _, s_bytes, d_bytes = workloads.reshard_layout(tensors, layers)
+    sp, dp = lib.mfrt_alloc_device(s_bytes), lib.mfrt_alloc_device(d_bytes)
+    if not sp or not dp:
+        return {"error": "allocation failed"}
+    segments, rects = workloads.reshard_plan(tensors, layers, sp, dp)
+    s_arr = native.u64_array([s for s, _, _ in segments])
+    d_arr = native.u64_array([d for _, d, _ in segments])
+    l_arr = native.u64_array([n for _, _, n in segments])
+    descs = (native.Copy2dDesc * len(rects))()
+    for i, r in enumerate(rects):
+        descs[i] = native.Copy2dDesc(*[int(v) for v in r])
+    timer = Timer(lib)
+
+    def run():
+        assert lib.mf_xcopy_batch(s_arr, d_arr, l_arr, len(segments), native.ROUTE_HBM, None) == 0
+        assert lib.mf_xcopy_2d_batch(descs, len(rects), native.ROUTE_HBM, None) == 0
+
+    us, _ = timer.run(run, 3, warm=1)
+    moved = sum(n for _, _, n in segments) + sum(r[2] * r[3] for r in rects)
+    hbm = 2 * moved / us / 1e3
+    lib.mfrt_device_sync()
+    lib.mfrt_free_device(sp)
+    lib.mfrt_free_device(dp)
+    return {"shape": "28 layers, hidden 3584, FFN 18944, 28 Q / 4 KV heads, TP8 storage -> TP4 layout",
+            "bytes_moved": moved, "source_bytes": s_bytes, "segments": len(segments), "rectangles": len(rects),
+            "us": round(us, 1), "hbm_GBps": round(hbm, 1), "frac_of_hbm_peak": frac(hbm, HBM_PEAK_GBPS)}
 
 
 def main():
@@ -124,15 +388,27 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=4000)
     ap.add_argument("--warmup", type=int, default=400)
-    ap.add_argument("--extras", action="store_true", help="also time H2D / D2H and synchronous calls")
+    ap.add_argument("--no-extras", action="store_true", help="headline only")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--calibrate", action="store_true", help="only run the plain copy kernel (counter calibration)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build is a single-GPU data plane (no collectives, no sharding); run with --gpus 1")
 
     lib = native.lib()
+    if args.calibrate:
+        # counter calibration load: five launches of the plain copy kernel, 1 GiB read + 1 GiB written each
+        assert lib.hybm_init(0, 0) == 0, native.last_error()
+        a, b = lib.mfrt_alloc_device(1 << 30), lib.mfrt_alloc_device(1 << 30)
+        for _ in range(5):
+            assert lib.mf_probe_hbm(0, b, a, 1 << 30, None) == 0
+        assert lib.mfrt_device_sync() == 0
+        print(json.dumps({"calibrate": "ProbeCopyKernel", "launches": 5, "bytes_read_per_launch": 1 << 30,
+                          "bytes_written_per_launch": 1 << 30}))
+        lib.hybm_uninit()
+        return
     assert bm.initialize("tcp://127.0.0.1:0", 1, 0) == 0, native.last_error()
-    want_host = POOL_BYTES if args.extras else 0
+    want_host = 0 if args.no_extras else POOL_BYTES
     pool = bm.create(0, want_host, POOL_BYTES)
     dev = pool.peer_rank_ptr(0, bm.BmMemType.DEVICE)
     fill_device_pool(lib, dev, POOL_BYTES, 0xC1)
@@ -163,7 +439,7 @@ def main():
         "config": {
             "workload": "DeepSeek-R1-style KV block batch: 122 segments (61x128KiB + 61x16KiB = 8994816 B), "
                         "4 KiB-aligned random offsets in a 4 GiB HBM pool, D2D, 64 rotating tables",
-            "api": "smem_bm_copy_batch(SMEMB_COPY_G2G, ASYNC_COPY_FLAG) + one wait",
+            "api": "smem_bm_copy_batch(SMEMB_COPY_G2G, ASYNC_COPY_FLAG) on one stream + one wait",
             "payload_bytes": payload,
             "cu_count": lib.mfrt_cu_count(),
         },
@@ -173,32 +449,26 @@ def main():
             "peak": HBM_PEAK_GBPS,
             "unit": "GB/s",
             "frac": achieved / HBM_PEAK_GBPS,
-            "traffic": None,
-            "kernel": "XcopyInlineKernel<HBM>",
+            "traffic": read_traffic(),
+            "kernel": "XcopyInlineKernel<true, 1> (one launch per batch)",
             "algorithmic_bytes_per_launch": 2 * payload,
             "avg_launch_us": per_launch_us,
         },
     }
 
-    if args.extras:
-        extras = {}
-        w2, m2 = timed_steps(lib, pool.handle, batches, g2g, max(200, args.steps // 10), 50, 0)
-        extras["d2d_sync_call_us"] = w2 * 1e6 / max(200, args.steps // 10)
-        host = pool.peer_rank_ptr(0, bm.BmMemType.HOST)
-        split = [workloads.kv_batch(0xD1 + b, POOL_BYTES, same_pool=False) for b in range(TABLES)]
-        h2d = [Batch(host + s, dev + d, l) for s, d, l in split]
-        d2h = [Batch(dev + s, host + d, l) for s, d, l in split]
-        for name, bs in (("h2d", h2d), ("d2h", d2h)):
-            k = max(100, args.steps // 20)
-            w, m = timed_steps(lib, pool.handle, bs, g2g, k, 20, native.ASYNC_COPY_FLAG)
-            gbps = payload * k / (m * 1e-3) / GB
-            extras[name] = {"GBps": gbps, "frac_of_link_peak": gbps / LINK_PEAK_GBPS, "us_per_batch": m * 1e3 / k}
+    if not args.no_extras:
+        extras, copy_ceiling = extras_block(lib, pool, dev, batches, tables, args.steps)
+        result["roofline"]["frac_of_measured_copy_ceiling"] = frac(achieved, copy_ceiling)
+    pool.destroy()  # give the pools back before the larger workloads allocate
+    if not args.no_extras:
+        extras["paged_kv_40GiB"] = extras_paged(lib)
+        extras["moe_local"] = extras_moe(lib)
+        extras["reshard_tp8_to_tp4"] = extras_reshard(lib)
         result["extras"] = extras
 
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(tables)
 
-    pool.destroy()
     bm.uninitialize()
     print(json.dumps(result))
 

@@ -98,6 +98,12 @@ int32_t mf_moe_dispatch(const void *x, const int32_t *topk, uint32_t tokens, uin
 int32_t mf_moe_combine(const void *rows, const int32_t *rowOf, const float *weights, uint32_t tokens, uint32_t hidden,
                        uint32_t topK, void *y, void *stream);
 
+/* Yardstick kernels of known traffic (grid-stride, 128-bit, nontemporal): kind 0
+ * copies `bytes` from src to dst, kind 1 fills dst, kind 2 reads src (dst: a
+ * 4-byte device sink).  They measure what this GPU sustains for a flat copy, a
+ * pure write and a pure read, and calibrate hardware byte counters. */
+int32_t mf_probe_hbm(int32_t kind, void *dst, const void *src, uint64_t bytes, void *stream);
+
 /* ---- runtime services (thin layer over HIP) ------------------------------ */
 int mfrt_init(int device);
 void mfrt_shutdown(void);
@@ -124,6 +130,7 @@ int mfrt_event_done(void *event);
 float mfrt_event_elapsed_ms(void *start, void *stop);
 int mfrt_memcpy(void *dst, const void *src, uint64_t bytes);
 int mfrt_memset(void *dst, int value, uint64_t bytes);
+int mfrt_memcpy_async(void *dst, const void *src, uint64_t bytes, void *stream);
 
 /* ---- address registry view (HybmVaManager counterpart,
  *      src/hybm/csrc/mm/hybm_va_manager.h:175-264) -------------------------- */

@@ -4,6 +4,7 @@
 #include "../../../include/mf_hip_dataplane.h"
 #include "../../../include/mf_xcopy_types.h"
 #include "copy_direction.h"
+#include "../rt/mf_rt.h"
 #include "gva_layout.h"
 #include "mf_log.h"
 #include "va_manager.h"
@@ -16,7 +17,7 @@ using namespace mf;
 MF_EXPORT int32_t mf_xcopy_batch(const uint64_t *src, const uint64_t *dst, const uint64_t *len, uint32_t n,
                                  int32_t route, void *stream)
 {
-    if ((n != 0 && (src == nullptr || dst == nullptr || len == nullptr)) || route < 0 || route > MF_ROUTE_HBM_THROUGH) {
+    if ((n != 0 && (src == nullptr || dst == nullptr || len == nullptr)) || route < 0 || route > 21) {
         MF_FAIL(BM_INVALID_PARAM, "mf_xcopy_batch: null array or unknown route " << route);
     }
     return XcopyEngine::Instance().Submit(src, dst, len, n, route, stream, nullptr, 0);
@@ -28,6 +29,26 @@ MF_EXPORT int32_t mf_xcopy_device_table(const void *triples, uint32_t n, int32_t
         MF_FAIL(BM_INVALID_PARAM, "mf_xcopy_device_table: null table or unknown route " << route);
     }
     return XcopyEngine::Instance().SubmitDeviceTable(triples, n, route, stream, nullptr, 0);
+}
+
+MF_EXPORT int32_t mf_probe_hbm(int32_t kind, void *dst, const void *src, uint64_t bytes, void *stream)
+{
+    XcopyEngine &engine = XcopyEngine::Instance();
+    if (!engine.Started()) {
+        MF_FAIL(BM_NOT_INITIALIZED, "GPU data plane is not running; call hybm_init first");
+    }
+    if (kind < 0 || kind > 2 || dst == nullptr || (kind != 1 && src == nullptr) || bytes == 0 || bytes % 16 != 0) {
+        MF_FAIL(BM_INVALID_PARAM, "mf_probe_hbm: bad kind, null buffer or size not a multiple of 16");
+    }
+    if (stream == nullptr) {
+        stream = engine.ThreadStream();
+    }
+    const uint32_t grid = (mfrt_cu_count() == 0 ? 256 : mfrt_cu_count()) * 64;
+    int err = mfk_probe(kind, dst, src, bytes, grid, stream);
+    if (err != 0) {
+        MF_FAIL(BM_ERROR, "probe launch failed");
+    }
+    return BM_OK;
 }
 
 MF_EXPORT void *mf_xcopy_thread_stream(void)

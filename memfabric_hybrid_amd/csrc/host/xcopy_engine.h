@@ -43,7 +43,7 @@ void NormalizeSegments(const uint64_t *src, const uint64_t *dst, const uint64_t 
 struct XcopyTuning {
     uint32_t unitsOverride = 0;  // 16-byte units per chunk, 0 = choose from batch size
     uint32_t wgPerCu = 16;       // workgroups launched per CU for HBM routes (grid cap)
-    uint32_t wgPerCuLink = 2;    // the same for routes bound by the host link
+    uint32_t wgPerCuLink = 1;    // the same for routes bound by the host link
     uint32_t minUnits = kXcopyThreads;
     uint32_t maxUnits = 16 * kXcopyThreads;
 };

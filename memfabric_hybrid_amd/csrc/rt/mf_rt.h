@@ -57,6 +57,7 @@ float mfrt_event_elapsed_ms(void *start, void *stop);
 
 int mfrt_memcpy(void *dst, const void *src, uint64_t bytes);  /* blocking hipMemcpy, direction inferred */
 int mfrt_memset(void *dst, int value, uint64_t bytes);
+int mfrt_memcpy_async(void *dst, const void *src, uint64_t bytes, void *stream);  /* the runtime's own DMA path */
 
 /* ---- xcopy launchers (kernels/xcopy.hip) --------------------------------- */
 int mfk_xcopy_inline(const void *inlinePlan, int route, uint32_t grid, void *mask, uint32_t maskValue, void *counter,
@@ -76,6 +77,9 @@ int mfk_moe_combine(const void *rows, const void *rowOf, const void *weights, ui
 
 /* ---- 2-D copy launcher (kernels/copy2d.hip) ----------------------------------- */
 int mfk_copy2d(const void *rectPlan, uint32_t grid, void *stream);
+
+/* ---- yardstick kernels (kernels/probe.hip) ------------------------------------ */
+int mfk_probe(int kind, void *dst, const void *src, uint64_t bytes, uint32_t grid, void *stream);
 
 #ifndef MF_RT_HIDDEN
 #pragma GCC visibility pop

@@ -243,3 +243,8 @@ extern "C" int mfrt_memset(void *dst, int value, uint64_t bytes)
     }
     return Code(hipDeviceSynchronize());
 }
+
+extern "C" int mfrt_memcpy_async(void *dst, const void *src, uint64_t bytes, void *stream)
+{
+    return Code(hipMemcpyAsync(dst, src, bytes, hipMemcpyDefault, static_cast<hipStream_t>(stream)));
+}

@@ -204,6 +204,8 @@ _SIGNATURES = {
     "mfrt_event_elapsed_ms": (ctypes.c_float, [vp, vp]),
     "mfrt_memcpy": (ctypes.c_int, [vp, vp, u64]),
     "mfrt_memset": (ctypes.c_int, [vp, ctypes.c_int, u64]),
+    "mfrt_memcpy_async": (ctypes.c_int, [vp, vp, u64, vp]),
+    "mf_probe_hbm": (i32, [i32, vp, vp, u64, vp]),
     "mf_va_clear": (None, []),
     "mf_va_add": (i32, [u64, u64, i32, u64, u32]),
     "mf_va_add_external": (i32, [u64, u64, i32, u64, u32, u32]),
