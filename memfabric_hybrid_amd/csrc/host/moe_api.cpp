@@ -52,6 +52,9 @@ MF_EXPORT int32_t mf_moe_dispatch(const void *x, const int32_t *topk, uint32_t t
     if ((reinterpret_cast<uint64_t>(x) | reinterpret_cast<uint64_t>(out)) % 16 != 0) {
         MF_FAIL(BM_INVALID_PARAM, "mf_moe_dispatch: token buffers must be 16-byte aligned");
     }
+    if (reinterpret_cast<uint64_t>(workspace) % 16 != 0) {
+        MF_FAIL(BM_INVALID_PARAM, "mf_moe_dispatch: workspace must be 16-byte aligned");
+    }
     if (workspaceBytes < mfk_moe_workspace_bytes(tokens, topK, experts)) {
         MF_FAIL(BM_INVALID_PARAM, "mf_moe_dispatch: workspace of " << workspaceBytes << " bytes is too small");
     }

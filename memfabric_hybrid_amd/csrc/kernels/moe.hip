@@ -62,6 +62,13 @@ __device__ __forceinline__ void SliceHistograms(const int32_t *__restrict__ topk
     const uint32_t lane = threadIdx.x & 63u;
     const uint32_t wave = threadIdx.x >> 6;
     const uint32_t bits = BitsFor(experts);
+    // all expert ids of this lane are requested before anything waits on them
+    int32_t ids[kRankRounds];
+#pragma unroll
+    for (uint32_t r = 0; r < kRankRounds; ++r) {
+        const uint32_t idx = blockBase + (wave + r * (kRankThreads / 64)) * 64 + lane;
+        ids[r] = idx < total ? topk[idx] : -1;
+    }
     for (uint32_t i = threadIdx.x; i < kRankSlices * experts; i += kRankThreads) {
         hist[i] = 0;
     }
@@ -70,10 +77,7 @@ __device__ __forceinline__ void SliceHistograms(const int32_t *__restrict__ topk
     for (uint32_t r = 0; r < kRankRounds; ++r) {
         const uint32_t slice = wave + r * (kRankThreads / 64);
         const uint32_t idx = blockBase + slice * 64 + lane;
-        int32_t e = -1;
-        if (idx < total) {
-            e = topk[idx];
-        }
+        const int32_t e = ids[r];
         const bool valid = e >= 0 && static_cast<uint32_t>(e) < experts;
         if (idx < total && !valid) {
             *bad = 1;
@@ -91,7 +95,7 @@ __device__ __forceinline__ void SliceHistograms(const int32_t *__restrict__ topk
 
 __global__ __launch_bounds__(kRankThreads) void MoeHistKernel(const int32_t *__restrict__ topk, uint32_t total,
                                                               uint32_t experts, uint32_t *__restrict__ blockHist,
-                                                              uint32_t *__restrict__ blockBad)
+                                                              uint32_t histStride, uint32_t *__restrict__ blockBad)
 {
     extern __shared__ uint32_t hist[];
     uint32_t e[kRankRounds];
@@ -103,7 +107,12 @@ __global__ __launch_bounds__(kRankThreads) void MoeHistKernel(const int32_t *__r
         for (uint32_t s = 0; s < kRankSlices; ++s) {
             sum += hist[s * experts + x];
         }
-        blockHist[static_cast<uint64_t>(x) * gridDim.x + blockIdx.x] = sum;  // [expert][block]
+        blockHist[static_cast<uint64_t>(x) * histStride + blockIdx.x] = sum;  // [expert][block], rows padded to 4
+        if (blockIdx.x == 0) {
+            for (uint32_t pad = gridDim.x; pad < histStride; ++pad) {
+                blockHist[static_cast<uint64_t>(x) * histStride + pad] = 0;
+            }
+        }
     }
     // every block reports, so the flags need no clearing between calls
     const uint32_t anyBad = __syncthreads_or(static_cast<int>(bad)) != 0 ? 1u : 0u;
@@ -114,7 +123,7 @@ __global__ __launch_bounds__(kRankThreads) void MoeHistKernel(const int32_t *__r
 
 __global__ __launch_bounds__(kRankThreads) void MoeRankKernel(const int32_t *__restrict__ topk, uint32_t total,
                                                               uint32_t experts, const uint32_t *__restrict__ blockHist,
-                                                              int32_t *__restrict__ counts, int32_t *__restrict__ offsets,
+                                                              uint32_t histStride, int32_t *__restrict__ counts, int32_t *__restrict__ offsets,
                                                               int32_t *__restrict__ rowOf, int32_t *__restrict__ srcOf,
                                                               const uint32_t *__restrict__ blockBad,
                                                               uint32_t *__restrict__ status)
@@ -128,12 +137,15 @@ __global__ __launch_bounds__(kRankThreads) void MoeRankKernel(const int32_t *__r
     uint32_t bad = 0;
     SliceHistograms(topk, total, experts, blockIdx.x * kRankBlock, hist, myExpert, myRank, &bad);
 
-    if (blockIdx.x == 0 && threadIdx.x == 0) {
+    if (blockIdx.x == 0) {
         uint32_t any = 0;
-        for (uint32_t blk = 0; blk < gridDim.x; ++blk) {
+        for (uint32_t blk = threadIdx.x; blk < gridDim.x; blk += kRankThreads) {
             any |= blockBad[blk];
         }
-        status[0] = any;  // 1: some expert id was outside [0, experts); those entries got row -1
+        any = __syncthreads_or(static_cast<int>(any)) != 0 ? 1u : 0u;
+        if (threadIdx.x == 0) {
+            status[0] = any;  // 1: some expert id was outside [0, experts); those entries got row -1
+        }
     }
     // totals and "entries of earlier blocks" per expert
     uint32_t tot[kMaxExperts / kRankThreads];
@@ -149,31 +161,40 @@ __global__ __launch_bounds__(kRankThreads) void MoeRankKernel(const int32_t *__r
     for (uint32_t j = 0; j < per; ++j) {
         const uint32_t x = threadIdx.x * per + j;
         if (x < experts) {
-            // one contiguous row of the [expert][block] table per expert: independent, coalescable loads
-            const uint32_t *rowHist = blockHist + static_cast<uint64_t>(x) * gridDim.x;
+            // one contiguous row of the [expert][block] table per expert, fetched 16 bytes at a time
+            const uint32_t *rowHist = blockHist + static_cast<uint64_t>(x) * histStride;
             uint32_t t = 0;
             uint32_t b = 0;
-#pragma unroll 16
-            for (uint32_t blk = 0; blk < gridDim.x; ++blk) {
-                const uint32_t v = rowHist[blk];
-                t += v;
-                b += blk < blockIdx.x ? v : 0u;
+            for (uint32_t blk = 0; blk < gridDim.x; blk += 4) {
+                const u32x4 v = *reinterpret_cast<const u32x4 *>(rowHist + blk);  // padded with zeros up to histStride
+#pragma unroll
+                for (uint32_t i = 0; i < 4; ++i) {
+                    t += v[i];
+                    b += blk + i < blockIdx.x ? v[i] : 0u;
+                }
             }
             tot[j] = t;
             before[j] = b;
             mine += t;
         }
     }
-    // exclusive scan of `mine` over the 256 threads
-    scan[threadIdx.x] = mine;
-    __syncthreads();
-    for (uint32_t step = 1; step < kRankThreads; step <<= 1) {
-        const uint32_t add = threadIdx.x >= step ? scan[threadIdx.x - step] : 0u;
-        __syncthreads();
-        scan[threadIdx.x] += add;
-        __syncthreads();
+    // exclusive scan of `mine` over the 256 threads: shuffles inside each wave, LDS across the four waves
+    uint32_t incl = mine;
+#pragma unroll
+    for (uint32_t step = 1; step < 64; step <<= 1) {
+        const uint32_t up = __shfl_up(incl, step, 64);
+        incl += (threadIdx.x & 63u) >= step ? up : 0u;
     }
-    uint32_t run = scan[threadIdx.x] - mine;
+    if ((threadIdx.x & 63u) == 63u) {
+        scan[threadIdx.x >> 6] = incl;
+    }
+    __syncthreads();
+    uint32_t waveBase = 0;
+    for (uint32_t wv = 0; wv < (threadIdx.x >> 6); ++wv) {
+        waveBase += scan[wv];
+    }
+    incl += waveBase;
+    uint32_t run = incl - mine;
     for (uint32_t j = 0; j < per; ++j) {
         const uint32_t x = threadIdx.x * per + j;
         if (x < experts) {
@@ -232,9 +253,13 @@ __device__ __forceinline__ void RowStore(MF_GLOBAL u32x4 *p, u32x4 v)
 template <uint32_t kThreads, uint32_t kHold, int kMode>
 __global__ __launch_bounds__(kThreads) void MoePermuteKernel(const u32x4 *__restrict__ x,
                                                              const int32_t *__restrict__ rowOf, uint32_t topK,
-                                                             uint32_t unitsPerRow, u32x4 *__restrict__ out)
+                                                             uint32_t unitsPerRow, uint32_t parts, u32x4 *__restrict__ out)
 {
-    const uint32_t token = blockIdx.x;
+    const uint32_t token = blockIdx.x / parts;
+    const uint32_t part = blockIdx.x - token * parts;
+    const uint32_t perPart = (unitsPerRow + parts - 1) / parts;
+    const uint32_t begin = part * perPart;
+    const uint32_t end = begin + perPart < unitsPerRow ? begin + perPart : unitsPerRow;
     const MF_GLOBAL u32x4 *src = reinterpret_cast<const MF_GLOBAL u32x4 *>(reinterpret_cast<uint64_t>(x)) +
                                  static_cast<uint64_t>(token) * unitsPerRow;
     int32_t rows[kMaxTopK];
@@ -242,12 +267,12 @@ __global__ __launch_bounds__(kThreads) void MoePermuteKernel(const u32x4 *__rest
     for (uint32_t k = 0; k < kMaxTopK; ++k) {
         rows[k] = k < topK ? rowOf[static_cast<uint64_t>(token) * topK + k] : -1;
     }
-    for (uint32_t u0 = 0; u0 < unitsPerRow; u0 += kHold * kThreads) {
+    for (uint32_t u0 = begin; u0 < end; u0 += kHold * kThreads) {
         u32x4 v[kHold];
 #pragma unroll
         for (uint32_t j = 0; j < kHold; ++j) {
             const uint32_t u = u0 + j * kThreads + threadIdx.x;
-            if (u < unitsPerRow) {
+            if (u < end) {
                 v[j] = __builtin_nontemporal_load(src + u);
             }
         }
@@ -259,7 +284,7 @@ __global__ __launch_bounds__(kThreads) void MoePermuteKernel(const u32x4 *__rest
 #pragma unroll
                 for (uint32_t j = 0; j < kHold; ++j) {
                     const uint32_t u = u0 + j * kThreads + threadIdx.x;
-                    if (u < unitsPerRow) {
+                    if (u < end) {
                         RowStore<kMode>(dst + u, v[j]);
                     }
                 }
@@ -288,13 +313,17 @@ __device__ __forceinline__ uint32_t ToBf16(float f)
     return (w + 0x7FFFu + ((w >> 16) & 1u)) >> 16;
 }
 
-template <uint32_t kTopK>
-__global__ __launch_bounds__(kRowThreads) void MoeCombineKernel(const u32x4 *__restrict__ rowsIn,
-                                                                const int32_t *__restrict__ rowOf,
-                                                                const float *__restrict__ weights, uint32_t topK,
-                                                                uint32_t unitsPerRow, u32x4 *__restrict__ y)
+template <uint32_t kTopK, uint32_t kThreads, bool kNtLoad>
+__global__ __launch_bounds__(kThreads) void MoeCombineKernel(const u32x4 *__restrict__ rowsIn,
+                                                             const int32_t *__restrict__ rowOf,
+                                                             const float *__restrict__ weights, uint32_t topK,
+                                                             uint32_t unitsPerRow, uint32_t parts, u32x4 *__restrict__ y)
 {
-    const uint32_t token = blockIdx.x;
+    const uint32_t token = blockIdx.x / parts;
+    const uint32_t part = blockIdx.x - token * parts;
+    const uint32_t perPart = (unitsPerRow + parts - 1) / parts;
+    const uint32_t begin = part * perPart;
+    const uint32_t end = begin + perPart < unitsPerRow ? begin + perPart : unitsPerRow;
     const uint32_t nk = kTopK != 0 ? kTopK : topK;
     constexpr uint32_t kSlots = kTopK != 0 ? kTopK : kMaxTopK;
     uint64_t rowBase[kSlots];
@@ -311,13 +340,14 @@ __global__ __launch_bounds__(kRowThreads) void MoeCombineKernel(const u32x4 *__r
         }
     }
     const MF_GLOBAL u32x4 *in = reinterpret_cast<const MF_GLOBAL u32x4 *>(reinterpret_cast<uint64_t>(rowsIn));
-    MF_GLOBAL u32x4 *dst = reinterpret_cast<MF_GLOBAL u32x4 *>(reinterpret_cast<uint64_t>(y)) + static_cast<uint64_t>(token) * unitsPerRow;
-    for (uint32_t u = threadIdx.x; u < unitsPerRow; u += kRowThreads) {
+    MF_GLOBAL u32x4 *dst = reinterpret_cast<MF_GLOBAL u32x4 *>(reinterpret_cast<uint64_t>(y)) +
+                           static_cast<uint64_t>(token) * unitsPerRow;
+    for (uint32_t u = begin + threadIdx.x; u < end; u += kThreads) {
         u32x4 v[kSlots];
 #pragma unroll
         for (uint32_t k = 0; k < kSlots; ++k) {
             if (k < nk) {
-                v[k] = __builtin_nontemporal_load(in + rowBase[k] + u);
+                v[k] = kNtLoad ? __builtin_nontemporal_load(in + rowBase[k] + u) : in[rowBase[k] + u];
             }
         }
         float acc[8];
@@ -348,16 +378,19 @@ __global__ __launch_bounds__(kRowThreads) void MoeCombineKernel(const u32x4 *__r
 }  // namespace mf
 
 static int g_permuteVariant = -1;  // -1: choose from the row width
-extern "C" void mfk_moe_tune(int permuteVariant)
+static int g_combineVariant = 0;
+extern "C" void mfk_moe_tune(int permuteVariant, int combineVariant)
 {
     g_permuteVariant = permuteVariant;
+    g_combineVariant = combineVariant;
 }
 
 extern "C" uint64_t mfk_moe_workspace_bytes(uint32_t tokens, uint32_t topK, uint32_t experts)
 {
     const uint64_t total = static_cast<uint64_t>(tokens) * topK;
     const uint64_t blocks = (total + mf::kRankBlock - 1) / mf::kRankBlock;
-    return 256 + blocks * sizeof(uint32_t) + blocks * experts * sizeof(uint32_t);
+    const uint64_t stride = (blocks + 3) / 4 * 4;
+    return 256 + stride * sizeof(uint32_t) + stride * experts * sizeof(uint32_t);
 }
 
 extern "C" int mfk_moe_dispatch(const void *x, const void *topk, uint32_t tokens, uint32_t hidden, uint32_t topK,
@@ -374,27 +407,46 @@ extern "C" int mfk_moe_dispatch(const void *x, const void *topk, uint32_t tokens
     const uint32_t blocks = (total + kRankBlock - 1) / kRankBlock;
     hipStream_t s = static_cast<hipStream_t>(stream);
     uint32_t *status = static_cast<uint32_t *>(workspace);
+    const uint32_t histStride = (blocks + 3) / 4 * 4;     // rows of the [expert][block] table, 16-byte granular
     uint32_t *blockBad = status + 64;
-    uint32_t *blockHist = blockBad + blocks;
+    uint32_t *blockHist = blockBad + histStride;
     const size_t histLds = static_cast<size_t>(kRankSlices) * experts * sizeof(uint32_t);
     const size_t rankLds = histLds + (experts + kRankThreads) * sizeof(uint32_t);
     hipLaunchKernelGGL(MoeHistKernel, dim3(blocks), dim3(kRankThreads), histLds, s, static_cast<const int32_t *>(topk),
-                       total, experts, blockHist, blockBad);
+                       total, experts, blockHist, histStride, blockBad);
     hipLaunchKernelGGL(MoeRankKernel, dim3(blocks), dim3(kRankThreads), rankLds, s, static_cast<const int32_t *>(topk),
-                       total, experts, blockHist, static_cast<int32_t *>(counts), static_cast<int32_t *>(offsets),
+                       total, experts, blockHist, histStride, static_cast<int32_t *>(counts), static_cast<int32_t *>(offsets),
                        static_cast<int32_t *>(rowOf), static_cast<int32_t *>(srcOf), blockBad, status);
     if (x != nullptr && out != nullptr && hidden != 0) {
         const u32x4 *xi = static_cast<const u32x4 *>(x);
         const int32_t *ro = static_cast<const int32_t *>(rowOf);
         u32x4 *oo = static_cast<u32x4 *>(out);
         const uint32_t upr = hidden / 8;
-        // One wave per token holding the whole row (14 pieces per lane covers 7168 elements)
-        // measured best for wide rows; narrow rows use four waves with fewer pieces each.
-        const int variant = g_permuteVariant >= 0 ? g_permuteVariant : (upr >= 512 ? 1 : 0);
-        if (variant == 1) {
-            hipLaunchKernelGGL((MoePermuteKernel<64, 14, 1>), dim3(tokens), dim3(64), 0, s, xi, ro, topK, upr, oo);
-        } else {
-            hipLaunchKernelGGL((MoePermuteKernel<256, 4, 1>), dim3(tokens), dim3(256), 0, s, xi, ro, topK, upr, oo);
+        // wide rows: two single-wave workgroups per token, 7 pieces per lane, plain stores (fastest of the
+        // shapes measured on 7168-element rows); narrow rows: one four-wave workgroup per token
+        const int variant = g_permuteVariant >= 0 ? g_permuteVariant : (upr >= 512 ? 6 : 0);
+        switch (variant) {
+            case 1:
+                hipLaunchKernelGGL((MoePermuteKernel<64, 14, 1>), dim3(tokens), dim3(64), 0, s, xi, ro, topK, upr, 1u, oo);
+                break;
+            case 2:
+                hipLaunchKernelGGL((MoePermuteKernel<64, 7, 1>), dim3(tokens * 2), dim3(64), 0, s, xi, ro, topK, upr, 2u, oo);
+                break;
+            case 3:
+                hipLaunchKernelGGL((MoePermuteKernel<64, 4, 1>), dim3(tokens * 4), dim3(64), 0, s, xi, ro, topK, upr, 4u, oo);
+                break;
+            case 4:
+                hipLaunchKernelGGL((MoePermuteKernel<64, 2, 1>), dim3(tokens * 7), dim3(64), 0, s, xi, ro, topK, upr, 7u, oo);
+                break;
+            case 5:
+                hipLaunchKernelGGL((MoePermuteKernel<64, 7, 2>), dim3(tokens * 2), dim3(64), 0, s, xi, ro, topK, upr, 2u, oo);
+                break;
+            case 6:
+                hipLaunchKernelGGL((MoePermuteKernel<64, 7, 0>), dim3(tokens * 2), dim3(64), 0, s, xi, ro, topK, upr, 2u, oo);
+                break;
+            default:
+                hipLaunchKernelGGL((MoePermuteKernel<256, 4, 1>), dim3(tokens), dim3(256), 0, s, xi, ro, topK, upr, 1u, oo);
+                break;
         }
     }
     return static_cast<int>(hipGetLastError());
@@ -412,10 +464,33 @@ extern "C" int mfk_moe_combine(const void *rows, const void *rowOf, const void *
     const int32_t *ro = static_cast<const int32_t *>(rowOf);
     const float *w = static_cast<const float *>(weights);
     u32x4 *o = static_cast<u32x4 *>(y);
+    const uint32_t upr = hidden / 8;
     if (topK == 8) {
-        hipLaunchKernelGGL(MoeCombineKernel<8>, dim3(tokens), dim3(kRowThreads), 0, s, in, ro, w, topK, hidden / 8, o);
+        switch (g_combineVariant) {
+            case 1:
+                hipLaunchKernelGGL((MoeCombineKernel<8, 128, true>), dim3(tokens), dim3(128), 0, s, in, ro, w, topK, upr, 1u, o);
+                break;
+            case 2:
+                hipLaunchKernelGGL((MoeCombineKernel<8, 64, true>), dim3(tokens), dim3(64), 0, s, in, ro, w, topK, upr, 1u, o);
+                break;
+            case 3:
+                hipLaunchKernelGGL((MoeCombineKernel<8, 64, true>), dim3(tokens * 2), dim3(64), 0, s, in, ro, w, topK, upr, 2u, o);
+                break;
+            case 4:
+                hipLaunchKernelGGL((MoeCombineKernel<8, 256, false>), dim3(tokens), dim3(256), 0, s, in, ro, w, topK, upr, 1u, o);
+                break;
+            case 5:
+                hipLaunchKernelGGL((MoeCombineKernel<8, 64, true>), dim3(tokens * 4), dim3(64), 0, s, in, ro, w, topK, upr, 4u, o);
+                break;
+            case 6:
+                hipLaunchKernelGGL((MoeCombineKernel<8, 128, true>), dim3(tokens * 2), dim3(128), 0, s, in, ro, w, topK, upr, 2u, o);
+                break;
+            default:
+                hipLaunchKernelGGL((MoeCombineKernel<8, 256, true>), dim3(tokens), dim3(256), 0, s, in, ro, w, topK, upr, 1u, o);
+                break;
+        }
     } else {
-        hipLaunchKernelGGL(MoeCombineKernel<0>, dim3(tokens), dim3(kRowThreads), 0, s, in, ro, w, topK, hidden / 8, o);
+        hipLaunchKernelGGL((MoeCombineKernel<0, 256, true>), dim3(tokens), dim3(256), 0, s, in, ro, w, topK, upr, 1u, o);
     }
     return static_cast<int>(hipGetLastError());
 }

@@ -219,17 +219,23 @@ __global__ __launch_bounds__(kXcopyThreads) void XcopyTableKernel(const uint64_t
                                                                   uint32_t maskValue, uint32_t *counter)
 {
     const uint32_t nchunk = nchunkDev != nullptr ? *nchunkDev : nchunkHost;
+    const uint32_t lane = threadIdx.x & 63u;
     for (uint32_t c = blockIdx.x; c < nchunk; c += gridDim.x) {
-        // upper_bound(first, c) - 1 over nseg + 1 prefix entries
+        // 64-ary search for the last prefix entry <= c: every level is one load per lane and a
+        // ballot, so 4096 segments resolve in two memory round trips (a binary search by one
+        // lane would chain twelve).  Invariant: first[lo] <= c < first[hi].
         uint32_t lo = 0;
-        uint32_t hi = nseg;  // invariant: first[lo] <= c < first[hi]
+        uint32_t hi = nseg;
         while (hi - lo > 1) {
-            const uint32_t mid = (lo + hi) >> 1;
-            if (first[mid] <= c) {
-                lo = mid;
-            } else {
-                hi = mid;
-            }
+            const uint32_t span = hi - lo;
+            const uint32_t step = (span + 63u) >> 6;            // entries per lane at this level
+            const uint32_t probe = lo + (lane + 1) * step;      // lanes probe lo+step, lo+2*step, ...
+            const bool inside = probe < hi;
+            const uint32_t v = inside ? first[probe] : 0xFFFFFFFFu;
+            const uint32_t hits = __popcll(__ballot(inside && v <= c));
+            lo += hits * step;
+            const uint32_t cap = lo + step;
+            hi = cap < hi ? cap : hi;
         }
         const uint64_t *t = triples + 3ull * lo;
         CopyChunk<kNtLoad, kStore>(t[0], t[1], t[2], c - first[lo], units);

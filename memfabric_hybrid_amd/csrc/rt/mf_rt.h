@@ -69,7 +69,7 @@ int mfk_xcopy_plan(const void *triples, uint32_t nseg, uint32_t units, void *fir
 
 /* ---- MoE launchers (kernels/moe.hip) ---------------------------------------- */
 uint64_t mfk_moe_workspace_bytes(uint32_t tokens, uint32_t topK, uint32_t experts);
-void mfk_moe_tune(int permuteVariant);
+void mfk_moe_tune(int permuteVariant, int combineVariant);
 int mfk_moe_dispatch(const void *x, const void *topk, uint32_t tokens, uint32_t hidden, uint32_t topK, uint32_t experts,
                      void *out, void *counts, void *offsets, void *rowOf, void *srcOf, void *workspace, void *stream);
 int mfk_moe_combine(const void *rows, const void *rowOf, const void *weights, uint32_t tokens, uint32_t hidden,
