@@ -79,14 +79,14 @@ ComposeDataOp::Ranked ComposeDataOp::Prioritised(const ExtOptions &) const
     const uint32_t reach = static_cast<uint32_t>(options_.bmDataOpType);
     Ranked out;
     if (intraNode_ != nullptr && (reach & HYBM_DOP_TYPE_SDMA) != 0) {
-        out.emplace_back(HYBM_DOP_TYPE_SDMA, intraNode_);
+        out.emplace_back(HYBM_DOP_TYPE_SDMA, intraNode_.get());
     }
     if (deviceRdma_ != nullptr && (reach & HYBM_DOP_TYPE_DEVICE_RDMA) != 0) {
-        out.emplace_back(HYBM_DOP_TYPE_DEVICE_RDMA, deviceRdma_);
+        out.emplace_back(HYBM_DOP_TYPE_DEVICE_RDMA, deviceRdma_.get());
     }
     for (hybm_data_op_type t : {HYBM_DOP_TYPE_HOST_RDMA, HYBM_DOP_TYPE_HOST_URMA, HYBM_DOP_TYPE_HOST_TCP}) {
         if (hostNet_ != nullptr && (reach & t) != 0) {
-            out.emplace_back(t, hostNet_);
+            out.emplace_back(t, hostNet_.get());
         }
     }
     return out;

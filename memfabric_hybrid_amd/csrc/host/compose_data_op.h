@@ -26,7 +26,27 @@ class ComposeDataOp : public ock::mf::DataOperator {
 public:
     using Result = ock::mf::Result;
     using ExtOptions = ock::mf::ExtOptions;
-    using Ranked = std::vector<std::pair<hybm_data_op_type, ock::mf::DataOperatorPtr>>;
+    // Engines in order of preference; raw pointers, the members below keep them alive.
+    struct Ranked {
+        std::pair<hybm_data_op_type, ock::mf::DataOperator *> item[5];
+        uint32_t count = 0;
+        bool empty() const
+        {
+            return count == 0;
+        }
+        const std::pair<hybm_data_op_type, ock::mf::DataOperator *> *begin() const
+        {
+            return item;
+        }
+        const std::pair<hybm_data_op_type, ock::mf::DataOperator *> *end() const
+        {
+            return item + count;
+        }
+        void emplace_back(hybm_data_op_type t, ock::mf::DataOperator *op)
+        {
+            item[count++] = {t, op};
+        }
+    };
 
     ComposeDataOp(const hybm_options &options, OperatorFactory factory);
     ~ComposeDataOp() override;

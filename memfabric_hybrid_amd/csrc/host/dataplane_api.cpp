@@ -1,4 +1,5 @@
 // Native C entry points declared in include/mf_hip_dataplane.h.
+#include <cstring>
 #include <vector>
 
 #include "../../../include/mf_hip_dataplane.h"
@@ -92,6 +93,14 @@ MF_EXPORT int64_t mf_xcopy_describe_plan(const uint64_t *src, const uint64_t *ds
     const bool fits = BuildInlinePlan(segs, units, plan);
     if (inlineForm != nullptr) {
         *inlineForm = fits ? 1 : 0;
+    }
+    {
+        // the one-pass planner of the submission path must produce the very same plan
+        InlinePlan direct;
+        const bool directFits = BuildInlineDirect(src, dst, len, n, units, direct);
+        if (directFits && (!fits || std::memcmp(&direct, &plan, sizeof(plan)) != 0)) {
+            return -2;
+        }
     }
     std::vector<uint64_t> triples(3ull * segs.Size() + 3);
     std::vector<uint32_t> first(segs.Size() + 1);

@@ -291,13 +291,13 @@ EntityRegistry &EntityRegistry::Instance()
 
 void EntityRegistry::SetFactory(OperatorFactory factory)
 {
-    std::lock_guard<std::mutex> guard(lock_);
+    std::unique_lock<std::shared_mutex> guard(lock_);
     factory_ = std::move(factory);
 }
 
 std::shared_ptr<MemEntity> EntityRegistry::Create(uint16_t id, const hybm_options &options, int &result)
 {
-    std::lock_guard<std::mutex> guard(lock_);
+    std::unique_lock<std::shared_mutex> guard(lock_);
     if (byId_.count(id) != 0) {
         result = BM_ERROR;
         MF_ERROR("pool id " << id << " already exists");
@@ -309,47 +309,38 @@ std::shared_ptr<MemEntity> EntityRegistry::Create(uint16_t id, const hybm_option
         return nullptr;
     }
     byId_[id] = entity;
-    byPtr_[entity.get()] = id;
+    byPtr_[entity.get()] = entity;
     return entity;
 }
 
 std::shared_ptr<MemEntity> EntityRegistry::FindById(uint16_t id)
 {
-    std::lock_guard<std::mutex> guard(lock_);
+    std::shared_lock<std::shared_mutex> guard(lock_);
     auto it = byId_.find(id);
     return it == byId_.end() ? nullptr : it->second;
 }
 
 std::shared_ptr<MemEntity> EntityRegistry::FindByPtr(const void *handle)
 {
-    std::lock_guard<std::mutex> guard(lock_);
+    std::shared_lock<std::shared_mutex> guard(lock_);
     auto it = byPtr_.find(handle);
-    if (it == byPtr_.end()) {
-        return nullptr;
-    }
-    auto e = byId_.find(it->second);
-    return e == byId_.end() ? nullptr : e->second;
+    return it == byPtr_.end() ? nullptr : it->second;
 }
 
 bool EntityRegistry::Remove(const void *handle)
 {
     std::shared_ptr<MemEntity> victim;
     {
-        std::lock_guard<std::mutex> guard(lock_);
+        std::unique_lock<std::shared_mutex> guard(lock_);
         auto it = byPtr_.find(handle);
         if (it == byPtr_.end()) {
             return false;
         }
-        auto e = byId_.find(it->second);
-        if (e != byId_.end()) {
-            victim = e->second;
-            byId_.erase(e);
-        }
+        victim = it->second;
+        byId_.erase(victim->Id());
         byPtr_.erase(it);
     }
-    if (victim != nullptr) {
-        victim->UnInitialize();
-    }
+    victim->UnInitialize();
     return true;
 }
 
@@ -357,7 +348,7 @@ void EntityRegistry::Clear()
 {
     std::map<uint16_t, std::shared_ptr<MemEntity>> victims;
     {
-        std::lock_guard<std::mutex> guard(lock_);
+        std::unique_lock<std::shared_mutex> guard(lock_);
         victims.swap(byId_);
         byPtr_.clear();
     }

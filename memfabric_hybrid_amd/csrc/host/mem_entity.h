@@ -9,6 +9,8 @@
 #include <map>
 #include <memory>
 #include <mutex>
+#include <shared_mutex>
+#include <unordered_map>
 #include <utility>
 
 #include "compose_data_op.h"
@@ -81,9 +83,9 @@ public:
     void SetFactory(OperatorFactory factory);
 
 private:
-    std::mutex lock_;
+    std::shared_mutex lock_;
     std::map<uint16_t, std::shared_ptr<MemEntity>> byId_;
-    std::map<const void *, uint16_t> byPtr_;
+    std::unordered_map<const void *, std::shared_ptr<MemEntity>> byPtr_;
     OperatorFactory factory_ = OperatorFactory::Default();
 };
 

@@ -9,6 +9,7 @@
 #include <memory>
 #include <mutex>
 #include <shared_mutex>
+#include <unordered_map>
 
 #include "../../../include/mf_xcopy_api.h"
 #include "copy_direction.h"
@@ -212,19 +213,15 @@ private:
 std::shared_mutex g_lock;
 bool g_inited = false;
 uint16_t g_deviceId = 0;
-std::mutex g_entriesLock;
+std::shared_mutex g_entriesLock;
 std::map<uint32_t, std::shared_ptr<BmEntry>> g_entriesById;
-std::map<const void *, uint32_t> g_entriesByPtr;
+std::unordered_map<const void *, std::shared_ptr<BmEntry>> g_entriesByPtr;
 
 std::shared_ptr<BmEntry> FindEntry(smem_bm_t handle)
 {
-    std::lock_guard<std::mutex> guard(g_entriesLock);
+    std::shared_lock<std::shared_mutex> guard(g_entriesLock);
     auto it = g_entriesByPtr.find(handle);
-    if (it == g_entriesByPtr.end()) {
-        return nullptr;
-    }
-    auto e = g_entriesById.find(it->second);
-    return e == g_entriesById.end() ? nullptr : e->second;
+    return it == g_entriesByPtr.end() ? nullptr : it->second;
 }
 
 bool ConfigValid(const smem_bm_config_t *c)
@@ -277,7 +274,7 @@ MF_EXPORT void smem_bm_uninit(uint32_t flags)
         return;
     }
     {
-        std::lock_guard<std::mutex> entries(g_entriesLock);
+        std::unique_lock<std::shared_mutex> entries(g_entriesLock);
         g_entriesByPtr.clear();
         g_entriesById.clear();  // releases every pool
     }
@@ -316,14 +313,14 @@ MF_EXPORT smem_bm_t smem_bm_create2(uint32_t id, const smem_bm_create_option_t *
     }
     std::shared_ptr<BmEntry> entry;
     {
-        std::lock_guard<std::mutex> entries(g_entriesLock);
+        std::unique_lock<std::shared_mutex> entries(g_entriesLock);
         if (g_entriesById.count(id) != 0) {
             MF_ERROR("smem_bm_create2: pool id " << id << " exists");
             return nullptr;
         }
         entry = std::make_shared<BmEntry>(id);
         g_entriesById[id] = entry;
-        g_entriesByPtr[entry.get()] = id;
+        g_entriesByPtr[entry.get()] = entry;
     }
     hybm_options options{};
     options.bmType = HYBM_TYPE_HOST_INITIATE;
@@ -352,7 +349,7 @@ MF_EXPORT smem_bm_t smem_bm_create2(uint32_t id, const smem_bm_create_option_t *
     std::memcpy(options.tag, option->tag, sizeof(options.tag));
     std::memcpy(options.tagOpInfo, option->tagOpInfo, sizeof(options.tagOpInfo));
     if (entry->Initialize(options) != SM_OK) {
-        std::lock_guard<std::mutex> entries(g_entriesLock);
+        std::unique_lock<std::shared_mutex> entries(g_entriesLock);
         g_entriesByPtr.erase(entry.get());
         g_entriesById.erase(id);
         return nullptr;
@@ -386,15 +383,17 @@ MF_EXPORT void smem_bm_destroy(smem_bm_t handle)
     }
     std::shared_ptr<BmEntry> entry;
     {
-        std::lock_guard<std::mutex> entries(g_entriesLock);
+        std::unique_lock<std::shared_mutex> entries(g_entriesLock);
         auto it = g_entriesByPtr.find(handle);
         if (it == g_entriesByPtr.end()) {
             return;
         }
-        auto e = g_entriesById.find(it->second);
-        if (e != g_entriesById.end()) {
-            entry = e->second;
-            g_entriesById.erase(e);
+        entry = it->second;
+        for (auto e = g_entriesById.begin(); e != g_entriesById.end(); ++e) {
+            if (e->second == entry) {
+                g_entriesById.erase(e);
+                break;
+            }
         }
         g_entriesByPtr.erase(it);
     }

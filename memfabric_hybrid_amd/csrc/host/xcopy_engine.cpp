@@ -215,6 +215,73 @@ bool BuildInlinePlan(const SegList &segs, uint32_t units, InlinePlan &plan)
     return true;
 }
 
+// Normalisation and inline planning in one pass over the caller's arrays, for the common case
+// of a batch that ends up with at most kInlineSegs segments below 4 GiB each.  Returns false
+// (plan contents undefined) when the batch needs the general path.
+bool BuildInlineDirect(const uint64_t *src, const uint64_t *dst, const uint64_t *len, uint32_t n, uint32_t units,
+                       InlinePlan &plan)
+{
+    const bool pow2 = (units & (units - 1)) == 0;
+    const uint32_t shift = pow2 ? static_cast<uint32_t>(__builtin_ctz(units)) : 0;
+    uint32_t used = 0;
+    uint64_t run = 0;
+    uint64_t curSrc = 0;
+    uint64_t curDst = 0;
+    uint64_t curLen = 0;
+    auto flush = [&]() -> bool {
+        if (curLen == 0) {
+            return true;
+        }
+        if (used == kInlineSegs || curLen > 0xFFFFFFFFull) {
+            return false;
+        }
+        uint64_t head = (0 - curDst) & (kUnitBytes - 1);
+        if (head > curLen) {
+            head = curLen;
+        }
+        const uint64_t body = (curLen - head) / kUnitBytes;
+        uint64_t chunks = pow2 ? (body + units - 1) >> shift : (body + units - 1) / units;
+        if (chunks == 0) {
+            chunks = 1;
+        }
+        plan.src[used] = curSrc;
+        plan.dst[used] = curDst;
+        plan.len[used] = static_cast<uint32_t>(curLen);
+        plan.first[used] = static_cast<uint32_t>(run);
+        run += chunks;
+        ++used;
+        return true;
+    };
+    for (uint32_t i = 0; i < n; ++i) {
+        const uint64_t l = len[i];
+        if (l == 0) {
+            continue;
+        }
+        if (curLen > 0 && curSrc + curLen == src[i] && curDst + curLen == dst[i]) {
+            curLen += l;
+            continue;
+        }
+        if (!flush()) {
+            return false;
+        }
+        curSrc = src[i];
+        curDst = dst[i];
+        curLen = l;
+    }
+    if (!flush() || run >= kNoChunk) {
+        return false;
+    }
+    for (uint32_t i = used; i < kInlineSegs; ++i) {
+        plan.src[i] = 0;
+        plan.dst[i] = 0;
+        plan.len[i] = 0;
+        plan.first[i] = kNoChunk;
+    }
+    plan.nchunk = static_cast<uint32_t>(run);
+    plan.units = units;
+    return true;
+}
+
 uint64_t BuildTablePlan(const SegList &segs, uint32_t units, uint64_t *triples, uint32_t *first)
 {
     const uint32_t n = segs.Size();
@@ -332,13 +399,25 @@ int XcopyEngine::Submit(const uint64_t *src, const uint64_t *dst, const uint64_t
         }
     }
     ThreadCtx &ctx = t_ctx;
-    NormalizeSegments(src, dst, len, n, kInlinePiece, ctx.segs);
     const uint32_t cu = mfrt_cu_count();
-    const uint32_t units = ChooseUnits(ctx.segs.totalBytes, cu, route, tuning_);
     void *counter = mask != nullptr ? NextCounter() : nullptr;
-
     InlinePlan plan;
-    if (BuildInlinePlan(ctx.segs, units, plan)) {
+    bool inlined = false;
+    uint32_t units = 0;
+    if (n <= 4 * kInlineSegs) {  // small enough that a failed attempt costs next to nothing
+        uint64_t total = 0;
+        for (uint32_t i = 0; i < n; ++i) {
+            total += len[i];
+        }
+        units = ChooseUnits(total, cu, route, tuning_);
+        inlined = BuildInlineDirect(src, dst, len, n, units, plan);
+    }
+    if (!inlined) {
+        NormalizeSegments(src, dst, len, n, kInlinePiece, ctx.segs);
+        units = ChooseUnits(ctx.segs.totalBytes, cu, route, tuning_);
+        inlined = BuildInlinePlan(ctx.segs, units, plan);
+    }
+    if (inlined) {
         const uint32_t grid = GridFor(plan.nchunk, cu, route, tuning_);
         int err = mfk_xcopy_inline(&plan, route, grid, mask, maskValue, counter, stream);
         if (err != 0) {

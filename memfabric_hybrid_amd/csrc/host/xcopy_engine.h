@@ -53,6 +53,12 @@ uint32_t ChooseUnits(uint64_t totalBytes, uint32_t cuCount, int route, const Xco
 // Returns false when the list does not fit the inline form.
 bool BuildInlinePlan(const SegList &segs, uint32_t units, InlinePlan &plan);
 
+// The same result as NormalizeSegments + BuildInlinePlan in one pass over the caller's arrays;
+// false when the batch does not fit the inline form (more than kInlineSegs merged segments, or
+// one of 4 GiB and more, which the general path cuts into pieces).
+bool BuildInlineDirect(const uint64_t *src, const uint64_t *dst, const uint64_t *len, uint32_t n, uint32_t units,
+                       InlinePlan &plan);
+
 // triples: 3 * segs.Size() words, first: segs.Size() + 1 words.  Returns total chunks.
 uint64_t BuildTablePlan(const SegList &segs, uint32_t units, uint64_t *triples, uint32_t *first);
 

@@ -1,0 +1,188 @@
+// TEST INFRASTRUCTURE ONLY.  A CPU stand-in for the thin runtime layer (csrc/rt/mf_rt.h) so that the
+// host stack above it - planner, staging ring, operator fallback, entity and C API - can be
+// exercised without a GPU, the way the reference's unit tests run against stub vendor libraries
+// (test/ut/mock/acl_stub.cpp of the reference).  "Device" memory is host memory, a launch executes
+// its plan at once with the SAME chunk geometry the kernels use (csrc/kernels/xcopy_plan.h), streams
+// and events are tokens.  Never linked into the product libraries.
+#include <cstdint>
+#include <cstdlib>
+#include <cstring>
+#include <map>
+#include <mutex>
+
+#include "../../memfabric_hybrid_amd/csrc/kernels/copy2d_plan.h"
+#include "../../memfabric_hybrid_amd/csrc/kernels/xcopy_plan.h"
+#include "../../memfabric_hybrid_amd/csrc/rt/mf_rt.h"
+
+namespace {
+std::mutex g_lock;
+std::map<uint64_t, std::pair<uint64_t, int>> g_allocs;  // base -> (size, kind)
+int g_device = -1;
+uint64_t g_launches = 0;
+uint64_t g_chunksRun = 0;
+
+void *Track(uint64_t bytes, int kind)
+{
+    void *p = nullptr;
+    if (posix_memalign(&p, 4096, bytes == 0 ? 4096 : bytes) != 0) {
+        return nullptr;
+    }
+    std::lock_guard<std::mutex> guard(g_lock);
+    g_allocs[reinterpret_cast<uint64_t>(p)] = {bytes, kind};
+    return p;
+}
+
+int Untrack(void *p)
+{
+    std::lock_guard<std::mutex> guard(g_lock);
+    auto it = g_allocs.find(reinterpret_cast<uint64_t>(p));
+    if (it == g_allocs.end()) {
+        return 1;
+    }
+    g_allocs.erase(it);
+    free(p);
+    return 0;
+}
+
+void RunChunk(uint64_t src, uint64_t dst, uint64_t len, uint64_t k, uint32_t units)
+{
+    const mf::SegGeom g = mf::SegmentGeometry(dst, len);
+    const uint64_t u0 = k * units;
+    const uint64_t left = g.body > u0 ? g.body - u0 : 0;
+    const uint64_t n = left < units ? left : units;
+    std::memmove(reinterpret_cast<void *>(dst + g.head + u0 * 16), reinterpret_cast<void *>(src + g.head + u0 * 16), n * 16);
+    if (k == 0) {
+        std::memmove(reinterpret_cast<void *>(dst), reinterpret_cast<void *>(src), g.head);
+    }
+    if (u0 + units >= g.body) {
+        const uint64_t off = g.head + g.body * 16;
+        std::memmove(reinterpret_cast<void *>(dst + off), reinterpret_cast<void *>(src + off), g.tail);
+    }
+    ++g_chunksRun;
+}
+}  // namespace
+
+extern "C" {
+uint64_t fake_rt_launches(void) { return g_launches; }
+uint64_t fake_rt_chunks(void) { return g_chunksRun; }
+
+int mfrt_init(int device)
+{
+    if (device != 0) {
+        return 101;
+    }
+    g_device = 0;
+    return 0;
+}
+int mfrt_current_device(void) { return 0; }
+int mfrt_bind_thread(void) { return g_device >= 0 ? 0 : 3; }
+void mfrt_shutdown(void) { g_device = -1; }
+int mfrt_is_initialised(void) { return g_device >= 0; }
+int mfrt_device_id(void) { return g_device; }
+uint32_t mfrt_cu_count(void) { return 256; }
+const char *mfrt_error_string(int) { return "fake runtime error"; }
+void *mfrt_alloc_device(uint64_t bytes) { return Track(bytes, MFRT_PTR_DEVICE); }
+int mfrt_free_device(void *p) { return Untrack(p); }
+void *mfrt_alloc_host(uint64_t bytes) { return Track(bytes, MFRT_PTR_PINNED_HOST); }
+int mfrt_free_host(void *p) { return Untrack(p); }
+int mfrt_pointer_kind(const void *p)
+{
+    std::lock_guard<std::mutex> guard(g_lock);
+    const uint64_t a = reinterpret_cast<uint64_t>(p);
+    auto it = g_allocs.upper_bound(a);
+    if (it == g_allocs.begin()) {
+        return MFRT_PTR_PAGEABLE;
+    }
+    --it;
+    return a < it->first + it->second.first ? it->second.second : MFRT_PTR_PAGEABLE;
+}
+void *mfrt_stream_create(void) { return malloc(8); }
+int mfrt_stream_destroy(void *s) { free(s); return 0; }
+int mfrt_stream_sync(void *) { return 0; }
+int mfrt_device_sync(void) { return 0; }
+void *mfrt_event_create(void) { return malloc(8); }
+int mfrt_event_destroy(void *e) { free(e); return 0; }
+int mfrt_event_record(void *, void *) { return 0; }
+int mfrt_event_sync(void *) { return 0; }
+int mfrt_event_done(void *) { return 1; }
+float mfrt_event_elapsed_ms(void *, void *) { return 0.0f; }
+int mfrt_memcpy(void *dst, const void *src, uint64_t bytes) { std::memmove(dst, src, bytes); return 0; }
+int mfrt_memcpy_async(void *dst, const void *src, uint64_t bytes, void *) { std::memmove(dst, src, bytes); return 0; }
+int mfrt_memset(void *dst, int value, uint64_t bytes) { std::memset(dst, value, bytes); return 0; }
+
+int mfk_xcopy_inline(const void *inlinePlan, int, uint32_t, void *mask, uint32_t maskValue, void *, void *)
+{
+    const mf::InlinePlan &p = *static_cast<const mf::InlinePlan *>(inlinePlan);
+    ++g_launches;
+    for (uint32_t c = 0; c < p.nchunk; ++c) {
+        uint32_t below = 0;
+        for (uint32_t i = 0; i < mf::kInlineSegs; ++i) {
+            below += p.first[i] <= c ? 1u : 0u;
+        }
+        const uint32_t s = below - 1;
+        RunChunk(p.src[s], p.dst[s], p.len[s], c - p.first[s], p.units);
+    }
+    if (mask != nullptr) {
+        *static_cast<uint64_t *>(mask) = maskValue;
+    }
+    return 0;
+}
+
+int mfk_xcopy_table(const void *triples, const void *first, const void *nchunkDev, uint32_t nseg, uint32_t nchunk,
+                    uint32_t units, int, uint32_t, void *mask, uint32_t maskValue, void *, void *)
+{
+    const uint64_t *t = static_cast<const uint64_t *>(triples);
+    const uint32_t *f = static_cast<const uint32_t *>(first);
+    const uint32_t total = nchunkDev != nullptr ? *static_cast<const uint32_t *>(nchunkDev) : nchunk;
+    ++g_launches;
+    uint32_t s = 0;
+    for (uint32_t c = 0; c < total; ++c) {
+        while (s + 1 <= nseg && f[s + 1] <= c) {
+            ++s;
+        }
+        RunChunk(t[3 * s], t[3 * s + 1], t[3 * s + 2], c - f[s], units);
+    }
+    if (mask != nullptr) {
+        *static_cast<uint64_t *>(mask) = maskValue;
+    }
+    return 0;
+}
+
+int mfk_xcopy_plan(const void *triples, uint32_t nseg, uint32_t units, void *first, void *nchunk, void *)
+{
+    const uint64_t *t = static_cast<const uint64_t *>(triples);
+    uint32_t *f = static_cast<uint32_t *>(first);
+    uint32_t run = 0;
+    for (uint32_t i = 0; i < nseg; ++i) {
+        f[i] = run;
+        run += static_cast<uint32_t>(mf::SegmentChunks(t[3 * i + 1], t[3 * i + 2], units));
+    }
+    f[nseg] = run;
+    *static_cast<uint32_t *>(nchunk) = run;
+    ++g_launches;
+    return 0;
+}
+
+int mfk_copy2d(const void *rectPlan, uint32_t, void *)
+{
+    const mf::RectPlan &p = *static_cast<const mf::RectPlan *>(rectPlan);
+    ++g_launches;
+    for (uint32_t r = 0; r < mf::kRectInline; ++r) {
+        if (p.first[r] == 0xFFFFFFFFu) {
+            break;
+        }
+        for (uint32_t row = 0; row < p.height[r]; ++row) {
+            std::memmove(reinterpret_cast<void *>(p.dst[r] + 16ull * p.dpitchUnits[r] * row),
+                         reinterpret_cast<void *>(p.src[r] + 16ull * p.spitchUnits[r] * row), 16ull * p.widthUnits[r]);
+        }
+    }
+    return 0;
+}
+
+uint64_t mfk_moe_workspace_bytes(uint32_t, uint32_t, uint32_t) { return 0; }
+int mfk_moe_dispatch(const void *, const void *, uint32_t, uint32_t, uint32_t, uint32_t, void *, void *, void *, void *, void *,
+                     void *, void *) { return -1; }
+int mfk_moe_combine(const void *, const void *, const void *, uint32_t, uint32_t, uint32_t, void *, void *) { return -1; }
+void mfk_moe_tune(int, int) {}
+int mfk_probe(int, void *, const void *, uint64_t, uint32_t, void *) { return -1; }
+}

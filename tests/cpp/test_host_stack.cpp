@@ -1,0 +1,280 @@
+// CPU unit tests of the host stack over the fake runtime (tests/cpp/fake_rt.cpp).
+// Part 1 restates the behaviours the reference pins for its operator set in
+// test/ut/testcase/hybm/data_operator/hybm_compose_data_op_test.cpp (init order and rollback,
+// intra-node engine first, fallback to the next engine on failure for copy / batch / async,
+// Wait only through the intra-node engine).  Part 2 drives the C API end to end and compares
+// bytes with memcpy.
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <random>
+#include <vector>
+
+#include "../../include/mf_hip_dataplane.h"
+#include "../../include/mf_xcopy_api.h"
+#include "../../memfabric_hybrid_amd/csrc/host/compose_data_op.h"
+#include "../../memfabric_hybrid_amd/csrc/host/mf_log.h"
+
+extern "C" uint64_t fake_rt_launches(void);
+
+using namespace mf;
+using ock::mf::DataOperatorPtr;
+using ock::mf::ExtOptions;
+
+static int g_failed = 0;
+#define CHECK(cond)                                                             \
+    do {                                                                        \
+        if (!(cond)) {                                                          \
+            std::printf("FAILED %s:%d: %s\n", __FILE__, __LINE__, #cond);       \
+            ++g_failed;                                                         \
+        }                                                                       \
+    } while (0)
+
+struct MockOp : ock::mf::DataOperator {
+    int initRet = 0, copyRet = 0, batchRet = 0, asyncRet = 0, waitRet = 0;
+    int inits = 0, uninits = 0, copies = 0, batches = 0, asyncs = 0, waits = 0, cleanups = 0;
+    uint32_t lastBatchSize = 0, lastSrcRank = 99, lastDstRank = 99;
+    ock::mf::Result Initialize() noexcept override { ++inits; return initRet; }
+    void UnInitialize() noexcept override { ++uninits; }
+    ock::mf::Result DataCopy(hybm_copy_params &, hybm_data_copy_direction, const ExtOptions &) noexcept override { ++copies; return copyRet; }
+    ock::mf::Result BatchDataCopy(hybm_batch_copy_params &p, hybm_data_copy_direction, const ExtOptions &o) noexcept override
+    {
+        ++batches;
+        lastBatchSize = p.batchSize;
+        lastSrcRank = o.srcRankId;
+        lastDstRank = o.destRankId;
+        return batchRet;
+    }
+    ock::mf::Result DataCopyAsync(hybm_copy_params &, hybm_data_copy_direction, const ExtOptions &) noexcept override { ++asyncs; return asyncRet; }
+    ock::mf::Result Wait(int32_t) noexcept override { ++waits; return waitRet; }
+    void CleanUp() noexcept override { ++cleanups; }
+};
+
+static hybm_options Options(uint32_t ops)
+{
+    hybm_options o{};
+    o.bmType = HYBM_TYPE_HOST_INITIATE;
+    o.bmDataOpType = static_cast<hybm_data_op_type>(ops);
+    o.rankCount = 1;
+    return o;
+}
+
+static void TestCompose()
+{
+    auto a = std::make_shared<MockOp>();
+    auto b = std::make_shared<MockOp>();
+    auto c = std::make_shared<MockOp>();
+    OperatorFactory f;
+    f.intraNode = [&]() -> DataOperatorPtr { return a; };
+    f.deviceRdma = [&]() -> DataOperatorPtr { return b; };
+    f.hostNet = [&]() -> DataOperatorPtr { return c; };
+    const uint32_t all = HYBM_DOP_TYPE_SDMA | HYBM_DOP_TYPE_DEVICE_RDMA | HYBM_DOP_TYPE_HOST_RDMA;
+    hybm_copy_params cp{reinterpret_cast<void *>(0x1000), reinterpret_cast<void *>(0x2000), 16};
+    void *srcs[3] = {cp.src, cp.src, cp.src};
+    void *dsts[3] = {cp.dest, cp.dest, cp.dest};
+    uint64_t lens[3] = {1, 2, 3};
+    hybm_batch_copy_params bp{srcs, dsts, lens, 3};
+    ExtOptions opt{};
+    opt.srcRankId = 0;
+    opt.destRankId = 0;
+    {
+        // only requested engines are created; device-initiated pools create none
+        ComposeDataOp only(Options(HYBM_DOP_TYPE_SDMA), f);
+        CHECK(only.Initialize() == BM_OK && a->inits == 1 && b->inits == 0 && c->inits == 0);
+        hybm_options ai = Options(all);
+        ai.bmType = HYBM_TYPE_AI_CORE_INITIATE;
+        ComposeDataOp none(ai, f);
+        CHECK(none.Initialize() == BM_OK && a->inits == 1);
+        CHECK(none.DataCopy(cp, HYBM_GLOBAL_DEVICE_TO_GLOBAL_DEVICE, opt) == BM_INVALID_PARAM);
+        CHECK(none.Wait(0) == BM_ERROR);
+    }
+    {
+        // a later engine failing to start drops the earlier ones and reports its code
+        *a = MockOp{};
+        *b = MockOp{};
+        *c = MockOp{};
+        c->initRet = BM_ERROR;
+        ComposeDataOp op(Options(all), f);
+        CHECK(op.Initialize() == BM_ERROR);
+        CHECK(a->inits == 1 && b->inits == 1 && c->inits == 1);
+        CHECK(op.DataCopy(cp, HYBM_GLOBAL_DEVICE_TO_GLOBAL_DEVICE, opt) == BM_INVALID_PARAM);  // nothing left
+    }
+    {
+        *a = MockOp{};
+        *b = MockOp{};
+        *c = MockOp{};
+        ComposeDataOp op(Options(all), f);
+        CHECK(op.Initialize() == BM_OK);
+        // first engine wins
+        CHECK(op.DataCopy(cp, HYBM_GLOBAL_DEVICE_TO_GLOBAL_DEVICE, opt) == BM_OK);
+        CHECK(a->copies == 1 && b->copies == 0 && c->copies == 0);
+        // failure falls through, in order
+        a->copyRet = BM_ERROR;
+        CHECK(op.DataCopy(cp, HYBM_GLOBAL_DEVICE_TO_GLOBAL_DEVICE, opt) == BM_OK);
+        CHECK(a->copies == 2 && b->copies == 1 && c->copies == 0);
+        b->copyRet = BM_TIMEOUT;
+        CHECK(op.DataCopy(cp, HYBM_GLOBAL_DEVICE_TO_GLOBAL_DEVICE, opt) == BM_OK);
+        CHECK(c->copies == 1);
+        c->copyRet = BM_NOT_SUPPORTED;
+        CHECK(op.DataCopy(cp, HYBM_GLOBAL_DEVICE_TO_GLOBAL_DEVICE, opt) == BM_NOT_SUPPORTED);  // last error is reported
+        // batch: whole batch to the intra-node engine, per rank pair to the others
+        CHECK(op.BatchDataCopy(bp, HYBM_GLOBAL_DEVICE_TO_GLOBAL_DEVICE, opt) == BM_OK);
+        CHECK(a->batches == 1 && a->lastBatchSize == 3 && b->batches == 0);
+        a->batchRet = BM_ERROR;
+        ExtOptions grouped = opt;
+        grouped.groupMap[{0, 1}] = {0, 2};
+        grouped.groupMap[{2, 0}] = {1};
+        CHECK(op.BatchDataCopy(bp, HYBM_GLOBAL_DEVICE_TO_GLOBAL_DEVICE, grouped) == BM_OK);
+        CHECK(b->batches == 2 && c->batches == 0);
+        b->batchRet = BM_ERROR;
+        CHECK(op.BatchDataCopy(bp, HYBM_GLOBAL_DEVICE_TO_GLOBAL_DEVICE, grouped) == BM_OK);
+        CHECK(c->batches == 2);
+        // an ungrouped batch reaches a network engine whole, between the two ranks named
+        c->batches = 0;
+        CHECK(op.BatchDataCopy(bp, HYBM_GLOBAL_DEVICE_TO_GLOBAL_DEVICE, opt) == BM_OK);
+        CHECK(c->batches == 1 && c->lastBatchSize == 3 && c->lastSrcRank == 0 && c->lastDstRank == 0);
+        // async: same fallback
+        CHECK(op.DataCopyAsync(cp, HYBM_GLOBAL_DEVICE_TO_GLOBAL_DEVICE, opt) == BM_OK && a->asyncs == 1 && b->asyncs == 0);
+        a->asyncRet = BM_ERROR;
+        CHECK(op.DataCopyAsync(cp, HYBM_GLOBAL_DEVICE_TO_GLOBAL_DEVICE, opt) == BM_OK && b->asyncs == 1);
+        // wait is routed to the intra-node engine only
+        CHECK(op.Wait(7) == BM_OK && a->waits == 1 && b->waits == 0 && c->waits == 0);
+        a->waitRet = BM_TIMEOUT;
+        CHECK(op.Wait(7) == BM_TIMEOUT);
+        op.CleanUp();
+        CHECK(a->cleanups == 1 && b->cleanups == 1 && c->cleanups == 1);
+        op.UnInitialize();
+        CHECK(a->uninits == 1 && b->uninits == 1 && c->uninits == 1);
+    }
+    {
+        // without the intra-node engine there is nothing to wait on
+        *b = MockOp{};
+        ComposeDataOp op(Options(HYBM_DOP_TYPE_DEVICE_RDMA), f);
+        CHECK(op.Initialize() == BM_OK);
+        CHECK(op.Wait(0) == BM_ERROR);
+        CHECK(op.DataCopy(cp, HYBM_GLOBAL_DEVICE_TO_GLOBAL_DEVICE, opt) == BM_OK && b->copies == 1);
+    }
+}
+
+static void Fill(std::vector<uint8_t> &v, uint32_t seed)
+{
+    std::mt19937 rng(seed);
+    for (auto &x : v) {
+        x = static_cast<uint8_t>(rng());
+    }
+}
+
+static void TestCApi()
+{
+    const uint64_t pool = 64ull << 20;
+    smem_bm_config_t cfg;
+    CHECK(smem_bm_config_init(&cfg) == SM_OK);
+    CHECK(smem_bm_init("tcp://127.0.0.1:1", 2, 0, &cfg) == SM_ERROR);  // a world of one only
+    CHECK(smem_bm_init("tcp://127.0.0.1:1", 1, 0, &cfg) == SM_OK);
+    CHECK(smem_bm_init("tcp://127.0.0.1:1", 1, 0, &cfg) == SM_OK);     // idempotent
+    CHECK(smem_bm_get_rank_id() == 0);
+    smem_bm_t bm = smem_bm_create(2, 1, SMEMB_DATA_OP_SDMA, pool, pool, 0);
+    CHECK(bm != nullptr);
+    CHECK(smem_bm_create(2, 1, SMEMB_DATA_OP_SDMA, pool, pool, 0) == nullptr);
+    CHECK(smem_bm_join(bm, 0) == SM_OK);
+    uint8_t *dev = static_cast<uint8_t *>(smem_bm_ptr_by_mem_type(bm, SMEM_MEM_TYPE_DEVICE, 0));
+    uint8_t *host = static_cast<uint8_t *>(smem_bm_ptr_by_mem_type(bm, SMEM_MEM_TYPE_HOST, 0));
+    CHECK(dev != nullptr && host != nullptr);
+    CHECK(smem_bm_ptr_by_mem_type(bm, SMEM_MEM_TYPE_DEVICE, 1) == nullptr);
+    CHECK(smem_bm_get_local_mem_size_by_mem_type(bm, SMEM_MEM_TYPE_HOST) == pool);
+    CHECK(smem_bm_get_rank_id_by_gva(bm, dev + 5) == 0);
+    CHECK(smem_bm_get_rank_id_by_gva(bm, &cfg) == UINT32_MAX);
+    CHECK(mf_va_infer_direction(reinterpret_cast<uint64_t>(host), reinterpret_cast<uint64_t>(dev)) == HYBM_GLOBAL_HOST_TO_GLOBAL_DEVICE);
+
+    std::vector<uint8_t> ref(pool);
+    Fill(ref, 1);
+    std::memcpy(host, ref.data(), pool);
+    std::memset(dev, 0, pool);
+    std::vector<uint8_t> model(pool, 0);
+
+    // 300 ragged segments (table form) host pool -> device pool
+    std::mt19937_64 rng(7);
+    std::vector<void *> s, d;
+    std::vector<uint64_t> l;
+    uint64_t cursor = 0;
+    for (int i = 0; i < 300; ++i) {
+        uint64_t len = i % 11 == 0 ? 0 : rng() % 50000;
+        uint64_t so = rng() % (pool - 60000);
+        s.push_back(host + so);
+        d.push_back(dev + cursor + (i % 16));
+        l.push_back(len);
+        std::memcpy(model.data() + cursor + (i % 16), ref.data() + so, len);
+        cursor += len + 64;
+    }
+    smem_batch_copy_params bp{s.data(), d.data(), l.data(), 300};
+    const uint64_t before = fake_rt_launches();
+    CHECK(smem_bm_copy_batch(bm, &bp, SMEMB_COPY_G2G, 0) == SM_OK);
+    CHECK(fake_rt_launches() - before == 2);  // descriptor staging + table kernel
+    CHECK(std::memcmp(dev, model.data(), pool) == 0);
+    // the same as an inline batch (first 100), asynchronous + wait, AUTO direction
+    std::memset(dev, 0, pool);
+    bp.batchSize = 100;
+    CHECK(smem_bm_copy_batch(bm, &bp, SMEMB_COPY_AUTO, ASYNC_COPY_FLAG) == SM_OK);
+    CHECK(smem_bm_wait(bm) == SM_OK);
+    std::vector<uint8_t> model2(pool, 0);
+    for (int i = 0; i < 100; ++i) {
+        std::memcpy(model2.data() + (static_cast<uint8_t *>(d[i]) - dev), ref.data() + (static_cast<uint8_t *>(s[i]) - host), l[i]);
+    }
+    CHECK(std::memcmp(dev, model2.data(), pool) == 0);
+    // pageable local memory: staged in rounds (70 MiB through a 32 MiB area would not fit the pool; use 40 MiB)
+    std::vector<uint8_t> big(40u << 20);
+    Fill(big, 3);
+    smem_copy_params one{big.data(), dev + 3, big.size()};
+    CHECK(smem_bm_copy(bm, &one, SMEMB_COPY_H2G, 0) == SM_OK);
+    CHECK(std::memcmp(dev + 3, big.data(), big.size()) == 0);
+    std::vector<uint8_t> back(big.size());
+    smem_copy_params two{dev + 3, back.data(), back.size()};
+    CHECK(smem_bm_copy(bm, &two, SMEMB_COPY_G2H, 0) == SM_OK);
+    CHECK(back == big);
+    // host pool <-> pageable: plain CPU copy
+    smem_copy_params three{big.data(), host + 9, 1000};
+    CHECK(smem_bm_copy(bm, &three, SMEMB_COPY_H2GH, 0) == SM_OK);
+    CHECK(std::memcmp(host + 9, big.data(), 1000) == 0);
+    // errors
+    smem_copy_params bad{dev, dev + pool - 8, 16};
+    CHECK(smem_bm_copy(bm, &bad, SMEMB_COPY_G2G, 0) == SM_INVALID_PARAM);  // leaves the window: unclassifiable
+    bad = {dev, host, 0};
+    CHECK(smem_bm_copy(bm, &bad, SMEMB_COPY_G2G, 0) == SM_INVALID_PARAM);
+    bad = {&cfg, host, 16};
+    CHECK(smem_bm_copy(bm, &bad, SMEMB_COPY_L2GH, 0) == SM_INVALID_PARAM);  // L2GH does not override the source
+    CHECK(smem_bm_copy(bm, &bad, SMEMB_COPY_BUTT, 0) == SM_INVALID_PARAM);
+    // 2-D copy, aligned and unaligned geometry
+    std::memset(dev, 0, pool);
+    mf_copy2d_desc rects[2] = {
+        {reinterpret_cast<uint64_t>(host), reinterpret_cast<uint64_t>(dev), 896, 100, 896, 1792},
+        {reinterpret_cast<uint64_t>(host) + 5, reinterpret_cast<uint64_t>(dev) + (1u << 20) + 3, 100, 50, 160, 300},
+    };
+    CHECK(mf_xcopy_2d_batch(rects, 2, MF_ROUTE_FROM_HOST, nullptr) == BM_OK);
+    bool ok = true;
+    for (int r = 0; r < 100; ++r) {
+        ok = ok && std::memcmp(dev + r * 1792, host + r * 896, 896) == 0;
+    }
+    for (int r = 0; r < 50; ++r) {
+        ok = ok && std::memcmp(dev + (1u << 20) + 3 + r * 300, host + 5 + r * 160, 100) == 0;
+    }
+    CHECK(ok);
+    CHECK(smem_bm_leave(bm, 0) == SM_OK);
+    smem_bm_destroy(bm);
+    CHECK(smem_bm_wait(bm) == SM_INVALID_PARAM);  // handle is gone
+    smem_bm_uninit(0);
+    CHECK(smem_bm_wait(bm) == SM_NOT_INITIALIZED);
+}
+
+int main()
+{
+    SetLogLevel(3);
+    SetLogSink([](int, const char *) {});
+    TestCompose();
+    TestCApi();
+    if (g_failed != 0) {
+        std::printf("%d check(s) failed\n", g_failed);
+        return 1;
+    }
+    std::printf("host stack tests passed\n");
+    return 0;
+}
