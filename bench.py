@@ -265,6 +265,38 @@ def extras_block(lib, pool, dev, batches, tables, steps):
     return out, copy_ceiling
 
 
+def extras_transfer(lib, dev, batches, steps):
+    """The same KV batches through the transfer front-end: a Prefill object writes into the pool
+    a Decode object registered, submitted on one stream (smem_trans_batch_write_submit)."""
+    from memfabric_hybrid_amd.transfer import TransferEngine
+    prefill, decode = TransferEngine(), TransferEngine()
+    if prefill.initialize("tcp://127.0.0.1:15432", "127.0.0.1:15321", "Prefill", 0) != 0 or \
+            decode.initialize("tcp://127.0.0.1:15432", "127.0.0.1:15322", "Decode", 0) != 0 or \
+            decode.register_memory(dev, POOL_BYTES) != 0:
+        return {"error": native.last_error()}
+    timer = Timer(lib)
+    peer = b"127.0.0.1:15322"
+    call, handle, stream = lib.smem_trans_batch_write_submit, prefill._handle, timer.stream
+    i = [0]
+
+    def step():
+        b = batches[i[0] % len(batches)]
+        i[0] += 1
+        if call(handle, b.srcs, peer, b.dsts, b.lens, b.n, stream, 0) != 0:
+            raise RuntimeError(native.last_error())
+
+    k = max(400, steps // 4)
+    us, wall_us = timer.run(step, k, warm=50)
+    hbm = 2 * batches[0].payload / us / 1e3
+    decode.unregister_memory(dev)
+    prefill.destroy()
+    decode.destroy()
+    prefill.unInitialize()
+    return {"api": "smem_trans_batch_write_submit, Prefill -> Decode object in one process, one stream",
+            "us_per_batch": round(us, 2), "wall_us_per_batch": round(wall_us, 2), "hbm_GBps": round(hbm, 1),
+            "frac_of_hbm_peak": frac(hbm, HBM_PEAK_GBPS)}
+
+
 def extras_paged(lib):
     """Paged KV gather/scatter: 4096 distinct 32 KiB pages out of a 40 GiB pool."""
     page, count = 32768, 4096
@@ -459,6 +491,7 @@ def main():
     if not args.no_extras:
         extras, copy_ceiling = extras_block(lib, pool, dev, batches, tables, args.steps)
         result["roofline"]["frac_of_measured_copy_ceiling"] = frac(achieved, copy_ceiling)
+        extras["kv122_transfer_write"] = extras_transfer(lib, dev, batches, args.steps)
     pool.destroy()  # give the pools back before the larger workloads allocate
     if not args.no_extras:
         extras["paged_kv_40GiB"] = extras_paged(lib)

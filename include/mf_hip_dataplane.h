@@ -159,6 +159,16 @@ int32_t mf_gva_contains(uint64_t base, uint64_t stride, uint64_t rankCount, uint
 uint32_t mf_gva_rank(uint64_t base, uint64_t stride, uint64_t rankCount, uint64_t rankSpace, uint64_t addr);
 uint64_t mf_gva_mask48(uint64_t addr);
 
+/* ---- transfer front-end arithmetic views ----------------------------------
+ * mf_trans_combine: union of n (start, size) pairs (pairs[2*n]) into sorted, disjoint runs
+ * written to out[2*k..] (room for n pairs); returns k.  mf_trans_translate: look one peer range
+ * up in n runs {start, size, mapped} (slices[3*n]); the mapped address or 0 when the range is not
+ * inside one run.  mf_trans_parse_name: 1 when the name is a valid "ip:port" / "[ipv6]:port" and,
+ * then, its 20-byte binary form in key. */
+uint32_t mf_trans_combine(const uint64_t *pairs, uint32_t n, uint64_t *out);
+uint64_t mf_trans_translate(const uint64_t *slices, uint32_t n, uint64_t remote, uint64_t size);
+int32_t mf_trans_parse_name(const char *name, uint8_t *key);
+
 #ifdef __cplusplus
 }
 #endif

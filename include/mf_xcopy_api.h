@@ -51,6 +51,11 @@ int32_t hybm_free_local_memory(hybm_entity_t e, hybm_mem_slice_t slice, uint32_t
 /* src/hybm/include/hybm_big_mem.h:96 */
 void *hybm_get_slice_va(hybm_entity_t e, hybm_mem_slice_t slice);
 
+/* src/hybm/include/hybm_big_mem.h:106 — make memory the caller owns (HBM from hipMalloc, or
+ * pinned host memory) part of the entity, so that pool-side range checks accept it.  Ordinary
+ * pageable memory is refused: it cannot be pinned after the fact on this platform. */
+hybm_mem_slice_t hybm_register_local_memory(hybm_entity_t e, const void *ptr, uint64_t size, uint32_t flags);
+
 /* src/hybm/include/hybm_data_op.h:36-37 — one contiguous copy.
  * BM_INVALID_PARAM for NULL e/params/src/dest, dataSize == 0, direction >= BUTT,
  * an AUTO direction that cannot be inferred, an unknown entity handle, or a
@@ -121,6 +126,48 @@ uint32_t smem_bm_get_rank_id_by_gva(smem_bm_t handle, void *gva);
 int32_t smem_set_extern_logger(void (*func)(int level, const char *msg));
 int32_t smem_set_log_level(int level);
 const char *smem_get_last_err_msg(void);
+
+/* ---- smem transfer front-end: one-sided read / write between transfer objects by name --------
+ * src/smem/include/host/smem_trans.h:24-239.  Objects of one process find each other through an
+ * in-process directory (the config store and its watch threads are not part of this library):
+ * a sender sees the memory receivers registered and the other way round, immediately, so
+ * registration does not sleep.  Remote addresses are the peer's own virtual addresses; they are
+ * translated through the slice map (src/smem/csrc/smem_trans/smem_trans_entry.cpp:307-372) and
+ * handed to hybm_data_batch_copy as one fused launch.  The copy direction follows what the
+ * memory really is (HBM or host) instead of assuming HBM on both sides. */
+int32_t smem_trans_config_init(smem_trans_config_t *config);                        /* smem_trans.h:30 */
+int32_t smem_trans_init(const smem_trans_config_t *config);                         /* :39 */
+void smem_trans_uninit(uint32_t flags);                                             /* :46 */
+/* uniqueId: "ip:port" or "[ipv6]:port"; storeUrl must be non-empty and is otherwise unused. */
+smem_trans_t smem_trans_create(const char *storeUrl, const char *uniqueId, const smem_trans_config_t *config); /* :57 */
+void smem_trans_destroy(smem_trans_t handle, uint32_t flags);                       /* :65 */
+/* Pinned, device-mapped host memory that is registered on return (size rounded up to 2 MiB). */
+void *smem_trans_malloc(smem_trans_t handle, size_t capacity);                      /* :74 */
+int32_t smem_trans_free(smem_trans_t handle, void *address);                        /* :84 */
+int32_t smem_trans_register_mem(smem_trans_t handle, void *address, size_t capacity, uint32_t flags); /* :95 */
+int32_t smem_trans_batch_register_mem(smem_trans_t handle, void *addresses[], size_t capacities[], uint32_t count,
+                                      uint32_t flags);                              /* :107-108 */
+/* Unlike the reference (a no-op there, smem_trans.cpp:210-217) this withdraws the memory. */
+int32_t smem_trans_deregister_mem(smem_trans_t handle, void *address);              /* :117 */
+int32_t smem_trans_write(smem_trans_t handle, const void *localAddr, const char *remoteUniqueId, void *remoteAddr,
+                         size_t dataSize, uint32_t flags);                          /* :130-131 */
+int32_t smem_trans_batch_write(smem_trans_t handle, const void *localAddrs[], const char *remoteUniqueId,
+                               void *remoteAddrs[], size_t dataSizes[], uint32_t batchSize, uint32_t flags); /* :145-146 */
+int32_t smem_trans_read(smem_trans_t handle, void *localAddr, const char *remoteUniqueId, const void *remoteAddr,
+                        size_t dataSize, uint32_t flags);                           /* :159-160 */
+int32_t smem_trans_batch_read(smem_trans_t handle, void *localAddrs[], const char *remoteUniqueId,
+                              const void *remoteAddrs[], size_t dataSizes[], uint32_t batchSize, uint32_t flags); /* :174-175 */
+/* The *_submit forms enqueue on the caller's hipStream_t (must not be NULL) and return at once. */
+int32_t smem_trans_read_submit(smem_trans_t handle, void *localAddr, const char *remoteUniqueId,
+                               const void *remoteAddr, size_t dataSize, void *stream, uint32_t flags);   /* :189-190 */
+int32_t smem_trans_write_submit(smem_trans_t handle, const void *localAddr, const char *remoteUniqueId,
+                                void *remoteAddr, size_t dataSize, void *stream, uint32_t flags);        /* :204-205 */
+int32_t smem_trans_batch_read_submit(smem_trans_t handle, void *localAddrs[], const char *remoteUniqueId,
+                                     const void *remoteAddrs[], size_t dataSizes[], uint32_t batchSize, void *stream,
+                                     uint32_t flags);                                                   /* :220-222 */
+int32_t smem_trans_batch_write_submit(smem_trans_t handle, const void *localAddrs[], const char *remoteUniqueId,
+                                      void *remoteAddrs[], size_t dataSizes[], uint32_t batchSize, void *stream,
+                                      uint32_t flags);                                                  /* :237-239 */
 
 #ifdef __cplusplus
 }

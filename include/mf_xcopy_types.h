@@ -259,6 +259,26 @@ enum {
     SM_GET_OBJIECT = -2011
 };
 
+/* ---- smem transfer front-end (src/smem/include/host/smem_trans_def.h:24-48) ---- */
+typedef void *smem_trans_t;
+
+typedef enum {
+    SMEM_TRANS_NONE = 0,
+    SMEM_TRANS_SENDER,
+    SMEM_TRANS_RECEIVER,
+    SMEM_TRANS_BOTH,
+    SMEM_TRANS_BUTT
+} smem_trans_role_t;
+
+typedef struct {
+    smem_trans_role_t role;          /* sender, receiver or both */
+    uint32_t initTimeout;            /* seconds; 120 by default */
+    uint32_t deviceId;               /* GPU ordinal */
+    uint32_t flags;
+    smem_bm_data_op_type dataOpType; /* engines to use; the copy kernels serve SMEMB_DATA_OP_SDMA */
+    bool startConfigServer;
+} smem_trans_config_t;
+
 #ifdef __cplusplus
 }
 #endif
@@ -285,6 +305,8 @@ MF_PIN(sizeof(smem_copy_params) == 24 && sizeof(smem_batch_copy_params) == 32);
 MF_PIN(sizeof(hybm_exchange_info) == 516);
 MF_PIN(offsetof(hybm_options, maxHBMSize) == 24 && offsetof(hybm_options, scene) == 56);
 MF_PIN(offsetof(smem_bm_create_option_t, dataOpType) == 32 && offsetof(smem_bm_create_option_t, tag) == 40);
+MF_PIN(SMEM_TRANS_SENDER == 1 && SMEM_TRANS_RECEIVER == 2 && SMEM_TRANS_BOTH == 3 && SMEM_TRANS_BUTT == 4);
+MF_PIN(sizeof(smem_trans_config_t) == 24 && offsetof(smem_trans_config_t, dataOpType) == 16);
 MF_PIN(BM_NOT_INITIALIZED == -9 && BM_NOT_SUPPORTED == -100 && SM_INVALID_PARAM == -2000 && SM_NOT_INITIALIZED == -2008);
 #undef MF_PIN
 

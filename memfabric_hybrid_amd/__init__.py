@@ -8,4 +8,4 @@ library and raises if it has not been built.
 
 from . import native  # noqa: F401
 
-__all__ = ["native", "bm", "workloads"]
+__all__ = ["native", "bm", "transfer", "workloads"]

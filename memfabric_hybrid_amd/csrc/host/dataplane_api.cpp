@@ -8,6 +8,7 @@
 #include "../rt/mf_rt.h"
 #include "gva_layout.h"
 #include "mf_log.h"
+#include "trans_entry.h"
 #include "va_manager.h"
 #include "xcopy_engine.h"
 
@@ -277,4 +278,45 @@ MF_EXPORT uint32_t mf_gva_rank(uint64_t base, uint64_t stride, uint64_t rankCoun
 MF_EXPORT uint64_t mf_gva_mask48(uint64_t addr)
 {
     return Mask48(addr);
+}
+
+MF_EXPORT uint32_t mf_trans_combine(const uint64_t *pairs, uint32_t n, uint64_t *out)
+{
+    if (pairs == nullptr || out == nullptr || n == 0) {
+        return 0;
+    }
+    std::vector<std::pair<uint64_t, uint64_t>> in;
+    in.reserve(n);
+    for (uint32_t i = 0; i < n; ++i) {
+        in.emplace_back(pairs[2 * i], pairs[2 * i + 1]);
+    }
+    const auto runs = CombineRanges(std::move(in));
+    for (size_t k = 0; k < runs.size(); ++k) {
+        out[2 * k] = runs[k].first;
+        out[2 * k + 1] = runs[k].second;
+    }
+    return static_cast<uint32_t>(runs.size());
+}
+
+MF_EXPORT uint64_t mf_trans_translate(const uint64_t *slices, uint32_t n, uint64_t remote, uint64_t size)
+{
+    PeerSliceMap map;
+    for (uint32_t i = 0; slices != nullptr && i < n; ++i) {
+        map.emplace(slices[3 * i], PeerSlice{slices[3 * i + 2], slices[3 * i + 1], HYBM_MEM_TYPE_DEVICE});
+    }
+    uint64_t mapped = 0;
+    hybm_mem_type type = HYBM_MEM_TYPE_BUTT;
+    return TranslatePeerAddress(map, remote, size, mapped, type) == SM_OK ? mapped : 0;
+}
+
+MF_EXPORT int32_t mf_trans_parse_name(const char *name, uint8_t *key)
+{
+    WorkerKey k;
+    if (name == nullptr || !ParseWorkerName(name, k)) {
+        return 0;
+    }
+    if (key != nullptr) {
+        std::memcpy(key, k.data(), k.size());
+    }
+    return 1;
 }

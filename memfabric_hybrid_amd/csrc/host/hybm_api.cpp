@@ -176,6 +176,17 @@ MF_EXPORT int32_t hybm_free_local_memory(hybm_entity_t e, hybm_mem_slice_t slice
     return entity == nullptr ? BM_INVALID_PARAM : entity->FreeLocal(static_cast<LocalSlice *>(slice));
 }
 
+MF_EXPORT hybm_mem_slice_t hybm_register_local_memory(hybm_entity_t e, const void *ptr, uint64_t size, uint32_t flags)
+{
+    (void)flags;
+    auto entity = EntityRegistry::Instance().FindByPtr(e);
+    if (entity == nullptr) {
+        MF_ERROR("hybm_register_local_memory: unknown pool handle");
+        return nullptr;
+    }
+    return entity->RegisterLocal(ptr, size);
+}
+
 MF_EXPORT void *hybm_get_slice_va(hybm_entity_t e, hybm_mem_slice_t slice)
 {
     auto entity = EntityRegistry::Instance().FindByPtr(e);

@@ -8,7 +8,20 @@ namespace mf {
 
 using ock::mf::ExtOptions;
 
-MemEntity::MemEntity(uint16_t id, const hybm_options &options) : id_(id), options_(options) {}
+namespace {
+// Every entity counts its range epochs in a block of its own, so a per-thread hit remembered for
+// an entity that is gone can never match a later entity that reuses its address.
+uint64_t NextEpochBlock()
+{
+    static std::atomic<uint64_t> block{1};
+    return block.fetch_add(1, std::memory_order_relaxed) << 32;
+}
+}  // namespace
+
+MemEntity::MemEntity(uint16_t id, const hybm_options &options) : id_(id), options_(options)
+{
+    rangeEpoch_.store(NextEpochBlock(), std::memory_order_release);
+}
 
 MemEntity::~MemEntity()
 {
@@ -41,6 +54,21 @@ void MemEntity::UnInitialize()
         dataOperator_->CleanUp();
         dataOperator_->UnInitialize();
         dataOperator_ = nullptr;
+    }
+    {
+        std::lock_guard<std::mutex> guard(sliceLock_);
+        for (auto &slice : looseSlices_) {
+            if (slice->ownsMemory) {
+                (void)mfrt_free_host(reinterpret_cast<void *>(slice->va));
+            }
+        }
+        looseSlices_.clear();
+    }
+    {
+        std::unique_lock<std::shared_mutex> guard(rangeLock_);
+        ranges_.clear();
+        rangeCount_.store(0, std::memory_order_release);
+        rangeEpoch_.fetch_add(1, std::memory_order_release);
     }
     (void)UnreserveSpace();
     initialized_ = false;
@@ -142,6 +170,32 @@ void *MemEntity::WindowBase(hybm_mem_type t) const
 
 LocalSlice *MemEntity::AllocLocal(hybm_mem_type t, uint64_t size)
 {
+    if (initialized_ && options_.scene == HYBM_SCENE_TRANS) {
+        // The transfer scene has no pre-sized window: every allocation is pinned host memory of
+        // its own (the reference carves it from a 128 GiB reservation,
+        // src/smem/csrc/smem_trans/smem_trans_entry.cpp:33,179-227).
+        if (t != HYBM_MEM_TYPE_HOST || size == 0) {
+            MF_ERROR("transfer-scene allocation needs host memory type and a size, got type " << t << " size " << size);
+            return nullptr;
+        }
+        if (mfrt_bind_thread() != 0) {
+            return nullptr;
+        }
+        const uint64_t bytes = (size + kLargePage - 1) / kLargePage * kLargePage;
+        void *p = mfrt_alloc_host(bytes);
+        if (p == nullptr) {
+            MF_ERROR("pinned allocation of " << bytes << " bytes failed");
+            return nullptr;
+        }
+        const uint64_t va = reinterpret_cast<uint64_t>(p);
+        if (AddRange(va, bytes, HYBM_MEM_TYPE_HOST) != BM_OK) {
+            (void)mfrt_free_host(p);
+            return nullptr;
+        }
+        std::lock_guard<std::mutex> guard(sliceLock_);
+        looseSlices_.emplace_back(new LocalSlice{HYBM_MEM_TYPE_HOST, va, bytes, true, true});
+        return looseSlices_.back().get();
+    }
     if (!initialized_ || !reserved_) {
         MF_ERROR("local allocation before the address space was reserved");
         return nullptr;
@@ -170,8 +224,115 @@ LocalSlice *MemEntity::AllocLocal(hybm_mem_type t, uint64_t size)
     return slot.get();
 }
 
+LocalSlice *MemEntity::RegisterLocal(const void *ptr, uint64_t size)
+{
+    if (!initialized_ || ptr == nullptr || size == 0) {
+        MF_ERROR("memory registration needs an initialised entity, an address and a size");
+        return nullptr;
+    }
+    if (mfrt_bind_thread() != 0) {
+        return nullptr;
+    }
+    const uint64_t va = reinterpret_cast<uint64_t>(ptr);
+    const int first = mfrt_pointer_kind(ptr);
+    const int last = mfrt_pointer_kind(reinterpret_cast<const void *>(va + size - 1));
+    if (first == MFRT_PTR_PAGEABLE || first != last) {
+        MF_ERROR("memory registration of [" << ptr << ", +" << size << ") refused: it must be one piece of HBM or of "
+                 "pinned host memory (ordinary host memory cannot be pinned after the fact here)");
+        return nullptr;
+    }
+    const hybm_mem_type t = first == MFRT_PTR_DEVICE ? HYBM_MEM_TYPE_DEVICE : HYBM_MEM_TYPE_HOST;
+    if (AddRange(va, size, t) != BM_OK) {
+        return nullptr;
+    }
+    std::lock_guard<std::mutex> guard(sliceLock_);
+    looseSlices_.emplace_back(new LocalSlice{t, va, size, false, true});
+    return looseSlices_.back().get();
+}
+
+int MemEntity::AddRange(uint64_t base, uint64_t size, hybm_mem_type t)
+{
+    if (base == 0 || size == 0 || base + size < base) {
+        return BM_INVALID_PARAM;
+    }
+    std::unique_lock<std::shared_mutex> guard(rangeLock_);
+    auto it = ranges_.find(base);
+    if (it != ranges_.end()) {
+        it->second.size = it->second.size > size ? it->second.size : size;
+        it->second.uses += 1;
+    } else {
+        ranges_.emplace(base, Range{size, t, 1});
+        rangeCount_.store(static_cast<uint32_t>(ranges_.size()), std::memory_order_release);
+    }
+    rangeEpoch_.fetch_add(1, std::memory_order_release);
+    return BM_OK;
+}
+
+int MemEntity::RemoveRange(uint64_t base)
+{
+    std::unique_lock<std::shared_mutex> guard(rangeLock_);
+    auto it = ranges_.find(base);
+    if (it == ranges_.end()) {
+        return BM_INVALID_PARAM;
+    }
+    if (--it->second.uses == 0) {
+        ranges_.erase(it);
+        rangeCount_.store(static_cast<uint32_t>(ranges_.size()), std::memory_order_release);
+    }
+    rangeEpoch_.fetch_add(1, std::memory_order_release);
+    return BM_OK;
+}
+
+bool MemEntity::InRanges(uint64_t a, uint64_t length) const
+{
+    // Batches walk one or two ranges; the last hit of this thread answers most calls without
+    // the lock.  The epoch makes a hit from before any change of the range set worthless.
+    struct Hit {
+        const MemEntity *owner = nullptr;
+        uint64_t epoch = 0;
+        uint64_t base = 0;
+        uint64_t end = 0;
+    };
+    thread_local Hit hit;
+    const uint64_t epoch = rangeEpoch_.load(std::memory_order_acquire);
+    if (hit.owner == this && hit.epoch == epoch && a >= hit.base && a + length <= hit.end && a + length >= a) {
+        return true;
+    }
+    std::shared_lock<std::shared_mutex> guard(rangeLock_);
+    auto it = ranges_.lower_bound(a);   // greatest start <= a
+    if (it == ranges_.end() || a + length < a || a + length > it->first + it->second.size) {
+        return false;
+    }
+    hit = Hit{this, rangeEpoch_.load(std::memory_order_acquire), it->first, it->first + it->second.size};
+    return true;
+}
+
 int MemEntity::FreeLocal(LocalSlice *slice)
 {
+    if (slice != nullptr && slice->outsideWindow) {
+        std::unique_ptr<LocalSlice> found;
+        {
+            std::lock_guard<std::mutex> guard(sliceLock_);
+            for (auto it = looseSlices_.begin(); it != looseSlices_.end(); ++it) {
+                if (it->get() == slice) {
+                    found = std::move(*it);
+                    looseSlices_.erase(it);
+                    break;
+                }
+            }
+        }
+        if (found == nullptr) {
+            return BM_INVALID_PARAM;
+        }
+        (void)RemoveRange(found->va);
+        if (found->ownsMemory) {
+            if (dataOperator_ != nullptr) {
+                dataOperator_->CleanUp();   // nothing may still be copying from or to it
+            }
+            (void)mfrt_free_host(reinterpret_cast<void *>(found->va));
+        }
+        return BM_OK;
+    }
     for (std::unique_ptr<LocalSlice> *slot : {&deviceSlice_, &hostSlice_}) {
         if (slot->get() == slice && slice != nullptr) {
             VaManager::Global().Remove(slice->va);
@@ -197,7 +358,7 @@ bool MemEntity::CheckAddressInEntity(const void *ptr, uint64_t length) const
     if (host_.Contains(a, length)) {
         return a + length <= host_.base + hostBacked_ || options_.rankCount > 1;
     }
-    return false;
+    return rangeCount_.load(std::memory_order_acquire) != 0 && InRanges(a, length);
 }
 
 void MemEntity::LocateAddrAndRank(void *&src, void *&dest, uint64_t length, std::pair<uint32_t, uint32_t> &ranks) const

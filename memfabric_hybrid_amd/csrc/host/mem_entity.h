@@ -6,12 +6,15 @@
 #ifndef MF_MEM_ENTITY_H
 #define MF_MEM_ENTITY_H
 
+#include <atomic>
+#include <functional>
 #include <map>
 #include <memory>
 #include <mutex>
 #include <shared_mutex>
 #include <unordered_map>
 #include <utility>
+#include <vector>
 
 #include "compose_data_op.h"
 #include "gva_layout.h"
@@ -25,6 +28,8 @@ struct LocalSlice {
     hybm_mem_type memType;
     uint64_t va;
     uint64_t size;
+    bool ownsMemory = false;    // allocated for this slice alone, released with it
+    bool outsideWindow = false; // user memory or a stand-alone allocation, known to the entity as a range
 };
 
 class MemEntity {
@@ -40,6 +45,18 @@ public:
     void *WindowBase(hybm_mem_type t) const;
     LocalSlice *AllocLocal(hybm_mem_type t, uint64_t size);
     int FreeLocal(LocalSlice *slice);
+    // Memory the caller owns becomes part of the entity (hybm_register_local_memory,
+    // src/hybm/csrc/hybm_big_mem_entry.cpp); pageable memory is refused.
+    LocalSlice *RegisterLocal(const void *ptr, uint64_t size);
+    // Address ranges outside the two windows that belong to the entity: registered user memory
+    // and memory of peers made addressable here (what hybm_import yields in the reference's
+    // transfer scene).  Ranges are counted, so the same range may be added more than once.
+    int AddRange(uint64_t base, uint64_t size, hybm_mem_type t);
+    int RemoveRange(uint64_t base);
+    uint32_t RangeCount() const
+    {
+        return rangeCount_.load(std::memory_order_acquire);
+    }
 
     bool CheckAddressInEntity(const void *ptr, uint64_t length) const;
     void LocateAddrAndRank(void *&src, void *&dest, uint64_t length, std::pair<uint32_t, uint32_t> &ranks) const;
@@ -69,6 +86,19 @@ private:
     std::unique_ptr<LocalSlice> deviceSlice_;
     std::unique_ptr<LocalSlice> hostSlice_;
     std::shared_ptr<ComposeDataOp> dataOperator_;
+
+    struct Range {
+        uint64_t size;
+        hybm_mem_type type;
+        uint32_t uses;
+    };
+    bool InRanges(uint64_t a, uint64_t length) const;
+    mutable std::shared_mutex rangeLock_;
+    std::map<uint64_t, Range, std::greater<uint64_t>> ranges_;   // by start, descending: lower_bound = covering candidate
+    std::atomic<uint32_t> rangeCount_{0};
+    std::atomic<uint64_t> rangeEpoch_{1};                        // bumped on every change; invalidates per-thread hits
+    std::mutex sliceLock_;
+    std::vector<std::unique_ptr<LocalSlice>> looseSlices_;       // slices that are not a window's backing
 };
 
 class EntityRegistry {

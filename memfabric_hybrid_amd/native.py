@@ -49,6 +49,10 @@ SMEMB_DATA_OP_HOST_TCP = 4
 SMEMB_DATA_OP_DEVICE_RDMA = 8
 SMEMB_DATA_OP_HOST_URMA = 16
 
+SMEM_TRANS_SENDER = 1
+SMEM_TRANS_RECEIVER = 2
+SMEM_TRANS_BOTH = 3
+
 SMEMB_COPY = {"L2G": 0, "G2L": 1, "G2H": 2, "H2G": 3, "L2GH": 4, "GH2L": 5, "GH2H": 6, "H2GH": 7, "G2G": 8,
               "AUTO": 9, "BUTT": 10}
 
@@ -112,6 +116,11 @@ class HybmCopyParams(ctypes.Structure):
     _fields_ = [("src", vp), ("dest", vp), ("dataSize", u64)]
 
 
+class SmemTransConfig(ctypes.Structure):
+    _fields_ = [("role", ctypes.c_int), ("initTimeout", u32), ("deviceId", u32), ("flags", u32),
+                ("dataOpType", ctypes.c_int), ("startConfigServer", ctypes.c_bool)]
+
+
 class HybmTlsConfig(SmemTlsConfig):
     pass
 
@@ -143,6 +152,7 @@ _SIGNATURES = {
     "hybm_alloc_local_memory": (vp, [vp, ctypes.c_int, u64, u32]),
     "hybm_free_local_memory": (i32, [vp, vp, u32, u32]),
     "hybm_get_slice_va": (vp, [vp, vp]),
+    "hybm_register_local_memory": (vp, [vp, vp, u64, u32]),
     "hybm_data_copy": (i32, [vp, ctypes.POINTER(HybmCopyParams), ctypes.c_int, vp, u32]),
     "hybm_data_batch_copy": (i32, [vp, ctypes.POINTER(BatchCopyParams), ctypes.c_int, vp, u32]),
     "hybm_wait": (i32, [vp]),
@@ -227,6 +237,30 @@ _SIGNATURES = {
     "mf_gva_contains": (i32, [u64, u64, u64, u64, u64]),
     "mf_gva_rank": (u32, [u64, u64, u64, u64, u64]),
     "mf_gva_mask48": (u64, [u64]),
+    "mf_trans_combine": (u32, [u64p, u32, u64p]),
+    "mf_trans_translate": (u64, [u64p, u32, u64, u64]),
+    "mf_trans_parse_name": (i32, [ctypes.c_char_p, u8p]),
+    # mf_xcopy_api.h, transfer front-end
+    "smem_trans_config_init": (i32, [ctypes.POINTER(SmemTransConfig)]),
+    "smem_trans_init": (i32, [ctypes.POINTER(SmemTransConfig)]),
+    "smem_trans_uninit": (None, [u32]),
+    "smem_trans_create": (vp, [ctypes.c_char_p, ctypes.c_char_p, ctypes.POINTER(SmemTransConfig)]),
+    "smem_trans_destroy": (None, [vp, u32]),
+    "smem_trans_malloc": (vp, [vp, ctypes.c_size_t]),
+    "smem_trans_free": (i32, [vp, vp]),
+    "smem_trans_register_mem": (i32, [vp, vp, ctypes.c_size_t, u32]),
+    "smem_trans_batch_register_mem": (i32, [vp, ctypes.POINTER(vp), u64p, u32, u32]),
+    "smem_trans_deregister_mem": (i32, [vp, vp]),
+    "smem_trans_write": (i32, [vp, vp, ctypes.c_char_p, vp, ctypes.c_size_t, u32]),
+    "smem_trans_batch_write": (i32, [vp, ctypes.POINTER(vp), ctypes.c_char_p, ctypes.POINTER(vp), u64p, u32, u32]),
+    "smem_trans_read": (i32, [vp, vp, ctypes.c_char_p, vp, ctypes.c_size_t, u32]),
+    "smem_trans_batch_read": (i32, [vp, ctypes.POINTER(vp), ctypes.c_char_p, ctypes.POINTER(vp), u64p, u32, u32]),
+    "smem_trans_read_submit": (i32, [vp, vp, ctypes.c_char_p, vp, ctypes.c_size_t, vp, u32]),
+    "smem_trans_write_submit": (i32, [vp, vp, ctypes.c_char_p, vp, ctypes.c_size_t, vp, u32]),
+    "smem_trans_batch_read_submit": (i32, [vp, ctypes.POINTER(vp), ctypes.c_char_p, ctypes.POINTER(vp), u64p, u32,
+                                           vp, u32]),
+    "smem_trans_batch_write_submit": (i32, [vp, ctypes.POINTER(vp), ctypes.c_char_p, ctypes.POINTER(vp), u64p, u32,
+                                            vp, u32]),
 }
 
 _PLUGIN_SIGNATURES = {

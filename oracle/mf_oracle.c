@@ -18,6 +18,11 @@
  *                                    and the reference's HybmVaManager in oracle/_ref
  *   orc_gva_* / orc_mask48           closed-form integer arithmetic, brute-forced in tests
  *   orc_coalesce                     invariant: byte result unchanged
+ *   orc_trans_*                      transfer front-end arithmetic; the reference's tests need two
+ *                                    processes and a config store and hold no vectors for it
+ *                                    ("parity unpinned" by reference tests) - pinned by closed forms
+ *                                    (page hull is the minimal aligned cover), a brute-force
+ *                                    page-bitmap union, and a linear-scan lookup
  *   orc_ref_kernel_*                 partition formulas of the AscendC kernel; pinned by coverage
  *                                    properties (no reference test exists)
  *   orc_moe_*                        NO reference implementation exists ("parity unpinned" by the
@@ -537,6 +542,78 @@ uint32_t orc_coalesce(const uint64_t *src, const uint64_t *dst, const uint64_t *
         out[3 * k] = s; out[3 * k + 1] = d; out[3 * k + 2] = l; ++k;
     }
     return k;
+}
+
+/* ------------------------------------------------------------------------
+ * Transfer front-end arithmetic (src/smem/csrc/smem_trans/smem_trans_entry.cpp).
+ * ---------------------------------------------------------------------- */
+/* SmemTransEntry::AlignMemory (:604-615): widen [*addr, *addr + *size) to whole 2 MiB pages. */
+void orc_trans_align(uint64_t *addr, uint64_t *size)
+{
+    const uint64_t page = 2ull * 1024 * 1024;
+    const uint64_t mask = ~(page - 1);
+    const uint64_t aligned = *addr & mask;
+    *size += *addr - aligned;
+    *size = (*size + page - 1) & mask;
+    *addr = aligned;
+}
+
+static int orc_pair_less(const void *a, const void *b)
+{
+    const uint64_t *x = (const uint64_t *)a, *y = (const uint64_t *)b;
+    if (x[0] != y[0]) {
+        return x[0] < y[0] ? -1 : 1;
+    }
+    return x[1] < y[1] ? -1 : (x[1] > y[1] ? 1 : 0);
+}
+
+/* SmemTransEntry::CombineMemories (:617-640): sort the (start, size) pairs, then fold every pair
+ * that starts inside or right at the end of the running one into it.  pairs[2*n] is sorted in
+ * place; merged pairs go to out[2*k..]; returns k.  n must be at least 1. */
+uint32_t orc_trans_combine(uint64_t *pairs, uint32_t n, uint64_t *out)
+{
+    qsort(pairs, n, 2 * sizeof(uint64_t), orc_pair_less);
+    uint64_t curStart = pairs[0], curSize = pairs[1];
+    uint32_t k = 0;
+    for (uint32_t i = 1; i < n; ++i) {
+        const uint64_t start = pairs[2 * i], size = pairs[2 * i + 1];
+        if (curStart + curSize >= start) {
+            const uint64_t diff = start - curStart;
+            if (diff > UINT64_MAX - size) {
+                out[2 * k] = curStart; out[2 * k + 1] = curSize; ++k;
+                curStart = start; curSize = size;
+                continue;
+            }
+            curSize = curSize > diff + size ? curSize : diff + size;
+        } else {
+            out[2 * k] = curStart; out[2 * k + 1] = curSize; ++k;
+            curStart = start; curSize = size;
+        }
+    }
+    out[2 * k] = curStart; out[2 * k + 1] = curSize; ++k;
+    return k;
+}
+
+/* Remote-address translation of SmemTransEntry::BatchSyncTransfer (:337-356).  The slice map is
+ * ordered by start address, descending (smem_trans_entry.h:123-124), so lower_bound(remote) is the
+ * slice with the greatest start <= remote.  slices[3*n] = {start, size, mapped}.  Returns the
+ * mapped address, or 0 where the reference returns SM_INVALID_PARAM. */
+uint64_t orc_trans_translate(const uint64_t *slices, uint32_t n, uint64_t remote, uint64_t size)
+{
+    int64_t best = -1;
+    for (uint32_t i = 0; i < n; ++i) {
+        if (slices[3 * i] <= remote && (best < 0 || slices[3 * i] > slices[3 * best])) {
+            best = i;
+        }
+    }
+    if (best < 0) {
+        return 0;
+    }
+    const uint64_t start = slices[3 * best], len = slices[3 * best + 1], mapped = slices[3 * best + 2];
+    if (remote + size > start + len) {
+        return 0;
+    }
+    return mapped + (remote - start);
 }
 
 /* ------------------------------------------------------------------------

@@ -3,7 +3,7 @@
 // test/ut/testcase/hybm/data_operator/hybm_compose_data_op_test.cpp (init order and rollback,
 // intra-node engine first, fallback to the next engine on failure for copy / batch / async,
 // Wait only through the intra-node engine).  Part 2 drives the C API end to end and compares
-// bytes with memcpy.
+// bytes with memcpy.  Part 3 does the same for the transfer front-end.
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
@@ -265,12 +265,157 @@ static void TestCApi()
     CHECK(smem_bm_wait(bm) == SM_NOT_INITIALIZED);
 }
 
+// Part 3: the transfer front-end.  Error codes are those the reference's unit tests pin
+// (test/ut/testcase/smem/smem_trans_test.cpp:145-168 create, :170-219 register, :1016-1098 batch
+// write); the data cases follow its two-object write / read tests (:272-373, :655-779) with both
+// objects in this process.
+static void TestTrans()
+{
+    const char *store = "tcp://127.0.0.1:5432";
+    const char *senderName = "127.0.0.1:5321";
+    const char *receiverName = "127.0.0.1:5322";
+    smem_trans_config_t sendCfg{};
+    CHECK(smem_trans_config_init(nullptr) == SM_INVALID_PARAM);
+    CHECK(smem_trans_config_init(&sendCfg) == SM_OK);
+    CHECK(sendCfg.role == SMEM_TRANS_SENDER && sendCfg.initTimeout == 120 && sendCfg.deviceId == UINT32_MAX &&
+          !sendCfg.startConfigServer);
+    sendCfg.deviceId = 0;
+    sendCfg.dataOpType = SMEMB_DATA_OP_SDMA;
+    smem_trans_config_t recvCfg = sendCfg;
+    recvCfg.role = SMEM_TRANS_RECEIVER;
+
+    CHECK(smem_trans_create(store, senderName, &sendCfg) == nullptr);   // not initialised
+    CHECK(smem_trans_init(nullptr) == SM_INVALID_PARAM);
+    CHECK(smem_trans_init(&sendCfg) == SM_OK);
+    CHECK(smem_trans_init(&sendCfg) == SM_OK);
+    CHECK(smem_trans_create(nullptr, senderName, &sendCfg) == nullptr);
+    CHECK(smem_trans_create(store, nullptr, &sendCfg) == nullptr);
+    CHECK(smem_trans_create(store, senderName, nullptr) == nullptr);
+    CHECK(smem_trans_create("", senderName, &sendCfg) == nullptr);
+    CHECK(smem_trans_create(store, "", &sendCfg) == nullptr);
+    CHECK(smem_trans_create(store, "127.0.0.1:80", &sendCfg) == nullptr);     // port not above 1024
+    CHECK(smem_trans_create(store, "0.0.0.0:5321", &sendCfg) == nullptr);
+    CHECK(smem_trans_create(store, "not-a-name", &sendCfg) == nullptr);
+
+    smem_trans_t sender = smem_trans_create(store, senderName, &sendCfg);
+    smem_trans_t receiver = smem_trans_create(store, receiverName, &recvCfg);
+    smem_trans_t v6 = smem_trans_create("tcp://[::1]:5432", "[::1]:5321", &recvCfg);
+    CHECK(sender != nullptr && receiver != nullptr && v6 != nullptr);
+    CHECK(smem_trans_create(store, senderName, &sendCfg) == nullptr);   // name taken
+
+    const size_t n = 3u << 20;
+    uint8_t *src = static_cast<uint8_t *>(mfrt_alloc_device(n));
+    uint8_t *dst = static_cast<uint8_t *>(mfrt_alloc_device(n));
+    uint8_t *pinned = static_cast<uint8_t *>(mfrt_alloc_host(n));
+    std::vector<uint8_t> pageable(n), pattern(n);
+    Fill(pattern, 77);
+    std::memcpy(src, pattern.data(), n);
+
+    CHECK(smem_trans_register_mem(nullptr, dst, n, 0) == SM_INVALID_PARAM);
+    CHECK(smem_trans_register_mem(receiver, nullptr, n, 0) == SM_INVALID_PARAM);
+    CHECK(smem_trans_register_mem(receiver, dst, 0, 0) == SM_INVALID_PARAM);
+    CHECK(smem_trans_register_mem(receiver, pageable.data(), n, 0) == SM_ERROR);   // cannot be pinned afterwards
+    CHECK(smem_trans_register_mem(receiver, dst + 4096, n - 8192, 0) == SM_OK);
+    CHECK(smem_trans_register_mem(receiver, dst + 4096, n - 8192, 0) == SM_OK);   // the same run again
+    CHECK(smem_trans_register_mem(receiver, dst, 8192, 0) == SM_INVALID_PARAM);    // overlaps it
+
+    const void *locals[3] = {src, src + 70001, src + (1u << 20)};
+    void *remotes[3] = {dst + 4096, dst + 200003, dst + (2u << 20)};
+    size_t sizes[3] = {70001, 4095, 1u << 19};
+    CHECK(smem_trans_batch_write(nullptr, locals, receiverName, remotes, sizes, 3, 0) == SM_INVALID_PARAM);
+    CHECK(smem_trans_batch_write(sender, nullptr, receiverName, remotes, sizes, 3, 0) == SM_INVALID_PARAM);
+    CHECK(smem_trans_batch_write(sender, locals, nullptr, remotes, sizes, 3, 0) == SM_INVALID_PARAM);
+    CHECK(smem_trans_batch_write(sender, locals, receiverName, nullptr, sizes, 3, 0) == SM_INVALID_PARAM);
+    CHECK(smem_trans_batch_write(sender, locals, receiverName, remotes, nullptr, 3, 0) == SM_INVALID_PARAM);
+    CHECK(smem_trans_batch_write(sender, locals, receiverName, remotes, sizes, 0, 0) == SM_INVALID_PARAM);
+    CHECK(smem_trans_batch_write(sender, locals, receiverName, remotes, sizes, 3, ASYNC_COPY_FLAG) == SM_INVALID_PARAM);
+    CHECK(smem_trans_batch_write(sender, locals, "127.0.0.1:9999", remotes, sizes, 3, 0) == SM_INVALID_PARAM);   // unknown peer
+    CHECK(smem_trans_batch_write(sender, locals, "garbage", remotes, sizes, 3, 0) == SM_ERROR);
+    CHECK(smem_trans_batch_write(sender, locals, senderName, remotes, sizes, 3, 0) == SM_INVALID_PARAM);   // senders see receivers only
+    CHECK(smem_trans_batch_write_submit(sender, locals, receiverName, remotes, sizes, 3, nullptr, 0) == SM_INVALID_PARAM);
+
+    std::memset(dst, 0, n);
+    const uint64_t before = fake_rt_launches();
+    CHECK(smem_trans_batch_write(sender, locals, receiverName, remotes, sizes, 3, 0) == SM_OK);
+    CHECK(fake_rt_launches() == before + 1);   // one fused launch for the batch
+    bool ok = true;
+    for (int i = 0; i < 3; ++i) {
+        ok = ok && std::memcmp(remotes[i], locals[i], sizes[i]) == 0;
+    }
+    CHECK(ok && dst[4095] == 0 && dst[4096 + 70001] == 0);
+
+    // ranges that leave the registered run: before it, past its end, and across its end
+    void *outside[1] = {dst};
+    size_t one[1] = {16};
+    const void *oneLocal[1] = {src};
+    CHECK(smem_trans_batch_write(sender, oneLocal, receiverName, outside, one, 1, 0) == SM_INVALID_PARAM);
+    outside[0] = dst + n - 4096;
+    CHECK(smem_trans_batch_write(sender, oneLocal, receiverName, outside, one, 1, 0) == SM_INVALID_PARAM);
+    outside[0] = dst + n - 4096 - 8;
+    CHECK(smem_trans_batch_write(sender, oneLocal, receiverName, outside, one, 1, 0) == SM_INVALID_PARAM);
+    one[0] = 8;
+    CHECK(smem_trans_batch_write(sender, oneLocal, receiverName, outside, one, 1, 0) == SM_OK);           // ends exactly at the end
+
+    // read back through the single-element calls, into pinned and into pageable memory
+    CHECK(smem_trans_read(sender, pinned, receiverName, dst + 4096, 70001, 0) == SM_OK);
+    CHECK(std::memcmp(pinned, src, 70001) == 0);
+    CHECK(smem_trans_read(sender, pageable.data(), receiverName, dst + (2u << 20), 1u << 19, 0) == SM_OK);
+    CHECK(std::memcmp(pageable.data(), src + (1u << 20), 1u << 19) == 0);
+    CHECK(smem_trans_write(sender, pageable.data(), receiverName, dst + 8192, 1000, 0) == SM_OK);
+    CHECK(std::memcmp(dst + 8192, pageable.data(), 1000) == 0);
+    void *stream = mfrt_stream_create();
+    CHECK(smem_trans_write_submit(sender, src + 5, receiverName, dst + 300000, 12345, stream, 0) == SM_OK);
+    CHECK(mfrt_stream_sync(stream) == 0 && std::memcmp(dst + 300000, src + 5, 12345) == 0);
+    CHECK(smem_trans_read_submit(sender, pinned, receiverName, dst + 300000, 12345, stream, 0) == SM_OK);
+    CHECK(mfrt_stream_sync(stream) == 0 && std::memcmp(pinned, src + 5, 12345) == 0);
+    mfrt_stream_destroy(stream);
+
+    // host memory from the object itself; batch registration merges touching pieces into one run
+    uint8_t *given = static_cast<uint8_t *>(smem_trans_malloc(v6, 1000));
+    CHECK(given != nullptr && mfrt_pointer_kind(given) == 2);
+    CHECK(smem_trans_malloc(nullptr, 1000) == nullptr && smem_trans_malloc(v6, 0) == nullptr);
+    CHECK(smem_trans_write(sender, src, "[::1]:5321", given + 100, 900, 0) == SM_OK && std::memcmp(given + 100, src, 900) == 0);
+    uint8_t *second = static_cast<uint8_t *>(mfrt_alloc_device(n));
+    void *pieces[3] = {second + 8192, second, second + 4096};
+    size_t pieceSizes[3] = {4096, 4096, 4096};
+    CHECK(smem_trans_batch_register_mem(v6, pieces, pieceSizes, 3, 0) == SM_OK);
+    CHECK(smem_trans_batch_register_mem(v6, pieces, pieceSizes, 0, 0) == SM_INVALID_PARAM);
+    pieces[1] = nullptr;
+    CHECK(smem_trans_batch_register_mem(v6, pieces, pieceSizes, 3, 0) == SM_INVALID_PARAM);
+    CHECK(smem_trans_write(sender, src, "[::1]:5321", second + 100, 12000, 0) == SM_OK);   // spans all three pieces
+    CHECK(std::memcmp(second + 100, src, 12000) == 0);
+    CHECK(smem_trans_write(sender, src, "[::1]:5321", second + 100, 12289 - 100, 0) == SM_INVALID_PARAM);
+
+    // withdrawing memory ends access to it; so does destroying its owner
+    CHECK(smem_trans_deregister_mem(receiver, nullptr) == SM_INVALID_PARAM);
+    CHECK(smem_trans_deregister_mem(receiver, dst + 4096) == SM_OK);
+    one[0] = 8;
+    outside[0] = dst + 8192;
+    CHECK(smem_trans_batch_write(sender, oneLocal, receiverName, outside, one, 1, 0) == SM_INVALID_PARAM);
+    CHECK(smem_trans_free(v6, nullptr) == SM_INVALID_PARAM);
+    CHECK(smem_trans_free(v6, second) == SM_ERROR);    // registered, not allocated by the object
+    CHECK(smem_trans_free(v6, given) == SM_OK);
+    smem_trans_destroy(v6, 0);
+    CHECK(smem_trans_write(sender, src, "[::1]:5321", second + 100, 100, 0) == SM_INVALID_PARAM);
+    CHECK(smem_trans_register_mem(v6, second, 16, 0) == SM_OBJECT_NOT_EXISTS);
+    smem_trans_destroy(nullptr, 0);
+    smem_trans_destroy(sender, 0);
+    smem_trans_destroy(receiver, 0);
+    smem_trans_uninit(0);
+    CHECK(smem_trans_register_mem(receiver, dst, 16, 0) == SM_INVALID_PARAM);   // not initialised
+    mfrt_free_device(src);
+    mfrt_free_device(dst);
+    mfrt_free_device(second);
+    mfrt_free_host(pinned);
+}
+
 int main()
 {
     SetLogLevel(3);
     SetLogSink([](int, const char *) {});
     TestCompose();
     TestCApi();
+    TestTrans();
     if (g_failed != 0) {
         std::printf("%d check(s) failed\n", g_failed);
         return 1;

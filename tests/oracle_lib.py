@@ -49,6 +49,9 @@ _ORACLE_SIG = {
     "orc_va_classify": (i32, [u64]),
     "orc_va_infer_direction": (i32, [u64, u64]),
     "orc_coalesce": (u32, [u64p, u64p, u64p, u32, u64p]),
+    "orc_trans_align": (None, [u64p, u64p]),
+    "orc_trans_combine": (u32, [u64p, u32, u64p]),
+    "orc_trans_translate": (u64, [u64p, u32, u64, u64]),
     "orc_ref_kernel_single_range": (None, [u64, u32, u32, u64p, u64p]),
     "orc_ref_kernel_batch_range": (None, [u32, u32, u32, ctypes.POINTER(u32), ctypes.POINTER(u32)]),
     "orc_moe_dispatch": (i32, [vp, vp, u32, u32, u32, u32, vp, vp, vp, vp, vp]),
