@@ -13,28 +13,10 @@ namespace {
 
 constexpr uint64_t kBounceBytes = 32ull << 20;
 
-// Pinned staging area for caller memory the GPU cannot address (ordinary
-// pageable host memory).  The reference allocates and frees a device buffer
-// per segment for these directions
-// (src/hybm/csrc/data_operation/host/hybm_data_op_sdma.cpp:171-221); here one
-// pinned area per thread is filled by the CPU and scattered by one launch.
-struct Bounce {
-    void *base = nullptr;
-    ~Bounce()
-    {
-        if (base != nullptr && mfrt_is_initialised() != 0) {
-            (void)mfrt_free_host(base);
-        }
-    }
-    uint8_t *Get()
-    {
-        if (base == nullptr) {
-            base = mfrt_alloc_host(kBounceBytes);
-        }
-        return static_cast<uint8_t *>(base);
-    }
-};
-thread_local Bounce t_bounce;
+// Caller memory the GPU cannot address (ordinary pageable host memory) goes through a pinned
+// staging area.  The reference allocates and frees a device buffer per segment for these
+// directions (src/hybm/csrc/data_operation/host/hybm_data_op_sdma.cpp:171-221); here one pinned
+// area per thread, owned by the engine, is filled by the CPU and scattered by one launch.
 
 struct Piece {
     uint64_t src;
@@ -168,7 +150,7 @@ HipDataOp::Result HipDataOp::Run(void *const *src, void *const *dst, const uint6
         return BM_OK;
     }
 
-    uint8_t *bounce = t_bounce.Get();
+    uint8_t *bounce = static_cast<uint8_t *>(engine.ThreadBounce(kBounceBytes));
     if (bounce == nullptr) {
         MF_FAIL(BM_MALLOC_FAILED, "pinned staging allocation failed");
     }

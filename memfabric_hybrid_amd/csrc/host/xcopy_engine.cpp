@@ -2,6 +2,8 @@
 
 #include <atomic>
 #include <cstring>
+#include <memory>
+#include <mutex>
 
 #include "../../../include/mf_xcopy_types.h"
 #include "../rt/mf_rt.h"
@@ -28,20 +30,20 @@ struct StagingSlot {
     bool pending = false;
 };
 
-struct ThreadCtx {
+// GPU resources of one calling thread: its stream, its staging slots, its bounce area.  They are
+// owned by the engine, not by the thread: a thread holds a lease, and when the thread ends the
+// lease goes back to the idle list without any GPU call (thread-exit destructors run when the
+// runtime, or a tool hooked into it, may already have torn down its own per-thread state).  The
+// next new thread takes an idle lease over; Stop() releases all of them.
+struct ThreadLease {
     void *stream = nullptr;
     StagingSlot slots[kSlots];
     uint32_t cursor = 0;
-    SegList segs;
-    ~ThreadCtx()
+    void *bounce = nullptr;
+    uint64_t bounceBytes = 0;
+
+    void Destroy()   // GPU calls: only from Stop(), on a thread that is alive and bound
     {
-        Release();
-    }
-    void Release()
-    {
-        if (mfrt_is_initialised() == 0) {
-            return;  // runtime already gone at process exit: nothing to hand back
-        }
         for (auto &slot : slots) {
             if (slot.event != nullptr) {
                 if (slot.pending) {
@@ -62,6 +64,85 @@ struct ThreadCtx {
             (void)mfrt_stream_destroy(stream);
             stream = nullptr;
         }
+        if (bounce != nullptr) {
+            (void)mfrt_free_host(bounce);
+            bounce = nullptr;
+            bounceBytes = 0;
+        }
+    }
+};
+
+struct LeasePool {
+    std::mutex lock;
+    std::vector<std::unique_ptr<ThreadLease>> all;
+    std::vector<ThreadLease *> idle;
+    uint64_t epoch = 1;   // bumped by Stop(): leases handed out before are gone
+
+    ThreadLease *Take(uint64_t &epochOut)
+    {
+        std::lock_guard<std::mutex> guard(lock);
+        epochOut = epoch;
+        if (!idle.empty()) {
+            ThreadLease *lease = idle.back();
+            idle.pop_back();
+            return lease;
+        }
+        all.emplace_back(new ThreadLease());
+        return all.back().get();
+    }
+    void GiveBack(ThreadLease *lease, uint64_t leaseEpoch)
+    {
+        std::lock_guard<std::mutex> guard(lock);
+        if (leaseEpoch == epoch) {
+            idle.push_back(lease);
+        }
+    }
+    void DestroyAll()
+    {
+        std::lock_guard<std::mutex> guard(lock);
+        for (auto &lease : all) {
+            lease->Destroy();
+        }
+        all.clear();
+        idle.clear();
+        ++epoch;
+    }
+    uint64_t Epoch()
+    {
+        std::lock_guard<std::mutex> guard(lock);
+        return epoch;
+    }
+};
+
+LeasePool &Leases()
+{
+    static LeasePool *pool = new LeasePool();   // never destroyed: threads may end after static destructors ran
+    return *pool;
+}
+
+std::atomic<uint64_t> g_leaseEpoch{1};   // copy of the pool's epoch that can be read without the lock
+
+struct ThreadCtx {
+    ThreadLease *lease = nullptr;
+    uint64_t epoch = 0;
+    SegList segs;
+    ~ThreadCtx()
+    {
+        if (lease != nullptr) {
+            Leases().GiveBack(lease, epoch);
+            lease = nullptr;
+        }
+    }
+    ThreadLease &Lease()
+    {
+        if (lease == nullptr || epoch != g_leaseEpoch.load(std::memory_order_acquire)) {
+            lease = Leases().Take(epoch);
+        }
+        return *lease;
+    }
+    bool HasLiveLease() const
+    {
+        return lease != nullptr && epoch == g_leaseEpoch.load(std::memory_order_acquire);
     }
 };
 
@@ -72,7 +153,7 @@ uint64_t RoundUp(uint64_t v, uint64_t to)
     return (v + to - 1) / to * to;
 }
 
-int AcquireSlot(ThreadCtx &ctx, uint64_t bytes, StagingSlot *&out)
+int AcquireSlot(ThreadLease &ctx, uint64_t bytes, StagingSlot *&out)
 {
     StagingSlot &slot = ctx.slots[ctx.cursor];
     ctx.cursor = (ctx.cursor + 1) % kSlots;
@@ -331,8 +412,10 @@ void XcopyEngine::Stop()
     if (!started_) {
         return;
     }
-    t_ctx.Release();
+    (void)mfrt_bind_thread();
     (void)mfrt_device_sync();
+    Leases().DestroyAll();   // every thread's stream and staging memory, not only the caller's
+    g_leaseEpoch.store(Leases().Epoch(), std::memory_order_release);
     if (counters_ != nullptr) {
         (void)mfrt_free_device(counters_);
         counters_ = nullptr;
@@ -354,13 +437,32 @@ void *XcopyEngine::NextCounter()
 
 void *XcopyEngine::ThreadStream()
 {
-    if (t_ctx.stream == nullptr) {
+    ThreadLease &lease = t_ctx.Lease();
+    if (lease.stream == nullptr) {
         if (mfrt_bind_thread() != 0) {
             return nullptr;
         }
-        t_ctx.stream = mfrt_stream_create();
+        lease.stream = mfrt_stream_create();
     }
-    return t_ctx.stream;
+    return lease.stream;
+}
+
+void *XcopyEngine::ThreadBounce(uint64_t bytes)
+{
+    ThreadLease &lease = t_ctx.Lease();
+    if (lease.bounceBytes < bytes) {
+        if (mfrt_bind_thread() != 0) {
+            return nullptr;
+        }
+        if (lease.bounce != nullptr) {
+            (void)mfrt_free_host(lease.bounce);
+            lease.bounce = nullptr;
+            lease.bounceBytes = 0;
+        }
+        lease.bounce = mfrt_alloc_host(bytes);
+        lease.bounceBytes = lease.bounce != nullptr ? bytes : 0;
+    }
+    return lease.bounce;
 }
 
 int XcopyEngine::DrainThread()
@@ -368,10 +470,10 @@ int XcopyEngine::DrainThread()
     if (!started_) {
         return BM_NOT_INITIALIZED;
     }
-    if (t_ctx.stream == nullptr) {
+    if (!t_ctx.HasLiveLease() || t_ctx.lease->stream == nullptr) {
         return BM_OK;
     }
-    int err = mfrt_stream_sync(t_ctx.stream);
+    int err = mfrt_stream_sync(t_ctx.lease->stream);
     if (err != 0) {
         MF_FAIL(BM_ERROR, "stream wait failed: " << mfrt_error_string(err));
     }
@@ -432,7 +534,7 @@ int XcopyEngine::Submit(const uint64_t *src, const uint64_t *dst, const uint64_t
     const uint64_t tripleBytes = 24ull * count;
     const uint64_t tableBytes = RoundUp(tripleBytes + 4ull * (count + 1), kUnitBytes);
     StagingSlot *slot = nullptr;
-    int ret = AcquireSlot(ctx, tableBytes, slot);
+    int ret = AcquireSlot(ctx.Lease(), tableBytes, slot);
     if (ret != BM_OK) {
         return ret;
     }
@@ -498,7 +600,7 @@ int XcopyEngine::SubmitDeviceTable(const void *triples, uint32_t n, int route, v
     ThreadCtx &ctx = t_ctx;
     StagingSlot *slot = nullptr;
     const uint64_t prefixBytes = RoundUp(4ull * (n + 2), kUnitBytes);
-    int ret = AcquireSlot(ctx, prefixBytes, slot);
+    int ret = AcquireSlot(ctx.Lease(), prefixBytes, slot);
     if (ret != BM_OK) {
         return ret;
     }

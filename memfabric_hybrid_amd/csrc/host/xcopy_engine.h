@@ -77,6 +77,9 @@ public:
 
     // The calling thread's own stream (created on first use).
     void *ThreadStream();
+    // Pinned, device-mapped staging memory of the calling thread, at least `bytes` long; it lives
+    // until Stop().  NULL when it cannot be allocated.
+    void *ThreadBounce(uint64_t bytes);
     // Wait for everything this thread enqueued on its own stream.
     int DrainThread();
 

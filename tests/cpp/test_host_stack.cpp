@@ -8,6 +8,7 @@
 #include <cstdlib>
 #include <cstring>
 #include <random>
+#include <thread>
 #include <vector>
 
 #include "../../include/mf_hip_dataplane.h"
@@ -409,6 +410,37 @@ static void TestTrans()
     mfrt_free_host(pinned);
 }
 
+// Per-thread GPU resources are leased from the engine: a thread that ends hands its stream back
+// without touching the runtime, the next new thread takes it over, and a stop / start cycle of the
+// library invalidates every lease, also those of threads that are still alive.
+static void TestLeases()
+{
+    CHECK(hybm_init(0, 0) == BM_OK);
+    void *mine = mf_xcopy_thread_stream();
+    CHECK(mine != nullptr && mf_xcopy_thread_stream() == mine);
+    void *first = nullptr, *second = nullptr;
+    std::thread([&] { first = mf_xcopy_thread_stream(); }).join();
+    std::thread([&] { second = mf_xcopy_thread_stream(); }).join();
+    CHECK(first != nullptr && first != mine && second == first);
+    void *a = nullptr, *b = nullptr;
+    std::thread ta([&] { a = mf_xcopy_thread_stream(); });
+    ta.join();
+    std::thread tb([&] {
+        b = mf_xcopy_thread_stream();
+        std::thread inner([&] { a = mf_xcopy_thread_stream(); });   // tb still holds its lease
+        inner.join();
+    });
+    tb.join();
+    CHECK(a != nullptr && b != nullptr && a != b);
+    hybm_uninit();
+    CHECK(mf_xcopy_thread_stream() == nullptr);   // not started
+    CHECK(hybm_init(0, 0) == BM_OK);
+    void *again = mf_xcopy_thread_stream();
+    CHECK(again != nullptr);
+    CHECK(hybm_wait(nullptr) == BM_INVALID_PARAM);
+    hybm_uninit();
+}
+
 int main()
 {
     SetLogLevel(3);
@@ -416,6 +448,7 @@ int main()
     TestCompose();
     TestCApi();
     TestTrans();
+    TestLeases();
     if (g_failed != 0) {
         std::printf("%d check(s) failed\n", g_failed);
         return 1;
