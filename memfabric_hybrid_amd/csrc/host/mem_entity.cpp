@@ -1,5 +1,8 @@
 #include "mem_entity.h"
 
+#include <cstdlib>
+#include <cstring>
+
 #include "../rt/mf_rt.h"
 #include "mf_log.h"
 #include "va_manager.h"
@@ -9,6 +12,16 @@ namespace mf {
 using ock::mf::ExtOptions;
 
 namespace {
+// The device window is reserved address space into which HBM is mapped piece by piece, so that no
+// other allocation can land inside the window.  MF_HIP_GVA_WINDOW=malloc selects the simpler
+// form instead: the local rank's share is one ordinary allocation and the rest of the window is
+// only arithmetic.
+bool WantMappedWindow()
+{
+    const char *mode = std::getenv("MF_HIP_GVA_WINDOW");
+    return mode == nullptr || std::strcmp(mode, "malloc") != 0;
+}
+
 // Every entity counts its range epochs in a block of its own, so a per-thread hit remembered for
 // an entity that is gone can never match a later entity that reuses its address.
 uint64_t NextEpochBlock()
@@ -87,7 +100,22 @@ int MemEntity::ReserveSpace()
     }
     // A world of one: the whole window is this rank's, so it is allocated in
     // one piece now and the address it lands on becomes the window base.
-    if ((options_.memType & HYBM_MEM_TYPE_DEVICE) != 0 && options_.deviceVASpace > 0) {
+    if ((options_.memType & HYBM_MEM_TYPE_DEVICE) != 0 && options_.maxHBMSize > 0 && WantMappedWindow()) {
+        const uint64_t granule = mfrt_window_granularity();
+        const uint64_t bytes = options_.maxHBMSize * options_.rankCount;
+        void *p = granule != 0 && options_.maxHBMSize % granule == 0 ? mfrt_window_reserve(bytes) : nullptr;
+        if (p == nullptr) {
+            MF_FAIL(BM_MALLOC_FAILED, "address window of " << bytes << " bytes could not be reserved (granularity "
+                                                            << granule << ")");
+        }
+        device_.base = reinterpret_cast<uint64_t>(p);
+        device_.stride = options_.maxHBMSize;
+        device_.rankCount = options_.rankCount;
+        device_.rankSpace = options_.maxHBMSize;
+        deviceBacked_ = 0;
+        deviceMapped_ = true;
+        deviceWindowBytes_ = bytes;
+    } else if ((options_.memType & HYBM_MEM_TYPE_DEVICE) != 0 && options_.deviceVASpace > 0) {
         void *p = mfrt_alloc_device(options_.deviceVASpace);
         if (p == nullptr) {
             MF_FAIL(BM_MALLOC_FAILED, "HBM pool allocation of " << options_.deviceVASpace << " bytes failed");
@@ -102,7 +130,12 @@ int MemEntity::ReserveSpace()
         void *p = mfrt_alloc_host(options_.hostVASpace);
         if (p == nullptr) {
             if (device_.base != 0) {
-                (void)mfrt_free_device(reinterpret_cast<void *>(device_.base));
+                if (deviceMapped_) {
+                    (void)mfrt_window_release(reinterpret_cast<void *>(device_.base), deviceWindowBytes_);
+                    deviceMapped_ = false;
+                } else {
+                    (void)mfrt_free_device(reinterpret_cast<void *>(device_.base));
+                }
                 device_ = GvaWindow{};
                 deviceBacked_ = 0;
             }
@@ -144,7 +177,14 @@ int MemEntity::UnreserveSpace()
     }
     if (device_.base != 0) {
         (void)mfrt_device_sync();
-        (void)mfrt_free_device(reinterpret_cast<void *>(device_.base));
+        if (deviceMapped_) {
+            UnmapAll();
+            (void)mfrt_window_release(reinterpret_cast<void *>(device_.base), deviceWindowBytes_);
+            deviceMapped_ = false;
+            deviceWindowBytes_ = 0;
+        } else {
+            (void)mfrt_free_device(reinterpret_cast<void *>(device_.base));
+        }
     }
     if (host_.base != 0) {
         (void)mfrt_free_host(reinterpret_cast<void *>(host_.base));
@@ -209,6 +249,9 @@ LocalSlice *MemEntity::AllocLocal(hybm_mem_type t, uint64_t size)
         MF_ERROR("local allocation with memory type " << t);
         return nullptr;
     }
+    if (device && deviceMapped_) {
+        return AllocMapped(size);
+    }
     const GvaWindow &w = device ? device_ : host_;
     std::unique_ptr<LocalSlice> &slot = device ? deviceSlice_ : hostSlice_;
     const uint64_t backed = device ? deviceBacked_ : hostBacked_;
@@ -222,6 +265,81 @@ LocalSlice *MemEntity::AllocLocal(hybm_mem_type t, uint64_t size)
     }
     slot.reset(new LocalSlice{t, va, size});
     return slot.get();
+}
+
+LocalSlice *MemEntity::AllocMapped(uint64_t size)
+{
+    const uint64_t granule = mfrt_window_granularity();
+    if (granule == 0 || size % granule != 0 || size > options_.maxHBMSize - deviceBacked_) {
+        MF_ERROR("local allocation of " << size << " bytes: not a multiple of " << granule << " or more than the "
+                 << options_.maxHBMSize - deviceBacked_ << " bytes left in this rank's window");
+        return nullptr;
+    }
+    if (mfrt_bind_thread() != 0) {
+        return nullptr;
+    }
+    const uint64_t va = device_.PtrOfRank(options_.rankId) + deviceBacked_;
+    void *mapping = mfrt_window_map(reinterpret_cast<void *>(va), size,
+                                    reinterpret_cast<void *>(device_.PtrOfRank(options_.rankId)), deviceBacked_ + size);
+    if (mapping == nullptr) {
+        MF_ERROR("HBM of " << size << " bytes could not be mapped into the window at offset " << deviceBacked_
+                 << " (step and code " << mfrt_window_last_error() << ")");
+        return nullptr;
+    }
+    if (VaManager::Global().AddOwn(va, size, HYBM_MEM_TYPE_DEVICE, va, options_.rankId) != BM_OK) {
+        (void)mfrt_window_unmap(reinterpret_cast<void *>(va), size, mapping);
+        return nullptr;
+    }
+    std::lock_guard<std::mutex> guard(sliceLock_);
+    mappedSlices_.emplace_back(new LocalSlice{HYBM_MEM_TYPE_DEVICE, va, size});
+    mappedSlices_.back()->mapping = mapping;
+    deviceBacked_ += size;
+    return mappedSlices_.back().get();
+}
+
+int MemEntity::FreeMapped(LocalSlice *slice)
+{
+    std::lock_guard<std::mutex> guard(sliceLock_);
+    bool mine = false;
+    for (auto &s : mappedSlices_) {
+        if (s.get() == slice && !s->released) {
+            s->released = true;
+            mine = true;
+        }
+    }
+    if (!mine) {
+        return BM_INVALID_PARAM;
+    }
+    // The backed bytes of a rank are one prefix of its window: memory goes back to the GPU from
+    // the top, once the slice and everything mapped after it have been released.
+    bool drained = false;
+    while (!mappedSlices_.empty() && mappedSlices_.back()->released) {
+        if (!drained) {
+            if (dataOperator_ != nullptr) {
+                dataOperator_->CleanUp();
+            }
+            (void)mfrt_device_sync();
+            drained = true;
+        }
+        LocalSlice &top = *mappedSlices_.back();
+        VaManager::Global().Remove(top.va);
+        (void)mfrt_window_unmap(reinterpret_cast<void *>(top.va), top.size, top.mapping);
+        deviceBacked_ -= top.size;
+        mappedSlices_.pop_back();
+    }
+    return BM_OK;
+}
+
+void MemEntity::UnmapAll()
+{
+    std::lock_guard<std::mutex> guard(sliceLock_);
+    while (!mappedSlices_.empty()) {
+        LocalSlice &top = *mappedSlices_.back();
+        VaManager::Global().Remove(top.va);
+        (void)mfrt_window_unmap(reinterpret_cast<void *>(top.va), top.size, top.mapping);
+        mappedSlices_.pop_back();
+    }
+    deviceBacked_ = 0;
 }
 
 LocalSlice *MemEntity::RegisterLocal(const void *ptr, uint64_t size)
@@ -331,6 +449,9 @@ int MemEntity::FreeLocal(LocalSlice *slice)
             }
             (void)mfrt_free_host(reinterpret_cast<void *>(found->va));
         }
+        return BM_OK;
+    }
+    if (slice != nullptr && deviceMapped_ && FreeMapped(slice) == BM_OK) {
         return BM_OK;
     }
     for (std::unique_ptr<LocalSlice> *slot : {&deviceSlice_, &hostSlice_}) {

@@ -30,6 +30,8 @@ struct LocalSlice {
     uint64_t size;
     bool ownsMemory = false;    // allocated for this slice alone, released with it
     bool outsideWindow = false; // user memory or a stand-alone allocation, known to the entity as a range
+    void *mapping = nullptr;    // physical memory mapped into a reserved window for this slice
+    bool released = false;      // given back by the caller, unmapped once every later slice is too
 };
 
 class MemEntity {
@@ -84,6 +86,16 @@ private:
     uint64_t deviceBacked_ = 0; // bytes of the local device window that are real memory
     uint64_t hostBacked_ = 0;
     std::unique_ptr<LocalSlice> deviceSlice_;
+    // Mapped-window mode (the default; MF_HIP_GVA_WINDOW=malloc turns it off): the device window is reserved address space of
+    // rankCount * maxHBMSize bytes, and every local allocation maps fresh HBM at the end of the
+    // local rank's backed prefix (the reference's HybmDevLegacySegment does the same with its
+    // driver's reserve / map calls, src/hybm/csrc/mm/hybm_dev_legacy_segment.cpp:123-181).
+    bool deviceMapped_ = false;
+    uint64_t deviceWindowBytes_ = 0;
+    std::vector<std::unique_ptr<LocalSlice>> mappedSlices_;   // in address order
+    LocalSlice *AllocMapped(uint64_t size);
+    int FreeMapped(LocalSlice *slice);
+    void UnmapAll();
     std::unique_ptr<LocalSlice> hostSlice_;
     std::shared_ptr<ComposeDataOp> dataOperator_;
 

@@ -43,6 +43,17 @@ void *mfrt_alloc_host(uint64_t bytes);  /* pinned + device-mapped + portable */
 int mfrt_free_host(void *p);
 int mfrt_pointer_kind(const void *p);
 
+/* Address windows: reserve virtual addresses first, back pieces of them with HBM later
+ * (hipMemAddressReserve / hipMemCreate / hipMemMap).  Sizes and offsets are multiples of
+ * mfrt_window_granularity().  A mapping is named by the handle mfrt_window_map returns;
+ * [accessBase, +accessBytes) is the contiguous mapped run that ends with the new piece. */
+uint64_t mfrt_window_granularity(void);
+void *mfrt_window_reserve(uint64_t bytes);
+int mfrt_window_release(void *base, uint64_t bytes);
+void *mfrt_window_map(void *addr, uint64_t bytes, void *accessBase, uint64_t accessBytes);  /* handle, NULL on failure */
+int mfrt_window_unmap(void *addr, uint64_t bytes, void *handle);
+int mfrt_window_last_error(void);                       /* failed step (1 create, 2 map, 3 access) * 10000 + hipError_t */
+
 void *mfrt_stream_create(void);
 int mfrt_stream_destroy(void *stream);
 int mfrt_stream_sync(void *stream);

@@ -7,6 +7,7 @@
 #include <hip/hip_runtime.h>
 
 #include <atomic>
+#include <cstring>
 #include <mutex>
 
 #include "mf_rt.h"
@@ -121,6 +122,100 @@ extern "C" void *mfrt_alloc_device(uint64_t bytes)
 extern "C" int mfrt_free_device(void *p)
 {
     return Code(hipFree(p));
+}
+
+namespace {
+hipMemAllocationProp WindowProp()
+{
+    hipMemAllocationProp prop{};
+    prop.type = hipMemAllocationTypePinned;
+    prop.location.type = hipMemLocationTypeDevice;
+    prop.location.id = g_device.load();
+    return prop;
+}
+}  // namespace
+
+extern "C" uint64_t mfrt_window_granularity(void)
+{
+    const hipMemAllocationProp prop = WindowProp();
+    size_t granularity = 0;
+    if (hipMemGetAllocationGranularity(&granularity, &prop, hipMemAllocationGranularityRecommended) != hipSuccess ||
+        granularity == 0) {
+        (void)hipGetLastError();
+        return 0;
+    }
+    return granularity;
+}
+
+extern "C" void *mfrt_window_reserve(uint64_t bytes)
+{
+    void *base = nullptr;
+    if (hipMemAddressReserve(&base, bytes, 0, nullptr, 0) != hipSuccess) {
+        (void)hipGetLastError();
+        return nullptr;
+    }
+    return base;
+}
+
+extern "C" int mfrt_window_release(void *base, uint64_t bytes)
+{
+    return Code(hipMemAddressFree(base, bytes));
+}
+
+namespace {
+thread_local int t_windowError = 0;   // step * 10000 + hipError_t of the last failed window call
+}  // namespace
+
+extern "C" int mfrt_window_last_error(void)
+{
+    return t_windowError;
+}
+
+extern "C" void *mfrt_window_map(void *addr, uint64_t bytes, void *accessBase, uint64_t accessBytes)
+{
+    const hipMemAllocationProp prop = WindowProp();
+    hipMemGenericAllocationHandle_t handle{};
+    hipError_t err = hipMemCreate(&handle, bytes, &prop, 0);
+    if (err != hipSuccess) {
+        t_windowError = 10000 + static_cast<int>(err);
+        (void)hipGetLastError();
+        return nullptr;
+    }
+    err = hipMemMap(addr, bytes, 0, handle, 0);
+    if (err != hipSuccess) {
+        t_windowError = 20000 + static_cast<int>(err);
+        (void)hipGetLastError();
+        (void)hipMemRelease(handle);
+        return nullptr;
+    }
+    hipMemAccessDesc access{};
+    access.location = prop.location;
+    access.flags = hipMemAccessFlagsProtReadWrite;
+    // Access is granted on the caller's whole backed run, not on the new piece alone: on this
+    // runtime a grant on a piece inside a reservation is refused (invalid value) unless the piece
+    // has the size of the reservation's first mapping, while a grant that starts at the first
+    // mapping and covers every mapped byte up to the new end is accepted.
+    err = hipMemSetAccess(accessBase, accessBytes, &access, 1);
+    if (err != hipSuccess) {
+        t_windowError = 30000 + static_cast<int>(err);
+        (void)hipGetLastError();
+        (void)hipMemUnmap(addr, bytes);
+        (void)hipMemRelease(handle);
+        return nullptr;
+    }
+    static_assert(sizeof(handle) == sizeof(void *), "allocation handles travel as pointers");
+    void *out = nullptr;
+    std::memcpy(&out, &handle, sizeof(out));
+    return out;
+}
+
+extern "C" int mfrt_window_unmap(void *addr, uint64_t bytes, void *handle)
+{
+    hipMemGenericAllocationHandle_t h{};
+    std::memcpy(&h, &handle, sizeof(h));
+    const int err = Code(hipMemUnmap(addr, bytes));
+    const int rel = Code(hipMemRelease(h));
+    return err != 0 ? err : rel;
 }
 
 extern "C" void *mfrt_alloc_host(uint64_t bytes)

@@ -10,6 +10,8 @@
 #include <map>
 #include <mutex>
 
+#include <sys/mman.h>
+
 #include "../../memfabric_hybrid_amd/csrc/kernels/copy2d_plan.h"
 #include "../../memfabric_hybrid_amd/csrc/kernels/xcopy_plan.h"
 #include "../../memfabric_hybrid_amd/csrc/rt/mf_rt.h"
@@ -85,6 +87,38 @@ void *mfrt_alloc_device(uint64_t bytes) { return Track(bytes, MFRT_PTR_DEVICE); 
 int mfrt_free_device(void *p) { return Untrack(p); }
 void *mfrt_alloc_host(uint64_t bytes) { return Track(bytes, MFRT_PTR_PINNED_HOST); }
 int mfrt_free_host(void *p) { return Untrack(p); }
+// Address windows: reserved as inaccessible pages, so a touch of an unmapped part ends the test
+// with a fault just as it would fault the GPU; mapping makes the pages usable.
+uint64_t mfrt_window_granularity(void) { return 2u << 20; }
+void *mfrt_window_reserve(uint64_t bytes)
+{
+    void *p = mmap(nullptr, bytes, PROT_NONE, MAP_PRIVATE | MAP_ANONYMOUS | MAP_NORESERVE, -1, 0);
+    return p == MAP_FAILED ? nullptr : p;
+}
+int mfrt_window_last_error(void) { return 0; }
+int mfrt_window_release(void *base, uint64_t bytes) { return munmap(base, bytes) == 0 ? 0 : 1; }
+void *mfrt_window_map(void *addr, uint64_t bytes, void *accessBase, uint64_t accessBytes)
+{
+    if (static_cast<char *>(accessBase) + accessBytes != static_cast<char *>(addr) + bytes) {
+        return nullptr;   // the access run must end with the new piece
+    }
+    if (mprotect(addr, bytes, PROT_READ | PROT_WRITE) != 0) {
+        return nullptr;
+    }
+    std::lock_guard<std::mutex> guard(g_lock);
+    g_allocs[reinterpret_cast<uint64_t>(addr)] = {bytes, MFRT_PTR_DEVICE};
+    return addr;
+}
+int mfrt_window_unmap(void *addr, uint64_t bytes, void *handle)
+{
+    if (handle != addr) {
+        return 1;
+    }
+    std::lock_guard<std::mutex> guard(g_lock);
+    g_allocs.erase(reinterpret_cast<uint64_t>(addr));
+    (void)madvise(addr, bytes, MADV_DONTNEED);
+    return mprotect(addr, bytes, PROT_NONE) == 0 ? 0 : 1;
+}
 int mfrt_pointer_kind(const void *p)
 {
     std::lock_guard<std::mutex> guard(g_lock);

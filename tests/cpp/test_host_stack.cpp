@@ -441,14 +441,68 @@ static void TestLeases()
     hybm_uninit();
 }
 
+// Mapped-window mode: the device window is reserved address space, local allocations map HBM
+// into it piece by piece, and only the mapped prefix passes the pool-side range check.
+static void TestMappedWindow()
+{
+    CHECK(hybm_init(0, 0) == BM_OK);
+    const uint64_t page = 2u << 20;
+    hybm_options o{};
+    o.bmType = HYBM_TYPE_HOST_INITIATE;
+    o.memType = HYBM_MEM_TYPE_DEVICE;
+    o.bmDataOpType = HYBM_DOP_TYPE_SDMA;
+    o.rankCount = 1;
+    o.maxHBMSize = 64 * page;      // window
+    o.deviceVASpace = 8 * page;    // what the caller intends to back
+    o.scene = HYBM_SCENE_DEFAULT;
+    o.dramShmFd = -1;
+    hybm_entity_t e = hybm_create_entity(300, &o, 0);
+    CHECK(e != nullptr);
+    CHECK(hybm_reserve_mem_space(e, 0) == BM_OK);
+    uint8_t *base = static_cast<uint8_t *>(hybm_get_memory_ptr(e, HYBM_MEM_TYPE_DEVICE));
+    CHECK(base != nullptr);
+    std::vector<uint8_t> local(4 * page);
+    Fill(local, 9);
+    hybm_copy_params cp{local.data(), base, page};
+    CHECK(hybm_data_copy(e, &cp, HYBM_LOCAL_HOST_TO_GLOBAL_DEVICE, nullptr, 0) == BM_INVALID_PARAM);   // nothing mapped yet
+    CHECK(hybm_alloc_local_memory(e, HYBM_MEM_TYPE_DEVICE, page + 4096, 0) == nullptr);               // not a granule multiple
+    hybm_mem_slice_t s1 = hybm_alloc_local_memory(e, HYBM_MEM_TYPE_DEVICE, 2 * page, 0);
+    hybm_mem_slice_t s2 = hybm_alloc_local_memory(e, HYBM_MEM_TYPE_DEVICE, 3 * page, 0);
+    CHECK(s1 != nullptr && s2 != nullptr);
+    CHECK(hybm_get_slice_va(e, s1) == base && hybm_get_slice_va(e, s2) == base + 2 * page);
+    CHECK(hybm_alloc_local_memory(e, HYBM_MEM_TYPE_DEVICE, 60 * page, 0) == nullptr);                  // window exhausted
+    cp = {local.data(), base + page, 3 * page};                                                         // spans both slices
+    CHECK(hybm_data_copy(e, &cp, HYBM_LOCAL_HOST_TO_GLOBAL_DEVICE, nullptr, 0) == BM_OK);
+    CHECK(std::memcmp(base + page, local.data(), 3 * page) == 0);
+    cp = {local.data(), base + 4 * page, 2 * page};                                                     // one page past the mapped prefix
+    CHECK(hybm_data_copy(e, &cp, HYBM_LOCAL_HOST_TO_GLOBAL_DEVICE, nullptr, 0) == BM_INVALID_PARAM);
+    CHECK(mf_va_infer_direction(reinterpret_cast<uint64_t>(base + 3 * page), reinterpret_cast<uint64_t>(local.data())) ==
+          HYBM_GLOBAL_DEVICE_TO_LOCAL_HOST);
+    // the lower slice stays mapped while the upper one is in use; both go when the upper is released
+    CHECK(hybm_free_local_memory(e, s1, 1, 0) == BM_OK);
+    cp = {base, local.data(), page};
+    CHECK(hybm_data_copy(e, &cp, HYBM_GLOBAL_DEVICE_TO_LOCAL_HOST, nullptr, 0) == BM_OK);
+    CHECK(hybm_free_local_memory(e, s1, 1, 0) == BM_INVALID_PARAM);
+    CHECK(hybm_free_local_memory(e, s2, 1, 0) == BM_OK);
+    CHECK(hybm_data_copy(e, &cp, HYBM_GLOBAL_DEVICE_TO_LOCAL_HOST, nullptr, 0) == BM_INVALID_PARAM);
+    hybm_mem_slice_t s3 = hybm_alloc_local_memory(e, HYBM_MEM_TYPE_DEVICE, page, 0);
+    CHECK(s3 != nullptr && hybm_get_slice_va(e, s3) == base);
+    hybm_destroy_entity(e, 0);
+    hybm_uninit();
+}
+
 int main()
 {
     SetLogLevel(3);
     SetLogSink([](int, const char *) {});
     TestCompose();
-    TestCApi();
+    TestCApi();                                  // device window: reserved address space, HBM mapped in
+    setenv("MF_HIP_GVA_WINDOW", "malloc", 1);
+    TestCApi();                                  // device window: one ordinary allocation
+    unsetenv("MF_HIP_GVA_WINDOW");
     TestTrans();
     TestLeases();
+    TestMappedWindow();
     if (g_failed != 0) {
         std::printf("%d check(s) failed\n", g_failed);
         return 1;
