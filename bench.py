@@ -250,6 +250,25 @@ def extras_block(lib, pool, dev, batches, tables, steps):
         us, _ = timer.run(lambda d=d, s=s: lib.mfrt_memcpy_async(d, s, 1 << 30, timer.stream), 3, warm=1)
         out[name + "_GBps"] = round((1 << 30) / us / 1e3, 2)   # the runtime's DMA engines, for comparison
 
+    # ---- pageable caller memory: CPU memcpy into a pinned ring overlapped with the launches (PCIe- and memcpy-inclusive)
+    page_host = np.empty(1 << 30, dtype=np.uint8)
+    page_host[:] = 7
+    php = page_host.ctypes.data
+    pageable = {}
+    for name, ct, params in (("h2d_1GiB", int(bm.BmCopyType.H2G), native.SmemCopyParams(php, dev, 1 << 30)),
+                             ("d2h_1GiB", int(bm.BmCopyType.G2H), native.SmemCopyParams(dev, php, 1 << 30))):
+        lib.smem_bm_copy(handle, ctypes.byref(params), ct, 0)
+        t0 = time.perf_counter()
+        for _ in range(2):
+            if lib.smem_bm_copy(handle, ctypes.byref(params), ct, 0) != 0:
+                raise RuntimeError(native.last_error())
+        pageable[name + "_GBps"] = round(2 * (1 << 30) / (time.perf_counter() - t0) / 1e9, 2)
+    t0 = time.perf_counter()
+    ctypes.memmove(php, php + (1 << 29), 1 << 29)
+    pageable["host_memmove_GBps"] = round((1 << 29) / (time.perf_counter() - t0) / 1e9, 2)
+    out["pageable_host_memory"] = pageable
+    del page_host
+
     # ---- large single copies through smem_bm_copy --------------------------------------------------------------
     big = {}
     for size_name, nbytes in (("1GiB", 1 << 30), ("2GiB", 2 << 30)):

@@ -11,7 +11,10 @@
 namespace mf {
 namespace {
 
-constexpr uint64_t kBounceBytes = 32ull << 20;
+constexpr uint32_t kRounds = 16;                       // slots of the staging ring
+constexpr uint64_t kRoundBytes = 2ull << 20;           // bytes per slot: ~70 us of CPU memcpy against ~40 us on the link
+constexpr uint64_t kBounceBytes = kRounds * kRoundBytes;
+static_assert(kRounds <= XcopyEngine::kBounceEvents, "one event per staging slot");
 
 // Caller memory the GPU cannot address (ordinary pageable host memory) goes through a pinned
 // staging area.  The reference allocates and frees a device buffer per segment for these
@@ -154,7 +157,11 @@ HipDataOp::Result HipDataOp::Run(void *const *src, void *const *dst, const uint6
     if (bounce == nullptr) {
         MF_FAIL(BM_MALLOC_FAILED, "pinned staging allocation failed");
     }
-    // Cut the batch into pieces that fit the staging area, then move it round by round.
+    // The staging area is a ring of kRounds slots.  The CPU side (memcpy between caller memory and
+    // a slot) and the GPU side (one fused launch per slot) overlap: towards the GPU the CPU fills
+    // slot r+1 while the launch of slot r runs, away from it the CPU empties slot r-1 while the
+    // launch that fills slot r runs.  An event per slot says when its launch has finished.
+    const uint64_t roundBytes = kRoundBytes;   // 512 KiB rounds were tried for small batches: slower (more launches)
     std::vector<Piece> pieces;
     pieces.reserve(n);
     for (uint32_t i = 0; i < n; ++i) {
@@ -162,58 +169,115 @@ HipDataOp::Result HipDataOp::Run(void *const *src, void *const *dst, const uint6
         uint64_t d = reinterpret_cast<uint64_t>(dst[i]);
         uint64_t left = len[i];
         while (left > 0) {
-            const uint64_t take = left > kBounceBytes ? kBounceBytes : left;
+            const uint64_t take = left > roundBytes ? roundBytes : left;
             pieces.push_back(Piece{s, d, take});
             s += take;
             d += take;
             left -= take;
         }
     }
+    struct Round {
+        size_t begin = 0;
+        size_t end = 0;
+        std::vector<uint64_t> staged;   // slot address of every piece of the round
+    };
+    Round rounds[kRounds];
     std::vector<uint64_t> a;
     std::vector<uint64_t> b;
     std::vector<uint64_t> l;
+    auto drain = [&](Round &round, uint32_t slot) -> int {   // GPU -> caller: wait for the slot's launch, empty it
+        if (round.begin == round.end) {
+            return BM_OK;
+        }
+        int err = mfrt_event_sync(engine.ThreadBounceEvent(slot));
+        if (err != 0) {
+            MF_FAIL(BM_ERROR, "copy failed on the GPU: " << mfrt_error_string(err));
+        }
+        for (size_t i = round.begin; i < round.end; ++i) {
+            std::memcpy(reinterpret_cast<void *>(pieces[i].dst), reinterpret_cast<const void *>(round.staged[i - round.begin]),
+                        pieces[i].len);
+        }
+        round.begin = round.end = 0;
+        return BM_OK;
+    };
+    const int route = srcPageable ? MFRT_ROUTE_FROM_HOST : MFRT_ROUTE_TO_HOST;
     size_t at = 0;
-    while (at < pieces.size()) {
+    uint32_t r = 0;
+    for (; at < pieces.size(); ++r) {
+        const uint32_t slot = r % kRounds;
+        Round &round = rounds[slot];
+        void *event = engine.ThreadBounceEvent(slot);
+        if (event == nullptr) {
+            MF_FAIL(BM_ERROR, "event creation failed");
+        }
+        if (r >= kRounds) {   // the slot's previous launch must be over before the slot is reused
+            if (dstPageable) {
+                int ret = drain(round, slot);
+                if (ret != BM_OK) {
+                    return ret;
+                }
+            } else {
+                int err = mfrt_event_sync(event);
+                if (err != 0) {
+                    MF_FAIL(BM_ERROR, "copy failed on the GPU: " << mfrt_error_string(err));
+                }
+            }
+        }
         a.clear();
         b.clear();
         l.clear();
+        round.staged.clear();
+        round.begin = at;
         uint64_t used = 0;
-        size_t end = at;
-        while (end < pieces.size()) {
-            const uint64_t padded = (pieces[end].len + 63) & ~63ull;  // keep staged pieces 64-byte aligned
-            if (used + padded > kBounceBytes) {
+        const uint64_t base = reinterpret_cast<uint64_t>(bounce) + static_cast<uint64_t>(slot) * kRoundBytes;
+        while (at < pieces.size()) {
+            const uint64_t padded = (pieces[at].len + 63) & ~63ull;  // keep staged pieces 64-byte aligned
+            if (used + padded > roundBytes) {
                 break;
             }
-            const uint64_t slot = reinterpret_cast<uint64_t>(bounce) + used;
+            const uint64_t where = base + used;
             if (srcPageable) {
-                std::memcpy(reinterpret_cast<void *>(slot), reinterpret_cast<const void *>(pieces[end].src),
-                            pieces[end].len);
-                a.push_back(slot);
-                b.push_back(pieces[end].dst);
+                std::memcpy(reinterpret_cast<void *>(where), reinterpret_cast<const void *>(pieces[at].src), pieces[at].len);
+                a.push_back(where);
+                b.push_back(pieces[at].dst);
             } else {
-                a.push_back(pieces[end].src);
-                b.push_back(slot);
+                a.push_back(pieces[at].src);
+                b.push_back(where);
+                round.staged.push_back(where);
             }
-            l.push_back(pieces[end].len);
+            l.push_back(pieces[at].len);
             used += padded;
-            ++end;
+            ++at;
         }
-        const int route = srcPageable ? MFRT_ROUTE_FROM_HOST : MFRT_ROUTE_TO_HOST;
+        round.end = at;
         int ret = engine.Submit(a.data(), b.data(), l.data(), static_cast<uint32_t>(l.size()), route, stream, nullptr, 0);
         if (ret != BM_OK) {
             return ret;
         }
-        int err = mfrt_stream_sync(stream);  // the staging area is reused next round
+        int err = mfrt_event_record(event, stream);
+        if (err != 0) {
+            MF_FAIL(BM_ERROR, "event record failed: " << mfrt_error_string(err));
+        }
+        if (dstPageable && r > 0) {   // while this launch runs, empty the slot of the one before
+            ret = drain(rounds[(r - 1) % kRounds], (r - 1) % kRounds);
+            if (ret != BM_OK) {
+                return ret;
+            }
+        }
+    }
+    if (dstPageable) {
+        for (uint32_t k = 0; k < kRounds; ++k) {   // what is still staged, oldest first
+            const uint32_t slot = (r + k) % kRounds;
+            int ret = drain(rounds[slot], slot);
+            if (ret != BM_OK) {
+                return ret;
+            }
+        }
+    } else {
+        int err = mfrt_stream_sync(stream);   // caller memory has been consumed; the copy itself is done as well
         if (err != 0) {
             MF_FAIL(BM_ERROR, "copy failed on the GPU: " << mfrt_error_string(err));
         }
-        if (dstPageable) {
-            for (size_t i = at; i < end; ++i) {
-                std::memcpy(reinterpret_cast<void *>(pieces[i].dst), reinterpret_cast<const void *>(b[i - at]),
-                            pieces[i].len);
-            }
-        }
-        at = end;
     }
     return BM_OK;
 }

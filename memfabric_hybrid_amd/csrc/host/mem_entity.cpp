@@ -567,8 +567,8 @@ int MemEntity::Wait()
 
 EntityRegistry &EntityRegistry::Instance()
 {
-    static EntityRegistry registry;
-    return registry;
+    static EntityRegistry *registry = new EntityRegistry();   // never destroyed: what is still alive at process exit is left to the operating system, no GPU call runs from a static destructor
+    return *registry;
 }
 
 void EntityRegistry::SetFactory(OperatorFactory factory)

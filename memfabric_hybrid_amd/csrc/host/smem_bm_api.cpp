@@ -214,8 +214,10 @@ std::shared_mutex g_lock;
 bool g_inited = false;
 uint16_t g_deviceId = 0;
 std::shared_mutex g_entriesLock;
-std::map<uint32_t, std::shared_ptr<BmEntry>> g_entriesById;
-std::unordered_map<const void *, std::shared_ptr<BmEntry>> g_entriesByPtr;
+// Both maps are never destroyed: a pool the caller did not destroy is left to the operating system at
+// process exit instead of being torn down (GPU calls included) from a static destructor.
+auto &g_entriesById = *new std::map<uint32_t, std::shared_ptr<BmEntry>>();
+auto &g_entriesByPtr = *new std::unordered_map<const void *, std::shared_ptr<BmEntry>>();
 
 std::shared_ptr<BmEntry> FindEntry(smem_bm_t handle)
 {

@@ -120,8 +120,8 @@ int TranslatePeerAddress(const PeerSliceMap &slices, uint64_t remote, uint64_t s
 
 TransDirectory &TransDirectory::Instance()
 {
-    static TransDirectory directory;
-    return directory;
+    static TransDirectory *directory = new TransDirectory();   // never destroyed, like the entity registry it refers to
+    return *directory;
 }
 
 bool TransDirectory::Interested(const TransEntry &watcher, const TransEntry &owner)

@@ -29,8 +29,8 @@ const typename Map::mapped_type *Floor(const Map &m, uint64_t va)
 
 VaManager &VaManager::Global()
 {
-    static VaManager manager;
-    return manager;
+    static VaManager *manager = new VaManager();   // never destroyed: entities that outlive main() may still refer to it
+    return *manager;
 }
 
 void VaManager::SetDeviceProbe(DeviceProbe probe)

@@ -41,6 +41,7 @@ struct ThreadLease {
     uint32_t cursor = 0;
     void *bounce = nullptr;
     uint64_t bounceBytes = 0;
+    void *bounceEvents[XcopyEngine::kBounceEvents] = {};
 
     void Destroy()   // GPU calls: only from Stop(), on a thread that is alive and bound
     {
@@ -68,6 +69,12 @@ struct ThreadLease {
             (void)mfrt_free_host(bounce);
             bounce = nullptr;
             bounceBytes = 0;
+        }
+        for (void *&event : bounceEvents) {
+            if (event != nullptr) {
+                (void)mfrt_event_destroy(event);
+                event = nullptr;
+            }
         }
     }
 };
@@ -463,6 +470,18 @@ void *XcopyEngine::ThreadBounce(uint64_t bytes)
         lease.bounceBytes = lease.bounce != nullptr ? bytes : 0;
     }
     return lease.bounce;
+}
+
+void *XcopyEngine::ThreadBounceEvent(uint32_t index)
+{
+    if (index >= kBounceEvents) {
+        return nullptr;
+    }
+    ThreadLease &lease = t_ctx.Lease();
+    if (lease.bounceEvents[index] == nullptr && mfrt_bind_thread() == 0) {
+        lease.bounceEvents[index] = mfrt_event_create();
+    }
+    return lease.bounceEvents[index];
 }
 
 int XcopyEngine::DrainThread()

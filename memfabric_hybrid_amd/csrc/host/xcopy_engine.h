@@ -80,6 +80,9 @@ public:
     // Pinned, device-mapped staging memory of the calling thread, at least `bytes` long; it lives
     // until Stop().  NULL when it cannot be allocated.
     void *ThreadBounce(uint64_t bytes);
+    // One of the calling thread's events for slots of that staging memory (index < kBounceEvents).
+    static constexpr uint32_t kBounceEvents = 16;
+    void *ThreadBounceEvent(uint32_t index);
     // Wait for everything this thread enqueued on its own stream.
     int DrainThread();
 

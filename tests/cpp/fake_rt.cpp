@@ -5,6 +5,7 @@
 // its plan at once with the SAME chunk geometry the kernels use (csrc/kernels/xcopy_plan.h), streams
 // and events are tokens.  Never linked into the product libraries.
 #include <cstdint>
+#include <cstdio>
 #include <cstdlib>
 #include <cstring>
 #include <map>
@@ -65,6 +66,17 @@ void RunChunk(uint64_t src, uint64_t dst, uint64_t len, uint64_t k, uint32_t uni
 }  // namespace
 
 extern "C" {
+// After this call any allocation, free, mapping or launch aborts: the test binary arms it at the
+// end of main() to prove that nothing touches the GPU runtime from static destructors.
+static bool g_sealed = false;
+void fake_rt_seal(void) { g_sealed = true; }
+static void Guard(const char *what)
+{
+    if (g_sealed) {
+        std::fprintf(stderr, "runtime call after main(): %s\n", what);
+        std::abort();
+    }
+}
 uint64_t fake_rt_launches(void) { return g_launches; }
 uint64_t fake_rt_chunks(void) { return g_chunksRun; }
 
@@ -84,9 +96,9 @@ int mfrt_device_id(void) { return g_device; }
 uint32_t mfrt_cu_count(void) { return 256; }
 const char *mfrt_error_string(int) { return "fake runtime error"; }
 void *mfrt_alloc_device(uint64_t bytes) { return Track(bytes, MFRT_PTR_DEVICE); }
-int mfrt_free_device(void *p) { return Untrack(p); }
+int mfrt_free_device(void *p) { Guard("mfrt_free_device"); return Untrack(p); }
 void *mfrt_alloc_host(uint64_t bytes) { return Track(bytes, MFRT_PTR_PINNED_HOST); }
-int mfrt_free_host(void *p) { return Untrack(p); }
+int mfrt_free_host(void *p) { Guard("mfrt_free_host"); return Untrack(p); }
 // Address windows: reserved as inaccessible pages, so a touch of an unmapped part ends the test
 // with a fault just as it would fault the GPU; mapping makes the pages usable.
 uint64_t mfrt_window_granularity(void) { return 2u << 20; }
@@ -96,7 +108,7 @@ void *mfrt_window_reserve(uint64_t bytes)
     return p == MAP_FAILED ? nullptr : p;
 }
 int mfrt_window_last_error(void) { return 0; }
-int mfrt_window_release(void *base, uint64_t bytes) { return munmap(base, bytes) == 0 ? 0 : 1; }
+int mfrt_window_release(void *base, uint64_t bytes) { Guard("mfrt_window_release"); return munmap(base, bytes) == 0 ? 0 : 1; }
 void *mfrt_window_map(void *addr, uint64_t bytes, void *accessBase, uint64_t accessBytes)
 {
     if (static_cast<char *>(accessBase) + accessBytes != static_cast<char *>(addr) + bytes) {
@@ -110,7 +122,7 @@ void *mfrt_window_map(void *addr, uint64_t bytes, void *accessBase, uint64_t acc
     return addr;
 }
 int mfrt_window_unmap(void *addr, uint64_t bytes, void *handle)
-{
+{ Guard("mfrt_window_unmap");
     if (handle != addr) {
         return 1;
     }
@@ -131,11 +143,11 @@ int mfrt_pointer_kind(const void *p)
     return a < it->first + it->second.first ? it->second.second : MFRT_PTR_PAGEABLE;
 }
 void *mfrt_stream_create(void) { return malloc(8); }
-int mfrt_stream_destroy(void *s) { free(s); return 0; }
-int mfrt_stream_sync(void *) { return 0; }
-int mfrt_device_sync(void) { return 0; }
+int mfrt_stream_destroy(void *s) { Guard("mfrt_stream_destroy"); free(s); return 0; }
+int mfrt_stream_sync(void *) { Guard("mfrt_stream_sync"); return 0; }
+int mfrt_device_sync(void) { Guard("mfrt_device_sync"); return 0; }
 void *mfrt_event_create(void) { return malloc(8); }
-int mfrt_event_destroy(void *e) { free(e); return 0; }
+int mfrt_event_destroy(void *e) { Guard("mfrt_event_destroy"); free(e); return 0; }
 int mfrt_event_record(void *, void *) { return 0; }
 int mfrt_event_sync(void *) { return 0; }
 int mfrt_event_done(void *) { return 1; }

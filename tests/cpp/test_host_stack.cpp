@@ -17,6 +17,7 @@
 #include "../../memfabric_hybrid_amd/csrc/host/mf_log.h"
 
 extern "C" uint64_t fake_rt_launches(void);
+extern "C" void fake_rt_seal(void);
 
 using namespace mf;
 using ock::mf::DataOperatorPtr;
@@ -507,6 +508,28 @@ int main()
         std::printf("%d check(s) failed\n", g_failed);
         return 1;
     }
+    // A caller that never tears down: a pool with memory, a transfer object with registered memory and
+    // a used stream stay alive past main().  Static destructors must leave the runtime alone.
+    smem_bm_config_t cfg;
+    smem_bm_config_init(&cfg);
+    CHECK(smem_bm_init("tcp://127.0.0.1:1", 1, 0, &cfg) == SM_OK);
+    smem_bm_t left = smem_bm_create(5, 1, SMEMB_DATA_OP_SDMA, 4u << 20, 4u << 20, 0);
+    CHECK(left != nullptr && smem_bm_join(left, 0) == SM_OK);
+    smem_copy_params cp{smem_bm_ptr_by_mem_type(left, SMEM_MEM_TYPE_HOST, 0), smem_bm_ptr_by_mem_type(left, SMEM_MEM_TYPE_DEVICE, 0), 4096};
+    CHECK(smem_bm_copy(left, &cp, SMEMB_COPY_G2G, ASYNC_COPY_FLAG) == SM_OK);
+    smem_trans_config_t tc;
+    smem_trans_config_init(&tc);
+    tc.deviceId = 0;
+    tc.role = SMEM_TRANS_BOTH;
+    CHECK(smem_trans_init(&tc) == SM_OK);
+    smem_trans_t leftTrans = smem_trans_create("tcp://127.0.0.1:5432", "127.0.0.1:5400", &tc);
+    CHECK(leftTrans != nullptr && smem_trans_malloc(leftTrans, 100) != nullptr);
+    if (g_failed != 0) {
+        std::printf("%d check(s) failed\n", g_failed);
+        return 1;
+    }
     std::printf("host stack tests passed\n");
+    std::fflush(stdout);
+    fake_rt_seal();
     return 0;
 }

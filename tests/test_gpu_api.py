@@ -144,6 +144,11 @@ def test_pageable_batches_go_through_staging(pool, lib, oracle):
     dst = dev + offs + np.arange(count) * 64 + 1
     assert pool.copy_data_batch((np_ptr(payload) + offs).tolist(), dst.tolist(), lens.tolist(), count,
                                 bm.BmCopyType.H2G) == 0, native.last_error()
+    landed = np.empty(total + count * 64 + 1, dtype=np.uint8)     # what is in the pool now, read by plain hipMemcpy
+    assert lib.mfrt_memcpy(np_ptr(landed), dev, len(landed)) == 0
+    for i in range(count):
+        at = int(offs[i]) + i * 64 + 1
+        assert np.array_equal(landed[at:at + int(lens[i])], payload[int(offs[i]):int(offs[i]) + int(lens[i])]), i
     back = np.zeros(total, dtype=np.uint8)
     assert pool.copy_data_batch(dst.tolist(), (np_ptr(back) + offs).tolist(), lens.tolist(), count,
                                 bm.BmCopyType.G2H) == 0
