@@ -580,6 +580,8 @@ int XcopyEngine::Submit(const uint64_t *src, const uint64_t *dst, const uint64_t
     err = mfk_xcopy_table(devBase, devBase + tripleBytes, nullptr, count, static_cast<uint32_t>(nchunk), units, route,
                           grid, mask, maskValue, counter, stream);
     if (err != 0) {
+        // the staging launch may still be reading the slot: keep it reserved until the stream has passed this point
+        slot->pending = mfrt_event_record(slot->event, stream) == 0;
         MF_FAIL(BM_ERROR, "xcopy table launch failed: " << mfrt_error_string(err));
     }
     // Both halves of the slot are free again once the table kernel has run.

@@ -1,0 +1,107 @@
+"""Concurrent callers on the GPU: eight host threads, each on its own stream and its own slice of
+one pool, mix small batches (descriptors in the kernel arguments), large batches (descriptor table
+staged through the thread's slot ring), pageable host memory (staging ring) and transfer-object
+writes, every result compared with the oracle.  A second generation of threads then reuses the
+streams and staging memory the first one handed back.  The reference serves concurrent callers the
+same way, one stream per calling thread (src/hybm/csrc/ts_engine/hybm_stream_manager.cpp:73-90)."""
+
+import threading
+
+import numpy as np
+import pytest
+
+from memfabric_hybrid_amd import bm, native, workloads
+from memfabric_hybrid_amd.transfer import TransferEngine
+from tests import gpu_util
+from tests.oracle_lib import np_ptr
+
+pytestmark = pytest.mark.gpu
+
+MIB = 1 << 20
+THREADS = 8
+SLICE = 32 * MIB                 # per thread: lower half sources, upper half destinations
+POOL = THREADS * SLICE
+DECODE = "127.0.0.1:16322"
+
+
+def _worker(tid, generation, lib, oracle, pool, prefill, data, errors):
+    try:
+        assert lib.mfrt_bind_thread() == 0
+        dev = pool.peer_rank_ptr(0, bm.BmMemType.DEVICE) + tid * SLICE
+        mine = data[tid * SLICE:(tid + 1) * SLICE]
+        half = SLICE // 2
+        scratch = np.zeros(half, dtype=np.uint8)          # ordinary pageable memory of this thread
+        for step in range(6):
+            seed = 0x7000 + generation * 1000 + tid * 10 + step
+            count = (100, 700, 60, 122, 3000, 40)[step]
+            src, dst, lens = workloads.ragged_batch(seed, SLICE, count, max_len=(SLICE // 4) // count)
+            want = np.zeros(half, dtype=np.uint8)
+            assert lib.mfrt_memset(dev + half, 0, half) == 0
+            kind = step % 3
+            if kind == 0:      # pool to pool, asynchronous, then wait
+                gpu_util.oracle_batch(oracle, mine, want, src, dst - half, lens)
+                ret = pool.copy_data_batch((dev + src).tolist(), (dev + dst).tolist(), lens.tolist(), count,
+                                           bm.BmCopyType.G2G, native.ASYNC_COPY_FLAG)
+                assert ret == 0, native.last_error()
+                assert pool.wait() == 0
+            elif kind == 1:    # pageable host memory into the pool and out again
+                scratch[:] = mine[:half]
+                gpu_util.oracle_batch(oracle, scratch, want, src, dst - half, lens)
+                ret = pool.copy_data_batch((np_ptr(scratch) + src).tolist(), (dev + dst).tolist(), lens.tolist(), count,
+                                           bm.BmCopyType.H2G)
+                assert ret == 0, native.last_error()
+                back = np.zeros(half, dtype=np.uint8)
+                ret = pool.copy_data_batch((dev + dst).tolist(), (np_ptr(back) + (dst - half)).tolist(), lens.tolist(),
+                                           count, bm.BmCopyType.G2H)
+                assert ret == 0, native.last_error()
+                assert np.array_equal(back, want), f"thread {tid} step {step}: read back through staging differs"
+            else:              # transfer-object write into the registered pool
+                keep = lens > 0
+                gpu_util.oracle_batch(oracle, mine, want, src[keep], dst[keep] - half, lens[keep])
+                ret = prefill.batch_transfer_sync_write(DECODE, (dev + src[keep]).tolist(), (dev + dst[keep]).tolist(),
+                                                        lens[keep].tolist())
+                assert ret == 0, native.last_error()
+            got = np.empty(half, dtype=np.uint8)
+            assert lib.mfrt_memcpy(np_ptr(got), dev + half, half) == 0
+            assert np.array_equal(got, want), f"thread {tid} generation {generation} step {step} kind {kind}"
+    except BaseException as exc:  # noqa: BLE001
+        errors.append((tid, generation, repr(exc)))
+
+
+def test_eight_threads_two_generations(lib, oracle):
+    assert bm.initialize("tcp://127.0.0.1:5432", 1, 0) == 0, native.last_error()
+    pool = bm.create(9, 0, POOL, bm.BmDataOpType.SDMA)
+    prefill, decode = TransferEngine(), TransferEngine()
+    try:
+        assert pool.join() == 0
+        dev = pool.peer_rank_ptr(0, bm.BmMemType.DEVICE)
+        data = np.empty(POOL, dtype=np.uint8)
+        oracle.orc_fill_random(np_ptr(data), POOL, 0x7EAD)
+        assert lib.mfrt_memcpy(dev, np_ptr(data), POOL) == 0
+        assert prefill.initialize("tcp://127.0.0.1:16432", "127.0.0.1:16321", "Prefill", 0) == 0
+        assert decode.initialize("tcp://127.0.0.1:16432", DECODE, "Decode", 0) == 0
+        assert decode.register_memory(dev, POOL) == 0, native.last_error()
+        launches = lib.mf_xcopy_launch_count()
+        for generation in range(2):
+            errors = []
+            threads = [threading.Thread(target=_worker, args=(t, generation, lib, oracle, pool, prefill, data, errors))
+                       for t in range(THREADS)]
+            for t in threads:
+                t.start()
+            for t in threads:
+                t.join(timeout=100)
+            assert not any(t.is_alive() for t in threads), "a worker is stuck"
+            assert not errors, errors
+            # sources were never written: the lower halves still hold the original bytes
+            check = np.empty(SLICE // 2, dtype=np.uint8)
+            for t in range(THREADS):
+                assert lib.mfrt_memcpy(np_ptr(check), dev + t * SLICE, SLICE // 2) == 0
+                assert np.array_equal(check, data[t * SLICE:t * SLICE + SLICE // 2]), t
+        assert lib.mf_xcopy_launch_count() > launches
+        assert decode.unregister_memory(dev) == 0
+    finally:
+        prefill.destroy()
+        decode.destroy()
+        prefill.unInitialize()
+        pool.destroy()
+        bm.uninitialize()
