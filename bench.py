@@ -316,6 +316,33 @@ def extras_transfer(lib, dev, batches, steps):
             "frac_of_hbm_peak": frac(hbm, HBM_PEAK_GBPS)}
 
 
+def extras_plugin(lib, dev, tables, steps):
+    """The same KV batches through the two-symbol plugin, as the reference's SDMA operator drives it:
+    a pinned parameter table per call, a completion word, 32 as the word's value."""
+    plug = native.plugin()
+    slot = 16384 * 24
+    params = lib.mfrt_alloc_host(len(tables) * slot + 4096)
+    if not params:
+        return {"error": "allocation failed"}
+    for b, (s, d, l) in enumerate(tables):
+        t = np.ctypeslib.as_array((ctypes.c_uint64 * (3 * len(l))).from_address(params + b * slot))
+        t[0::3], t[1::3], t[2::3] = dev + s, dev + d, l
+    mask = params + len(tables) * slot
+    timer = Timer(lib)
+    i = [0]
+
+    def step():
+        plug.hybm_batch_copy_extend(params + (i[0] % len(tables)) * slot, len(tables[0][2]), mask, 32, timer.stream)
+        i[0] += 1
+
+    us, _ = timer.run(step, max(400, steps // 4), warm=50)
+    hbm = 2 * int(tables[0][2].sum()) / us / 1e3
+    ok = ctypes.c_uint64.from_address(mask).value == 32
+    lib.mfrt_free_host(params)
+    return {"api": "hybm_batch_copy_extend(pinned table, 122, mask, 32, stream)", "us_per_batch": round(us, 2),
+            "hbm_GBps": round(hbm, 1), "frac_of_hbm_peak": frac(hbm, HBM_PEAK_GBPS), "mask_ok": ok}
+
+
 def extras_paged(lib):
     """Paged KV gather/scatter: 4096 distinct 32 KiB pages out of a 40 GiB pool."""
     page, count = 32768, 4096
@@ -511,6 +538,7 @@ def main():
         extras, copy_ceiling = extras_block(lib, pool, dev, batches, tables, args.steps)
         result["roofline"]["frac_of_measured_copy_ceiling"] = frac(achieved, copy_ceiling)
         extras["kv122_transfer_write"] = extras_transfer(lib, dev, batches, args.steps)
+        extras["kv122_plugin"] = extras_plugin(lib, dev, tables, args.steps)
     pool.destroy()  # give the pools back before the larger workloads allocate
     if not args.no_extras:
         extras["paged_kv_40GiB"] = extras_paged(lib)

@@ -34,7 +34,8 @@ void hybm_copy_extend(void *src, void *dst, uint64_t len, uint32_t dim, void *st
  *        count <= 16384 per call in the reference, any count here.
  * mask:  device-accessible address of one uint64_t that the caller zeroed.
  *        When the last byte of the batch has been written and `param` will
- *        not be read again, the kernel stores `dim` into it (the reference's
+ *        not be read again, a one-lane launch queued right behind the copy on
+ *        the same stream stores `dim` into it (the reference's
  *        "slot is free again" marker, hybm_data_op_sdma.cpp:487-497 and
  *        hybm_copy_kernel.cpp:113-118).  May be NULL.
  * Enqueues on `stream` and returns without waiting. */

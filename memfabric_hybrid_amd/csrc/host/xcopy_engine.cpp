@@ -12,11 +12,9 @@
 namespace mf {
 namespace {
 
-constexpr uint32_t kCounters = 4096;          // completion counters shared by launches that carry a mask
 constexpr uint32_t kSlots = 4;                // table staging slots per thread
 constexpr uint64_t kInlinePiece = 1ull << 30; // cut for segments the 32-bit inline length cannot hold
 
-std::atomic<uint32_t> g_counterCursor{0};
 std::atomic<uint64_t> g_launches{0};
 
 // One descriptor table in flight: host fills `host`, a copy kernel moves it to
@@ -400,16 +398,6 @@ int XcopyEngine::Start(int device)
     if (started_) {
         return BM_OK;
     }
-    counters_ = mfrt_alloc_device(kCounters * sizeof(uint32_t));
-    if (counters_ == nullptr) {
-        MF_FAIL(BM_MALLOC_FAILED, "completion counter allocation failed");
-    }
-    err = mfrt_memset(counters_, 0, kCounters * sizeof(uint32_t));
-    if (err != 0) {
-        (void)mfrt_free_device(counters_);
-        counters_ = nullptr;
-        MF_FAIL(BM_ERROR, "completion counter clear failed: " << mfrt_error_string(err));
-    }
     started_ = true;
     return BM_OK;
 }
@@ -423,10 +411,6 @@ void XcopyEngine::Stop()
     (void)mfrt_device_sync();
     Leases().DestroyAll();   // every thread's stream and staging memory, not only the caller's
     g_leaseEpoch.store(Leases().Epoch(), std::memory_order_release);
-    if (counters_ != nullptr) {
-        (void)mfrt_free_device(counters_);
-        counters_ = nullptr;
-    }
     started_ = false;
     mfrt_shutdown();
 }
@@ -434,12 +418,6 @@ void XcopyEngine::Stop()
 bool XcopyEngine::Started() const
 {
     return started_;
-}
-
-void *XcopyEngine::NextCounter()
-{
-    const uint32_t idx = g_counterCursor.fetch_add(1, std::memory_order_relaxed) % kCounters;
-    return static_cast<uint32_t *>(counters_) + idx;
 }
 
 void *XcopyEngine::ThreadStream()
@@ -521,7 +499,6 @@ int XcopyEngine::Submit(const uint64_t *src, const uint64_t *dst, const uint64_t
     }
     ThreadCtx &ctx = t_ctx;
     const uint32_t cu = mfrt_cu_count();
-    void *counter = mask != nullptr ? NextCounter() : nullptr;
     InlinePlan plan;
     bool inlined = false;
     uint32_t units = 0;
@@ -540,7 +517,7 @@ int XcopyEngine::Submit(const uint64_t *src, const uint64_t *dst, const uint64_t
     }
     if (inlined) {
         const uint32_t grid = GridFor(plan.nchunk, cu, route, tuning_);
-        int err = mfk_xcopy_inline(&plan, route, grid, mask, maskValue, counter, stream);
+        int err = mfk_xcopy_inline(&plan, route, grid, mask, maskValue, stream);
         if (err != 0) {
             MF_FAIL(BM_ERROR, "xcopy launch failed: " << mfrt_error_string(err));
         }
@@ -571,14 +548,14 @@ int XcopyEngine::Submit(const uint64_t *src, const uint64_t *dst, const uint64_t
     InlinePlan stagePlan;
     const uint32_t stageUnits = kXcopyThreads;
     (void)BuildInlinePlan(stage, stageUnits, stagePlan);
-    int err = mfk_xcopy_inline(&stagePlan, MFRT_ROUTE_FROM_HOST, stagePlan.nchunk, nullptr, 0, nullptr, stream);
+    int err = mfk_xcopy_inline(&stagePlan, MFRT_ROUTE_FROM_HOST, stagePlan.nchunk, nullptr, 0, stream);
     if (err != 0) {
         MF_FAIL(BM_ERROR, "descriptor staging launch failed: " << mfrt_error_string(err));
     }
     const uint32_t grid = GridFor(nchunk, cu, route, tuning_);
     const uint8_t *devBase = static_cast<const uint8_t *>(slot->dev);
     err = mfk_xcopy_table(devBase, devBase + tripleBytes, nullptr, count, static_cast<uint32_t>(nchunk), units, route,
-                          grid, mask, maskValue, counter, stream);
+                          grid, mask, maskValue, stream);
     if (err != 0) {
         // the staging launch may still be reading the slot: keep it reserved until the stream has passed this point
         slot->pending = mfrt_event_record(slot->event, stream) == 0;
@@ -609,12 +586,11 @@ int XcopyEngine::SubmitDeviceTable(const void *triples, uint32_t n, int route, v
             MF_FAIL(BM_ERROR, "cannot create the thread's stream");
         }
     }
-    void *counter = mask != nullptr ? NextCounter() : nullptr;
     if (n == 0) {
         InlinePlan empty;
         SegList none;
         (void)BuildInlinePlan(none, kXcopyThreads, empty);
-        int err = mfk_xcopy_inline(&empty, route, 1, mask, maskValue, counter, stream);
+        int err = mfk_xcopy_inline(&empty, route, 1, mask, maskValue, stream);
         return err == 0 ? BM_OK : BM_ERROR;
     }
     // The prefix is computed on the GPU; its slot is only ever touched by kernels of this stream.
@@ -635,7 +611,7 @@ int XcopyEngine::SubmitDeviceTable(const void *triples, uint32_t n, int route, v
     }
     const uint32_t cu = mfrt_cu_count();
     const uint32_t grid = GridFor(~0ull, cu, route, tuning_);
-    err = mfk_xcopy_table(triples, first, nchunkDev, n, 0, units, route, grid, mask, maskValue, counter, stream);
+    err = mfk_xcopy_table(triples, first, nchunkDev, n, 0, units, route, grid, mask, maskValue, stream);
     if (err != 0) {
         MF_FAIL(BM_ERROR, "xcopy table launch failed: " << mfrt_error_string(err));
     }

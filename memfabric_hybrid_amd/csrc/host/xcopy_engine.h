@@ -99,10 +99,8 @@ public:
 
 private:
     XcopyEngine() = default;
-    void *NextCounter();
 
     XcopyTuning tuning_;
-    void *counters_ = nullptr;   // device uint32[kCounters], all zero between launches
     bool started_ = false;
 };
 

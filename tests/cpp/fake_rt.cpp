@@ -156,7 +156,7 @@ int mfrt_memcpy(void *dst, const void *src, uint64_t bytes) { std::memmove(dst, 
 int mfrt_memcpy_async(void *dst, const void *src, uint64_t bytes, void *) { std::memmove(dst, src, bytes); return 0; }
 int mfrt_memset(void *dst, int value, uint64_t bytes) { std::memset(dst, value, bytes); return 0; }
 
-int mfk_xcopy_inline(const void *inlinePlan, int, uint32_t, void *mask, uint32_t maskValue, void *, void *)
+int mfk_xcopy_inline(const void *inlinePlan, int, uint32_t, void *mask, uint32_t maskValue, void *)
 {
     const mf::InlinePlan &p = *static_cast<const mf::InlinePlan *>(inlinePlan);
     ++g_launches;
@@ -175,7 +175,7 @@ int mfk_xcopy_inline(const void *inlinePlan, int, uint32_t, void *mask, uint32_t
 }
 
 int mfk_xcopy_table(const void *triples, const void *first, const void *nchunkDev, uint32_t nseg, uint32_t nchunk,
-                    uint32_t units, int, uint32_t, void *mask, uint32_t maskValue, void *, void *)
+                    uint32_t units, int, uint32_t, void *mask, uint32_t maskValue, void *)
 {
     const uint64_t *t = static_cast<const uint64_t *>(triples);
     const uint32_t *f = static_cast<const uint32_t *>(first);
