@@ -90,6 +90,52 @@ def test_every_small_length_and_alignment_in_one_launch(gpu, oracle):
     _check_d2d(gpu, oracle, 2 * half, np.array(src_off), np.array(dst_off), np.array(lens), 0xA1)
 
 
+@pytest.mark.parametrize("count", [16384, 70000])
+def test_batches_at_and_beyond_the_reference_slot_size(gpu, oracle, count):
+    """16 384 segments fill one parameter slot of the reference (hybm_data_op_sdma.cpp:25-31 there);
+    this path takes any count in one call."""
+    pool = 96 * MIB
+    src, dst, lens = workloads.ragged_batch(count, pool, count, max_len=600)
+    _check_d2d(gpu, oracle, pool, src, dst, lens, count)
+
+
+def test_one_segment_longer_than_4gib(gpu, oracle):
+    """A single copy whose length does not fit 32 bits (5 GiB + 5 bytes, odd offsets on both sides):
+    the planner cuts it into pieces.  Source blocks differ from each other, so a piece that lands
+    at a wrong offset cannot go unnoticed; the bytes around the destination must stay untouched."""
+    n = 5 * (1 << 30) + 5
+    block = _random_bytes(oracle, 64 * MIB, 0x5A1)
+    blocks = (n + len(block) - 1) // len(block) + 1
+    src = gpu_util.DeviceBuffer(gpu, blocks * len(block))
+    dst = gpu_util.DeviceBuffer(gpu, n + 4096)
+    try:
+        for i in range(blocks):
+            src.upload(block ^ np.uint8((i * 29 + 3) & 0xFF), i * len(block))
+        dst.fill(0xEE)
+        gpu_util.xcopy(gpu, np.array([src.ptr + 7], dtype=np.uint64), np.array([dst.ptr + 1001], dtype=np.uint64),
+                       np.array([n], dtype=np.uint64), native.ROUTE_HBM)
+        edge = dst.download(0, 1001)
+        assert np.all(edge == 0xEE)
+        edge = dst.download(1001 + n, 4096 - 1001)
+        assert np.all(edge == 0xEE)
+        step = 256 * MIB
+        for at in range(0, n, step):
+            take = min(step, n - at)
+            got = dst.download(1001 + at, take)
+            want = np.empty(take, dtype=np.uint8)
+            pos = 0
+            while pos < take:                      # rebuild the source bytes [7 + at + pos, ...) from the block pattern
+                absolute = 7 + at + pos
+                i, off = divmod(absolute, len(block))
+                m = min(len(block) - off, take - pos)
+                want[pos:pos + m] = block[off:off + m] ^ np.uint8((i * 29 + 3) & 0xFF)
+                pos += m
+            assert np.array_equal(got, want), at
+    finally:
+        src.free()
+        dst.free()
+
+
 def test_single_large_copy_with_odd_edges(gpu, oracle):
     pool = 192 * MIB
     _check_d2d(gpu, oracle, pool, np.array([3]), np.array([96 * MIB + 5]), np.array([80 * MIB + 123]), 0xB2)
