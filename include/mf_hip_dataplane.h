@@ -59,8 +59,9 @@ typedef struct {
 int32_t mf_xcopy_2d_batch(const mf_copy2d_desc *descs, uint32_t n, int32_t route, void *stream);
 
 /* Launch-shape knobs.  units: 16-byte units per workgroup chunk (0 = choose
- * per batch); wgPerCu / wgPerCuLink: resident workgroups per CU for HBM and
- * host-link routes (0 = keep). */
+ * per batch); wgPerCu: grid cap in workgroups per CU on HBM routes (0 = the
+ * default: one workgroup per chunk, no cap); wgPerCuLink: workgroups per CU
+ * on host-link routes (0 = the default, 1). */
 int32_t mf_xcopy_tune(uint32_t units, uint32_t wgPerCu, uint32_t wgPerCuLink);
 uint32_t mf_xcopy_choose_units(uint64_t totalBytes, uint32_t cuCount, int32_t route);
 uint64_t mf_xcopy_launch_count(void);
@@ -98,7 +99,7 @@ int32_t mf_moe_dispatch(const void *x, const int32_t *topk, uint32_t tokens, uin
 int32_t mf_moe_combine(const void *rows, const int32_t *rowOf, const float *weights, uint32_t tokens, uint32_t hidden,
                        uint32_t topK, void *y, void *stream);
 
-/* Yardstick kernels of known traffic (grid-stride, 128-bit, nontemporal): kind 0
+/* Yardstick kernels of known traffic (one workgroup per 16 KiB tile, 128-bit, nontemporal): kind 0
  * copies `bytes` from src to dst, kind 1 fills dst, kind 2 reads src (dst: a
  * 4-byte device sink).  They measure what this GPU sustains for a flat copy, a
  * pure write and a pure read, and calibrate hardware byte counters. */

@@ -69,7 +69,8 @@ MF_EXPORT int32_t mf_xcopy_2d_batch(const mf_copy2d_desc *descs, uint32_t n, int
             plan.first[i] = 0xFFFFFFFFu;
         }
         plan.nchunk = static_cast<uint32_t>(run);
-        const uint64_t cap = static_cast<uint64_t>(cu) * engine.Tuning().wgPerCu;
+        const uint32_t perCu = engine.Tuning().wgPerCu;   // 0: one workgroup per row group
+        const uint64_t cap = perCu == 0 ? run : static_cast<uint64_t>(cu) * perCu;
         int err = mfk_copy2d(&plan, static_cast<uint32_t>(run < cap ? run : cap), stream);
         used = 0;
         run = 0;

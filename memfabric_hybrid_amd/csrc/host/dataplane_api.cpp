@@ -45,8 +45,7 @@ MF_EXPORT int32_t mf_probe_hbm(int32_t kind, void *dst, const void *src, uint64_
     if (stream == nullptr) {
         stream = engine.ThreadStream();
     }
-    const uint32_t grid = (mfrt_cu_count() == 0 ? 256 : mfrt_cu_count()) * 64;
-    int err = mfk_probe(kind, dst, src, bytes, grid, stream);
+    int err = mfk_probe(kind, dst, src, bytes, 0, stream);   // one workgroup per 16 KiB tile
     if (err != 0) {
         MF_FAIL(BM_ERROR, "probe launch failed");
     }
@@ -63,12 +62,8 @@ MF_EXPORT int32_t mf_xcopy_tune(uint32_t units, uint32_t wgPerCu, uint32_t wgPer
 {
     XcopyTuning &t = XcopyEngine::Instance().Tuning();
     t.unitsOverride = units;
-    if (wgPerCu != 0) {
-        t.wgPerCu = wgPerCu;
-    }
-    if (wgPerCuLink != 0) {
-        t.wgPerCuLink = wgPerCuLink;
-    }
+    t.wgPerCu = wgPerCu;                               // 0: no cap, one workgroup per chunk
+    t.wgPerCuLink = wgPerCuLink == 0 ? 1 : wgPerCuLink;
     return BM_OK;
 }
 

@@ -199,9 +199,17 @@ int AcquireSlot(ThreadLease &ctx, uint64_t bytes, StagingSlot *&out)
 
 uint32_t GridFor(uint64_t nchunk, uint32_t cuCount, int route, const XcopyTuning &tuning)
 {
+    // HBM routes: one workgroup per chunk unless a cap is set.  Measured on 128 MiB ... 4 GiB copies:
+    // letting the hardware dispatcher hand out 16 KiB chunks one by one sustains 6.0-6.2 TB/s, a
+    // grid capped at 16 workgroups per CU that strides over the chunks 5.3-5.7 TB/s (its static
+    // assignment leaves a tail).  Link routes: one workgroup per CU, more only adds contention.
     const bool link = route == MFRT_ROUTE_TO_HOST || route == MFRT_ROUTE_FROM_HOST || route >= 16;
-    const uint32_t perCu = link ? tuning.wgPerCuLink : tuning.wgPerCu;
-    uint64_t cap = static_cast<uint64_t>(cuCount == 0 ? 256 : cuCount) * (perCu == 0 ? 1 : perCu);
+    const uint32_t perCu = link ? (tuning.wgPerCuLink == 0 ? 1 : tuning.wgPerCuLink) : tuning.wgPerCu;
+    const uint64_t limit = 0x7FFFFFFFull;
+    uint64_t cap = perCu == 0 ? limit : static_cast<uint64_t>(cuCount == 0 ? 256 : cuCount) * perCu;
+    if (cap > limit) {
+        cap = limit;
+    }
     uint64_t grid = nchunk < cap ? nchunk : cap;
     return grid == 0 ? 1u : static_cast<uint32_t>(grid);
 }
@@ -250,9 +258,9 @@ uint32_t ChooseUnits(uint64_t totalBytes, uint32_t cuCount, int route, const Xco
         return static_cast<uint32_t>(RoundUp(tuning.unitsOverride, kXcopyThreads));
     }
     // Measured on MI355X (256 CUs): 16 KiB per workgroup step (four 128-bit accesses per lane, one
-    // full tile) is the sweet spot from a few MiB up to a GiB; it also divides the usual power-of-two
-    // block sizes, so no workgroup runs a ragged tile.  Below 1 MiB the batch is latency bound and
-    // 4 KiB chunks put more CUs to work; beyond 1 GiB fewer, longer chunks save lookups.
+    // full tile) is the sweet spot from a few MiB to at least 4 GiB (32 and 64 KiB chunks: 3-10 %
+    // slower); it also divides the usual power-of-two block sizes, so no workgroup runs a ragged
+    // tile.  Below 1 MiB the batch is latency bound and 4 KiB chunks put more CUs to work.
     if (route == MFRT_ROUTE_TO_HOST || route == MFRT_ROUTE_FROM_HOST) {
         // The host link, not the GPU, is the bound: one workgroup per CU with small chunks keeps
         // the link busy without flooding it (measured: 56 GB/s out, 55 GB/s in on a Gen5 x16 link).
@@ -264,10 +272,7 @@ uint32_t ChooseUnits(uint64_t totalBytes, uint32_t cuCount, int route, const Xco
     if (totalBytes < (1ull << 20)) {
         return tuning.minUnits;
     }
-    if (totalBytes <= (1ull << 30)) {
-        return 4 * kXcopyThreads;
-    }
-    return tuning.maxUnits;
+    return 4 * kXcopyThreads;
 }
 
 bool BuildInlinePlan(const SegList &segs, uint32_t units, InlinePlan &plan)
@@ -610,7 +615,7 @@ int XcopyEngine::SubmitDeviceTable(const void *triples, uint32_t n, int route, v
         MF_FAIL(BM_ERROR, "xcopy plan launch failed: " << mfrt_error_string(err));
     }
     const uint32_t cu = mfrt_cu_count();
-    const uint32_t grid = GridFor(~0ull, cu, route, tuning_);
+    const uint32_t grid = GridFor(static_cast<uint64_t>(cu == 0 ? 256 : cu) * 64, cu, route, tuning_);   // chunk count is only known on the GPU
     err = mfk_xcopy_table(triples, first, nchunkDev, n, 0, units, route, grid, mask, maskValue, stream);
     if (err != 0) {
         MF_FAIL(BM_ERROR, "xcopy table launch failed: " << mfrt_error_string(err));

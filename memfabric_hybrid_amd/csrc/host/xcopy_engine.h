@@ -42,8 +42,8 @@ void NormalizeSegments(const uint64_t *src, const uint64_t *dst, const uint64_t 
 
 struct XcopyTuning {
     uint32_t unitsOverride = 0;  // 16-byte units per chunk, 0 = choose from batch size
-    uint32_t wgPerCu = 16;       // workgroups launched per CU for HBM routes (grid cap)
-    uint32_t wgPerCuLink = 1;    // the same for routes bound by the host link
+    uint32_t wgPerCu = 0;        // HBM routes: grid cap in workgroups per CU, 0 = one workgroup per chunk
+    uint32_t wgPerCuLink = 1;    // routes bound by the host link: workgroups per CU
     uint32_t minUnits = kXcopyThreads;
     uint32_t maxUnits = 16 * kXcopyThreads;
 };

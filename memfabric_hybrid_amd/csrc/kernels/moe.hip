@@ -313,7 +313,7 @@ __device__ __forceinline__ uint32_t ToBf16(float f)
     return (w + 0x7FFFu + ((w >> 16) & 1u)) >> 16;
 }
 
-template <uint32_t kTopK, uint32_t kThreads, bool kNtLoad>
+template <uint32_t kTopK, uint32_t kThreads, bool kNtLoad, uint32_t kBatch = 1>
 __global__ __launch_bounds__(kThreads) void MoeCombineKernel(const u32x4 *__restrict__ rowsIn,
                                                              const int32_t *__restrict__ rowOf,
                                                              const float *__restrict__ weights, uint32_t topK,
@@ -342,35 +342,48 @@ __global__ __launch_bounds__(kThreads) void MoeCombineKernel(const u32x4 *__rest
     const MF_GLOBAL u32x4 *in = reinterpret_cast<const MF_GLOBAL u32x4 *>(reinterpret_cast<uint64_t>(rowsIn));
     MF_GLOBAL u32x4 *dst = reinterpret_cast<MF_GLOBAL u32x4 *>(reinterpret_cast<uint64_t>(y)) +
                            static_cast<uint64_t>(token) * unitsPerRow;
-    for (uint32_t u = begin + threadIdx.x; u < end; u += kThreads) {
-        u32x4 v[kSlots];
+    // kBatch column positions per lane are requested together (kBatch * K loads in flight per lane)
+    // before any of them is consumed.
+    for (uint32_t u0 = begin + threadIdx.x; u0 < end; u0 += kBatch * kThreads) {
+        u32x4 v[kBatch][kSlots];
 #pragma unroll
-        for (uint32_t k = 0; k < kSlots; ++k) {
-            if (k < nk) {
-                v[k] = kNtLoad ? __builtin_nontemporal_load(in + rowBase[k] + u) : in[rowBase[k] + u];
-            }
-        }
-        float acc[8];
+        for (uint32_t b = 0; b < kBatch; ++b) {
+            const uint32_t u = u0 + b * kThreads;
 #pragma unroll
-        for (uint32_t i = 0; i < 8; ++i) {
-            acc[i] = 0.0f;
-        }
-#pragma unroll
-        for (uint32_t k = 0; k < kSlots; ++k) {
-            if (k < nk) {
-#pragma unroll
-                for (uint32_t i = 0; i < 4; ++i) {
-                    acc[2 * i] = __builtin_fmaf(w[k], Bf16Lo(v[k][i]), acc[2 * i]);
-                    acc[2 * i + 1] = __builtin_fmaf(w[k], Bf16Hi(v[k][i]), acc[2 * i + 1]);
+            for (uint32_t k = 0; k < kSlots; ++k) {
+                if (k < nk && u < end) {
+                    v[b][k] = kNtLoad ? __builtin_nontemporal_load(in + rowBase[k] + u) : in[rowBase[k] + u];
                 }
             }
         }
-        u32x4 o;
 #pragma unroll
-        for (uint32_t i = 0; i < 4; ++i) {
-            o[i] = ToBf16(acc[2 * i]) | (ToBf16(acc[2 * i + 1]) << 16);
+        for (uint32_t b = 0; b < kBatch; ++b) {
+            const uint32_t u = u0 + b * kThreads;
+            if (u >= end) {
+                break;
+            }
+            float acc[8];
+#pragma unroll
+            for (uint32_t i = 0; i < 8; ++i) {
+                acc[i] = 0.0f;
+            }
+#pragma unroll
+            for (uint32_t k = 0; k < kSlots; ++k) {
+                if (k < nk) {
+#pragma unroll
+                    for (uint32_t i = 0; i < 4; ++i) {
+                        acc[2 * i] = __builtin_fmaf(w[k], Bf16Lo(v[b][k][i]), acc[2 * i]);
+                        acc[2 * i + 1] = __builtin_fmaf(w[k], Bf16Hi(v[b][k][i]), acc[2 * i + 1]);
+                    }
+                }
+            }
+            u32x4 o;
+#pragma unroll
+            for (uint32_t i = 0; i < 4; ++i) {
+                o[i] = ToBf16(acc[2 * i]) | (ToBf16(acc[2 * i + 1]) << 16);
+            }
+            __builtin_nontemporal_store(o, dst + u);
         }
-        __builtin_nontemporal_store(o, dst + u);
     }
 }
 
@@ -378,7 +391,7 @@ __global__ __launch_bounds__(kThreads) void MoeCombineKernel(const u32x4 *__rest
 }  // namespace mf
 
 static int g_permuteVariant = -1;  // -1: choose from the row width
-static int g_combineVariant = 0;
+static int g_combineVariant = -1;  // -1: choose from the row width
 extern "C" void mfk_moe_tune(int permuteVariant, int combineVariant)
 {
     g_permuteVariant = permuteVariant;
@@ -424,25 +437,29 @@ extern "C" int mfk_moe_dispatch(const void *x, const void *topk, uint32_t tokens
         const uint32_t upr = hidden / 8;
         // wide rows: two single-wave workgroups per token, 7 pieces per lane, plain stores (fastest of the
         // shapes measured on 7168-element rows); narrow rows: one four-wave workgroup per token
-        const int variant = g_permuteVariant >= 0 ? g_permuteVariant : (upr >= 512 ? 6 : 0);
+        // Wide rows: single-wave workgroups that hold up to 14 pieces per lane (a whole 7168-element
+        // row) and write them with plain stores, the fastest of the shapes measured on such rows
+        // (214 us; two waves per row 221 us; four-wave workgroups with nontemporal stores 237 us).
+        // Narrow rows: one four-wave workgroup per token.
+        const int variant = g_permuteVariant >= 0 ? g_permuteVariant : (upr >= 512 ? 10 : 0);
+        const uint32_t wideParts = (upr + 64 * 14 - 1) / (64 * 14);
         switch (variant) {
             case 1:
-                hipLaunchKernelGGL((MoePermuteKernel<64, 14, 1>), dim3(tokens), dim3(64), 0, s, xi, ro, topK, upr, 1u, oo);
+                hipLaunchKernelGGL((MoePermuteKernel<64, 14, 1>), dim3(tokens * wideParts), dim3(64), 0, s, xi, ro, topK, upr,
+                                   wideParts, oo);
                 break;
-            case 2:
-                hipLaunchKernelGGL((MoePermuteKernel<64, 7, 1>), dim3(tokens * 2), dim3(64), 0, s, xi, ro, topK, upr, 2u, oo);
+            case 6: {
+                const uint32_t parts = (upr + 64 * 7 - 1) / (64 * 7);
+                hipLaunchKernelGGL((MoePermuteKernel<64, 7, 0>), dim3(tokens * parts), dim3(64), 0, s, xi, ro, topK, upr, parts, oo);
                 break;
-            case 3:
-                hipLaunchKernelGGL((MoePermuteKernel<64, 4, 1>), dim3(tokens * 4), dim3(64), 0, s, xi, ro, topK, upr, 4u, oo);
+            }
+            case 7:
+                hipLaunchKernelGGL((MoePermuteKernel<128, 7, 0>), dim3(tokens * wideParts), dim3(128), 0, s, xi, ro, topK, upr,
+                                   wideParts, oo);
                 break;
-            case 4:
-                hipLaunchKernelGGL((MoePermuteKernel<64, 2, 1>), dim3(tokens * 7), dim3(64), 0, s, xi, ro, topK, upr, 7u, oo);
-                break;
-            case 5:
-                hipLaunchKernelGGL((MoePermuteKernel<64, 7, 2>), dim3(tokens * 2), dim3(64), 0, s, xi, ro, topK, upr, 2u, oo);
-                break;
-            case 6:
-                hipLaunchKernelGGL((MoePermuteKernel<64, 7, 0>), dim3(tokens * 2), dim3(64), 0, s, xi, ro, topK, upr, 2u, oo);
+            case 10:
+                hipLaunchKernelGGL((MoePermuteKernel<64, 14, 0>), dim3(tokens * wideParts), dim3(64), 0, s, xi, ro, topK, upr,
+                                   wideParts, oo);
                 break;
             default:
                 hipLaunchKernelGGL((MoePermuteKernel<256, 4, 1>), dim3(tokens), dim3(256), 0, s, xi, ro, topK, upr, 1u, oo);
@@ -466,25 +483,31 @@ extern "C" int mfk_moe_combine(const void *rows, const void *rowOf, const void *
     u32x4 *o = static_cast<u32x4 *>(y);
     const uint32_t upr = hidden / 8;
     if (topK == 8) {
-        switch (g_combineVariant) {
-            case 1:
-                hipLaunchKernelGGL((MoeCombineKernel<8, 128, true>), dim3(tokens), dim3(128), 0, s, in, ro, w, topK, upr, 1u, o);
+        // Wide rows: single-wave workgroups, each on a 128-unit slice of the row with two column
+        // positions per lane in flight (16 loads), the fastest shape measured on 7168-element rows
+        // (178 us; one four-wave workgroup per token 188 us; plain instead of nontemporal loads 194 us).
+        const int variant = g_combineVariant >= 0 ? g_combineVariant : (upr >= 256 ? 11 : 0);
+        switch (variant) {
+            case 3: {
+                const uint32_t parts = (upr + 447) / 448;
+                hipLaunchKernelGGL((MoeCombineKernel<8, 64, true>), dim3(tokens * parts), dim3(64), 0, s, in, ro, w, topK, upr, parts, o);
                 break;
-            case 2:
-                hipLaunchKernelGGL((MoeCombineKernel<8, 64, true>), dim3(tokens), dim3(64), 0, s, in, ro, w, topK, upr, 1u, o);
-                break;
-            case 3:
-                hipLaunchKernelGGL((MoeCombineKernel<8, 64, true>), dim3(tokens * 2), dim3(64), 0, s, in, ro, w, topK, upr, 2u, o);
-                break;
+            }
             case 4:
                 hipLaunchKernelGGL((MoeCombineKernel<8, 256, false>), dim3(tokens), dim3(256), 0, s, in, ro, w, topK, upr, 1u, o);
                 break;
-            case 5:
-                hipLaunchKernelGGL((MoeCombineKernel<8, 64, true>), dim3(tokens * 4), dim3(64), 0, s, in, ro, w, topK, upr, 4u, o);
+            case 11: {
+                const uint32_t parts = (upr + 127) / 128;
+                hipLaunchKernelGGL((MoeCombineKernel<8, 64, true, 2>), dim3(tokens * parts), dim3(64), 0, s, in, ro, w, topK, upr,
+                                   parts, o);
                 break;
-            case 6:
-                hipLaunchKernelGGL((MoeCombineKernel<8, 128, true>), dim3(tokens * 2), dim3(128), 0, s, in, ro, w, topK, upr, 2u, o);
+            }
+            case 13: {
+                const uint32_t parts = (upr + 63) / 64;
+                hipLaunchKernelGGL((MoeCombineKernel<8, 64, true, 1>), dim3(tokens * parts), dim3(64), 0, s, in, ro, w, topK, upr,
+                                   parts, o);
                 break;
+            }
             default:
                 hipLaunchKernelGGL((MoeCombineKernel<8, 256, true>), dim3(tokens), dim3(256), 0, s, in, ro, w, topK, upr, 1u, o);
                 break;

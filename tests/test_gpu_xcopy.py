@@ -20,7 +20,7 @@ MIB = 1 << 20
 def gpu(lib):
     assert lib.hybm_init(0, 0) == 0, native.last_error()
     yield lib
-    lib.mf_xcopy_tune(0, 16, 1)
+    lib.mf_xcopy_tune(0, 0, 0)
     lib.hybm_uninit()
 
 
@@ -31,7 +31,7 @@ def _random_bytes(oracle, nbytes, seed):
 
 
 def _check_d2d(gpu, oracle, pool_bytes, src_off, dst_off, lens, seed, units=0):
-    gpu.mf_xcopy_tune(units, 16, 1)
+    gpu.mf_xcopy_tune(units, 16 if units else 0, 0)
     init = _random_bytes(oracle, pool_bytes, seed)
     buf = gpu_util.DeviceBuffer(gpu, pool_bytes)
     try:

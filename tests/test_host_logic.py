@@ -160,7 +160,7 @@ def test_choose_units_policy(lib):
     assert lib.mf_xcopy_choose_units(64 * 1024, 256, native.ROUTE_HBM) == 256
     assert lib.mf_xcopy_choose_units(workloads.KV_PAYLOAD, 256, native.ROUTE_HBM) == 1024
     assert lib.mf_xcopy_choose_units(1 << 30, 256, native.ROUTE_HBM) == 1024
-    assert lib.mf_xcopy_choose_units(2 << 30, 256, native.ROUTE_HBM) == 4096
+    assert lib.mf_xcopy_choose_units(2 << 30, 256, native.ROUTE_HBM) == 1024
 
 
 # ---- error contracts that need no GPU (test/ut/testcase/smem/smem_bm_test.cpp:59-201 of the reference) ----
