@@ -435,11 +435,11 @@ extern "C" int mfk_moe_dispatch(const void *x, const void *topk, uint32_t tokens
         const int32_t *ro = static_cast<const int32_t *>(rowOf);
         u32x4 *oo = static_cast<u32x4 *>(out);
         const uint32_t upr = hidden / 8;
-        // wide rows: two single-wave workgroups per token, 7 pieces per lane, plain stores (fastest of the
-        // shapes measured on 7168-element rows); narrow rows: one four-wave workgroup per token
         // Wide rows: single-wave workgroups that hold up to 14 pieces per lane (a whole 7168-element
         // row) and write them with plain stores, the fastest of the shapes measured on such rows
-        // (214 us; two waves per row 221 us; four-wave workgroups with nontemporal stores 237 us).
+        // (214 us; two waves per row 221 us; four-wave workgroups with nontemporal stores 237 us; the
+        // destination-side form, one workgroup per output row reading x[srcOf[row]], 271 us: its
+        // eight reads of every token row are not absorbed by the caches).
         // Narrow rows: one four-wave workgroup per token.
         const int variant = g_permuteVariant >= 0 ? g_permuteVariant : (upr >= 512 ? 10 : 0);
         const uint32_t wideParts = (upr + 64 * 14 - 1) / (64 * 14);
