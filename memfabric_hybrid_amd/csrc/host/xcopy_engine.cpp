@@ -255,24 +255,23 @@ uint32_t ChooseUnits(uint64_t totalBytes, uint32_t cuCount, int route, const Xco
 {
     (void)cuCount;
     if (tuning.unitsOverride != 0) {
-        return static_cast<uint32_t>(RoundUp(tuning.unitsOverride, kXcopyThreads));
+        return static_cast<uint32_t>(RoundUp(tuning.unitsOverride, 64));
     }
-    // Measured on MI355X (256 CUs): 16 KiB per workgroup step (four 128-bit accesses per lane, one
-    // full tile) is the sweet spot from a few MiB to at least 4 GiB (32 and 64 KiB chunks: 3-10 %
-    // slower); it also divides the usual power-of-two block sizes, so no workgroup runs a ragged
-    // tile.  Below 1 MiB the batch is latency bound and 4 KiB chunks put more CUs to work.
+    // Measured on MI355X (256 CUs).  HBM routes: 4 KiB chunks, which the launcher gives to single-wave
+    // workgroups, one workgroup per chunk: the fastest shape from a 1 MiB copy (3.4 us against 4.5 us
+    // with four-wave workgroups on 16 KiB chunks) over the 9 MB KV batch (4.8 against 5.5 us) to a
+    // 1 GiB copy (6.4 against 6.25 TB/s).  4 KiB also divides the usual power-of-two block sizes, so
+    // no workgroup runs a ragged tile.
     if (route == MFRT_ROUTE_TO_HOST || route == MFRT_ROUTE_FROM_HOST) {
-        // The host link, not the GPU, is the bound: one workgroup per CU with small chunks keeps
-        // the link busy without flooding it (measured: 56 GB/s out, 55 GB/s in on a Gen5 x16 link).
+        // The host link, not the GPU, is the bound: one four-wave workgroup per CU with small chunks
+        // keeps the link busy without flooding it (measured: 56 GB/s out, 55 GB/s in on a Gen5 x16 link).
         if (totalBytes > (256ull << 20)) {
             return 4 * kXcopyThreads;
         }
         return route == MFRT_ROUTE_TO_HOST ? kXcopyThreads : 2 * kXcopyThreads;
     }
-    if (totalBytes < (1ull << 20)) {
-        return tuning.minUnits;
-    }
-    return 4 * kXcopyThreads;
+    (void)totalBytes;
+    return tuning.minUnits;
 }
 
 bool BuildInlinePlan(const SegList &segs, uint32_t units, InlinePlan &plan)

@@ -44,8 +44,7 @@ struct XcopyTuning {
     uint32_t unitsOverride = 0;  // 16-byte units per chunk, 0 = choose from batch size
     uint32_t wgPerCu = 0;        // HBM routes: grid cap in workgroups per CU, 0 = one workgroup per chunk
     uint32_t wgPerCuLink = 1;    // routes bound by the host link: workgroups per CU
-    uint32_t minUnits = kXcopyThreads;
-    uint32_t maxUnits = 16 * kXcopyThreads;
+    uint32_t minUnits = kXcopyThreads;   // 4 KiB: the chunk of HBM routes
 };
 
 uint32_t ChooseUnits(uint64_t totalBytes, uint32_t cuCount, int route, const XcopyTuning &tuning);

@@ -156,11 +156,14 @@ def test_plan_splits_segments_the_inline_form_cannot_hold(lib):
 
 
 def test_choose_units_policy(lib):
-    # latency-bound batches use the smallest chunk, the bulk 16 KiB, multi-GiB copies the largest
+    # HBM routes: 4 KiB chunks (single-wave workgroups) at every size; link routes: their own small chunks
     assert lib.mf_xcopy_choose_units(64 * 1024, 256, native.ROUTE_HBM) == 256
-    assert lib.mf_xcopy_choose_units(workloads.KV_PAYLOAD, 256, native.ROUTE_HBM) == 1024
-    assert lib.mf_xcopy_choose_units(1 << 30, 256, native.ROUTE_HBM) == 1024
-    assert lib.mf_xcopy_choose_units(2 << 30, 256, native.ROUTE_HBM) == 1024
+    assert lib.mf_xcopy_choose_units(workloads.KV_PAYLOAD, 256, native.ROUTE_HBM) == 256
+    assert lib.mf_xcopy_choose_units(1 << 30, 256, native.ROUTE_HBM) == 256
+    assert lib.mf_xcopy_choose_units(2 << 30, 256, native.ROUTE_HBM) == 256
+    assert lib.mf_xcopy_choose_units(workloads.KV_PAYLOAD, 256, native.ROUTE_TO_HOST) == 256
+    assert lib.mf_xcopy_choose_units(workloads.KV_PAYLOAD, 256, native.ROUTE_FROM_HOST) == 512
+    assert lib.mf_xcopy_choose_units(1 << 30, 256, native.ROUTE_FROM_HOST) == 1024
 
 
 # ---- error contracts that need no GPU (test/ut/testcase/smem/smem_bm_test.cpp:59-201 of the reference) ----
