@@ -89,16 +89,16 @@ def timed_steps(lib, handle, batches, copy_type, steps, warmup, flags):
     start, stop = lib.mfrt_event_create(), lib.mfrt_event_create()
     call = lib.smem_bm_copy_batch
     nb = len(batches)
+    refs = [b.ref for b in batches]
     for i in range(warmup):
-        ret = call(handle, batches[i % nb].ref, copy_type, flags)
+        ret = call(handle, refs[i % nb], copy_type, flags)
         assert ret == 0, native.last_error()
     assert lib.mfrt_stream_sync(stream) == 0
     assert lib.mfrt_device_sync() == 0
     t0 = time.perf_counter()
     lib.mfrt_event_record(start, stream)
     for i in range(steps):
-        ret = call(handle, batches[i % nb].ref, copy_type, flags)
-        if ret != 0:
+        if call(handle, refs[i % nb], copy_type, flags) != 0:
             raise RuntimeError(native.last_error())
     lib.mfrt_event_record(stop, stream)
     assert lib.mfrt_stream_sync(stream) == 0

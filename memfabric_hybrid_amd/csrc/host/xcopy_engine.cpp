@@ -50,6 +50,7 @@ struct ThreadLease {
                 }
                 (void)mfrt_event_destroy(slot.event);
             }
+
             if (slot.host != nullptr) {
                 (void)mfrt_free_host(slot.host);
             }
@@ -63,6 +64,7 @@ struct ThreadLease {
             (void)mfrt_stream_destroy(stream);
             stream = nullptr;
         }
+
         if (bounce != nullptr) {
             (void)mfrt_free_host(bounce);
             bounce = nullptr;
@@ -387,6 +389,60 @@ uint64_t BuildTablePlan(const SegList &segs, uint32_t units, uint64_t *triples, 
     return run;
 }
 
+// Normalisation (empty segments dropped, neighbours that continue each other merged) and table
+// planning in one pass over the caller's arrays, straight into the staging slot: a 4096-segment
+// batch costs the host about as long as the GPU needs to copy it, so nothing is built twice.
+// triples: room for 3 * n words, first: room for n + 1.  Returns the chunk count, count = segments.
+uint64_t BuildTableDirect(const uint64_t *src, const uint64_t *dst, const uint64_t *len, uint32_t n, uint32_t units,
+                          uint64_t *triples, uint32_t *first, uint32_t &count)
+{
+    const bool pow2 = (units & (units - 1)) == 0;
+    const uint32_t shift = pow2 ? static_cast<uint32_t>(__builtin_ctz(units)) : 0;
+    uint32_t used = 0;
+    uint64_t run = 0;
+    uint64_t curSrc = 0;
+    uint64_t curDst = 0;
+    uint64_t curLen = 0;
+    auto flush = [&]() {
+        if (curLen == 0) {
+            return;
+        }
+        uint64_t head = (0 - curDst) & (kUnitBytes - 1);
+        if (head > curLen) {
+            head = curLen;
+        }
+        const uint64_t body = (curLen - head) / kUnitBytes;
+        uint64_t chunks = pow2 ? (body + units - 1) >> shift : (body + units - 1) / units;
+        if (chunks == 0) {
+            chunks = 1;
+        }
+        triples[3 * used] = curSrc;
+        triples[3 * used + 1] = curDst;
+        triples[3 * used + 2] = curLen;
+        first[used] = static_cast<uint32_t>(run < kNoChunk ? run : kNoChunk);
+        run += chunks;
+        ++used;
+    };
+    for (uint32_t i = 0; i < n; ++i) {
+        const uint64_t l = len[i];
+        if (l == 0) {
+            continue;
+        }
+        if (curLen > 0 && curSrc + curLen == src[i] && curDst + curLen == dst[i]) {
+            curLen += l;
+            continue;
+        }
+        flush();
+        curSrc = src[i];
+        curDst = dst[i];
+        curLen = l;
+    }
+    flush();
+    first[used] = static_cast<uint32_t>(run < kNoChunk ? run : kNoChunk);
+    count = used;
+    return run;
+}
+
 XcopyEngine &XcopyEngine::Instance()
 {
     static XcopyEngine engine;
@@ -514,7 +570,8 @@ int XcopyEngine::Submit(const uint64_t *src, const uint64_t *dst, const uint64_t
         units = ChooseUnits(total, cu, route, tuning_);
         inlined = BuildInlineDirect(src, dst, len, n, units, plan);
     }
-    if (!inlined) {
+    if (!inlined && n <= 4 * kInlineSegs) {
+        // merging or a segment of 4 GiB and more made the one-pass attempt give up: the general inline path
         NormalizeSegments(src, dst, len, n, kInlinePiece, ctx.segs);
         units = ChooseUnits(ctx.segs.totalBytes, cu, route, tuning_);
         inlined = BuildInlinePlan(ctx.segs, units, plan);
@@ -529,10 +586,17 @@ int XcopyEngine::Submit(const uint64_t *src, const uint64_t *dst, const uint64_t
         return BM_OK;
     }
 
-    // Table form: stage {triples, prefix} through a pinned slot into HBM, then search it there.
-    const uint32_t count = ctx.segs.Size();
-    const uint64_t tripleBytes = 24ull * count;
-    const uint64_t tableBytes = RoundUp(tripleBytes + 4ull * (count + 1), kUnitBytes);
+    // Table form: {triples, prefix} are built in a pinned slot, moved to HBM by a copy launch and
+    // searched there.  The slot is sized for n segments; merging can only make the table shorter.
+    if (units == 0 || n > 4 * kInlineSegs) {
+        uint64_t total = 0;
+        for (uint32_t i = 0; i < n; ++i) {
+            total += len[i];
+        }
+        units = ChooseUnits(total, cu, route, tuning_);
+    }
+    const uint64_t tripleBytes = 24ull * n;
+    const uint64_t tableBytes = RoundUp(tripleBytes + 4ull * (n + 1), kUnitBytes);
     StagingSlot *slot = nullptr;
     int ret = AcquireSlot(ctx.Lease(), tableBytes, slot);
     if (ret != BM_OK) {
@@ -540,18 +604,27 @@ int XcopyEngine::Submit(const uint64_t *src, const uint64_t *dst, const uint64_t
     }
     uint64_t *triples = static_cast<uint64_t *>(slot->host);
     uint32_t *first = reinterpret_cast<uint32_t *>(static_cast<uint8_t *>(slot->host) + tripleBytes);
-    const uint64_t nchunk = BuildTablePlan(ctx.segs, units, triples, first);
+    uint32_t count = 0;
+    const uint64_t nchunk = BuildTableDirect(src, dst, len, n, units, triples, first, count);
     if (nchunk >= kNoChunk) {
         MF_FAIL(BM_INVALID_PARAM, "batch too large for one launch: " << nchunk << " chunks");
     }
+    if (count == 0) {   // nothing but empty segments
+        InlinePlan empty;
+        SegList none;
+        (void)BuildInlinePlan(none, kXcopyThreads, empty);
+        int err = mfk_xcopy_inline(&empty, route, 1, mask, maskValue, stream);
+        return err == 0 ? BM_OK : BM_ERROR;
+    }
 
-    SegList stage;
     const uint64_t hostAddr = reinterpret_cast<uint64_t>(slot->host);
     const uint64_t devAddr = reinterpret_cast<uint64_t>(slot->dev);
-    NormalizeSegments(&hostAddr, &devAddr, &tableBytes, 1, 0, stage);
     InlinePlan stagePlan;
-    const uint32_t stageUnits = kXcopyThreads;
-    (void)BuildInlinePlan(stage, stageUnits, stagePlan);
+    if (!BuildInlineDirect(&hostAddr, &devAddr, &tableBytes, 1, kXcopyThreads, stagePlan)) {
+        MF_FAIL(BM_INVALID_PARAM, "descriptor table of " << tableBytes << " bytes is too large");
+    }
+    // (Uploading on a stream of its own, with the copy stream waiting for an event, was measured: the
+    // two extra queue operations cost what the overlap gains, 56 us per 4096-page gather either way.)
     int err = mfk_xcopy_inline(&stagePlan, MFRT_ROUTE_FROM_HOST, stagePlan.nchunk, nullptr, 0, stream);
     if (err != 0) {
         MF_FAIL(BM_ERROR, "descriptor staging launch failed: " << mfrt_error_string(err));
