@@ -678,8 +678,7 @@ int XcopyEngine::SubmitDeviceTable(const void *triples, uint32_t n, int route, v
     if (ret != BM_OK) {
         return ret;
     }
-    const uint32_t units = tuning_.unitsOverride != 0 ? static_cast<uint32_t>(RoundUp(tuning_.unitsOverride, kXcopyThreads))
-                                                      : 4 * kXcopyThreads;
+    const uint32_t units = ChooseUnits(0, mfrt_cu_count(), route, tuning_);   // sizes are only known on the GPU
     uint32_t *first = static_cast<uint32_t *>(slot->dev);
     uint32_t *nchunkDev = first + n + 1;
     int err = mfk_xcopy_plan(triples, n, units, first, nchunkDev, stream);
@@ -687,7 +686,7 @@ int XcopyEngine::SubmitDeviceTable(const void *triples, uint32_t n, int route, v
         MF_FAIL(BM_ERROR, "xcopy plan launch failed: " << mfrt_error_string(err));
     }
     const uint32_t cu = mfrt_cu_count();
-    const uint32_t grid = GridFor(static_cast<uint64_t>(cu == 0 ? 256 : cu) * 64, cu, route, tuning_);   // chunk count is only known on the GPU
+    const uint32_t grid = GridFor(static_cast<uint64_t>(cu == 0 ? 256 : cu) * 256, cu, route, tuning_);   // chunk count is only known on the GPU; surplus workgroups leave at once
     err = mfk_xcopy_table(triples, first, nchunkDev, n, 0, units, route, grid, mask, maskValue, stream);
     if (err != 0) {
         MF_FAIL(BM_ERROR, "xcopy table launch failed: " << mfrt_error_string(err));
