@@ -259,23 +259,25 @@ MF_EXPORT int32_t hybm_data_batch_copy(hybm_entity_t e, hybm_batch_copy_params *
     if (entity == nullptr) {
         MF_FAIL(BM_INVALID_PARAM, "hybm_data_batch_copy: unknown pool handle");
     }
-    const bool checkDst = MustCheckDestination(direction);
-    const bool checkSrc = MustCheckSource(direction);
-    for (uint32_t i = 0; i < params->batchSize; ++i) {
-        if (params->sources[i] == nullptr || params->destinations[i] == nullptr) {
-            MF_FAIL(BM_INVALID_PARAM, "batch element " << i << " has a null address");
+    const uint32_t n = params->batchSize;
+    uint32_t bad = n;
+    if (MustCheckDestination(direction)) {
+        bad = entity->FirstOutside(params->destinations, params->dataSizes, n);
+    }
+    if (bad == n && MustCheckSource(direction)) {
+        bad = entity->FirstOutside(params->sources, params->dataSizes, n);
+    }
+    if (bad == n) {   // sides that are not checked against the pool must at least not be null
+        for (uint32_t i = 0; i < n; ++i) {
+            if (params->sources[i] == nullptr || params->destinations[i] == nullptr) {
+                MF_FAIL(BM_INVALID_PARAM, "batch element " << i << " has a null address");
+            }
         }
-        bool ok = true;
-        if (checkDst) {
-            ok = entity->CheckAddressInEntity(params->destinations[i], params->dataSizes[i]);
-        }
-        if (checkSrc) {
-            ok = ok && entity->CheckAddressInEntity(params->sources[i], params->dataSizes[i]);
-        }
-        if (!ok) {
-            MF_FAIL(BM_INVALID_PARAM, "batch element " << i << " (" << params->dataSizes[i]
-                                                       << " bytes) leaves the pool, direction " << direction);
-        }
+    } else if (params->sources[bad] == nullptr || params->destinations[bad] == nullptr) {
+        MF_FAIL(BM_INVALID_PARAM, "batch element " << bad << " has a null address");
+    } else {
+        MF_FAIL(BM_INVALID_PARAM, "batch element " << bad << " (" << params->dataSizes[bad]
+                                                   << " bytes) leaves the pool, direction " << direction);
     }
     return entity->BatchCopyData(*params, direction, stream, flags);
 }

@@ -482,6 +482,38 @@ bool MemEntity::CheckAddressInEntity(const void *ptr, uint64_t length) const
     return rangeCount_.load(std::memory_order_acquire) != 0 && InRanges(a, length);
 }
 
+uint32_t MemEntity::FirstOutside(void *const *ptrs, const uint64_t *lengths, uint32_t n) const
+{
+    if (!initialized_ || options_.rankCount > 1) {
+        for (uint32_t i = 0; i < n; ++i) {
+            if (ptrs[i] == nullptr || !CheckAddressInEntity(ptrs[i], lengths[i])) {
+                return i;
+            }
+        }
+        return n;
+    }
+    // One rank: an address is inside when it lies in the backed part of one of the two windows
+    // (or in a registered range).  The bounds stay in registers for the whole batch.
+    const uint64_t devLo = device_.base;
+    const uint64_t devHi = device_.base == 0 ? 0 : device_.base + (deviceBacked_ < device_.Span() ? deviceBacked_ : device_.Span());
+    const uint64_t hostLo = host_.base;
+    const uint64_t hostHi = host_.base == 0 ? 0 : host_.base + (hostBacked_ < host_.Span() ? hostBacked_ : host_.Span());
+    const bool haveRanges = rangeCount_.load(std::memory_order_acquire) != 0;
+    for (uint32_t i = 0; i < n; ++i) {
+        const uint64_t a = reinterpret_cast<uint64_t>(ptrs[i]);
+        const uint64_t end = a + lengths[i];
+        const bool inDevice = a >= devLo && end <= devHi;
+        const bool inHost = a >= hostLo && end <= hostHi;
+        if (a != 0 && end >= a && (inDevice || inHost)) {
+            continue;
+        }
+        if (a == 0 || !haveRanges || !InRanges(a, lengths[i])) {
+            return i;
+        }
+    }
+    return n;
+}
+
 void MemEntity::LocateAddrAndRank(void *&src, void *&dest, uint64_t length, std::pair<uint32_t, uint32_t> &ranks) const
 {
     auto owner = [&](uint64_t a) -> uint32_t {

@@ -61,6 +61,9 @@ public:
     }
 
     bool CheckAddressInEntity(const void *ptr, uint64_t length) const;
+    // The same test for every element of a batch in one pass; the index of the first element that
+    // is null or leaves the entity, n when all are inside.
+    uint32_t FirstOutside(void *const *ptrs, const uint64_t *lengths, uint32_t n) const;
     void LocateAddrAndRank(void *&src, void *&dest, uint64_t length, std::pair<uint32_t, uint32_t> &ranks) const;
 
     int CopyData(hybm_copy_params &params, hybm_data_copy_direction direction, void *stream, uint32_t flags);
