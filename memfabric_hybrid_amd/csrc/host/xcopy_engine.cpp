@@ -202,12 +202,12 @@ int AcquireSlot(ThreadLease &ctx, uint64_t bytes, StagingSlot *&out)
 uint32_t GridFor(uint64_t nchunk, uint32_t cuCount, int route, const XcopyTuning &tuning)
 {
     // HBM routes: one workgroup per chunk unless a cap is set.  Measured on 128 MiB ... 4 GiB copies:
-    // letting the hardware dispatcher hand out 16 KiB chunks one by one sustains 6.0-6.2 TB/s, a
+    // letting the hardware dispatcher hand out the chunks one by one sustains 6.0-6.2 TB/s, a
     // grid capped at 16 workgroups per CU that strides over the chunks 5.3-5.7 TB/s (its static
     // assignment leaves a tail).  Link routes: one workgroup per CU, more only adds contention.
     const bool link = route == MFRT_ROUTE_TO_HOST || route == MFRT_ROUTE_FROM_HOST || route >= 16;
     const uint32_t perCu = link ? (tuning.wgPerCuLink == 0 ? 1 : tuning.wgPerCuLink) : tuning.wgPerCu;
-    const uint64_t limit = 0x7FFFFFFFull;
+    const uint64_t limit = (1ull << 24) - 1;   // grid size in lanes must stay below 2^32 with up to 256 lanes per workgroup
     uint64_t cap = perCu == 0 ? limit : static_cast<uint64_t>(cuCount == 0 ? 256 : cuCount) * perCu;
     if (cap > limit) {
         cap = limit;

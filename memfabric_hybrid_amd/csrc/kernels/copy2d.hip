@@ -89,6 +89,9 @@ extern "C" int mfk_copy2d(const void *rectPlan, uint32_t grid, void *stream)
     if (grid == 0 || grid > plan.nchunk) {
         grid = plan.nchunk;
     }
+    if (grid > (1u << 24) - 1) {
+        grid = (1u << 24) - 1;   // the grid size in lanes must stay below 2^32; workgroups loop over the rest
+    }
     hipLaunchKernelGGL(mf::Copy2dKernel, dim3(grid), dim3(mf::kRectThreads), 0, static_cast<hipStream_t>(stream), plan);
     return static_cast<int>(hipGetLastError());
 }

@@ -91,11 +91,9 @@ extern "C" int mfk_probe(int kind, void *dst, const void *src, uint64_t bytes, u
     hipStream_t s = static_cast<hipStream_t>(stream);
     const uint64_t units = bytes / 16;
     const uint64_t tiles = (units + kTile - 1) / kTile;
-    if (tiles > 0x7FFFFFFFull) {
-        return -1;
-    }
+    const uint64_t most = (1ull << 24) - 1;   // the grid size in lanes must stay below 2^32; the kernels loop over what is left
     if (grid == 0 || grid > tiles) {
-        grid = static_cast<uint32_t>(tiles);
+        grid = static_cast<uint32_t>(tiles < most ? tiles : most);
     }
     switch (kind) {
         case 0:

@@ -360,6 +360,9 @@ extern "C" int mfk_xcopy_inline(const void *inlinePlan, int route, uint32_t grid
     if (grid == 0 || grid > plan.nchunk) {
         grid = plan.nchunk;
     }
+    if (grid > (1u << 24) - 1) {
+        grid = (1u << 24) - 1;   // the grid size in lanes must stay below 2^32; workgroups loop over the rest
+    }
     const int err = mf::WithPolicy(mf::PolicyOf(route), [&](auto ntLoad, auto store) {
         return mf::LaunchInline<decltype(ntLoad)::value, decltype(store)::value>(plan, grid, mf::LanesFor(plan.units, route), s);
     });

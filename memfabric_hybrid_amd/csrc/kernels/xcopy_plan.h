@@ -24,7 +24,7 @@
 
 namespace mf {
 
-constexpr uint32_t kXcopyThreads = 256;       // lanes per workgroup (4 wave64)
+constexpr uint32_t kXcopyThreads = 256;       // most lanes a copy workgroup has (4 wave64); 4 KiB chunks get one wave
 constexpr uint32_t kUnitBytes = 16;           // one 128-bit access
 constexpr uint32_t kInlineSegs = 128;         // segments that fit in the kernel-argument block: 2 table rows per lane of a wave64
 constexpr uint32_t kNoChunk = 0xFFFFFFFFu;    // sentinel prefix for unused slots
@@ -74,7 +74,7 @@ struct InlinePlan {
     uint32_t len[kInlineSegs];          // inline path carries segments < 4 GiB only
     uint32_t first[kInlineSegs];        // exclusive prefix of chunk counts, kNoChunk past the end
     uint32_t nchunk;
-    uint32_t units;                     // 16-byte units per chunk, multiple of kXcopyThreads
+    uint32_t units;                     // 16-byte units per chunk, a multiple of 64
 };
 
 // A table-driven launch: triples and prefix live in device memory.
