@@ -61,6 +61,11 @@ bool BuildInlineDirect(const uint64_t *src, const uint64_t *dst, const uint64_t 
 // triples: 3 * segs.Size() words, first: segs.Size() + 1 words.  Returns total chunks.
 uint64_t BuildTablePlan(const SegList &segs, uint32_t units, uint64_t *triples, uint32_t *first);
 
+// The same result as NormalizeSegments (no piece limit) + BuildTablePlan in one pass over the
+// caller's arrays.  triples: room for 3 * n words, first: room for n + 1; count = segments written.
+uint64_t BuildTableDirect(const uint64_t *src, const uint64_t *dst, const uint64_t *len, uint32_t n, uint32_t units,
+                          uint64_t *triples, uint32_t *first, uint32_t &count);
+
 class XcopyEngine {
 public:
     static XcopyEngine &Instance();

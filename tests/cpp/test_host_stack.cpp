@@ -15,6 +15,7 @@
 #include "../../include/mf_xcopy_api.h"
 #include "../../memfabric_hybrid_amd/csrc/host/compose_data_op.h"
 #include "../../memfabric_hybrid_amd/csrc/host/mf_log.h"
+#include "../../memfabric_hybrid_amd/csrc/host/xcopy_engine.h"
 
 extern "C" uint64_t fake_rt_launches(void);
 extern "C" void fake_rt_seal(void);
@@ -492,11 +493,57 @@ static void TestMappedWindow()
     hybm_uninit();
 }
 
+// The one-pass planners must produce exactly what normalisation followed by planning produces.
+static void TestPlanners()
+{
+    std::mt19937_64 rng(0x9142);
+    for (int trial = 0; trial < 400; ++trial) {
+        const uint32_t n = 1 + rng() % (trial % 3 == 0 ? 600 : 140);
+        const uint32_t units = 64u << (rng() % 6);
+        std::vector<uint64_t> src(n), dst(n), len(n);
+        uint64_t s = 0x7f1000000000ull + rng() % 4096, d = 0x7f8000000000ull + rng() % 4096;
+        for (uint32_t i = 0; i < n; ++i) {
+            const uint32_t kind = rng() % 8;
+            len[i] = kind == 0 ? 0 : (kind == 1 ? rng() % 40 : rng() % 300000);
+            if (kind != 2) {   // kind 2: continue the previous segment on both sides
+                s += rng() % 70000;
+                d += rng() % 70000;
+            }
+            src[i] = s;
+            dst[i] = d;
+            s += len[i];
+            d += len[i];
+        }
+        SegList segs;
+        NormalizeSegments(src.data(), dst.data(), len.data(), n, 0, segs);
+        std::vector<uint64_t> t1(3 * segs.Size() + 3), t2(3 * n + 3);
+        std::vector<uint32_t> f1(segs.Size() + 1), f2(n + 1);
+        const uint64_t c1 = BuildTablePlan(segs, units, t1.data(), f1.data());
+        uint32_t count = 0;
+        const uint64_t c2 = BuildTableDirect(src.data(), dst.data(), len.data(), n, units, t2.data(), f2.data(), count);
+        bool same = c1 == c2 && count == segs.Size();
+        for (uint32_t i = 0; same && i < count; ++i) {
+            same = t1[3 * i] == t2[3 * i] && t1[3 * i + 1] == t2[3 * i + 1] && t1[3 * i + 2] == t2[3 * i + 2] && f1[i] == f2[i];
+        }
+        same = same && f1[segs.Size()] == f2[count];
+        CHECK(same);
+        InlinePlan a, b;
+        NormalizeSegments(src.data(), dst.data(), len.data(), n, 1ull << 30, segs);
+        const bool fitsA = BuildInlinePlan(segs, units, a);
+        const bool fitsB = BuildInlineDirect(src.data(), dst.data(), len.data(), n, units, b);
+        CHECK(fitsA == fitsB);
+        if (fitsA && fitsB) {
+            CHECK(std::memcmp(&a, &b, sizeof(a)) == 0);
+        }
+    }
+}
+
 int main()
 {
     SetLogLevel(3);
     SetLogSink([](int, const char *) {});
     TestCompose();
+    TestPlanners();
     TestCApi();                                  // device window: reserved address space, HBM mapped in
     setenv("MF_HIP_GVA_WINDOW", "malloc", 1);
     TestCApi();                                  // device window: one ordinary allocation
