@@ -394,12 +394,14 @@ uint64_t BuildTablePlan(const SegList &segs, uint32_t units, uint64_t *triples, 
 // batch costs the host about as long as the GPU needs to copy it, so nothing is built twice.
 // triples: room for 3 * n words, first: room for n + 1.  Returns the chunk count, count = segments.
 uint64_t BuildTableDirect(const uint64_t *src, const uint64_t *dst, const uint64_t *len, uint32_t n, uint32_t units,
-                          uint64_t *triples, uint32_t *first, uint32_t &count)
+                          uint64_t *triples, uint32_t *first, uint32_t &count, uint32_t *perSegment)
 {
     const bool pow2 = (units & (units - 1)) == 0;
     const uint32_t shift = pow2 ? static_cast<uint32_t>(__builtin_ctz(units)) : 0;
     uint32_t used = 0;
     uint64_t run = 0;
+    uint64_t firstChunks = 0;
+    uint64_t differing = 0;   // OR of (chunks ^ firstChunks): stays 0 while all segments agree
     uint64_t curSrc = 0;
     uint64_t curDst = 0;
     uint64_t curLen = 0;
@@ -420,6 +422,10 @@ uint64_t BuildTableDirect(const uint64_t *src, const uint64_t *dst, const uint64
         triples[3 * used + 1] = curDst;
         triples[3 * used + 2] = curLen;
         first[used] = static_cast<uint32_t>(run < kNoChunk ? run : kNoChunk);
+        if (used == 0) {
+            firstChunks = chunks;
+        }
+        differing |= chunks ^ firstChunks;
         run += chunks;
         ++used;
     };
@@ -440,6 +446,9 @@ uint64_t BuildTableDirect(const uint64_t *src, const uint64_t *dst, const uint64
     flush();
     first[used] = static_cast<uint32_t>(run < kNoChunk ? run : kNoChunk);
     count = used;
+    if (perSegment != nullptr) {
+        *perSegment = used != 0 && differing == 0 && firstChunks < kNoChunk ? static_cast<uint32_t>(firstChunks) : 0;
+    }
     return run;
 }
 
@@ -605,7 +614,8 @@ int XcopyEngine::Submit(const uint64_t *src, const uint64_t *dst, const uint64_t
     uint64_t *triples = static_cast<uint64_t *>(slot->host);
     uint32_t *first = reinterpret_cast<uint32_t *>(static_cast<uint8_t *>(slot->host) + tripleBytes);
     uint32_t count = 0;
-    const uint64_t nchunk = BuildTableDirect(src, dst, len, n, units, triples, first, count);
+    uint32_t perSegment = 0;
+    const uint64_t nchunk = BuildTableDirect(src, dst, len, n, units, triples, first, count, &perSegment);
     if (nchunk >= kNoChunk) {
         MF_FAIL(BM_INVALID_PARAM, "batch too large for one launch: " << nchunk << " chunks");
     }
@@ -619,8 +629,10 @@ int XcopyEngine::Submit(const uint64_t *src, const uint64_t *dst, const uint64_t
 
     const uint64_t hostAddr = reinterpret_cast<uint64_t>(slot->host);
     const uint64_t devAddr = reinterpret_cast<uint64_t>(slot->dev);
+    // Segments of one size (pages) need no prefix on the GPU: only the descriptors travel.
+    const uint64_t uploadBytes = perSegment != 0 ? 24ull * count : tableBytes;
     InlinePlan stagePlan;
-    if (!BuildInlineDirect(&hostAddr, &devAddr, &tableBytes, 1, kXcopyThreads, stagePlan)) {
+    if (!BuildInlineDirect(&hostAddr, &devAddr, &uploadBytes, 1, kXcopyThreads, stagePlan)) {
         MF_FAIL(BM_INVALID_PARAM, "descriptor table of " << tableBytes << " bytes is too large");
     }
     // (Uploading on a stream of its own, with the copy stream waiting for an event, was measured: the
@@ -631,8 +643,8 @@ int XcopyEngine::Submit(const uint64_t *src, const uint64_t *dst, const uint64_t
     }
     const uint32_t grid = GridFor(nchunk, cu, route, tuning_);
     const uint8_t *devBase = static_cast<const uint8_t *>(slot->dev);
-    err = mfk_xcopy_table(devBase, devBase + tripleBytes, nullptr, count, static_cast<uint32_t>(nchunk), units, route,
-                          grid, mask, maskValue, stream);
+    err = mfk_xcopy_table(devBase, devBase + tripleBytes, nullptr, count, static_cast<uint32_t>(nchunk), units, perSegment,
+                          route, grid, mask, maskValue, stream);
     if (err != 0) {
         // the staging launch may still be reading the slot: keep it reserved until the stream has passed this point
         slot->pending = mfrt_event_record(slot->event, stream) == 0;
@@ -687,7 +699,7 @@ int XcopyEngine::SubmitDeviceTable(const void *triples, uint32_t n, int route, v
     }
     const uint32_t cu = mfrt_cu_count();
     const uint32_t grid = GridFor(static_cast<uint64_t>(cu == 0 ? 256 : cu) * 256, cu, route, tuning_);   // chunk count is only known on the GPU; surplus workgroups leave at once
-    err = mfk_xcopy_table(triples, first, nchunkDev, n, 0, units, route, grid, mask, maskValue, stream);
+    err = mfk_xcopy_table(triples, first, nchunkDev, n, 0, units, 0, route, grid, mask, maskValue, stream);
     if (err != 0) {
         MF_FAIL(BM_ERROR, "xcopy table launch failed: " << mfrt_error_string(err));
     }

@@ -293,6 +293,83 @@ __global__ __launch_bounds__(kThreads) void MoePermuteKernel(const u32x4 *__rest
     }
 }
 
+// Single-wave workgroups that walk items (token, part) with stride gridDim.x and fetch the next
+// item's pieces before they store the current one's: after the first item of every wave, reads of
+// x overlap the eight-fold stores instead of preceding them.
+template <uint32_t kHold>
+__global__ __launch_bounds__(64) void MoePermuteLoopKernel(const u32x4 *__restrict__ x, const int32_t *__restrict__ rowOf,
+                                                           uint32_t topK, uint32_t unitsPerRow, uint32_t parts,
+                                                           uint32_t items, u32x4 *__restrict__ out)
+{
+    const uint32_t perPart = (unitsPerRow + parts - 1) / parts;
+    const MF_GLOBAL u32x4 *xg = reinterpret_cast<const MF_GLOBAL u32x4 *>(reinterpret_cast<uint64_t>(x));
+    MF_GLOBAL u32x4 *og = reinterpret_cast<MF_GLOBAL u32x4 *>(reinterpret_cast<uint64_t>(out));
+    auto fetch = [&](uint32_t item, u32x4(&v)[kHold], int32_t(&rows)[kMaxTopK]) {
+        const uint32_t token = item / parts;
+        const uint32_t begin = (item - token * parts) * perPart;
+        const uint32_t end = begin + perPart < unitsPerRow ? begin + perPart : unitsPerRow;
+#pragma unroll
+        for (uint32_t k = 0; k < kMaxTopK; ++k) {
+            rows[k] = k < topK ? rowOf[static_cast<uint64_t>(token) * topK + k] : -1;
+        }
+#pragma unroll
+        for (uint32_t j = 0; j < kHold; ++j) {
+            const uint32_t u = begin + j * 64 + threadIdx.x;
+            if (u < end) {
+                v[j] = __builtin_nontemporal_load(xg + static_cast<uint64_t>(token) * unitsPerRow + u);
+            }
+        }
+    };
+    auto spread = [&](uint32_t item, const u32x4(&v)[kHold], const int32_t(&rows)[kMaxTopK]) {
+        const uint32_t token = item / parts;
+        const uint32_t begin = (item - token * parts) * perPart;
+        const uint32_t end = begin + perPart < unitsPerRow ? begin + perPart : unitsPerRow;
+#pragma unroll
+        for (uint32_t k = 0; k < kMaxTopK; ++k) {
+            if (k < topK && rows[k] >= 0) {
+                MF_GLOBAL u32x4 *dst = og + static_cast<uint64_t>(rows[k]) * unitsPerRow;
+#pragma unroll
+                for (uint32_t j = 0; j < kHold; ++j) {
+                    const uint32_t u = begin + j * 64 + threadIdx.x;
+                    if (u < end) {
+                        dst[u] = v[j];
+                    }
+                }
+            }
+        }
+    };
+    // two register sets, a and b, alternate between "being fetched" and "being stored"
+    uint32_t ia = blockIdx.x;
+    if (ia >= items) {
+        return;
+    }
+    u32x4 a[kHold];
+    u32x4 b[kHold];
+    int32_t ra[kMaxTopK];
+    int32_t rb[kMaxTopK];
+    fetch(ia, a, ra);
+    while (true) {
+        const uint32_t ib = ia + gridDim.x;
+        const bool hasB = ib < items;
+        if (hasB) {
+            fetch(ib, b, rb);
+        }
+        spread(ia, a, ra);
+        if (!hasB) {
+            break;
+        }
+        ia = ib + gridDim.x;
+        const bool hasA = ia < items;
+        if (hasA) {
+            fetch(ia, a, ra);
+        }
+        spread(ib, b, rb);
+        if (!hasA) {
+            break;
+        }
+    }
+}
+
 __device__ __forceinline__ float Bf16Lo(uint32_t w)
 {
     return __uint_as_float(w << 16);
@@ -436,12 +513,16 @@ extern "C" int mfk_moe_dispatch(const void *x, const void *topk, uint32_t tokens
         u32x4 *oo = static_cast<u32x4 *>(out);
         const uint32_t upr = hidden / 8;
         // Wide rows: single-wave workgroups that hold up to 14 pieces per lane (a whole 7168-element
-        // row) and write them with plain stores, the fastest of the shapes measured on such rows
-        // (214 us; two waves per row 221 us; four-wave workgroups with nontemporal stores 237 us; the
-        // destination-side form, one workgroup per output row reading x[srcOf[row]], 271 us: its
-        // eight reads of every token row are not absorbed by the caches).
+        // row) and write them with plain stores.  Storing alone takes 177 us of the 200 us such a
+        // kernel needs when every wave reads its row first; with sixteen waves per CU that each
+        // take several tokens and fetch the next row while they store the current one (variant 12)
+        // the dispatch takes 207 us instead of 215.  Other shapes measured on these rows: two waves
+        // per row 221 us; four-wave workgroups with nontemporal stores 237 us; buffer-addressed
+        // stores at eight waves per SIMD 224 us; the destination-side form, one workgroup per output
+        // row reading x[srcOf[row]], 271 us: its eight reads of every token row are not absorbed by
+        // the caches.
         // Narrow rows: one four-wave workgroup per token.
-        const int variant = g_permuteVariant >= 0 ? g_permuteVariant : (upr >= 512 ? 10 : 0);
+        const int variant = g_permuteVariant >= 0 ? g_permuteVariant : (upr >= 512 ? 12 : 0);
         const uint32_t wideParts = (upr + 64 * 14 - 1) / (64 * 14);
         switch (variant) {
             case 1:
@@ -461,6 +542,14 @@ extern "C" int mfk_moe_dispatch(const void *x, const void *topk, uint32_t tokens
                 hipLaunchKernelGGL((MoePermuteKernel<64, 14, 0>), dim3(tokens * wideParts), dim3(64), 0, s, xi, ro, topK, upr,
                                    wideParts, oo);
                 break;
+            case 12: {
+                // 123 vector registers per lane: four waves per SIMD, sixteen per CU, all resident at once
+                const uint32_t items = tokens * wideParts;
+                const uint32_t waves = static_cast<uint32_t>(mfrt_cu_count() > 0 ? mfrt_cu_count() : 256) * 16u;
+                hipLaunchKernelGGL((MoePermuteLoopKernel<14>), dim3(items < waves ? items : waves), dim3(64), 0, s, xi, ro, topK, upr,
+                                   wideParts, items, oo);
+                break;
+            }
             default:
                 hipLaunchKernelGGL((MoePermuteKernel<256, 4, 1>), dim3(tokens), dim3(256), 0, s, xi, ro, topK, upr, 1u, oo);
                 break;

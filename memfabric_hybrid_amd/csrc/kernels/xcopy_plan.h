@@ -84,6 +84,7 @@ struct TablePlan {
     uint32_t nseg;
     uint32_t nchunk;
     uint32_t units;
+    uint32_t perSegment;                // != 0: every segment has this many chunks and `first` is not read
 };
 
 }  // namespace mf

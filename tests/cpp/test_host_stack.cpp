@@ -502,7 +502,15 @@ static void TestPlanners()
         const uint32_t units = 64u << (rng() % 6);
         std::vector<uint64_t> src(n), dst(n), len(n);
         uint64_t s = 0x7f1000000000ull + rng() % 4096, d = 0x7f8000000000ull + rng() % 4096;
+        const bool pages = trial % 5 == 4;   // equal-size segments at page-aligned places
+        const uint64_t pageBytes = 4096ull << (rng() % 5);
         for (uint32_t i = 0; i < n; ++i) {
+            if (pages) {
+                len[i] = pageBytes;
+                src[i] = 0x7f1000000000ull + pageBytes * (2 * (rng() % 100000));
+                dst[i] = 0x7f8000000000ull + pageBytes * (2 * i);
+                continue;
+            }
             const uint32_t kind = rng() % 8;
             len[i] = kind == 0 ? 0 : (kind == 1 ? rng() % 40 : rng() % 300000);
             if (kind != 2) {   // kind 2: continue the previous segment on both sides
@@ -520,7 +528,17 @@ static void TestPlanners()
         std::vector<uint32_t> f1(segs.Size() + 1), f2(n + 1);
         const uint64_t c1 = BuildTablePlan(segs, units, t1.data(), f1.data());
         uint32_t count = 0;
-        const uint64_t c2 = BuildTableDirect(src.data(), dst.data(), len.data(), n, units, t2.data(), f2.data(), count);
+        uint32_t perSegment = 77;
+        const uint64_t c2 = BuildTableDirect(src.data(), dst.data(), len.data(), n, units, t2.data(), f2.data(), count,
+                                             &perSegment);
+        uint32_t expectPer = segs.Size() != 0 ? f1[1] - f1[0] : 0;
+        for (uint32_t i = 0; i < segs.Size(); ++i) {
+            if (f1[i + 1] - f1[i] != expectPer) {
+                expectPer = 0;
+            }
+        }
+        CHECK(perSegment == expectPer);
+        CHECK(!pages || perSegment != 0);
         bool same = c1 == c2 && count == segs.Size();
         for (uint32_t i = 0; same && i < count; ++i) {
             same = t1[3 * i] == t2[3 * i] && t1[3 * i + 1] == t2[3 * i + 1] && t1[3 * i + 2] == t2[3 * i + 2] && f1[i] == f2[i];

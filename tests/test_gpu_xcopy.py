@@ -90,6 +90,18 @@ def test_every_small_length_and_alignment_in_one_launch(gpu, oracle):
     _check_d2d(gpu, oracle, 2 * half, np.array(src_off), np.array(dst_off), np.array(lens), 0xA1)
 
 
+@pytest.mark.parametrize("length,count", [(5000, 300), (32768, 700), (12288 + 7, 2000)])
+def test_equal_sized_segments_at_ragged_places(gpu, oracle, length, count):
+    """Segments of one size have equal chunk counts whatever their alignment: the launch that
+    finds a chunk's segment by division instead of a search must move the same bytes."""
+    rng = np.random.default_rng(length)
+    slot = (length + 64 + 4095) // 4096 * 4096
+    half = slot * count
+    src_off = rng.permutation(count) * slot + rng.integers(0, 48, count)
+    dst_off = half + np.arange(count) * slot + rng.integers(0, 48, count)
+    _check_d2d(gpu, oracle, 2 * half, src_off, dst_off, np.full(count, length), length)
+
+
 @pytest.mark.parametrize("count", [16384, 70000])
 def test_batches_at_and_beyond_the_reference_slot_size(gpu, oracle, count):
     """16 384 segments fill one parameter slot of the reference (hybm_data_op_sdma.cpp:25-31 there);
