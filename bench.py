@@ -402,6 +402,25 @@ def extras_paged(lib):
     res["shape"] = "4096 x 32 KiB pages, 40 GiB pool, one K-or-V plane of one layer per call (134 217 728 B)"
     lib.mfrt_device_sync()
     lib.mfrt_free_device(buf)
+    # The whole set of a 32-layer model (K and V planes: 64 x 4096 pages) as ONE call of 262 144 descriptors.
+    planes = 64
+    big = lib.mfrt_alloc_device(planes * count * page)
+    if big:
+        ids = np.concatenate([workloads.page_ids(0xC3 + 16 + b, pool_bytes // page, count) for b in range(planes)])
+        total = planes * count
+        s_all = native.u64_array((pool + ids * page).tolist())
+        d_all = native.u64_array((big + np.arange(total, dtype=np.uint64) * page).tolist())
+        l_all = native.u64_array([page] * total)
+
+        def gather_all():
+            assert lib.mf_xcopy_batch(s_all, d_all, l_all, total, native.ROUTE_HBM, None) == 0
+
+        us, _ = timer.run(gather_all, 8, warm=5)   # the warm-up sizes all four descriptor staging slots
+        hbm = 2 * total * page / us / 1e3
+        res["gather_full_set_one_call"] = {"descriptors": total, "us": round(us, 1), "hbm_GBps": round(hbm, 1),
+                                           "frac_of_hbm_peak": frac(hbm, HBM_PEAK_GBPS)}
+        lib.mfrt_device_sync()
+        lib.mfrt_free_device(big)
     lib.mfrt_free_device(pool)
     return res
 
