@@ -1,4 +1,5 @@
 #include "hip_data_op.h"
+#include "host_copy.h"
 
 #include <cstring>
 #include <vector>
@@ -176,6 +177,7 @@ HipDataOp::Result HipDataOp::Run(void *const *src, void *const *dst, const uint6
             left -= take;
         }
     }
+    HostCopyHelper &copier = HostCopyHelper::Instance();   // large pieces are copied by two cores
     struct Round {
         size_t begin = 0;
         size_t end = 0;
@@ -185,6 +187,7 @@ HipDataOp::Result HipDataOp::Run(void *const *src, void *const *dst, const uint6
     std::vector<uint64_t> a;
     std::vector<uint64_t> b;
     std::vector<uint64_t> l;
+    std::vector<HostCopyHelper::Task> tasks;   // the CPU copies of one round
     auto drain = [&](Round &round, uint32_t slot) -> int {   // GPU -> caller: wait for the slot's launch, empty it
         if (round.begin == round.end) {
             return BM_OK;
@@ -193,10 +196,12 @@ HipDataOp::Result HipDataOp::Run(void *const *src, void *const *dst, const uint6
         if (err != 0) {
             MF_FAIL(BM_ERROR, "copy failed on the GPU: " << mfrt_error_string(err));
         }
+        tasks.clear();
         for (size_t i = round.begin; i < round.end; ++i) {
-            std::memcpy(reinterpret_cast<void *>(pieces[i].dst), reinterpret_cast<const void *>(round.staged[i - round.begin]),
-                        pieces[i].len);
+            tasks.push_back(HostCopyHelper::Task{reinterpret_cast<void *>(pieces[i].dst),
+                                                 reinterpret_cast<const void *>(round.staged[i - round.begin]), pieces[i].len});
         }
+        copier.CopySet(tasks.data(), tasks.size());
         round.begin = round.end = 0;
         return BM_OK;
     };
@@ -226,6 +231,7 @@ HipDataOp::Result HipDataOp::Run(void *const *src, void *const *dst, const uint6
         a.clear();
         b.clear();
         l.clear();
+        tasks.clear();
         round.staged.clear();
         round.begin = at;
         uint64_t used = 0;
@@ -237,7 +243,8 @@ HipDataOp::Result HipDataOp::Run(void *const *src, void *const *dst, const uint6
             }
             const uint64_t where = base + used;
             if (srcPageable) {
-                std::memcpy(reinterpret_cast<void *>(where), reinterpret_cast<const void *>(pieces[at].src), pieces[at].len);
+                tasks.push_back(HostCopyHelper::Task{reinterpret_cast<void *>(where), reinterpret_cast<const void *>(pieces[at].src),
+                                                     pieces[at].len});
                 a.push_back(where);
                 b.push_back(pieces[at].dst);
             } else {
@@ -250,6 +257,9 @@ HipDataOp::Result HipDataOp::Run(void *const *src, void *const *dst, const uint6
             ++at;
         }
         round.end = at;
+        if (srcPageable) {
+            copier.CopySet(tasks.data(), tasks.size());
+        }
         int ret = engine.Submit(a.data(), b.data(), l.data(), static_cast<uint32_t>(l.size()), route, stream, nullptr, 0);
         if (ret != BM_OK) {
             return ret;

@@ -16,6 +16,7 @@
 #include "../../memfabric_hybrid_amd/csrc/host/compose_data_op.h"
 #include "../../memfabric_hybrid_amd/csrc/host/mf_log.h"
 #include "../../memfabric_hybrid_amd/csrc/host/xcopy_engine.h"
+#include "../../memfabric_hybrid_amd/csrc/host/host_copy.h"
 
 extern "C" uint64_t fake_rt_launches(void);
 extern "C" void fake_rt_seal(void);
@@ -556,12 +557,69 @@ static void TestPlanners()
     }
 }
 
+// Copies shared with the helper thread move exactly the bytes memcpy would, also when two
+// callers compete for the helper and when pieces are just below and above the split size.
+static void TestHostCopy()
+{
+    HostCopyHelper &helper = HostCopyHelper::Instance();
+    auto worker = [&](uint64_t seed, int rounds) {
+        std::mt19937_64 rng(seed);
+        std::vector<uint8_t> src(5u << 20), dst(5u << 20), expect(5u << 20);
+        for (auto &b : src) {
+            b = static_cast<uint8_t>(rng());
+        }
+        for (int r = 0; r < rounds; ++r) {
+            const size_t edge = HostCopyHelper::kSplitMin;
+            const size_t lens[] = {0, 1, 4095, edge - 1, edge, edge + 1, (2u << 20), (2u << 20) + 77, 3000001};
+            const size_t len = lens[r % 9];
+            const size_t so = rng() % 4097, dof = rng() % 4097;
+            std::memset(dst.data(), 0xCD, dst.size());
+            std::memset(expect.data(), 0xCD, expect.size());
+            std::memcpy(expect.data() + dof, src.data() + so, len);
+            helper.Copy(dst.data() + dof, src.data() + so, len);
+            CHECK(dst == expect);
+        }
+    };
+    worker(1, 27);
+    CHECK(helper.SharedCopies() > 0);
+    // sets of pieces: the cut falls between pieces, inside one, and after empty ones
+    {
+        std::mt19937_64 rng(9);
+        std::vector<uint8_t> src(6u << 20), dst(6u << 20), expect(6u << 20);
+        for (auto &b : src) {
+            b = static_cast<uint8_t>(rng());
+        }
+        for (int trial = 0; trial < 40; ++trial) {
+            std::vector<HostCopyHelper::Task> set;
+            std::memset(dst.data(), 0xEE, dst.size());
+            std::memset(expect.data(), 0xEE, expect.size());
+            size_t at = 0;
+            const int pieces = 1 + static_cast<int>(rng() % 40);
+            for (int i = 0; i < pieces && at < (5u << 20); ++i) {
+                const uint32_t kind = static_cast<uint32_t>(rng() % 6);
+                const size_t len = kind == 0 ? 0 : (kind == 1 ? 1u << 20 : rng() % 200000);
+                const size_t so = rng() % ((6u << 20) - len);
+                set.push_back(HostCopyHelper::Task{dst.data() + at, src.data() + so, len});
+                std::memcpy(expect.data() + at, src.data() + so, len);
+                at += len + rng() % 64;
+            }
+            helper.CopySet(set.data(), set.size());
+            CHECK(dst == expect);
+        }
+        helper.CopySet(nullptr, 0);
+    }
+    std::thread other(worker, 2, 27);
+    worker(3, 27);
+    other.join();
+}
+
 int main()
 {
     SetLogLevel(3);
     SetLogSink([](int, const char *) {});
     TestCompose();
     TestPlanners();
+    TestHostCopy();
     TestCApi();                                  // device window: reserved address space, HBM mapped in
     setenv("MF_HIP_GVA_WINDOW", "malloc", 1);
     TestCApi();                                  // device window: one ordinary allocation
