@@ -162,7 +162,14 @@ HipDataOp::Result HipDataOp::Run(void *const *src, void *const *dst, const uint6
     // a slot) and the GPU side (one fused launch per slot) overlap: towards the GPU the CPU fills
     // slot r+1 while the launch of slot r runs, away from it the CPU empties slot r-1 while the
     // launch that fills slot r runs.  An event per slot says when its launch has finished.
-    const uint64_t roundBytes = kRoundBytes;   // 512 KiB rounds were tried for small batches: slower (more launches)
+    // 512 KiB rounds were tried for small batches: slower (more launches).  Large transfers take
+    // slots of twice the size: the launch and the event of a round cost the host about 10 us.
+    uint64_t totalBytes = 0;
+    for (uint32_t i = 0; i < n; ++i) {
+        totalBytes += len[i];
+    }
+    const uint64_t roundBytes = totalBytes >= (64ull << 20) ? 2 * kRoundBytes : kRoundBytes;
+    const uint32_t ringSlots = static_cast<uint32_t>(kBounceBytes / roundBytes);
     std::vector<Piece> pieces;
     pieces.reserve(n);
     for (uint32_t i = 0; i < n; ++i) {
@@ -209,13 +216,13 @@ HipDataOp::Result HipDataOp::Run(void *const *src, void *const *dst, const uint6
     size_t at = 0;
     uint32_t r = 0;
     for (; at < pieces.size(); ++r) {
-        const uint32_t slot = r % kRounds;
+        const uint32_t slot = r % ringSlots;
         Round &round = rounds[slot];
         void *event = engine.ThreadBounceEvent(slot);
         if (event == nullptr) {
             MF_FAIL(BM_ERROR, "event creation failed");
         }
-        if (r >= kRounds) {   // the slot's previous launch must be over before the slot is reused
+        if (r >= ringSlots) {   // the slot's previous launch must be over before the slot is reused
             if (dstPageable) {
                 int ret = drain(round, slot);
                 if (ret != BM_OK) {
@@ -235,7 +242,7 @@ HipDataOp::Result HipDataOp::Run(void *const *src, void *const *dst, const uint6
         round.staged.clear();
         round.begin = at;
         uint64_t used = 0;
-        const uint64_t base = reinterpret_cast<uint64_t>(bounce) + static_cast<uint64_t>(slot) * kRoundBytes;
+        const uint64_t base = reinterpret_cast<uint64_t>(bounce) + static_cast<uint64_t>(slot) * roundBytes;
         while (at < pieces.size()) {
             const uint64_t padded = (pieces[at].len + 63) & ~63ull;  // keep staged pieces 64-byte aligned
             if (used + padded > roundBytes) {
@@ -269,15 +276,15 @@ HipDataOp::Result HipDataOp::Run(void *const *src, void *const *dst, const uint6
             MF_FAIL(BM_ERROR, "event record failed: " << mfrt_error_string(err));
         }
         if (dstPageable && r > 0) {   // while this launch runs, empty the slot of the one before
-            ret = drain(rounds[(r - 1) % kRounds], (r - 1) % kRounds);
+            ret = drain(rounds[(r - 1) % ringSlots], (r - 1) % ringSlots);
             if (ret != BM_OK) {
                 return ret;
             }
         }
     }
     if (dstPageable) {
-        for (uint32_t k = 0; k < kRounds; ++k) {   // what is still staged, oldest first
-            const uint32_t slot = (r + k) % kRounds;
+        for (uint32_t k = 0; k < ringSlots; ++k) {   // what is still staged, oldest first
+            const uint32_t slot = (r + k) % ringSlots;
             int ret = drain(rounds[slot], slot);
             if (ret != BM_OK) {
                 return ret;
