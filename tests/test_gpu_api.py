@@ -155,6 +155,18 @@ def test_pageable_batches_go_through_staging(pool, lib, oracle):
     assert np.array_equal(back, payload)
 
 
+def test_pageable_copy_that_wraps_the_ring_of_small_slots(pool, lib, oracle):
+    """48 MiB is below the size that switches to large staging slots and above what the ring of
+    small ones holds, so slots are reused in both directions."""
+    dev = pool.peer_rank_ptr(0, bm.BmMemType.DEVICE)
+    n = 48 * MIB + 5
+    payload = _rand(oracle, n, 0xD4)
+    assert pool.copy_data(np_ptr(payload), dev + 3, n, bm.BmCopyType.H2G) == 0, native.last_error()
+    back = np.zeros(n, dtype=np.uint8)
+    assert pool.copy_data(dev + 3, np_ptr(back), n, bm.BmCopyType.G2H) == 0
+    assert np.array_equal(back, payload)
+
+
 def test_reference_example_pattern_round_trip(pool, lib, oracle):
     """The check the reference's own example performs (example/bm/BmCpp/main.cpp:142-197 of the
     reference): fill with the LCG pattern, copy host -> pool -> host, compare word by word."""
