@@ -83,13 +83,17 @@ def fill_device_pool(lib, dev, nbytes, seed):
         assert err == 0, lib.mfrt_error_string(err)
 
 
-def timed_steps(lib, handle, batches, copy_type, steps, warmup, flags):
-    """K batch copies between two events on the launch stream; returns (wall s, event ms)."""
+def timed_steps(lib, handle, batches, copy_type, steps, warmup, flags, caller="c"):
+    """K batch copies between two events on the launch stream; returns (wall s, event ms).
+    caller "c": the K calls of smem_bm_copy_batch are issued by a C loop inside the library
+    (mf_bm_copy_batch_replay), as a C or C++ program would issue them; "python": one ctypes call
+    per batch, which adds about 1 us of interpreter time to every call."""
     stream = lib.mf_xcopy_thread_stream()
     start, stop = lib.mfrt_event_create(), lib.mfrt_event_create()
     call = lib.smem_bm_copy_batch
     nb = len(batches)
     refs = [b.ref for b in batches]
+    table = (ctypes.POINTER(native.BatchCopyParams) * nb)(*[ctypes.pointer(b.params) for b in batches])
     for i in range(warmup):
         ret = call(handle, refs[i % nb], copy_type, flags)
         assert ret == 0, native.last_error()
@@ -97,9 +101,13 @@ def timed_steps(lib, handle, batches, copy_type, steps, warmup, flags):
     assert lib.mfrt_device_sync() == 0
     t0 = time.perf_counter()
     lib.mfrt_event_record(start, stream)
-    for i in range(steps):
-        if call(handle, refs[i % nb], copy_type, flags) != 0:
+    if caller == "c":
+        if lib.mf_bm_copy_batch_replay(handle, table, nb, steps, copy_type, flags) != 0:
             raise RuntimeError(native.last_error())
+    else:
+        for i in range(steps):
+            if call(handle, refs[i % nb], copy_type, flags) != 0:
+                raise RuntimeError(native.last_error())
     lib.mfrt_event_record(stop, stream)
     assert lib.mfrt_stream_sync(stream) == 0
     assert lib.mfrt_device_sync() == 0
@@ -252,6 +260,10 @@ def extras_block(lib, pool, dev, batches, tables, steps):
     k = max(200, steps // 10)
     w, _ = timed_steps(lib, handle, batches, g2g, k, 50, 0)
     out["kv122_d2d_sync_call_us"] = round(w * 1e6 / k, 2)
+    wp, msp = timed_steps(lib, handle, batches, g2g, steps, 100, native.ASYNC_COPY_FLAG, caller="python")
+    out["kv122_python_caller"] = {"us_per_batch_wall": round(wp * 1e6 / steps, 2),
+                                  "us_per_batch_events": round(msp * 1e3 / steps, 2),
+                                  "note": "the headline loop with one ctypes call per batch instead of the C loop"}
     conc = {}
     for threads in (2, 4, 8):
         wall = threaded_steps(lib, handle, batches, g2g, steps, threads)
@@ -560,7 +572,8 @@ def main():
         "config": {
             "workload": "DeepSeek-R1-style KV block batch: 122 segments (61x128KiB + 61x16KiB = 8994816 B), "
                         "4 KiB-aligned random offsets in a 4 GiB HBM pool, D2D, 64 rotating tables",
-            "api": "smem_bm_copy_batch(SMEMB_COPY_G2G, ASYNC_COPY_FLAG) on one stream + one wait",
+            "api": "smem_bm_copy_batch(SMEMB_COPY_G2G, ASYNC_COPY_FLAG) on one stream + one wait; the K calls are "
+                   "issued by a C loop (mf_bm_copy_batch_replay), extras.kv122_python_caller has one ctypes call per batch",
             "payload_bytes": payload,
             "cu_count": lib.mfrt_cu_count(),
         },

@@ -15,6 +15,8 @@
 
 #include <stdint.h>
 
+#include "mf_xcopy_types.h"
+
 #ifdef __cplusplus
 extern "C" {
 #endif
@@ -34,6 +36,14 @@ extern "C" {
  * device-accessible.  Does not wait. */
 int32_t mf_xcopy_batch(const uint64_t *src, const uint64_t *dst, const uint64_t *len, uint32_t n, int32_t route,
                        void *stream);
+
+/* `steps` calls of smem_bm_copy_batch(handle, batches[i % count], t, flags), i = 0 .. steps-1,
+ * issued from C: what the loop of a C or C++ caller does (the reference's benchmark,
+ * example/bm/BmBenchmark/band_width_calculator.cpp:530-590, is such a loop), for callers
+ * written in an interpreted language whose per-call overhead would otherwise set the pace.
+ * Stops at the first call that fails and returns its code. */
+int32_t mf_bm_copy_batch_replay(smem_bm_t handle, smem_batch_copy_params *const *batches, uint32_t count,
+                                uint32_t steps, smem_bm_copy_type t, uint32_t flags);
 
 /* Same for a {src,dst,len} triple table that already lives in device memory. */
 int32_t mf_xcopy_device_table(const void *triples, uint32_t n, int32_t route, void *stream);

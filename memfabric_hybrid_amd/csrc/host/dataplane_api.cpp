@@ -52,6 +52,23 @@ MF_EXPORT int32_t mf_probe_hbm(int32_t kind, void *dst, const void *src, uint64_
     return BM_OK;
 }
 
+MF_EXPORT int32_t mf_bm_copy_batch_replay(smem_bm_t handle, smem_batch_copy_params *const *batches, uint32_t count,
+                                          uint32_t steps, smem_bm_copy_type t, uint32_t flags)
+{
+    if (batches == nullptr || count == 0) {
+        MF_FAIL(SM_INVALID_PARAM, "mf_bm_copy_batch_replay: no batches");
+    }
+    uint32_t at = 0;
+    for (uint32_t i = 0; i < steps; ++i) {
+        const int32_t ret = smem_bm_copy_batch(handle, batches[at], t, flags);
+        if (ret != 0) {
+            return ret;
+        }
+        at = at + 1 == count ? 0 : at + 1;
+    }
+    return 0;
+}
+
 MF_EXPORT void *mf_xcopy_thread_stream(void)
 {
     XcopyEngine &engine = XcopyEngine::Instance();
