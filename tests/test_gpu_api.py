@@ -194,6 +194,47 @@ def test_async_copy_completes_on_wait(pool, lib, oracle):
     assert np.array_equal(got, block)
 
 
+def test_replayed_batches_keep_stream_order(pool, lib, oracle):
+    """mf_bm_copy_batch_replay issues the same calls a loop would: three batches, each reading what
+    the one before wrote, cycled for seven steps on one stream, against the oracle applied in order."""
+    dev = pool.peer_rank_ptr(0, bm.BmMemType.DEVICE)
+    n = 24 * MIB
+    init = _rand(oracle, n, 0xD6)
+    assert lib.mfrt_memcpy(dev, np_ptr(init), n) == 0
+    region = 8 * MIB
+    rng = np.random.default_rng(11)
+    tables = []
+    for b in range(3):   # batch b moves 40 ragged pieces from region b to region (b + 1) % 3
+        lens = rng.integers(1, 150000, 40)
+        src = b * region + np.cumsum(lens) - lens + rng.integers(0, 7)
+        dst = ((b + 1) % 3) * region + np.cumsum(lens) - lens + rng.integers(0, 7)
+        tables.append((src, dst, lens))
+    keep = []
+    blocks = []
+    for src, dst, lens in tables:
+        srcs = native.ptr_array((dev + src).tolist())
+        dsts = native.ptr_array((dev + dst).tolist())
+        sizes = native.u64_array(lens.tolist())
+        params = native.BatchCopyParams(srcs, dsts, sizes, len(lens))
+        keep.append((srcs, dsts, sizes))
+        blocks.append(params)
+    table = (ctypes.POINTER(native.BatchCopyParams) * 3)(*[ctypes.pointer(p) for p in blocks])
+    steps = 7
+    assert lib.mf_bm_copy_batch_replay(pool.handle, table, 3, steps, int(bm.BmCopyType.G2G),
+                                       native.ASYNC_COPY_FLAG) == 0, native.last_error()
+    assert pool.wait() == 0
+    expect = init.copy()
+    for i in range(steps):
+        src, dst, lens = tables[i % 3]
+        before = expect.copy()
+        gpu_util.oracle_batch(oracle, before, expect, src, dst, lens)
+    got = np.empty(n, dtype=np.uint8)
+    assert lib.mfrt_memcpy(np_ptr(got), dev, n) == 0
+    assert np.array_equal(got, expect)
+    assert lib.mf_bm_copy_batch_replay(pool.handle, None, 3, 1, int(bm.BmCopyType.G2G), 0) == native.SM_INVALID_PARAM
+    assert lib.mf_bm_copy_batch_replay(pool.handle, table, 3, 0, int(bm.BmCopyType.G2G), 0) == 0
+
+
 def test_range_and_argument_errors(pool, lib):
     dev = pool.peer_rank_ptr(0, bm.BmMemType.DEVICE)
     host = pool.peer_rank_ptr(0, bm.BmMemType.HOST)
