@@ -264,6 +264,9 @@ def extras_block(lib, pool, dev, batches, tables, steps):
     out["kv122_python_caller"] = {"us_per_batch_wall": round(wp * 1e6 / steps, 2),
                                   "us_per_batch_events": round(msp * 1e3 / steps, 2),
                                   "note": "the headline loop with one ctypes call per batch instead of the C loop"}
+    reps = sorted(timed_steps(lib, handle, batches, g2g, 256, 16, native.ASYNC_COPY_FLAG)[1] * 1e3 / 256 for _ in range(20))
+    out["kv122_d2d_repetitions"] = {"n": 20, "launches_each": 256, "median_us": round(reps[10], 2), "min_us": round(reps[0], 2),
+                                    "max_us": round(reps[-1], 2)}
     conc = {}
     for threads in (2, 4, 8):
         wall = threaded_steps(lib, handle, batches, g2g, steps, threads)
