@@ -105,8 +105,12 @@ void HostCopyHelper::CopySet(const Task *tasks, size_t count)
         std::memcpy(tasks[i].dst, tasks[i].src, tasks[i].len);
     }
     std::memcpy(tasks[cut].dst, tasks[cut].src, within);
-    while (done_.load(std::memory_order_acquire) != ticket) {
-        CpuRelax();
+    for (int spins = 0; done_.load(std::memory_order_acquire) != ticket; ++spins) {
+        if (spins < kSpinRounds) {
+            CpuRelax();
+        } else {
+            std::this_thread::yield();   // the helper has not been scheduled: do not hold the core it may need
+        }
     }
     shared_.fetch_add(1, std::memory_order_relaxed);
 }
