@@ -148,8 +148,17 @@ HipDataOp::Result HipDataOp::Run(void *const *src, void *const *dst, const uint6
         if (err != 0) {
             MF_FAIL(BM_ERROR, "stream wait failed: " << mfrt_error_string(err));
         }
+        // Elements whose own source and destination overlap are moved in place; the rest is shared
+        // with the helper thread, one element at a time (elements may depend on one another only
+        // if the caller broke the rule that destinations overlap nothing else in the batch).
         for (uint32_t i = 0; i < n; ++i) {
-            std::memmove(dst[i], src[i], len[i]);
+            const uint64_t s = reinterpret_cast<uint64_t>(src[i]);
+            const uint64_t d = reinterpret_cast<uint64_t>(dst[i]);
+            if (s < d + len[i] && d < s + len[i]) {
+                std::memmove(dst[i], src[i], len[i]);
+            } else {
+                HostCopyHelper::Instance().Copy(dst[i], src[i], len[i]);
+            }
         }
         return BM_OK;
     }
