@@ -517,7 +517,8 @@ extern "C" int mfk_moe_dispatch(const void *x, const void *topk, uint32_t tokens
         // kernel needs when every wave reads its row first; with sixteen waves per CU that each
         // take several tokens and fetch the next row while they store the current one (variant 12)
         // the dispatch takes 207 us instead of 215.  Other shapes measured on these rows: two waves
-        // per row 221 us; four-wave workgroups with nontemporal stores 237 us; buffer-addressed
+        // per row 221 us; four-wave workgroups with nontemporal stores 237 us; the row staged in LDS
+        // instead of registers 221 us (one wave) and 227 us (four waves); buffer-addressed
         // stores at eight waves per SIMD 224 us; the destination-side form, one workgroup per output
         // row reading x[srcOf[row]], 271 us: its eight reads of every token row are not absorbed by
         // the caches.
