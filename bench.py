@@ -275,6 +275,23 @@ def extras_block(lib, pool, dev, batches, tables, steps):
                                       "frac_of_hbm_peak": frac(hbm, HBM_PEAK_GBPS)}
     out["kv122_d2d_concurrent_streams"] = conc
 
+    # ---- the grid the reference publishes for its transfer benchmark (example/trans/perf/README.md:61-70 there:
+    # 32 equal blocks per batch, blocking calls, GB/s = block * 32 / time per call), here HBM to HBM on one GPU
+    grid = []
+    for block in (32 << 10, 64 << 10, 128 << 10, 256 << 10, 512 << 10, 1 << 20, 2 << 20, 4 << 20, 8 << 20, 16 << 20):
+        src_off = np.arange(32, dtype=np.uint64) * block
+        dst_off = (POOL_BYTES // 2) + np.arange(32, dtype=np.uint64) * block
+        b = Batch(dev + src_off, dev + dst_off, np.full(32, block, dtype=np.uint64))
+        for _ in range(5):
+            lib.smem_bm_copy_batch(handle, b.ref, g2g, 0)
+        t0 = time.perf_counter()
+        for _ in range(30):
+            lib.smem_bm_copy_batch(handle, b.ref, g2g, 0)
+        per_call = (time.perf_counter() - t0) / 30
+        grid.append({"block_KiB": block >> 10, "us_per_call": round(per_call * 1e6, 1),
+                     "payload_GBps": round(32 * block / per_call / GB, 1)})
+    out["batch32_blocking_calls_d2d"] = grid
+
     # ---- KV batch over the host link ------------------------------------------------------------------------
     host = pool.peer_rank_ptr(0, bm.BmMemType.HOST)
     split = [workloads.kv_batch(0xD1 + b, POOL_BYTES, same_pool=False) for b in range(16)]
