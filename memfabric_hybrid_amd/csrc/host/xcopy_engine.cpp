@@ -597,12 +597,25 @@ int XcopyEngine::Submit(const uint64_t *src, const uint64_t *dst, const uint64_t
 
     // Table form: {triples, prefix} are built in a pinned slot; the general form moves them to HBM
     // with a copy launch and searches them there.  The slot is sized for n segments; merging can only make the table shorter.
-    if (units == 0 || n > 4 * kInlineSegs) {
+    {
         uint64_t total = 0;
+        uint64_t longest = 0;
         for (uint32_t i = 0; i < n; ++i) {
             total += len[i];
+            longest = len[i] > longest ? len[i] : longest;
         }
         units = ChooseUnits(total, cu, route, tuning_);
+        // Many short segments: a chunk size that holds the longest of them gives every segment exactly
+        // one chunk, which is the equal-count form below (no prefix, no search, no upload): 16 384
+        // segments of 2-14 KB take 62 us instead of 74 us.
+        if (tuning_.unitsOverride == 0 && longest != 0) {
+            for (uint32_t u = units; u <= 4 * kXcopyThreads; u *= 2) {
+                if (longest <= static_cast<uint64_t>(u) * kUnitBytes - kUnitBytes) {
+                    units = u;
+                    break;
+                }
+            }
+        }
     }
     const uint64_t tripleBytes = 24ull * n;
     const uint64_t tableBytes = RoundUp(tripleBytes + 4ull * (n + 1), kUnitBytes);
