@@ -394,14 +394,15 @@ uint64_t BuildTablePlan(const SegList &segs, uint32_t units, uint64_t *triples, 
 // batch costs the host about as long as the GPU needs to copy it, so nothing is built twice.
 // triples: room for 3 * n words, first: room for n + 1.  Returns the chunk count, count = segments.
 uint64_t BuildTableDirect(const uint64_t *src, const uint64_t *dst, const uint64_t *len, uint32_t n, uint32_t units,
-                          uint64_t *triples, uint32_t *first, uint32_t &count, uint32_t *perSegment)
+                          uint64_t *triples, uint32_t *first, uint32_t &count, ChunkPattern *pattern)
 {
     const bool pow2 = (units & (units - 1)) == 0;
     const uint32_t shift = pow2 ? static_cast<uint32_t>(__builtin_ctz(units)) : 0;
     uint32_t used = 0;
     uint64_t run = 0;
-    uint64_t firstChunks = 0;
-    uint64_t differing = 0;   // OR of (chunks ^ firstChunks): stays 0 while all segments agree
+    uint64_t recent[kMaxPeriod] = {};   // chunk counts of the last kMaxPeriod segments, by index modulo kMaxPeriod
+    uint64_t leading[kMaxPeriod] = {};  // and of the first ones
+    uint32_t alive = 0x1FEu;            // bit p: the counts so far repeat with period p (1 .. kMaxPeriod)
     uint64_t curSrc = 0;
     uint64_t curDst = 0;
     uint64_t curLen = 0;
@@ -422,10 +423,17 @@ uint64_t BuildTableDirect(const uint64_t *src, const uint64_t *dst, const uint64
         triples[3 * used + 1] = curDst;
         triples[3 * used + 2] = curLen;
         first[used] = static_cast<uint32_t>(run < kNoChunk ? run : kNoChunk);
-        if (used == 0) {
-            firstChunks = chunks;
+        if (alive != 0) {
+            for (uint32_t p = 1; p <= kMaxPeriod; ++p) {
+                if (used >= p && recent[(used - p) % kMaxPeriod] != chunks) {
+                    alive &= ~(1u << p);
+                }
+            }
+            recent[used % kMaxPeriod] = chunks;
+            if (used < kMaxPeriod) {
+                leading[used] = chunks;
+            }
         }
-        differing |= chunks ^ firstChunks;
         run += chunks;
         ++used;
     };
@@ -446,8 +454,19 @@ uint64_t BuildTableDirect(const uint64_t *src, const uint64_t *dst, const uint64
     flush();
     first[used] = static_cast<uint32_t>(run < kNoChunk ? run : kNoChunk);
     count = used;
-    if (perSegment != nullptr) {
-        *perSegment = used != 0 && differing == 0 && firstChunks < kNoChunk ? static_cast<uint32_t>(firstChunks) : 0;
+    if (pattern != nullptr) {
+        *pattern = ChunkPattern{};
+        if (used != 0 && alive != 0 && run < kNoChunk) {
+            const uint32_t period = static_cast<uint32_t>(__builtin_ctz(alive));
+            uint32_t sum = 0;
+            for (uint32_t i = 0; i < period; ++i) {
+                pattern->start[i] = sum;
+                sum += static_cast<uint32_t>(leading[i]);   // the shortest period never exceeds the segment count
+            }
+            pattern->start[period] = sum;
+            pattern->period = period;
+            pattern->chunksPerPeriod = sum;
+        }
     }
     return run;
 }
@@ -627,8 +646,8 @@ int XcopyEngine::Submit(const uint64_t *src, const uint64_t *dst, const uint64_t
     uint64_t *triples = static_cast<uint64_t *>(slot->host);
     uint32_t *first = reinterpret_cast<uint32_t *>(static_cast<uint8_t *>(slot->host) + tripleBytes);
     uint32_t count = 0;
-    uint32_t perSegment = 0;
-    const uint64_t nchunk = BuildTableDirect(src, dst, len, n, units, triples, first, count, &perSegment);
+    ChunkPattern pattern;
+    const uint64_t nchunk = BuildTableDirect(src, dst, len, n, units, triples, first, count, &pattern);
     if (nchunk >= kNoChunk) {
         MF_FAIL(BM_INVALID_PARAM, "batch too large for one launch: " << nchunk << " chunks");
     }
@@ -642,14 +661,15 @@ int XcopyEngine::Submit(const uint64_t *src, const uint64_t *dst, const uint64_t
 
     const uint32_t grid = GridFor(nchunk, cu, route, tuning_);
     int err = 0;
-    if (perSegment != 0) {
-        // Segments of one size (pages): a workgroup finds its descriptor by a division, so the only
+    if (pattern.period != 0) {
+        // Chunk counts that repeat (pages of one size, K and V blocks in turn): a workgroup finds its
+        // descriptor by a division and a few comparisons, so the only
         // thing it needs from the table is that one descriptor, and it reads it straight out of
         // the pinned slot.  No upload launch, nothing serial in front of the copy: a 4096-page gather
         // takes 50 us instead of 55, the 64 bytes per workgroup that cross the host link stay below
         // 2 % of the payload rate.  (With the chunk prefix in host memory as well the search of the
         // general form pays a link round trip per level: 16 384 ragged segments 135 us against 74.)
-        err = mfk_xcopy_table(slot->host, nullptr, nullptr, count, static_cast<uint32_t>(nchunk), units, perSegment, route,
+        err = mfk_xcopy_table(slot->host, nullptr, nullptr, count, static_cast<uint32_t>(nchunk), units, &pattern, route,
                               grid, mask, maskValue, stream);
         g_launches.fetch_add(1, std::memory_order_relaxed);
     } else {
@@ -666,7 +686,7 @@ int XcopyEngine::Submit(const uint64_t *src, const uint64_t *dst, const uint64_t
             MF_FAIL(BM_ERROR, "descriptor staging launch failed: " << mfrt_error_string(err));
         }
         const uint8_t *devBase = static_cast<const uint8_t *>(slot->dev);
-        err = mfk_xcopy_table(devBase, devBase + tripleBytes, nullptr, count, static_cast<uint32_t>(nchunk), units, 0, route,
+        err = mfk_xcopy_table(devBase, devBase + tripleBytes, nullptr, count, static_cast<uint32_t>(nchunk), units, nullptr, route,
                               grid, mask, maskValue, stream);
         g_launches.fetch_add(2, std::memory_order_relaxed);
     }
@@ -723,7 +743,7 @@ int XcopyEngine::SubmitDeviceTable(const void *triples, uint32_t n, int route, v
     }
     const uint32_t cu = mfrt_cu_count();
     const uint32_t grid = GridFor(static_cast<uint64_t>(cu == 0 ? 256 : cu) * 256, cu, route, tuning_);   // chunk count is only known on the GPU; surplus workgroups leave at once
-    err = mfk_xcopy_table(triples, first, nchunkDev, n, 0, units, 0, route, grid, mask, maskValue, stream);
+    err = mfk_xcopy_table(triples, first, nchunkDev, n, 0, units, nullptr, route, grid, mask, maskValue, stream);
     if (err != 0) {
         MF_FAIL(BM_ERROR, "xcopy table launch failed: " << mfrt_error_string(err));
     }

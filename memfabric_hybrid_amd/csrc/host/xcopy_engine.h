@@ -63,9 +63,10 @@ uint64_t BuildTablePlan(const SegList &segs, uint32_t units, uint64_t *triples, 
 
 // The same result as NormalizeSegments (no piece limit) + BuildTablePlan in one pass over the
 // caller's arrays.  triples: room for 3 * n words, first: room for n + 1; count = segments written.
-// perSegment (optional) receives the chunk count shared by all segments, or 0 when they differ.
+// pattern (optional) receives the shortest period (up to kMaxPeriod) with which the chunk counts
+// of the segments repeat, period 0 when there is none.
 uint64_t BuildTableDirect(const uint64_t *src, const uint64_t *dst, const uint64_t *len, uint32_t n, uint32_t units,
-                          uint64_t *triples, uint32_t *first, uint32_t &count, uint32_t *perSegment = nullptr);
+                          uint64_t *triples, uint32_t *first, uint32_t &count, ChunkPattern *pattern = nullptr);
 
 class XcopyEngine {
 public:

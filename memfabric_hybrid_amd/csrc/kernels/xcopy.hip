@@ -202,17 +202,20 @@ template <bool kNtLoad, int kStore>
 __global__ __launch_bounds__(kXcopyThreads) void XcopyTableKernel(const uint64_t *__restrict__ triples,
                                                                   const uint32_t *__restrict__ first,
                                                                   const uint32_t *__restrict__ nchunkDev, uint32_t nseg,
-                                                                  uint32_t nchunkHost, uint32_t units, uint32_t perSegment)
+                                                                  uint32_t nchunkHost, uint32_t units, const ChunkPattern pattern)
 {
     const uint32_t nchunk = nchunkDev != nullptr ? *nchunkDev : nchunkHost;
     const uint32_t lane = threadIdx.x & 63u;
     for (uint32_t c = blockIdx.x; c < nchunk; c += gridDim.x) {
-        if (perSegment != 0) {
-            // Equal chunk counts (pages of one size): the owner follows from a division and the
-            // only memory round trip before the copy is the fetch of its descriptor.
-            const uint32_t seg = c / perSegment;
+        if (pattern.period != 0) {
+            // Chunk counts that repeat (pages of one size, K and V blocks in turn): the owner follows
+            // from a division and a few comparisons on kernel arguments, and the only memory round
+            // trip before the copy is the fetch of its descriptor.
+            uint32_t seg;
+            uint32_t k;
+            PatternOwner(pattern, c, seg, k);
             const uint64_t *t = triples + 3ull * seg;
-            CopyChunk<kNtLoad, kStore>(t[0], t[1], t[2], c - seg * perSegment, units);
+            CopyChunk<kNtLoad, kStore>(t[0], t[1], t[2], k, units);
             continue;
         }
         // 64-ary search for the last prefix entry <= c: every level is one load per lane and a
@@ -341,7 +344,7 @@ template <bool kNtLoad, int kStore>
 int LaunchTable(const TablePlan &plan, const uint32_t *nchunkDev, uint32_t grid, uint32_t lanes, hipStream_t stream)
 {
     hipLaunchKernelGGL((XcopyTableKernel<kNtLoad, kStore>), dim3(grid), dim3(lanes), 0, stream, plan.triples,
-                       plan.first, nchunkDev, plan.nseg, plan.nchunk, plan.units, plan.perSegment);
+                       plan.first, nchunkDev, plan.nseg, plan.nchunk, plan.units, plan.pattern);
     return static_cast<int>(hipGetLastError());
 }
 
@@ -378,15 +381,22 @@ extern "C" int mfk_xcopy_inline(const void *inlinePlan, int route, uint32_t grid
 }
 
 extern "C" int mfk_xcopy_table(const void *triples, const void *first, const void *nchunkDev, uint32_t nseg,
-                               uint32_t nchunk, uint32_t units, uint32_t perSegment, int route, uint32_t grid, void *mask,
+                               uint32_t nchunk, uint32_t units, const void *pattern, int route, uint32_t grid, void *mask,
                                uint32_t maskValue, void *stream)
 {
-    if (nseg == 0 || grid == 0 || (perSegment == 0 && first == nullptr) ||
-        (perSegment != 0 && (nchunkDev != nullptr || static_cast<uint64_t>(perSegment) * nseg != nchunk))) {
+    mf::ChunkPattern pat{};
+    if (pattern != nullptr) {
+        pat = *static_cast<const mf::ChunkPattern *>(pattern);
+    }
+    if (nseg == 0 || grid == 0 || (pat.period == 0 && first == nullptr)) {
         return -1;
     }
-    mf::TablePlan plan{static_cast<const uint64_t *>(triples), static_cast<const uint32_t *>(first), nseg, nchunk, units,
-                       perSegment};
+    if (pat.period != 0 && (pat.period > mf::kMaxPeriod || pat.chunksPerPeriod == 0 || nchunkDev != nullptr ||
+                            pat.start[0] != 0 || pat.start[pat.period] != pat.chunksPerPeriod ||
+                            mf::PatternChunks(pat, nseg) != nchunk)) {
+        return -1;
+    }
+    mf::TablePlan plan{static_cast<const uint64_t *>(triples), static_cast<const uint32_t *>(first), nseg, nchunk, units, pat};
     const uint32_t *nd = static_cast<const uint32_t *>(nchunkDev);
     hipStream_t s = static_cast<hipStream_t>(stream);
     const int err = mf::WithPolicy(mf::PolicyOf(route), [&](auto ntLoad, auto store) {

@@ -77,14 +77,44 @@ struct InlinePlan {
     uint32_t units;                     // 16-byte units per chunk, a multiple of 64
 };
 
+// Chunk counts that repeat with a short period: pages of one size (period 1), K and V blocks
+// taking turns (period 2), ...  With such a pattern the owner of a chunk follows from a division
+// and at most kMaxPeriod comparisons, and no chunk prefix is needed.
+constexpr uint32_t kMaxPeriod = 8;
+
+struct ChunkPattern {
+    uint32_t period;                    // 0: no pattern, the chunk prefix is searched
+    uint32_t chunksPerPeriod;
+    uint32_t start[kMaxPeriod + 1];     // exclusive prefix of the counts inside one period; start[period] == chunksPerPeriod
+};
+
+// Segment and chunk-in-segment of global chunk c under a pattern.
+MF_HD inline void PatternOwner(const ChunkPattern &p, uint32_t c, uint32_t &seg, uint32_t &k)
+{
+    const uint32_t group = c / p.chunksPerPeriod;
+    const uint32_t r = c - group * p.chunksPerPeriod;
+    uint32_t j = 0;
+    for (uint32_t i = 1; i < kMaxPeriod; ++i) {
+        j += (i < p.period && p.start[i] <= r) ? 1u : 0u;
+    }
+    seg = group * p.period + j;
+    k = r - p.start[j];
+}
+
+// Chunks of the first nseg segments under a pattern.
+MF_HD inline uint64_t PatternChunks(const ChunkPattern &p, uint32_t nseg)
+{
+    return static_cast<uint64_t>(nseg / p.period) * p.chunksPerPeriod + p.start[nseg % p.period];
+}
+
 // A table-driven launch: triples and prefix live in device memory.
 struct TablePlan {
     const uint64_t *triples;            // {src,dst,len} * nseg
-    const uint32_t *first;              // nseg + 1 entries, first[nseg] == nchunk
+    const uint32_t *first;              // nseg + 1 entries, first[nseg] == nchunk; not read under a pattern
     uint32_t nseg;
     uint32_t nchunk;
     uint32_t units;
-    uint32_t perSegment;                // != 0: every segment has this many chunks and `first` is not read
+    ChunkPattern pattern;
 };
 
 }  // namespace mf

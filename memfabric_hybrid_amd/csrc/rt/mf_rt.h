@@ -72,9 +72,10 @@ int mfrt_memcpy_async(void *dst, const void *src, uint64_t bytes, void *stream);
 
 /* ---- xcopy launchers (kernels/xcopy.hip) --------------------------------- */
 int mfk_xcopy_inline(const void *inlinePlan, int route, uint32_t grid, void *mask, uint32_t maskValue, void *stream);
-/* perSegment != 0: every segment has exactly that many chunks, `first` is not read (may be NULL). */
+/* pattern: NULL, or a mf::ChunkPattern (kernels/xcopy_plan.h) that the chunk counts of the segments follow;
+ * then `first` is not read (may be NULL) and `triples` may live in pinned host memory. */
 int mfk_xcopy_table(const void *triples, const void *first, const void *nchunkDev, uint32_t nseg, uint32_t nchunk,
-                    uint32_t units, uint32_t perSegment, int route, uint32_t grid, void *mask, uint32_t maskValue,
+                    uint32_t units, const void *pattern, int route, uint32_t grid, void *mask, uint32_t maskValue,
                     void *stream);
 int mfk_xcopy_plan(const void *triples, uint32_t nseg, uint32_t units, void *first, void *nchunk, void *stream);
 

@@ -179,18 +179,27 @@ int mfk_xcopy_inline(const void *inlinePlan, int, uint32_t, void *mask, uint32_t
 }
 
 int mfk_xcopy_table(const void *triples, const void *first, const void *nchunkDev, uint32_t nseg, uint32_t nchunk,
-                    uint32_t units, uint32_t perSegment, int, uint32_t, void *mask, uint32_t maskValue, void *)
+                    uint32_t units, const void *pattern, int, uint32_t, void *mask, uint32_t maskValue, void *)
 {
     const uint64_t *t = static_cast<const uint64_t *>(triples);
     const uint32_t *f = static_cast<const uint32_t *>(first);
     const uint32_t total = nchunkDev != nullptr ? *static_cast<const uint32_t *>(nchunkDev) : nchunk;
     ++g_launches;
     uint32_t s = 0;
-    for (uint32_t c = 0; perSegment != 0 && c < total; ++c) {   // as the kernel: owner by division, no prefix
-        const uint32_t seg = c / perSegment;
-        RunChunk(t[3 * seg], t[3 * seg + 1], t[3 * seg + 2], c - seg * perSegment, units);
+    mf::ChunkPattern pat{};
+    if (pattern != nullptr) {
+        pat = *static_cast<const mf::ChunkPattern *>(pattern);
+        if (pat.period == 0 || pat.period > mf::kMaxPeriod || mf::PatternChunks(pat, nseg) != total) {
+            return -1;
+        }
     }
-    for (uint32_t c = 0; perSegment == 0 && c < total; ++c) {
+    for (uint32_t c = 0; pat.period != 0 && c < total; ++c) {   // as the kernel: owner by division, no prefix
+        uint32_t seg = 0;
+        uint32_t k = 0;
+        mf::PatternOwner(pat, c, seg, k);
+        RunChunk(t[3 * seg], t[3 * seg + 1], t[3 * seg + 2], k, units);
+    }
+    for (uint32_t c = 0; pat.period == 0 && c < total; ++c) {
         while (s + 1 <= nseg && f[s + 1] <= c) {
             ++s;
         }

@@ -504,12 +504,18 @@ static void TestPlanners()
         std::vector<uint64_t> src(n), dst(n), len(n);
         uint64_t s = 0x7f1000000000ull + rng() % 4096, d = 0x7f8000000000ull + rng() % 4096;
         const bool pages = trial % 5 == 4;   // equal-size segments at page-aligned places
+        const bool turns = trial % 5 == 3;   // a few sizes taking turns (K and V blocks)
         const uint64_t pageBytes = 4096ull << (rng() % 5);
+        const uint32_t sizes = 2 + static_cast<uint32_t>(rng() % 7);
+        uint64_t turnBytes[8];
+        for (auto &t : turnBytes) {
+            t = 4096ull * (1 + rng() % 40);
+        }
         for (uint32_t i = 0; i < n; ++i) {
-            if (pages) {
-                len[i] = pageBytes;
-                src[i] = 0x7f1000000000ull + pageBytes * (2 * (rng() % 100000));
-                dst[i] = 0x7f8000000000ull + pageBytes * (2 * i);
+            if (pages || turns) {
+                len[i] = pages ? pageBytes : turnBytes[i % sizes];
+                src[i] = 0x7f1000000000ull + 4096ull * (400 * (rng() % 100000));
+                dst[i] = 0x7f8000000000ull + 4096ull * (400 * i);
                 continue;
             }
             const uint32_t kind = rng() % 8;
@@ -529,17 +535,37 @@ static void TestPlanners()
         std::vector<uint32_t> f1(segs.Size() + 1), f2(n + 1);
         const uint64_t c1 = BuildTablePlan(segs, units, t1.data(), f1.data());
         uint32_t count = 0;
-        uint32_t perSegment = 77;
+        ChunkPattern pattern;
+        pattern.period = 99;
         const uint64_t c2 = BuildTableDirect(src.data(), dst.data(), len.data(), n, units, t2.data(), f2.data(), count,
-                                             &perSegment);
-        uint32_t expectPer = segs.Size() != 0 ? f1[1] - f1[0] : 0;
-        for (uint32_t i = 0; i < segs.Size(); ++i) {
-            if (f1[i + 1] - f1[i] != expectPer) {
-                expectPer = 0;
+                                             &pattern);
+        uint32_t expectPeriod = 0;
+        for (uint32_t p = 1; p <= kMaxPeriod && expectPeriod == 0 && segs.Size() != 0; ++p) {
+            bool repeats = true;
+            for (uint32_t i = p; i < segs.Size() && repeats; ++i) {
+                repeats = f1[i + 1] - f1[i] == f1[i + 1 - p] - f1[i - p];
+            }
+            expectPeriod = repeats ? p : 0;
+        }
+        CHECK(pattern.period == expectPeriod);
+        CHECK(!pages || pattern.period == 1);
+        CHECK(!turns || pattern.period != 0);
+        if (pattern.period != 0) {
+            CHECK(PatternChunks(pattern, segs.Size()) == c1);
+            uint32_t seg = 0;
+            for (uint32_t c = 0; c < c1; ++c) {   // every chunk lands on the segment the prefix names
+                while (f1[seg + 1] <= c) {
+                    ++seg;
+                }
+                uint32_t gotSeg = 0;
+                uint32_t gotK = 0;
+                PatternOwner(pattern, c, gotSeg, gotK);
+                if (gotSeg != seg || gotK != c - f1[seg]) {
+                    CHECK(false);
+                    break;
+                }
             }
         }
-        CHECK(perSegment == expectPer);
-        CHECK(!pages || perSegment != 0);
         bool same = c1 == c2 && count == segs.Size();
         for (uint32_t i = 0; same && i < count; ++i) {
             same = t1[3 * i] == t2[3 * i] && t1[3 * i + 1] == t2[3 * i + 1] && t1[3 * i + 2] == t2[3 * i + 2] && f1[i] == f2[i];

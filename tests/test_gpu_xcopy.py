@@ -102,6 +102,19 @@ def test_equal_sized_segments_at_ragged_places(gpu, oracle, length, count):
     _check_d2d(gpu, oracle, 2 * half, src_off, dst_off, np.full(count, length), length)
 
 
+@pytest.mark.parametrize("sizes,count", [((131072, 16384), 610), ((5000, 70000, 12288), 999), ((4096,) * 7 + (40960,), 1203)])
+def test_sizes_taking_turns_above_the_inline_limit(gpu, oracle, sizes, count):
+    """K and V blocks in turn, several requests in one call: the chunk counts repeat with a short
+    period, which the launch uses instead of a chunk prefix.  Placement is random, alignment ragged."""
+    rng = np.random.default_rng(count)
+    lens = np.array([sizes[i % len(sizes)] for i in range(count)])
+    slot = (max(sizes) + 64 + 4095) // 4096 * 4096
+    half = slot * count
+    src_off = rng.permutation(count) * slot + rng.integers(0, 16, count) * (1 if min(sizes) % 4096 else 0)
+    dst_off = half + rng.permutation(count) * slot + rng.integers(0, 16, count) * (1 if min(sizes) % 4096 else 0)
+    _check_d2d(gpu, oracle, 2 * half, src_off, dst_off, lens, count)
+
+
 @pytest.mark.parametrize("count", [16384, 70000])
 def test_batches_at_and_beyond_the_reference_slot_size(gpu, oracle, count):
     """16 384 segments fill one parameter slot of the reference (hybm_data_op_sdma.cpp:25-31 there);
