@@ -428,7 +428,7 @@ def extras_paged(lib):
 
     res = {}
     for name, fn in (("gather", gather), ("scatter", scatter)):
-        us, _ = timer.run(fn, 40, warm=4)
+        us, _ = timer.run(fn, 40, warm=10)   # the warm-up sizes all staging slots of the thread
         hbm = 2 * count * page / us / 1e3
         res[name] = {"us": round(us, 1), "hbm_GBps": round(hbm, 1), "frac_of_hbm_peak": frac(hbm, HBM_PEAK_GBPS)}
     res["shape"] = "4096 x 32 KiB pages, 40 GiB pool, one K-or-V plane of one layer per call (134 217 728 B)"
@@ -447,7 +447,7 @@ def extras_paged(lib):
         def gather_all():
             assert lib.mf_xcopy_batch(s_all, d_all, l_all, total, native.ROUTE_HBM, None) == 0
 
-        us, _ = timer.run(gather_all, 8, warm=5)   # the warm-up sizes all four descriptor staging slots
+        us, _ = timer.run(gather_all, 8, warm=9)   # the warm-up sizes all descriptor staging slots
         hbm = 2 * total * page / us / 1e3
         res["gather_full_set_one_call"] = {"descriptors": total, "us": round(us, 1), "hbm_GBps": round(hbm, 1),
                                            "frac_of_hbm_peak": frac(hbm, HBM_PEAK_GBPS)}
@@ -525,7 +525,7 @@ def extras_reshard(lib):
         assert lib.mf_xcopy_batch(s_arr, d_arr, l_arr, len(segments), native.ROUTE_HBM, None) == 0
         assert lib.mf_xcopy_2d_batch(descs, len(rects), native.ROUTE_HBM, None) == 0
 
-    us, _ = timer.run(run, 3, warm=1)
+    us, _ = timer.run(run, 5, warm=8)   # the warm-up sizes all staging slots of the thread
     moved = sum(n for _, _, n in segments) + sum(r[2] * r[3] for r in rects)
     hbm = 2 * moved / us / 1e3
     lib.mfrt_device_sync()

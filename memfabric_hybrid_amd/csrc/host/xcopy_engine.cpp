@@ -12,20 +12,26 @@
 namespace mf {
 namespace {
 
-constexpr uint32_t kSlots = 4;                // table staging slots per thread
+constexpr uint32_t kSlots = 8;                // table staging slots per thread
+constexpr uint32_t kGuardEvery = 4;           // one event is recorded per this many table launches
 constexpr uint64_t kInlinePiece = 1ull << 30; // cut for segments the 32-bit inline length cannot hold
 
 std::atomic<uint64_t> g_launches{0};
 
-// One descriptor table in flight: host fills `host`, a copy kernel moves it to
-// `dev`, the table kernel reads `dev`.  `event` marks the point on the stream
-// after which `host` may be rewritten.
+// One descriptor table in flight: the host fills `host`; the table kernel reads it there, or a copy
+// kernel moves it to `dev` first.  The slot may be rewritten once an event recorded behind its
+// kernels has fired.  Recording an event costs the stream about 3 us, as much as the launch gap
+// it sits in, so one event guards kGuardEvery consecutive launches: a slot is Queued until that
+// event is recorded and Guarded (by the slot that owns the event) afterwards.
 struct StagingSlot {
+    enum State : uint8_t { kFree, kQueued, kGuarded };
     void *host = nullptr;
     void *dev = nullptr;
-    uint64_t capacity = 0;
+    uint64_t capacity = 0;      // of host
+    uint64_t devCapacity = 0;
     void *event = nullptr;
-    bool pending = false;
+    State state = kFree;
+    StagingSlot *guard = nullptr;
 };
 
 // GPU resources of one calling thread: its stream, its staging slots, its bounce area.  They are
@@ -37,17 +43,28 @@ struct ThreadLease {
     void *stream = nullptr;
     StagingSlot slots[kSlots];
     uint32_t cursor = 0;
+    uint32_t queued = 0;            // slots in state kQueued; their kernels all run on queuedStream
+    void *queuedStream = nullptr;
+    StagingSlot *lastQueued = nullptr;
+    bool adopted = false;           // taken over from a thread that ended: its queued kernels ran on streams unknown here
     void *bounce = nullptr;
     uint64_t bounceBytes = 0;
     void *bounceEvents[XcopyEngine::kBounceEvents] = {};
 
     void Destroy()   // GPU calls: only from Stop(), on a thread that is alive and bound
     {
+        bool busy = false;
+        for (auto &slot : slots) {
+            busy = busy || slot.state != StagingSlot::kFree;
+        }
+        if (busy) {
+            (void)mfrt_device_sync();   // kernels that read the slots may run on streams of the callers
+        }
+        queued = 0;
+        queuedStream = nullptr;
+        lastQueued = nullptr;
         for (auto &slot : slots) {
             if (slot.event != nullptr) {
-                if (slot.pending) {
-                    (void)mfrt_event_sync(slot.event);
-                }
                 (void)mfrt_event_destroy(slot.event);
             }
 
@@ -92,6 +109,7 @@ struct LeasePool {
         if (!idle.empty()) {
             ThreadLease *lease = idle.back();
             idle.pop_back();
+            lease->adopted = true;
             return lease;
         }
         all.emplace_back(new ThreadLease());
@@ -160,30 +178,98 @@ uint64_t RoundUp(uint64_t v, uint64_t to)
     return (v + to - 1) / to * to;
 }
 
-int AcquireSlot(ThreadLease &ctx, uint64_t bytes, StagingSlot *&out)
+// Records the event that guards every queued slot.  If the record fails the stream is drained instead.
+int SealQueued(ThreadLease &ctx)
 {
+    if (ctx.queued == 0) {
+        return BM_OK;
+    }
+    StagingSlot *owner = ctx.lastQueued;
+    const bool recorded = owner != nullptr && owner->event != nullptr && mfrt_event_record(owner->event, ctx.queuedStream) == 0;
+    if (!recorded && mfrt_stream_sync(ctx.queuedStream) != 0) {
+        const int err = mfrt_device_sync();
+        if (err != 0) {
+            MF_FAIL(BM_ERROR, "staging slots could not be released: " << mfrt_error_string(err));
+        }
+    }
+    for (auto &slot : ctx.slots) {
+        if (slot.state == StagingSlot::kQueued) {
+            slot.state = recorded ? StagingSlot::kGuarded : StagingSlot::kFree;
+            slot.guard = recorded ? owner : nullptr;
+        }
+    }
+    ctx.queued = 0;
+    ctx.lastQueued = nullptr;
+    return BM_OK;
+}
+
+// The kernels just launched on `stream` read `slot`.  Only launches on the lease's own stream wait
+// for a shared event: a caller's stream may be gone by the time the next launch comes.
+int MarkQueued(ThreadLease &ctx, StagingSlot *slot, void *stream, bool sealNow)
+{
+    sealNow = sealNow || stream != ctx.stream;
+    slot->state = StagingSlot::kQueued;
+    slot->guard = nullptr;
+    ctx.queuedStream = stream;
+    ctx.lastQueued = slot;
+    ++ctx.queued;
+    return sealNow || ctx.queued >= kGuardEvery ? SealQueued(ctx) : BM_OK;
+}
+
+// The next slot of the ring, free to be rewritten, with at least `bytes` of pinned host memory.
+int AcquireSlot(ThreadLease &ctx, uint64_t bytes, void *stream, StagingSlot *&out)
+{
+    if (ctx.adopted) {
+        // The thread that filled these slots is gone, and with it the knowledge which streams its
+        // last launches went to: wait for the whole device once.
+        bool busy = false;
+        for (auto &slot : ctx.slots) {
+            busy = busy || slot.state != StagingSlot::kFree;
+        }
+        if (busy) {
+            const int err = mfrt_device_sync();
+            if (err != 0) {
+                MF_FAIL(BM_ERROR, "device wait failed: " << mfrt_error_string(err));
+            }
+            for (auto &slot : ctx.slots) {
+                slot.state = StagingSlot::kFree;
+                slot.guard = nullptr;
+            }
+        }
+        ctx.queued = 0;
+        ctx.lastQueued = nullptr;
+        ctx.adopted = false;
+    }
     StagingSlot &slot = ctx.slots[ctx.cursor];
     ctx.cursor = (ctx.cursor + 1) % kSlots;
-    if (slot.pending) {
-        int err = mfrt_event_sync(slot.event);
+    if (ctx.queued != 0 && (slot.state == StagingSlot::kQueued || ctx.queuedStream != stream)) {
+        // one event guards launches of one stream only; and a slot about to be reused needs its guard now
+        const int ret = SealQueued(ctx);
+        if (ret != BM_OK) {
+            return ret;
+        }
+    }
+    if (slot.state == StagingSlot::kGuarded) {
+        StagingSlot *guard = slot.guard;
+        const int err = mfrt_event_sync(guard->event);
         if (err != 0) {
             MF_FAIL(BM_ERROR, "staging slot wait failed: " << mfrt_error_string(err));
         }
-        slot.pending = false;
+        for (auto &other : ctx.slots) {   // everything that event guarded is free now
+            if (other.state == StagingSlot::kGuarded && other.guard == guard) {
+                other.state = StagingSlot::kFree;
+                other.guard = nullptr;
+            }
+        }
     }
     if (slot.capacity < bytes) {
         if (slot.host != nullptr) {
             (void)mfrt_free_host(slot.host);
             slot.host = nullptr;
         }
-        if (slot.dev != nullptr) {
-            (void)mfrt_free_device(slot.dev);
-            slot.dev = nullptr;
-        }
         const uint64_t cap = RoundUp(bytes < 65536 ? 65536 : bytes, 65536);
         slot.host = mfrt_alloc_host(cap);
-        slot.dev = mfrt_alloc_device(cap);
-        if (slot.host == nullptr || slot.dev == nullptr) {
+        if (slot.host == nullptr) {
             slot.capacity = 0;
             MF_FAIL(BM_MALLOC_FAILED, "descriptor staging allocation of " << cap << " bytes failed");
         }
@@ -196,6 +282,26 @@ int AcquireSlot(ThreadLease &ctx, uint64_t bytes, StagingSlot *&out)
         }
     }
     out = &slot;
+    return BM_OK;
+}
+
+// Device half of a slot, for the forms that need the table or the prefix in HBM.
+int EnsureDevice(StagingSlot &slot, uint64_t bytes)
+{
+    if (slot.devCapacity >= bytes) {
+        return BM_OK;
+    }
+    if (slot.dev != nullptr) {
+        (void)mfrt_free_device(slot.dev);
+        slot.dev = nullptr;
+        slot.devCapacity = 0;
+    }
+    const uint64_t cap = RoundUp(bytes < 65536 ? 65536 : bytes, 65536);
+    slot.dev = mfrt_alloc_device(cap);
+    if (slot.dev == nullptr) {
+        MF_FAIL(BM_MALLOC_FAILED, "descriptor staging allocation of " << cap << " bytes in HBM failed");
+    }
+    slot.devCapacity = cap;
     return BM_OK;
 }
 
@@ -639,7 +745,8 @@ int XcopyEngine::Submit(const uint64_t *src, const uint64_t *dst, const uint64_t
     const uint64_t tripleBytes = 24ull * n;
     const uint64_t tableBytes = RoundUp(tripleBytes + 4ull * (n + 1), kUnitBytes);
     StagingSlot *slot = nullptr;
-    int ret = AcquireSlot(ctx.Lease(), tableBytes, slot);
+    ThreadLease &lease = ctx.Lease();
+    int ret = AcquireSlot(lease, tableBytes, stream, slot);
     if (ret != BM_OK) {
         return ret;
     }
@@ -673,6 +780,10 @@ int XcopyEngine::Submit(const uint64_t *src, const uint64_t *dst, const uint64_t
                               grid, mask, maskValue, stream);
         g_launches.fetch_add(1, std::memory_order_relaxed);
     } else {
+        ret = EnsureDevice(*slot, tableBytes);
+        if (ret != BM_OK) {
+            return ret;
+        }
         const uint64_t hostAddr = reinterpret_cast<uint64_t>(slot->host);
         const uint64_t devAddr = reinterpret_cast<uint64_t>(slot->dev);
         InlinePlan stagePlan;
@@ -692,16 +803,10 @@ int XcopyEngine::Submit(const uint64_t *src, const uint64_t *dst, const uint64_t
     }
     if (err != 0) {
         // an earlier launch may still be reading the slot: keep it reserved until the stream has passed this point
-        slot->pending = mfrt_event_record(slot->event, stream) == 0;
+        (void)MarkQueued(lease, slot, stream, true);
         MF_FAIL(BM_ERROR, "xcopy table launch failed: " << mfrt_error_string(err));
     }
-    // Both halves of the slot are free again once the table kernel has run.
-    err = mfrt_event_record(slot->event, stream);
-    if (err != 0) {
-        MF_FAIL(BM_ERROR, "event record failed: " << mfrt_error_string(err));
-    }
-    slot->pending = true;
-    return BM_OK;
+    return MarkQueued(lease, slot, stream, false);
 }
 
 int XcopyEngine::SubmitDeviceTable(const void *triples, uint32_t n, int route, void *stream, void *mask,
@@ -730,7 +835,11 @@ int XcopyEngine::SubmitDeviceTable(const void *triples, uint32_t n, int route, v
     ThreadCtx &ctx = t_ctx;
     StagingSlot *slot = nullptr;
     const uint64_t prefixBytes = RoundUp(4ull * (n + 2), kUnitBytes);
-    int ret = AcquireSlot(ctx.Lease(), prefixBytes, slot);
+    ThreadLease &lease = ctx.Lease();
+    int ret = AcquireSlot(lease, 0, stream, slot);
+    if (ret == BM_OK) {
+        ret = EnsureDevice(*slot, prefixBytes);
+    }
     if (ret != BM_OK) {
         return ret;
     }
@@ -745,15 +854,11 @@ int XcopyEngine::SubmitDeviceTable(const void *triples, uint32_t n, int route, v
     const uint32_t grid = GridFor(static_cast<uint64_t>(cu == 0 ? 256 : cu) * 256, cu, route, tuning_);   // chunk count is only known on the GPU; surplus workgroups leave at once
     err = mfk_xcopy_table(triples, first, nchunkDev, n, 0, units, nullptr, route, grid, mask, maskValue, stream);
     if (err != 0) {
+        (void)MarkQueued(lease, slot, stream, true);   // the plan launch writes the slot
         MF_FAIL(BM_ERROR, "xcopy table launch failed: " << mfrt_error_string(err));
     }
-    err = mfrt_event_record(slot->event, stream);
-    if (err != 0) {
-        MF_FAIL(BM_ERROR, "event record failed: " << mfrt_error_string(err));
-    }
-    slot->pending = true;
     g_launches.fetch_add(2, std::memory_order_relaxed);
-    return BM_OK;
+    return MarkQueued(lease, slot, stream, false);
 }
 
 }  // namespace mf

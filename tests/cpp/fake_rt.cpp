@@ -7,6 +7,7 @@
 #include <cstdint>
 #include <cstdio>
 #include <cstdlib>
+#include <vector>
 #include <cstring>
 #include <map>
 #include <mutex>
@@ -63,6 +64,47 @@ void RunChunk(uint64_t src, uint64_t dst, uint64_t len, uint64_t k, uint32_t uni
     }
     ++g_chunksRun;
 }
+// Descriptor tables stay "in flight" until something the host has waited for covers their launch:
+// an event recorded later, or a stream / device wait.  A table that changed in the meantime was
+// rewritten while a kernel could still read it.
+struct InFlight {
+    uint64_t seq;
+    const void *table;
+    std::vector<uint8_t> snapshot;
+};
+std::mutex g_flightLock;
+std::vector<InFlight> g_inFlight;
+uint64_t g_flightSeq = 0;
+uint64_t g_violations = 0;
+
+void TrackTable(const void *table, size_t bytes)
+{
+    std::lock_guard<std::mutex> guard(g_flightLock);
+    InFlight f{++g_flightSeq, table, {}};
+    f.snapshot.assign(static_cast<const uint8_t *>(table), static_cast<const uint8_t *>(table) + bytes);
+    g_inFlight.push_back(std::move(f));
+}
+
+void Retire(uint64_t upTo)
+{
+    std::lock_guard<std::mutex> guard(g_flightLock);
+    size_t keep = 0;
+    for (size_t i = 0; i < g_inFlight.size(); ++i) {
+        InFlight &f = g_inFlight[i];
+        if (f.seq <= upTo) {
+            if (std::memcmp(f.table, f.snapshot.data(), f.snapshot.size()) != 0) {
+                ++g_violations;
+            }
+        } else {
+            if (keep != i) {
+                g_inFlight[keep] = std::move(f);
+            }
+            ++keep;
+        }
+    }
+    g_inFlight.resize(keep);
+}
+
 }  // namespace
 
 extern "C" {
@@ -96,9 +138,9 @@ int mfrt_device_id(void) { return g_device; }
 uint32_t mfrt_cu_count(void) { return 256; }
 const char *mfrt_error_string(int) { return "fake runtime error"; }
 void *mfrt_alloc_device(uint64_t bytes) { return Track(bytes, MFRT_PTR_DEVICE); }
-int mfrt_free_device(void *p) { Guard("mfrt_free_device"); return Untrack(p); }
+int mfrt_free_device(void *p) { Guard("mfrt_free_device"); Retire(~0ull); return Untrack(p); }   // hipFree waits for the device
 void *mfrt_alloc_host(uint64_t bytes) { return Track(bytes, MFRT_PTR_PINNED_HOST); }
-int mfrt_free_host(void *p) { Guard("mfrt_free_host"); return Untrack(p); }
+int mfrt_free_host(void *p) { Guard("mfrt_free_host"); Retire(~0ull); return Untrack(p); }
 // Address windows: reserved as inaccessible pages, so a touch of an unmapped part ends the test
 // with a fault just as it would fault the GPU; mapping makes the pages usable.
 uint64_t mfrt_window_granularity(void) { return 2u << 20; }
@@ -144,12 +186,24 @@ int mfrt_pointer_kind(const void *p)
 }
 void *mfrt_stream_create(void) { return malloc(8); }
 int mfrt_stream_destroy(void *s) { Guard("mfrt_stream_destroy"); free(s); return 0; }
-int mfrt_stream_sync(void *) { Guard("mfrt_stream_sync"); return 0; }
-int mfrt_device_sync(void) { Guard("mfrt_device_sync"); return 0; }
-void *mfrt_event_create(void) { return malloc(8); }
+uint64_t fake_rt_violations(void) { return g_violations; }
+uint64_t fake_rt_in_flight(void)
+{
+    std::lock_guard<std::mutex> guard(g_flightLock);
+    return g_inFlight.size();
+}
+
+int mfrt_stream_sync(void *) { Guard("mfrt_stream_sync"); Retire(~0ull); return 0; }
+int mfrt_device_sync(void) { Guard("mfrt_device_sync"); Retire(~0ull); return 0; }
+void *mfrt_event_create(void) { return calloc(1, 8); }
 int mfrt_event_destroy(void *e) { Guard("mfrt_event_destroy"); free(e); return 0; }
-int mfrt_event_record(void *, void *) { return 0; }
-int mfrt_event_sync(void *) { return 0; }
+int mfrt_event_record(void *e, void *)
+{
+    std::lock_guard<std::mutex> guard(g_flightLock);
+    *static_cast<uint64_t *>(e) = g_flightSeq;
+    return 0;
+}
+int mfrt_event_sync(void *e) { Retire(*static_cast<uint64_t *>(e)); return 0; }
 int mfrt_event_done(void *) { return 1; }
 float mfrt_event_elapsed_ms(void *, void *) { return 0.0f; }
 int mfrt_memcpy(void *dst, const void *src, uint64_t bytes) { std::memmove(dst, src, bytes); return 0; }
@@ -186,6 +240,7 @@ int mfk_xcopy_table(const void *triples, const void *first, const void *nchunkDe
     const uint32_t total = nchunkDev != nullptr ? *static_cast<const uint32_t *>(nchunkDev) : nchunk;
     ++g_launches;
     uint32_t s = 0;
+    TrackTable(triples, 24ull * nseg);
     mf::ChunkPattern pat{};
     if (pattern != nullptr) {
         pat = *static_cast<const mf::ChunkPattern *>(pattern);

@@ -20,6 +20,8 @@
 
 extern "C" uint64_t fake_rt_launches(void);
 extern "C" void fake_rt_seal(void);
+extern "C" uint64_t fake_rt_violations(void);
+extern "C" uint64_t fake_rt_in_flight(void);
 
 using namespace mf;
 using ock::mf::DataOperatorPtr;
@@ -639,6 +641,71 @@ static void TestHostCopy()
     other.join();
 }
 
+// Descriptor staging slots are recycled behind events that several launches share.  The stand-in
+// runtime keeps every table "in flight" until a wait covers its launch and counts tables that were
+// rewritten before that.
+static void TestSlotRing()
+{
+    CHECK(hybm_init(0, 0) == BM_OK);
+    const size_t pool = 8u << 20;
+    uint8_t *a = static_cast<uint8_t *>(mfrt_alloc_device(pool));
+    uint8_t *b = static_cast<uint8_t *>(mfrt_alloc_device(pool));
+    std::mt19937_64 rng(0x51);
+    for (size_t i = 0; i < pool; ++i) {
+        a[i] = static_cast<uint8_t>(rng());
+    }
+    std::memset(b, 0, pool);
+    std::vector<uint8_t> model(pool, 0);
+    auto batch = [&](uint32_t n, bool pages, void *stream) {
+        std::vector<uint64_t> s(n), d(n), l(n);
+        const uint64_t slot = pool / n / 64 * 64;
+        for (uint32_t i = 0; i < n; ++i) {
+            l[i] = pages ? 4096 : 1 + rng() % (slot - 1);
+            s[i] = reinterpret_cast<uint64_t>(a) + (rng() % n) * slot;
+            d[i] = reinterpret_cast<uint64_t>(b) + static_cast<uint64_t>(i) * slot;
+            std::memcpy(model.data() + static_cast<uint64_t>(i) * slot, reinterpret_cast<const void *>(s[i]), l[i]);
+        }
+        CHECK(mf_xcopy_batch(s.data(), d.data(), l.data(), n, MF_ROUTE_HBM, stream) == BM_OK);
+    };
+    const uint64_t before = fake_rt_violations();
+    for (int i = 0; i < 45; ++i) {   // the ring wraps five times; forms with and without a chunk prefix alternate irregularly
+        batch(200 + static_cast<uint32_t>(rng() % 300), i % 3 == 1, nullptr);
+    }
+    CHECK(fake_rt_in_flight() > 0);      // nothing waited for the last launches yet
+    void *other = mfrt_stream_create();  // a caller's stream: every launch is followed by its own event
+    for (int i = 0; i < 20; ++i) {
+        batch(300, i % 2 == 0, i % 4 < 2 ? other : nullptr);
+    }
+    CHECK(mfrt_stream_sync(mf_xcopy_thread_stream()) == 0);
+    CHECK(mfrt_stream_sync(other) == 0);
+    CHECK(fake_rt_in_flight() == 0);
+    CHECK(fake_rt_violations() == before);
+    CHECK(std::memcmp(b, model.data(), pool) == 0);
+    // a thread that ends with launches queued hands its lease to the next thread
+    std::thread first([&] {
+        mfrt_bind_thread();
+        for (int i = 0; i < 3; ++i) {
+            batch(260, false, nullptr);
+        }
+    });
+    first.join();
+    std::thread second([&] {
+        mfrt_bind_thread();
+        for (int i = 0; i < 12; ++i) {
+            batch(260, i % 2 == 0, nullptr);
+        }
+        CHECK(mfrt_stream_sync(mf_xcopy_thread_stream()) == 0);
+    });
+    second.join();
+    CHECK(mfrt_device_sync() == 0);
+    CHECK(fake_rt_violations() == before);
+    CHECK(std::memcmp(b, model.data(), pool) == 0);
+    mfrt_stream_destroy(other);
+    mfrt_free_device(a);
+    mfrt_free_device(b);
+    hybm_uninit();
+}
+
 int main()
 {
     SetLogLevel(3);
@@ -646,6 +713,7 @@ int main()
     TestCompose();
     TestPlanners();
     TestHostCopy();
+    TestSlotRing();
     TestCApi();                                  // device window: reserved address space, HBM mapped in
     setenv("MF_HIP_GVA_WINDOW", "malloc", 1);
     TestCApi();                                  // device window: one ordinary allocation
