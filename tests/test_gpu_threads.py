@@ -105,3 +105,71 @@ def test_eight_threads_two_generations(lib, oracle):
         prefill.unInitialize()
         pool.destroy()
         bm.uninitialize()
+
+
+def _chain_worker(tid, lib, dev, data, errors):
+    """24 asynchronous table batches in a row, each reading what the one before wrote: page
+    permutations (descriptors read from the staging slot while the kernel runs) take turns with ragged
+    batches (table uploaded first).  The host runs ahead of the GPU, so the staging ring wraps while
+    kernels still read it; a slot rewritten too early would scramble a later batch."""
+    try:
+        assert lib.mfrt_bind_thread() == 0
+        region = 32 * MIB
+        base = dev + tid * 3 * region
+        model = [data[(tid * 3 + r) * region:(tid * 3 + r + 1) * region].copy() for r in range(3)]
+        rng = np.random.default_rng(0x600 + tid)
+        keep = []
+        for step in range(24):
+            s_reg, d_reg = step % 3, (step + 1) % 3
+            if step % 2 == 0:
+                page = 16384
+                pages = region // page
+                order = rng.permutation(pages)
+                src = order.astype(np.uint64) * page
+                dst = np.arange(pages, dtype=np.uint64) * page
+                lens = np.full(pages, page, dtype=np.uint64)
+                model[d_reg] = model[s_reg].reshape(pages, page)[order].reshape(-1).copy()
+            else:
+                count = 1500
+                slot = region // count
+                lens = rng.integers(1, slot, count).astype(np.uint64)
+                src = rng.permutation(count).astype(np.uint64) * slot
+                dst = np.arange(count, dtype=np.uint64) * slot
+                out = model[d_reg].copy()
+                for i in range(count):
+                    out[int(dst[i]):int(dst[i]) + int(lens[i])] = model[s_reg][int(src[i]):int(src[i]) + int(lens[i])]
+                model[d_reg] = out
+            arrays = (native.u64_array((base + s_reg * region + src).tolist()),
+                      native.u64_array((base + d_reg * region + dst).tolist()), native.u64_array(lens.tolist()))
+            keep.append((arrays, len(lens)))
+        for arrays, count in keep:   # all at once: the host finishes queueing long before the GPU is through
+            assert lib.mf_xcopy_batch(arrays[0], arrays[1], arrays[2], count, native.ROUTE_HBM, None) == 0, native.last_error()
+        assert lib.mfrt_stream_sync(lib.mf_xcopy_thread_stream()) == 0
+        got = np.empty(region, dtype=np.uint8)
+        for r in range(3):
+            assert lib.mfrt_memcpy(np_ptr(got), base + r * region, region) == 0
+            assert np.array_equal(got, model[r]), f"thread {tid} region {r}"
+    except BaseException as exc:  # noqa: BLE001
+        errors.append((tid, repr(exc)))
+
+
+def test_table_batches_in_a_row_keep_their_descriptors(lib, oracle):
+    threads_n = 3
+    assert lib.hybm_init(0, 0) == 0, native.last_error()
+    total = threads_n * 3 * 32 * MIB
+    buf = gpu_util.DeviceBuffer(lib, total)
+    try:
+        data = np.empty(total, dtype=np.uint8)
+        oracle.orc_fill_random(np_ptr(data), total, 0x7EAE)
+        buf.upload(data)
+        errors = []
+        threads = [threading.Thread(target=_chain_worker, args=(t, lib, buf.ptr, data, errors)) for t in range(threads_n)]
+        for t in threads:
+            t.start()
+        for t in threads:
+            t.join(timeout=100)
+        assert not any(t.is_alive() for t in threads), "a worker is stuck"
+        assert not errors, errors
+    finally:
+        buf.free()
+        lib.hybm_uninit()
