@@ -696,16 +696,18 @@ int XcopyEngine::Submit(const uint64_t *src, const uint64_t *dst, const uint64_t
     InlinePlan plan;
     bool inlined = false;
     uint32_t units = 0;
+    bool oversized = false;      // a run the 32-bit length of the inline table cannot hold is possible
     if (n <= 4 * kInlineSegs) {  // small enough that a failed attempt costs next to nothing
         uint64_t total = 0;
         for (uint32_t i = 0; i < n; ++i) {
             total += len[i];
         }
+        oversized = total > 0xFFFFFFFFull;
         units = ChooseUnits(total, cu, route, tuning_);
         inlined = BuildInlineDirect(src, dst, len, n, units, plan);
     }
-    if (!inlined && n <= 4 * kInlineSegs) {
-        // merging or a segment of 4 GiB and more made the one-pass attempt give up: the general inline path
+    if (!inlined && oversized) {
+        // a run of 4 GiB and more may have made the one-pass attempt give up: the general inline path cuts it into pieces
         NormalizeSegments(src, dst, len, n, kInlinePiece, ctx.segs);
         units = ChooseUnits(ctx.segs.totalBytes, cu, route, tuning_);
         inlined = BuildInlinePlan(ctx.segs, units, plan);
