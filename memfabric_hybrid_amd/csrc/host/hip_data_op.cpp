@@ -15,6 +15,7 @@ namespace {
 constexpr uint32_t kRounds = 16;                       // slots of the staging ring
 constexpr uint64_t kRoundBytes = 2ull << 20;           // bytes per slot: ~70 us of CPU memcpy against ~40 us on the link
 constexpr uint64_t kBounceBytes = kRounds * kRoundBytes;
+constexpr uint32_t kAhead = 2;                        // launches queued beyond the slot being emptied (device to pageable memory)
 static_assert(kRounds <= XcopyEngine::kBounceEvents, "one event per staging slot");
 
 // Caller memory the GPU cannot address (ordinary pageable host memory) goes through a pinned
@@ -284,8 +285,10 @@ HipDataOp::Result HipDataOp::Run(void *const *src, void *const *dst, const uint6
         if (err != 0) {
             MF_FAIL(BM_ERROR, "event record failed: " << mfrt_error_string(err));
         }
-        if (dstPageable && r > 0) {   // while this launch runs, empty the slot of the one before
-            ret = drain(rounds[(r - 1) % ringSlots], (r - 1) % ringSlots);
+        // Two launches stay queued while an older slot is emptied: with only one, the next launch is
+        // submitted just as the running one ends, and any delay leaves the GPU idle.
+        if (dstPageable && r >= kAhead) {
+            ret = drain(rounds[(r - kAhead) % ringSlots], (r - kAhead) % ringSlots);
             if (ret != BM_OK) {
                 return ret;
             }

@@ -25,32 +25,39 @@ HostCopyHelper &HostCopyHelper::Instance()
     return *helper;
 }
 
-void HostCopyHelper::Loop()
+void HostCopyHelper::Run(const Share &share)
+{
+    for (size_t i = share.begin.piece; i < share.count && i <= share.end.piece; ++i) {
+        const size_t from = i == share.begin.piece ? share.begin.offset : 0;
+        const size_t to = i == share.end.piece ? share.end.offset : share.tasks[i].len;
+        if (to > from) {
+            std::memcpy(static_cast<uint8_t *>(share.tasks[i].dst) + from, static_cast<const uint8_t *>(share.tasks[i].src) + from,
+                        to - from);
+        }
+    }
+}
+
+void HostCopyHelper::Loop(Worker *worker)
 {
     uint64_t seen = 0;
     for (;;) {
         bool posted = false;
         for (int i = 0; i < kSpinRounds; ++i) {
-            if (seq_.load(std::memory_order_acquire) != seen) {
+            if (worker->seq.load(std::memory_order_acquire) != seen) {
                 posted = true;
                 break;
             }
             CpuRelax();
         }
         if (!posted) {
-            std::unique_lock<std::mutex> lock(m_);
-            sleeping_.store(true, std::memory_order_seq_cst);
-            cv_.wait(lock, [&] { return seq_.load(std::memory_order_seq_cst) != seen; });
-            sleeping_.store(false, std::memory_order_seq_cst);
+            std::unique_lock<std::mutex> lock(worker->m);
+            worker->sleeping.store(true, std::memory_order_seq_cst);
+            worker->cv.wait(lock, [&] { return worker->seq.load(std::memory_order_seq_cst) != seen; });
+            worker->sleeping.store(false, std::memory_order_seq_cst);
         }
-        seen = seq_.load(std::memory_order_acquire);   // one task is outstanding at most: the caller waits for it
-        size_t skip = skip_;
-        for (size_t i = first_; i < count_; ++i) {
-            std::memcpy(static_cast<uint8_t *>(tasks_[i].dst) + skip, static_cast<const uint8_t *>(tasks_[i].src) + skip,
-                        tasks_[i].len - skip);
-            skip = 0;
-        }
-        done_.store(seen, std::memory_order_release);
+        seen = worker->seq.load(std::memory_order_acquire);   // one share is outstanding at most: the caller waits for it
+        Run(worker->share);
+        worker->done.store(seen, std::memory_order_release);
     }
 }
 
@@ -70,46 +77,55 @@ void HostCopyHelper::CopySet(const Task *tasks, size_t count)
         return;
     }
     std::lock_guard<std::mutex> owner(owner_, std::adopt_lock);
-    if (!started_ && !unavailable_) {
+    while (started_ < kWorkers && !unavailable_) {
         try {
-            std::thread(&HostCopyHelper::Loop, this).detach();
-            started_ = true;
+            std::thread(&HostCopyHelper::Loop, this, &workers_[started_]).detach();
+            ++started_;
         } catch (...) {
             unavailable_ = true;
         }
     }
-    if (!started_) {
+    if (started_ == 0) {
         alone();
         return;
     }
-    // the cut: piece `cut`, byte `within` (a multiple of 4096 so that both sides stay page-aligned
-    // relative to the piece)
-    const size_t half = total / 2;
-    size_t cut = 0;
-    size_t before = 0;
-    while (cut < count && before + tasks[cut].len <= half) {
-        before += tasks[cut].len;
-        ++cut;
+    // Equal shares by bytes; a cut inside a piece is moved down to a multiple of 4096 so that every
+    // share stays page-aligned relative to the piece.  Share 0 is the caller's.
+    const uint32_t parts = started_ + 1;
+    Cut cuts[kWorkers + 2];
+    cuts[parts] = Cut{count, 0};
+    size_t piece = 0;
+    size_t before = 0;      // bytes of the pieces in front of `piece`
+    for (uint32_t p = 1; p < parts; ++p) {
+        const size_t at = total / parts * p;
+        while (piece < count && before + tasks[piece].len <= at) {
+            before += tasks[piece].len;
+            ++piece;
+        }
+        cuts[p] = piece < count ? Cut{piece, (at - before) & ~static_cast<size_t>(4095)} : Cut{count, 0};
     }
-    const size_t within = (half - before) & ~static_cast<size_t>(4095);   // half < total, so cut < count here
-    tasks_ = tasks;
-    first_ = cut;
-    count_ = count;
-    skip_ = within;
-    const uint64_t ticket = seq_.fetch_add(1, std::memory_order_seq_cst) + 1;
-    if (sleeping_.load(std::memory_order_seq_cst)) {
-        std::lock_guard<std::mutex> lock(m_);
-        cv_.notify_one();
+    Share shares[kWorkers + 1];
+    for (uint32_t p = 0; p < parts; ++p) {
+        shares[p] = Share{tasks, count, cuts[p], cuts[p + 1]};
     }
-    for (size_t i = 0; i < cut; ++i) {
-        std::memcpy(tasks[i].dst, tasks[i].src, tasks[i].len);
+    uint64_t tickets[kWorkers];
+    for (uint32_t w = 0; w < started_; ++w) {
+        Worker &worker = workers_[w];
+        worker.share = shares[w + 1];
+        tickets[w] = worker.seq.fetch_add(1, std::memory_order_seq_cst) + 1;
+        if (worker.sleeping.load(std::memory_order_seq_cst)) {
+            std::lock_guard<std::mutex> lock(worker.m);
+            worker.cv.notify_one();
+        }
     }
-    std::memcpy(tasks[cut].dst, tasks[cut].src, within);
-    for (int spins = 0; done_.load(std::memory_order_acquire) != ticket; ++spins) {
-        if (spins < kSpinRounds) {
-            CpuRelax();
-        } else {
-            std::this_thread::yield();   // the helper has not been scheduled: do not hold the core it may need
+    Run(shares[0]);
+    for (uint32_t w = 0; w < started_; ++w) {
+        for (int spins = 0; workers_[w].done.load(std::memory_order_acquire) != tickets[w]; ++spins) {
+            if (spins < kSpinRounds) {
+                CpuRelax();
+            } else {
+                std::this_thread::yield();   // the helper has not been scheduled: do not hold the core it may need
+            }
         }
     }
     shared_.fetch_add(1, std::memory_order_relaxed);
