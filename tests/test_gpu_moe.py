@@ -85,6 +85,7 @@ def _inputs(oracle, seed, T, H, K, E):
 @pytest.mark.parametrize("T,H,K,E", [
     (1, 8, 1, 1), (7, 64, 2, 4), (300, 64, 4, 16), (1000, 520, 8, 256), (129, 1024, 8, 300),
     (2050, 72, 16, 512), (4096, 2048, 8, 256), (511, 16384, 3, 37),
+    (40000, 64, 8, 300),   # 320 000 entries in 313 rank blocks
     (5000, 8192, 2, 8),    # wide rows in two parts: every wave of the permute takes two or three (token, part) items
 ])
 def test_dispatch_and_combine_match_the_specification(gpu, oracle, T, H, K, E):
