@@ -457,14 +457,13 @@ def extras_paged(lib):
     return res
 
 
+MOE_SHAPE = (8192, 7168, 8, 256)   # tokens, hidden, top-k, experts
+
+
 def extras_moe(lib):
-    from tests import oracle_lib
-    oracle = oracle_lib.oracle()
-    T, H, K, E = 8192, 7168, 8, 256
+    T, H, K, E = MOE_SHAPE
     x, logits = workloads.moe_inputs(0xC4, T, H, E, K)
-    topk = np.zeros((T, K), dtype=np.int32)
-    w = np.zeros((T, K), dtype=np.float32)
-    oracle.orc_moe_route(logits.ctypes.data, T, E, K, topk.ctypes.data, w.ctypes.data)  # input synthesis only
+    topk, w = workloads.moe_route(logits, K)
 
     def dev_of(a):
         p = lib.mfrt_alloc_device(a.nbytes)
@@ -503,6 +502,32 @@ def extras_moe(lib):
     for p in (dx, dt, dw, out, y, counts, offs, row, src, ws):
         lib.mfrt_free_device(p)
     return res
+
+
+def cpu_baseline_moe():
+    """The MoE workload on one host core: the oracle's dispatch (stable counting sort + row copies)
+    and combine (fp32 FMA chain, one rounding to bf16), one pass each at full size."""
+    from tests import oracle_lib
+    oracle = oracle_lib.oracle()
+    T, H, K, E = MOE_SHAPE
+    x, logits = workloads.moe_inputs(0xC4, T, H, E, K)
+    topk, w = workloads.moe_route(logits, K)
+    out = np.zeros((T * K, H), dtype=np.uint16)
+    counts, offsets = np.zeros(E, dtype=np.int32), np.zeros(E, dtype=np.int32)
+    row_of, src_of = np.zeros(T * K, dtype=np.int32), np.zeros(T * K, dtype=np.int32)
+    y = np.zeros((T, H), dtype=np.uint16)
+    t0 = time.perf_counter()
+    ret = oracle.orc_moe_dispatch(x.ctypes.data, topk.ctypes.data, T, H, K, E, out.ctypes.data, counts.ctypes.data,
+                                  offsets.ctypes.data, row_of.ctypes.data, src_of.ctypes.data)
+    t1 = time.perf_counter()
+    assert ret == 0
+    oracle.orc_moe_combine(out.ctypes.data, row_of.ctypes.data, w.ctypes.data, T, H, K, y.ctypes.data)
+    t2 = time.perf_counter()
+    d_bytes = T * H * 2 + T * K * H * 2 + T * K * 4
+    c_bytes = T * K * H * 2 + T * K * 4 + T * K * 4 + T * H * 2
+    return {"cores": 1, "kind": "port", "sample": "one pass each at the full shape",
+            "dispatch": {"ms": round((t1 - t0) * 1e3, 1), "GBps": round(d_bytes / (t1 - t0) / GB, 2)},
+            "combine": {"ms": round((t2 - t1) * 1e3, 1), "GBps": round(c_bytes / (t2 - t1) / GB, 2)}}
 
 
 def extras_reshard(lib):
@@ -624,6 +649,8 @@ def main():
 
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(tables)
+        if not args.no_extras:
+            result["cpu_baseline"]["moe_local"] = cpu_baseline_moe()
 
     bm.uninitialize()
     print(json.dumps(result))

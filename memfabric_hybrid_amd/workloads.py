@@ -120,6 +120,15 @@ def moe_inputs(seed, tokens, hidden, experts, topk):
     return f32_to_bf16_words(x), logits
 
 
+def moe_route(logits, topk):
+    """Top-k experts per token by logit, ties to the lower expert id, and the softmax of the
+    selected logits in fp32 (the routing the MoE workload is specified with)."""
+    order = np.argsort(-logits, axis=1, kind="stable")[:, :topk].astype(np.int32)
+    picked = np.take_along_axis(logits, order, axis=1).astype(np.float32)
+    e = np.exp(picked - picked.max(axis=1, keepdims=True), dtype=np.float32)
+    return np.ascontiguousarray(order), np.ascontiguousarray(e / e.sum(axis=1, keepdims=True, dtype=np.float32))
+
+
 def f32_to_bf16_words(a):
     w = np.ascontiguousarray(a, dtype=np.float32).view(np.uint32)
     bias = np.uint32(0x7FFF) + ((w >> np.uint32(16)) & np.uint32(1))

@@ -351,3 +351,18 @@ def test_fill_random_is_reproducible_and_seed_sensitive(oracle):
     assert int.from_bytes(z.tobytes(), "little") == 0xE220A8397B1DCDAF
     hist = np.bincount(a, minlength=256)
     assert hist.max() < 20
+
+
+def test_numpy_routing_equals_the_oracle_routing(oracle):
+    """bench.py synthesises its MoE inputs with numpy (workloads.moe_route); the oracle's routing,
+    which the parity tests use, must pick the same experts and the same weights."""
+    from memfabric_hybrid_amd import workloads
+    T, H, K, E = 700, 16, 8, 256
+    _, logits = workloads.moe_inputs(0xC4, T, H, E, K)
+    logits[5, 17] = logits[5, 3]          # a tie goes to the lower expert id
+    topk, w = workloads.moe_route(logits, K)
+    topk2 = np.zeros((T, K), dtype=np.int32)
+    w2 = np.zeros((T, K), dtype=np.float32)
+    oracle.orc_moe_route(np_ptr(logits), T, E, K, np_ptr(topk2), np_ptr(w2))
+    assert np.array_equal(topk, topk2)
+    assert np.allclose(w, w2, rtol=0, atol=1e-6)
