@@ -221,7 +221,9 @@ extern "C" int mfrt_window_unmap(void *addr, uint64_t bytes, void *handle)
 extern "C" void *mfrt_alloc_host(uint64_t bytes)
 {
     void *p = nullptr;
-    if (hipHostMalloc(&p, bytes, hipHostMallocMapped | hipHostMallocPortable) != hipSuccess) {
+    // Coherent on purpose, whatever HIP_HOST_COHERENT says: kernels read descriptor tables out of this memory
+    // that the CPU rewrites between launches, and the CPU reads staged data the moment an event has fired.
+    if (hipHostMalloc(&p, bytes, hipHostMallocMapped | hipHostMallocPortable | hipHostMallocCoherent) != hipSuccess) {
         (void)hipGetLastError();
         return nullptr;
     }
