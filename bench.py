@@ -246,11 +246,12 @@ def extras_block(lib, pool, dev, batches, tables, steps):
 
     # ---- yardsticks: what this GPU sustains for flat streaming kernels --------------------------------
     half = POOL_BYTES // 2
+    yard_lib = native.yardstick()
     sink = lib.mfrt_alloc_device(256)
     yard = {}
     for kind, name, factor in ((0, "copy", 2), (1, "fill", 1), (2, "read", 1)):
         dst = sink if kind == 2 else dev + half
-        us, _ = timer.run(lambda k=kind, d=dst: lib.mf_probe_hbm(k, d, dev, 1 << 30, None), 10)
+        us, _ = timer.run(lambda k=kind, d=dst: yard_lib.mf_probe_hbm(k, d, dev, 1 << 30, timer.stream), 10)
         yard[name + "_GBps"] = round(factor * (1 << 30) / us / 1e3, 1)
     lib.mfrt_free_device(sink)
     out["hbm_yardstick_1GiB"] = yard
@@ -596,7 +597,7 @@ def main():
         assert lib.hybm_init(0, 0) == 0, native.last_error()
         a, b = lib.mfrt_alloc_device(1 << 30), lib.mfrt_alloc_device(1 << 30)
         for _ in range(5):
-            assert lib.mf_probe_hbm(0, b, a, 1 << 30, None) == 0
+            assert native.yardstick().mf_probe_hbm(0, b, a, 1 << 30, None) == 0
         assert lib.mfrt_device_sync() == 0
         print(json.dumps({"calibrate": "ProbeCopyKernel", "launches": 5, "bytes_read_per_launch": 1 << 30,
                           "bytes_written_per_launch": 1 << 30}))

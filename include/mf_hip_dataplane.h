@@ -25,8 +25,6 @@ extern "C" {
 #define MF_ROUTE_HBM 0
 #define MF_ROUTE_TO_HOST 1
 #define MF_ROUTE_FROM_HOST 2
-#define MF_ROUTE_HBM_CACHED 3  /* HBM to HBM through the caches, for data that is re-read soon */
-#define MF_ROUTE_HBM_THROUGH 4 /* HBM to HBM, destination written through while the copy runs */
 
 /* Enqueue `n` independent copies dst[i][0..len[i]) = src[i][0..len[i]) as one
  * fused launch on `stream` (NULL: the calling thread's stream).  This is the
@@ -68,6 +66,13 @@ typedef struct {
 } mf_copy2d_desc;
 int32_t mf_xcopy_2d_batch(const mf_copy2d_desc *descs, uint32_t n, int32_t route, void *stream);
 
+/* Host-only views of the 2-D kernel's index arithmetic, for tests.  mf_copy2d_describe: rows one
+ * workgroup takes and the division constant for rows of `width` bytes.  mf_copy2d_rowcol_mismatches:
+ * how many of the units 0 .. unitsInChunk-1 of a chunk the kernel's (row, column) formula places
+ * differently from u / widthUnits, u % widthUnits (0 for every plan the library builds). */
+void mf_copy2d_describe(uint64_t width, uint32_t *rowsPerChunk, uint32_t *magic);
+uint32_t mf_copy2d_rowcol_mismatches(uint32_t widthUnits, uint32_t rowsPerChunk, uint32_t magic, uint32_t unitsInChunk);
+
 /* Launch-shape knobs.  units: 16-byte units per workgroup chunk (0 = choose
  * per batch); wgPerCu: grid cap in workgroups per CU on HBM routes (0 = the
  * default: one workgroup per chunk, no cap); wgPerCuLink: workgroups per CU
@@ -108,12 +113,6 @@ int32_t mf_moe_dispatch(const void *x, const int32_t *topk, uint32_t tokens, uin
  * round-to-nearest-even; entries with rowOf < 0 contribute nothing. */
 int32_t mf_moe_combine(const void *rows, const int32_t *rowOf, const float *weights, uint32_t tokens, uint32_t hidden,
                        uint32_t topK, void *y, void *stream);
-
-/* Yardstick kernels of known traffic (one workgroup per 16 KiB tile, 128-bit, nontemporal): kind 0
- * copies `bytes` from src to dst, kind 1 fills dst, kind 2 reads src (dst: a
- * 4-byte device sink).  They measure what this GPU sustains for a flat copy, a
- * pure write and a pure read, and calibrate hardware byte counters. */
-int32_t mf_probe_hbm(int32_t kind, void *dst, const void *src, uint64_t bytes, void *stream);
 
 /* ---- runtime services (thin layer over HIP) ------------------------------ */
 int mfrt_init(int device);

@@ -10,6 +10,11 @@
  * of the reference tree.  The _Static_assert block at the end pins each value
  * so that an accidental edit fails the build instead of silently breaking a
  * caller compiled against the original headers.
+ *
+ * MF_WITH_REFERENCE_HEADERS: for a build inside the reference tree (its
+ * include directories on the search path).  The reference's own headers then
+ * define every type and this file only adds the pins, so code written against
+ * this header and code written against theirs share one set of definitions.
  */
 #ifndef MF_XCOPY_TYPES_H
 #define MF_XCOPY_TYPES_H
@@ -17,6 +22,23 @@
 #include <stdbool.h>
 #include <stddef.h>
 #include <stdint.h>
+
+#ifdef MF_WITH_REFERENCE_HEADERS
+
+#include "hybm_def.h"
+#include "hybm_data_op.h"
+#include "smem.h"
+#include "smem_bm_def.h"
+#include "smem_trans_def.h"
+#ifdef __cplusplus
+/* the return codes are C++ enumerations of the reference's namespaces */
+#include "hybm_types.h"
+#include "smem_types.h"
+using namespace ock::mf;
+using namespace ock::smem;
+#endif
+
+#else /* definitions of this build */
 
 #ifdef __cplusplus
 extern "C" {
@@ -283,6 +305,8 @@ typedef struct {
 }
 #endif
 
+#endif /* MF_WITH_REFERENCE_HEADERS */
+
 /* ---- contract pins ------------------------------------------------------ */
 #ifdef __cplusplus
 #define MF_PIN(expr) static_assert(expr, #expr)
@@ -307,7 +331,9 @@ MF_PIN(offsetof(hybm_options, maxHBMSize) == 24 && offsetof(hybm_options, scene)
 MF_PIN(offsetof(smem_bm_create_option_t, dataOpType) == 32 && offsetof(smem_bm_create_option_t, tag) == 40);
 MF_PIN(SMEM_TRANS_SENDER == 1 && SMEM_TRANS_RECEIVER == 2 && SMEM_TRANS_BOTH == 3 && SMEM_TRANS_BUTT == 4);
 MF_PIN(sizeof(smem_trans_config_t) == 24 && offsetof(smem_trans_config_t, dataOpType) == 16);
+#if !defined(MF_WITH_REFERENCE_HEADERS) || defined(__cplusplus)
 MF_PIN(BM_NOT_INITIALIZED == -9 && BM_NOT_SUPPORTED == -100 && SM_INVALID_PARAM == -2000 && SM_NOT_INITIALIZED == -2008);
+#endif
 #undef MF_PIN
 
 #endif /* MF_XCOPY_TYPES_H */

@@ -17,19 +17,34 @@ using namespace mf;
 
 namespace {
 
-constexpr uint32_t kChunkBytes = 16384;
-
 bool Aligned16(const mf_copy2d_desc &d)
 {
-    return ((d.src | d.dst | d.width | d.spitch | d.dpitch) & 15u) == 0 && d.width / 16 <= 0xFFFFu &&
-           d.spitch / 16 <= 0xFFFFFFFFull && d.dpitch / 16 <= 0xFFFFFFFFull && d.height <= 0xFFFFFFFFull;
+    return RectFitsPlan(d.src, d.dst, d.width, d.height, d.spitch, d.dpitch);
 }
 
 }  // namespace
 
+MF_EXPORT void mf_copy2d_describe(uint64_t width, uint32_t *rowsPerChunk, uint32_t *magic)
+{
+    *rowsPerChunk = RectRowsPerChunk(width);
+    *magic = RectMagic(static_cast<uint32_t>(width / 16));
+}
+
+MF_EXPORT uint32_t mf_copy2d_rowcol_mismatches(uint32_t widthUnits, uint32_t rowsPerChunk, uint32_t magic, uint32_t unitsInChunk)
+{
+    uint32_t bad = 0;
+    for (uint32_t u = 0; u < unitsInChunk; ++u) {
+        uint32_t row = 0;
+        uint32_t col = 0;
+        RectRowCol(u, widthUnits, rowsPerChunk, magic, row, col);
+        bad += (row != u / widthUnits || col != u % widthUnits) ? 1u : 0u;
+    }
+    return bad;
+}
+
 MF_EXPORT int32_t mf_xcopy_2d_batch(const mf_copy2d_desc *descs, uint32_t n, int32_t route, void *stream)
 {
-    if ((n != 0 && descs == nullptr) || route < 0 || route > MF_ROUTE_HBM_THROUGH) {
+    if ((n != 0 && descs == nullptr) || route < 0 || route > MF_ROUTE_FROM_HOST) {
         MF_FAIL(BM_INVALID_PARAM, "mf_xcopy_2d_batch: null descriptors or unknown route");
     }
     XcopyEngine &engine = XcopyEngine::Instance();
@@ -90,10 +105,7 @@ MF_EXPORT int32_t mf_xcopy_2d_batch(const mf_copy2d_desc *descs, uint32_t n, int
             continue;
         }
         const uint32_t wu = static_cast<uint32_t>(d.width / 16);
-        uint32_t rpc = kChunkBytes / static_cast<uint32_t>(d.width);
-        if (rpc == 0) {
-            rpc = 1;
-        }
+        const uint32_t rpc = RectRowsPerChunk(d.width);
         const uint64_t chunks = (d.height + rpc - 1) / rpc;
         if (run + chunks >= 0xFFFFFFFFull || used == kRectInline) {
             int err = flush();
@@ -108,7 +120,7 @@ MF_EXPORT int32_t mf_xcopy_2d_batch(const mf_copy2d_desc *descs, uint32_t n, int
         plan.widthUnits[used] = wu;
         plan.height[used] = static_cast<uint32_t>(d.height);
         plan.rowsPerChunk[used] = rpc;
-        plan.magic[used] = wu == 1 ? 0u : static_cast<uint32_t>((1ull << 32) / wu) + 1u;
+        plan.magic[used] = RectMagic(wu);
         plan.first[used] = static_cast<uint32_t>(run);
         run += chunks;
         ++used;

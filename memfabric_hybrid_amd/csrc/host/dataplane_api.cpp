@@ -19,7 +19,7 @@ using namespace mf;
 MF_EXPORT int32_t mf_xcopy_batch(const uint64_t *src, const uint64_t *dst, const uint64_t *len, uint32_t n,
                                  int32_t route, void *stream)
 {
-    if ((n != 0 && (src == nullptr || dst == nullptr || len == nullptr)) || route < 0 || route > 21) {
+    if ((n != 0 && (src == nullptr || dst == nullptr || len == nullptr)) || route < 0 || route > MF_ROUTE_FROM_HOST) {
         MF_FAIL(BM_INVALID_PARAM, "mf_xcopy_batch: null array or unknown route " << route);
     }
     return XcopyEngine::Instance().Submit(src, dst, len, n, route, stream, nullptr, 0);
@@ -27,29 +27,10 @@ MF_EXPORT int32_t mf_xcopy_batch(const uint64_t *src, const uint64_t *dst, const
 
 MF_EXPORT int32_t mf_xcopy_device_table(const void *triples, uint32_t n, int32_t route, void *stream)
 {
-    if ((n != 0 && triples == nullptr) || route < 0 || route > MF_ROUTE_HBM_THROUGH) {
+    if ((n != 0 && triples == nullptr) || route < 0 || route > MF_ROUTE_FROM_HOST) {
         MF_FAIL(BM_INVALID_PARAM, "mf_xcopy_device_table: null table or unknown route " << route);
     }
     return XcopyEngine::Instance().SubmitDeviceTable(triples, n, route, stream, nullptr, 0);
-}
-
-MF_EXPORT int32_t mf_probe_hbm(int32_t kind, void *dst, const void *src, uint64_t bytes, void *stream)
-{
-    XcopyEngine &engine = XcopyEngine::Instance();
-    if (!engine.Started()) {
-        MF_FAIL(BM_NOT_INITIALIZED, "GPU data plane is not running; call hybm_init first");
-    }
-    if (kind < 0 || kind > 2 || dst == nullptr || (kind != 1 && src == nullptr) || bytes == 0 || bytes % 16 != 0) {
-        MF_FAIL(BM_INVALID_PARAM, "mf_probe_hbm: bad kind, null buffer or size not a multiple of 16");
-    }
-    if (stream == nullptr) {
-        stream = engine.ThreadStream();
-    }
-    int err = mfk_probe(kind, dst, src, bytes, 0, stream);   // one workgroup per 16 KiB tile
-    if (err != 0) {
-        MF_FAIL(BM_ERROR, "probe launch failed");
-    }
-    return BM_OK;
 }
 
 MF_EXPORT int32_t mf_bm_copy_batch_replay(smem_bm_t handle, smem_batch_copy_params *const *batches, uint32_t count,

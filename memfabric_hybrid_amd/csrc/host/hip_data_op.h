@@ -5,7 +5,13 @@
 #ifndef MF_HIP_DATA_OP_H
 #define MF_HIP_DATA_OP_H
 
+#include <atomic>
+
+#ifdef MF_WITH_REFERENCE_HEADERS
+#include "hybm_data_operator.h"   // the reference's own contract, from its include path
+#else
 #include "data_operator.h"
+#endif
 
 namespace mf {
 
@@ -28,7 +34,7 @@ public:
 private:
     Result Run(void *const *src, void *const *dst, const uint64_t *len, uint32_t n, hybm_data_copy_direction direction,
                const ExtOptions &options, bool async) noexcept;
-    bool inited_ = false;
+    std::atomic<bool> inited_{false};   // operators are shared by all calling threads
 };
 
 }  // namespace mf

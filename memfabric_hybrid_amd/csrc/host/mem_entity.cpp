@@ -254,7 +254,7 @@ LocalSlice *MemEntity::AllocLocal(hybm_mem_type t, uint64_t size)
     }
     const GvaWindow &w = device ? device_ : host_;
     std::unique_ptr<LocalSlice> &slot = device ? deviceSlice_ : hostSlice_;
-    const uint64_t backed = device ? deviceBacked_ : hostBacked_;
+    const uint64_t backed = device ? deviceBacked_.load(std::memory_order_acquire) : hostBacked_.load(std::memory_order_acquire);
     if (w.base == 0 || slot != nullptr || size > backed) {
         MF_ERROR("local allocation of " << size << " bytes does not fit the reserved window of " << backed);
         return nullptr;
@@ -270,19 +270,21 @@ LocalSlice *MemEntity::AllocLocal(hybm_mem_type t, uint64_t size)
 LocalSlice *MemEntity::AllocMapped(uint64_t size)
 {
     const uint64_t granule = mfrt_window_granularity();
-    if (granule == 0 || size % granule != 0 || size > options_.maxHBMSize - deviceBacked_) {
+    std::lock_guard<std::mutex> guard(sliceLock_);   // the backed prefix grows under the lock: two allocations must not pick the same offset
+    const uint64_t backed = deviceBacked_.load(std::memory_order_acquire);
+    if (granule == 0 || size % granule != 0 || size > options_.maxHBMSize - backed) {
         MF_ERROR("local allocation of " << size << " bytes: not a multiple of " << granule << " or more than the "
-                 << options_.maxHBMSize - deviceBacked_ << " bytes left in this rank's window");
+                 << options_.maxHBMSize - backed << " bytes left in this rank's window");
         return nullptr;
     }
     if (mfrt_bind_thread() != 0) {
         return nullptr;
     }
-    const uint64_t va = device_.PtrOfRank(options_.rankId) + deviceBacked_;
+    const uint64_t va = device_.PtrOfRank(options_.rankId) + backed;
     void *mapping = mfrt_window_map(reinterpret_cast<void *>(va), size,
-                                    reinterpret_cast<void *>(device_.PtrOfRank(options_.rankId)), deviceBacked_ + size);
+                                    reinterpret_cast<void *>(device_.PtrOfRank(options_.rankId)), backed + size);
     if (mapping == nullptr) {
-        MF_ERROR("HBM of " << size << " bytes could not be mapped into the window at offset " << deviceBacked_
+        MF_ERROR("HBM of " << size << " bytes could not be mapped into the window at offset " << backed
                  << " (step and code " << mfrt_window_last_error() << ")");
         return nullptr;
     }
@@ -290,10 +292,9 @@ LocalSlice *MemEntity::AllocMapped(uint64_t size)
         (void)mfrt_window_unmap(reinterpret_cast<void *>(va), size, mapping);
         return nullptr;
     }
-    std::lock_guard<std::mutex> guard(sliceLock_);
     mappedSlices_.emplace_back(new LocalSlice{HYBM_MEM_TYPE_DEVICE, va, size});
     mappedSlices_.back()->mapping = mapping;
-    deviceBacked_ += size;
+    deviceBacked_.store(backed + size, std::memory_order_release);   // published once the mapping exists
     return mappedSlices_.back().get();
 }
 
@@ -312,19 +313,25 @@ int MemEntity::FreeMapped(LocalSlice *slice)
     }
     // The backed bytes of a rank are one prefix of its window: memory goes back to the GPU from
     // the top, once the slice and everything mapped after it have been released.
-    bool drained = false;
+    uint64_t going = 0;
+    for (auto it = mappedSlices_.rbegin(); it != mappedSlices_.rend() && (*it)->released; ++it) {
+        going += (*it)->size;
+    }
+    if (going == 0) {
+        return BM_OK;
+    }
+    // First the bound comes down, so that no new copy passes the range check for these bytes; then
+    // the copies already queued drain; only then the memory goes.  (A copy into a slice that is
+    // being freed is a caller error all the same: it may now fail its range check.)
+    deviceBacked_.store(deviceBacked_.load(std::memory_order_acquire) - going, std::memory_order_release);
+    if (dataOperator_ != nullptr) {
+        dataOperator_->CleanUp();
+    }
+    (void)mfrt_device_sync();
     while (!mappedSlices_.empty() && mappedSlices_.back()->released) {
-        if (!drained) {
-            if (dataOperator_ != nullptr) {
-                dataOperator_->CleanUp();
-            }
-            (void)mfrt_device_sync();
-            drained = true;
-        }
         LocalSlice &top = *mappedSlices_.back();
         VaManager::Global().Remove(top.va);
         (void)mfrt_window_unmap(reinterpret_cast<void *>(top.va), top.size, top.mapping);
-        deviceBacked_ -= top.size;
         mappedSlices_.pop_back();
     }
     return BM_OK;
@@ -473,11 +480,14 @@ bool MemEntity::CheckAddressInEntity(const void *ptr, uint64_t length) const
     // Window test as in the reference, narrowed to the bytes that are real
     // memory: an address in the unbacked remainder of a window would fault
     // the GPU instead of failing a remote transfer.
+    if (a + length < a) {
+        return false;   // wraps round the address space
+    }
     if (device_.Contains(a, length)) {
-        return a + length <= device_.base + deviceBacked_ || options_.rankCount > 1;
+        return a + length <= device_.base + deviceBacked_.load(std::memory_order_acquire) || options_.rankCount > 1;
     }
     if (host_.Contains(a, length)) {
-        return a + length <= host_.base + hostBacked_ || options_.rankCount > 1;
+        return a + length <= host_.base + hostBacked_.load(std::memory_order_acquire) || options_.rankCount > 1;
     }
     return rangeCount_.load(std::memory_order_acquire) != 0 && InRanges(a, length);
 }
@@ -495,9 +505,11 @@ uint32_t MemEntity::FirstOutside(void *const *ptrs, const uint64_t *lengths, uin
     // One rank: an address is inside when it lies in the backed part of one of the two windows
     // (or in a registered range).  The bounds stay in registers for the whole batch.
     const uint64_t devLo = device_.base;
-    const uint64_t devHi = device_.base == 0 ? 0 : device_.base + (deviceBacked_ < device_.Span() ? deviceBacked_ : device_.Span());
+    const uint64_t devBacked = deviceBacked_.load(std::memory_order_acquire);
+    const uint64_t hostBacked = hostBacked_.load(std::memory_order_acquire);
+    const uint64_t devHi = device_.base == 0 ? 0 : device_.base + (devBacked < device_.Span() ? devBacked : device_.Span());
     const uint64_t hostLo = host_.base;
-    const uint64_t hostHi = host_.base == 0 ? 0 : host_.base + (hostBacked_ < host_.Span() ? hostBacked_ : host_.Span());
+    const uint64_t hostHi = host_.base == 0 ? 0 : host_.base + (hostBacked < host_.Span() ? hostBacked : host_.Span());
     const bool haveRanges = rangeCount_.load(std::memory_order_acquire) != 0;
     for (uint32_t i = 0; i < n; ++i) {
         const uint64_t a = reinterpret_cast<uint64_t>(ptrs[i]);

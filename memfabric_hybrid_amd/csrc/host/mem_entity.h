@@ -86,8 +86,12 @@ private:
     bool reserved_ = false;
     GvaWindow device_;          // stride = maxHBMSize
     GvaWindow host_;            // stride = maxDRAMSize
-    uint64_t deviceBacked_ = 0; // bytes of the local device window that are real memory
-    uint64_t hostBacked_ = 0;
+    // Bytes of the local windows that are real memory.  Written under sliceLock_ (or during
+    // Initialize / UnInitialize), read without a lock by the range check of every copy: a map is
+    // published with a release store after it exists, an unmap lowers the bound before it waits
+    // for the GPU, so no new copy is admitted into memory that is about to go away.
+    std::atomic<uint64_t> deviceBacked_{0};
+    std::atomic<uint64_t> hostBacked_{0};
     std::unique_ptr<LocalSlice> deviceSlice_;
     // Mapped-window mode (the default; MF_HIP_GVA_WINDOW=malloc turns it off): the device window is reserved address space of
     // rankCount * maxHBMSize bytes, and every local allocation maps fresh HBM at the end of the

@@ -311,7 +311,7 @@ uint32_t GridFor(uint64_t nchunk, uint32_t cuCount, int route, const XcopyTuning
     // letting the hardware dispatcher hand out the chunks one by one sustains 6.0-6.2 TB/s, a
     // grid capped at 16 workgroups per CU that strides over the chunks 5.3-5.7 TB/s (its static
     // assignment leaves a tail).  Link routes: one workgroup per CU, more only adds contention.
-    const bool link = route == MFRT_ROUTE_TO_HOST || route == MFRT_ROUTE_FROM_HOST || route >= 16;
+    const bool link = route == MFRT_ROUTE_TO_HOST || route == MFRT_ROUTE_FROM_HOST;
     const uint32_t perCu = link ? (tuning.wgPerCuLink == 0 ? 1 : tuning.wgPerCuLink) : tuning.wgPerCu;
     const uint64_t limit = (1ull << 24) - 1;   // grid size in lanes must stay below 2^32 with up to 256 lanes per workgroup
     uint64_t cap = perCu == 0 ? limit : static_cast<uint64_t>(cuCount == 0 ? 256 : cuCount) * perCu;
@@ -589,29 +589,26 @@ int XcopyEngine::Start(int device)
     if (err != 0) {
         MF_FAIL(BM_ERROR, "GPU runtime start on device " << device << " failed: " << mfrt_error_string(err));
     }
-    if (started_) {
-        return BM_OK;
-    }
-    started_ = true;
+    started_.store(true, std::memory_order_release);
     return BM_OK;
 }
 
 void XcopyEngine::Stop()
 {
-    if (!started_) {
+    if (!started_.load(std::memory_order_acquire)) {
         return;
     }
     (void)mfrt_bind_thread();
     (void)mfrt_device_sync();
     Leases().DestroyAll();   // every thread's stream and staging memory, not only the caller's
     g_leaseEpoch.store(Leases().Epoch(), std::memory_order_release);
-    started_ = false;
+    started_.store(false, std::memory_order_release);
     mfrt_shutdown();
 }
 
 bool XcopyEngine::Started() const
 {
-    return started_;
+    return started_.load(std::memory_order_acquire);
 }
 
 void *XcopyEngine::ThreadStream()
@@ -658,7 +655,7 @@ void *XcopyEngine::ThreadBounceEvent(uint32_t index)
 
 int XcopyEngine::DrainThread()
 {
-    if (!started_) {
+    if (!Started()) {
         return BM_NOT_INITIALIZED;
     }
     if (!t_ctx.HasLiveLease() || t_ctx.lease->stream == nullptr) {
@@ -679,7 +676,7 @@ uint64_t XcopyEngine::LaunchCount() const
 int XcopyEngine::Submit(const uint64_t *src, const uint64_t *dst, const uint64_t *len, uint32_t n, int route,
                         void *stream, void *mask, uint32_t maskValue)
 {
-    if (!started_) {
+    if (!Started()) {
         MF_FAIL(BM_NOT_INITIALIZED, "xcopy engine not started");
     }
     if (mfrt_bind_thread() != 0) {
@@ -814,7 +811,7 @@ int XcopyEngine::Submit(const uint64_t *src, const uint64_t *dst, const uint64_t
 int XcopyEngine::SubmitDeviceTable(const void *triples, uint32_t n, int route, void *stream, void *mask,
                                    uint32_t maskValue)
 {
-    if (!started_) {
+    if (!Started()) {
         MF_FAIL(BM_NOT_INITIALIZED, "xcopy engine not started");
     }
     if (mfrt_bind_thread() != 0) {

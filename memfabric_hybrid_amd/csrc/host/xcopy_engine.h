@@ -8,6 +8,7 @@
 
 #include <stdint.h>
 
+#include <atomic>
 #include <vector>
 
 #include "../kernels/xcopy_plan.h"
@@ -107,7 +108,7 @@ private:
     XcopyEngine() = default;
 
     XcopyTuning tuning_;
-    bool started_ = false;
+    std::atomic<bool> started_{false};   // read by every calling thread, flipped by Start / Stop
 };
 
 }  // namespace mf

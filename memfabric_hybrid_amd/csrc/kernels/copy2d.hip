@@ -59,8 +59,7 @@ __global__ __launch_bounds__(kRectThreads) void Copy2dKernel(const RectPlan p)
 #pragma unroll
             for (uint32_t j = 0; j < 4; ++j) {
                 const uint32_t u = u0 + j * kRectThreads + threadIdx.x;
-                row[j] = rwu == 1 ? u : __umulhi(u, rmg);
-                col[j] = u - row[j] * rwu;
+                RectRowCol(u, rwu, rrpc, rmg, row[j], col[j]);
                 if (u < units) {
                     v[j] = __builtin_nontemporal_load(s + static_cast<uint64_t>(row[j]) * rsp + col[j]);
                 }

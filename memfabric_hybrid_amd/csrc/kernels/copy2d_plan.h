@@ -22,10 +22,55 @@ struct RectPlan {
     uint32_t widthUnits[kRectInline];
     uint32_t height[kRectInline];
     uint32_t rowsPerChunk[kRectInline];
-    uint32_t magic[kRectInline];          // floor(2^32 / widthUnits) + 1: row = (u * magic) >> 32
+    uint32_t magic[kRectInline];          // floor(2^32 / widthUnits) + 1, see RectRowCol; unused when rowsPerChunk == 1
     uint32_t first[kRectInline];          // exclusive prefix of chunk counts, 0xFFFFFFFF past the end
     uint32_t nchunk;
 };
+
+#if defined(__HIPCC__)
+#define MF_RECT_HD __host__ __device__
+#else
+#define MF_RECT_HD
+#endif
+
+constexpr uint32_t kRectChunkBytes = 16384;   // a workgroup's share: this many bytes of whole rows, or one wider row
+
+// Rows one workgroup takes for rows of `width` bytes (a multiple of 16).
+MF_RECT_HD inline uint32_t RectRowsPerChunk(uint64_t width)
+{
+    const uint64_t rows = width == 0 ? 1 : kRectChunkBytes / width;
+    return rows == 0 ? 1u : static_cast<uint32_t>(rows);
+}
+
+MF_RECT_HD inline uint32_t RectMagic(uint32_t widthUnits)
+{
+    return widthUnits <= 1 ? 0u : static_cast<uint32_t>((1ull << 32) / widthUnits) + 1u;
+}
+
+// Row (relative to the chunk's first row) and column, in 16-byte units, of unit u of a chunk.
+// A chunk that holds a single row needs no division, whatever the width; a chunk of several rows
+// has rows of at most kRectChunkBytes / 2 bytes, so u < 1024 and widthUnits <= 512, where the
+// multiply-high by floor(2^32 / widthUnits) + 1 is exact (it is for all u, widthUnits < 65536).
+MF_RECT_HD inline void RectRowCol(uint32_t u, uint32_t widthUnits, uint32_t rowsPerChunk, uint32_t magic, uint32_t &row,
+                                  uint32_t &col)
+{
+    if (rowsPerChunk == 1) {
+        row = 0;
+        col = u;
+        return;
+    }
+    row = widthUnits == 1 ? u : static_cast<uint32_t>((static_cast<uint64_t>(u) * magic) >> 32);
+    col = u - row * widthUnits;
+}
+
+// Whether a rectangle can take the 2-D kernel: everything a multiple of 16 and, in 16-byte units
+// (rows: in rows), within the 32-bit fields of the plan.
+MF_RECT_HD inline bool RectFitsPlan(uint64_t src, uint64_t dst, uint64_t width, uint64_t height, uint64_t spitch,
+                                    uint64_t dpitch)
+{
+    return ((src | dst | width | spitch | dpitch) & 15u) == 0 && width / 16 <= 0xFFFFFFFFull &&
+           spitch / 16 <= 0xFFFFFFFFull && dpitch / 16 <= 0xFFFFFFFFull && height <= 0xFFFFFFFFull;
+}
 
 }  // namespace mf
 

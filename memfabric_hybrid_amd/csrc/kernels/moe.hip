@@ -405,12 +405,17 @@ __global__ __launch_bounds__(kThreads) void MoeCombineKernel(const u32x4 *__rest
     constexpr uint32_t kSlots = kTopK != 0 ? kTopK : kMaxTopK;
     uint64_t rowBase[kSlots];
     float w[kSlots];
+    // Slots without a row (an expert id that dispatch flagged) are skipped: neither loaded nor
+    // multiplied, so whatever lies in row 0 (an infinity, a NaN) cannot reach y through 0 * x.
+    // The mask is the same for every lane of the workgroup.
+    uint32_t live = 0;
 #pragma unroll
     for (uint32_t k = 0; k < kSlots; ++k) {
         if (k < nk) {
             const int32_t row = rowOf[static_cast<uint64_t>(token) * nk + k];
             rowBase[k] = static_cast<uint64_t>(row < 0 ? 0 : row) * unitsPerRow;
-            w[k] = row < 0 ? 0.0f : weights[static_cast<uint64_t>(token) * nk + k];
+            w[k] = weights[static_cast<uint64_t>(token) * nk + k];
+            live |= row < 0 ? 0u : 1u << k;
         } else {
             rowBase[k] = 0;
             w[k] = 0.0f;
@@ -428,7 +433,7 @@ __global__ __launch_bounds__(kThreads) void MoeCombineKernel(const u32x4 *__rest
             const uint32_t u = u0 + b * kThreads;
 #pragma unroll
             for (uint32_t k = 0; k < kSlots; ++k) {
-                if (k < nk && u < end) {
+                if (((live >> k) & 1u) != 0 && u < end) {
                     v[b][k] = kNtLoad ? __builtin_nontemporal_load(in + rowBase[k] + u) : in[rowBase[k] + u];
                 }
             }
@@ -446,7 +451,7 @@ __global__ __launch_bounds__(kThreads) void MoeCombineKernel(const u32x4 *__rest
             }
 #pragma unroll
             for (uint32_t k = 0; k < kSlots; ++k) {
-                if (k < nk) {
+                if (((live >> k) & 1u) != 0) {
 #pragma unroll
                     for (uint32_t i = 0; i < 4; ++i) {
                         acc[2 * i] = __builtin_fmaf(w[k], Bf16Lo(v[b][k][i]), acc[2 * i]);
@@ -466,14 +471,6 @@ __global__ __launch_bounds__(kThreads) void MoeCombineKernel(const u32x4 *__rest
 
 }  // namespace
 }  // namespace mf
-
-static int g_permuteVariant = -1;  // -1: choose from the row width
-static int g_combineVariant = -1;  // -1: choose from the row width
-extern "C" void mfk_moe_tune(int permuteVariant, int combineVariant)
-{
-    g_permuteVariant = permuteVariant;
-    g_combineVariant = combineVariant;
-}
 
 extern "C" uint64_t mfk_moe_workspace_bytes(uint32_t tokens, uint32_t topK, uint32_t experts)
 {
@@ -515,7 +512,7 @@ extern "C" int mfk_moe_dispatch(const void *x, const void *topk, uint32_t tokens
         // Wide rows: single-wave workgroups that hold up to 14 pieces per lane (a whole 7168-element
         // row) and write them with plain stores.  Storing alone takes 177 us of the 200 us such a
         // kernel needs when every wave reads its row first; with sixteen waves per CU that each
-        // take several tokens and fetch the next row while they store the current one (variant 12)
+        // take several tokens and fetch the next row while they store the current one
         // the dispatch takes 207 us instead of 215.  Other shapes measured on these rows: two waves
         // per row 221 us; four-wave workgroups with nontemporal stores 237 us; the row staged in LDS
         // instead of registers 221 us (one wave) and 227 us (four waves); buffer-addressed
@@ -523,37 +520,15 @@ extern "C" int mfk_moe_dispatch(const void *x, const void *topk, uint32_t tokens
         // row reading x[srcOf[row]], 271 us: its eight reads of every token row are not absorbed by
         // the caches.
         // Narrow rows: one four-wave workgroup per token.
-        const int variant = g_permuteVariant >= 0 ? g_permuteVariant : (upr >= 512 ? 12 : 0);
-        const uint32_t wideParts = (upr + 64 * 14 - 1) / (64 * 14);
-        switch (variant) {
-            case 1:
-                hipLaunchKernelGGL((MoePermuteKernel<64, 14, 1>), dim3(tokens * wideParts), dim3(64), 0, s, xi, ro, topK, upr,
-                                   wideParts, oo);
-                break;
-            case 6: {
-                const uint32_t parts = (upr + 64 * 7 - 1) / (64 * 7);
-                hipLaunchKernelGGL((MoePermuteKernel<64, 7, 0>), dim3(tokens * parts), dim3(64), 0, s, xi, ro, topK, upr, parts, oo);
-                break;
-            }
-            case 7:
-                hipLaunchKernelGGL((MoePermuteKernel<128, 7, 0>), dim3(tokens * wideParts), dim3(128), 0, s, xi, ro, topK, upr,
-                                   wideParts, oo);
-                break;
-            case 10:
-                hipLaunchKernelGGL((MoePermuteKernel<64, 14, 0>), dim3(tokens * wideParts), dim3(64), 0, s, xi, ro, topK, upr,
-                                   wideParts, oo);
-                break;
-            case 12: {
-                // 123 vector registers per lane: four waves per SIMD, sixteen per CU, all resident at once
-                const uint32_t items = tokens * wideParts;
-                const uint32_t waves = static_cast<uint32_t>(mfrt_cu_count() > 0 ? mfrt_cu_count() : 256) * 16u;
-                hipLaunchKernelGGL((MoePermuteLoopKernel<14>), dim3(items < waves ? items : waves), dim3(64), 0, s, xi, ro, topK, upr,
-                                   wideParts, items, oo);
-                break;
-            }
-            default:
-                hipLaunchKernelGGL((MoePermuteKernel<256, 4, 1>), dim3(tokens), dim3(256), 0, s, xi, ro, topK, upr, 1u, oo);
-                break;
+        if (upr >= 512) {
+            // 123 vector registers per lane: four waves per SIMD, sixteen per CU, all resident at once
+            const uint32_t wideParts = (upr + 64 * 14 - 1) / (64 * 14);
+            const uint32_t items = tokens * wideParts;
+            const uint32_t waves = static_cast<uint32_t>(mfrt_cu_count() > 0 ? mfrt_cu_count() : 256) * 16u;
+            hipLaunchKernelGGL((MoePermuteLoopKernel<14>), dim3(items < waves ? items : waves), dim3(64), 0, s, xi, ro, topK, upr,
+                               wideParts, items, oo);
+        } else {
+            hipLaunchKernelGGL((MoePermuteKernel<256, 4, 1>), dim3(tokens), dim3(256), 0, s, xi, ro, topK, upr, 1u, oo);
         }
     }
     return static_cast<int>(hipGetLastError());
@@ -576,31 +551,12 @@ extern "C" int mfk_moe_combine(const void *rows, const void *rowOf, const void *
         // Wide rows: single-wave workgroups, each on a 128-unit slice of the row with two column
         // positions per lane in flight (16 loads), the fastest shape measured on 7168-element rows
         // (178 us; one four-wave workgroup per token 188 us; plain instead of nontemporal loads 194 us).
-        const int variant = g_combineVariant >= 0 ? g_combineVariant : (upr >= 256 ? 11 : 0);
-        switch (variant) {
-            case 3: {
-                const uint32_t parts = (upr + 447) / 448;
-                hipLaunchKernelGGL((MoeCombineKernel<8, 64, true>), dim3(tokens * parts), dim3(64), 0, s, in, ro, w, topK, upr, parts, o);
-                break;
-            }
-            case 4:
-                hipLaunchKernelGGL((MoeCombineKernel<8, 256, false>), dim3(tokens), dim3(256), 0, s, in, ro, w, topK, upr, 1u, o);
-                break;
-            case 11: {
-                const uint32_t parts = (upr + 127) / 128;
-                hipLaunchKernelGGL((MoeCombineKernel<8, 64, true, 2>), dim3(tokens * parts), dim3(64), 0, s, in, ro, w, topK, upr,
-                                   parts, o);
-                break;
-            }
-            case 13: {
-                const uint32_t parts = (upr + 63) / 64;
-                hipLaunchKernelGGL((MoeCombineKernel<8, 64, true, 1>), dim3(tokens * parts), dim3(64), 0, s, in, ro, w, topK, upr,
-                                   parts, o);
-                break;
-            }
-            default:
-                hipLaunchKernelGGL((MoeCombineKernel<8, 256, true>), dim3(tokens), dim3(256), 0, s, in, ro, w, topK, upr, 1u, o);
-                break;
+        if (upr >= 256) {
+            const uint32_t parts = (upr + 127) / 128;
+            hipLaunchKernelGGL((MoeCombineKernel<8, 64, true, 2>), dim3(tokens * parts), dim3(64), 0, s, in, ro, w, topK, upr,
+                               parts, o);
+        } else {
+            hipLaunchKernelGGL((MoeCombineKernel<8, 256, true>), dim3(tokens), dim3(256), 0, s, in, ro, w, topK, upr, 1u, o);
         }
     } else {
         hipLaunchKernelGGL((MoeCombineKernel<0, 256, true>), dim3(tokens), dim3(256), 0, s, in, ro, w, topK, upr, 1u, o);

@@ -108,21 +108,19 @@ __global__ __launch_bounds__(kThreads) void ProbeReadKernel(const u32x4 *__restr
 }  // namespace
 }  // namespace mf
 
-// kind: 0 copy (bytes read + bytes written), 1 fill (bytes written), 2 read (bytes read; dst = 4-byte sink).
-// grid: workgroups to launch, 0 = one per 16 KiB tile.
-extern "C" int mfk_probe(int kind, void *dst, const void *src, uint64_t bytes, uint32_t grid, void *stream)
+// Declared in include/mf_hip_yardstick.h.  Enqueues only; the caller owns the stream.
+extern "C" __attribute__((visibility("default"))) int32_t mf_probe_hbm(int32_t kind, void *dst, const void *src,
+                                                                         uint64_t bytes, void *stream)
 {
     using namespace mf;
-    if (bytes % 16 != 0 || bytes == 0) {
-        return -1;
+    if (kind < 0 || kind > 2 || dst == nullptr || (kind != 1 && src == nullptr) || bytes % 16 != 0 || bytes == 0) {
+        return -2;
     }
     hipStream_t s = static_cast<hipStream_t>(stream);
     const uint64_t units = bytes / 16;
     const uint64_t tiles = (units + kTile - 1) / kTile;
     const uint64_t most = (1ull << 24) - 1;   // the grid size in lanes must stay below 2^32; the kernels loop over what is left
-    if (grid == 0 || grid > tiles) {
-        grid = static_cast<uint32_t>(tiles < most ? tiles : most);
-    }
+    const uint32_t grid = static_cast<uint32_t>(tiles < most ? tiles : most);   // one workgroup per 16 KiB tile
     const uint32_t span = kXcdSpan;
     switch (kind) {
         case 0:
@@ -132,12 +130,10 @@ extern "C" int mfk_probe(int kind, void *dst, const void *src, uint64_t bytes, u
         case 1:
             hipLaunchKernelGGL(ProbeFillKernel, dim3(grid), dim3(kThreads), 0, s, static_cast<u32x4 *>(dst), units, 0x5Au, span);
             break;
-        case 2:
+        default:
             hipLaunchKernelGGL(ProbeReadKernel, dim3(grid), dim3(kThreads), 0, s, static_cast<const u32x4 *>(src), units,
                                static_cast<uint32_t *>(dst), span);
             break;
-        default:
-            return -1;
     }
-    return static_cast<int>(hipGetLastError());
+    return hipGetLastError() == hipSuccess ? 0 : -1;
 }

@@ -294,9 +294,6 @@ __global__ __launch_bounds__(kPlanThreads) void XcopyPlanKernel(const uint64_t *
 
 Policy PolicyOf(int route)
 {
-    if (route >= 16) {  // explicit policy for experiments: 16 + ntLoad + 2 * store mode
-        return Policy{((route - 16) & 1) != 0, ((route - 16) >> 1) % 3};
-    }
     switch (route) {
         case MFRT_ROUTE_TO_HOST:
             // measured over the host link with 122-segment batches: write-through 56.0 GB/s,
@@ -304,11 +301,9 @@ Policy PolicyOf(int route)
             return Policy{false, kStoreThrough};
         case MFRT_ROUTE_FROM_HOST:
             return Policy{true, kStorePlain};
-        case MFRT_ROUTE_HBM_CACHED:
-            return Policy{false, kStorePlain};
-        case MFRT_ROUTE_HBM_THROUGH:
-            return Policy{true, kStoreThrough};
         default:
+            // HBM to HBM, measured on the 9 MB batch: streaming loads and stores 5.2 us, plain 6.3 us,
+            // stores written through 6.5 us (they are 4 % faster on a 1 GiB copy only)
             return Policy{true, kStoreStream};
     }
 }

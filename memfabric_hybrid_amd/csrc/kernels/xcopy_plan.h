@@ -29,7 +29,7 @@ constexpr uint32_t kUnitBytes = 16;           // one 128-bit access
 constexpr uint32_t kInlineSegs = 128;         // segments that fit in the kernel-argument block: 2 table rows per lane of a wave64
 constexpr uint32_t kNoChunk = 0xFFFFFFFFu;    // sentinel prefix for unused slots
 
-#if defined(__HIPCC__) || defined(__CUDACC__)
+#if defined(__HIPCC__)
 #define MF_HD __host__ __device__
 #else
 #define MF_HD

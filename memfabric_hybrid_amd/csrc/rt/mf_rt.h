@@ -20,8 +20,6 @@ extern "C" {
 #define MFRT_ROUTE_HBM 0        /* source and destination in HBM            */
 #define MFRT_ROUTE_TO_HOST 1    /* destination in pinned, mapped host DRAM  */
 #define MFRT_ROUTE_FROM_HOST 2  /* source in pinned, mapped host DRAM       */
-#define MFRT_ROUTE_HBM_CACHED 3 /* HBM to HBM through the caches (data that is re-read soon) */
-#define MFRT_ROUTE_HBM_THROUGH 4 /* HBM to HBM, destination written through as it is produced */
 
 #define MFRT_PTR_PAGEABLE 0     /* ordinary host memory the GPU cannot address */
 #define MFRT_PTR_DEVICE 1
@@ -81,7 +79,6 @@ int mfk_xcopy_plan(const void *triples, uint32_t nseg, uint32_t units, void *fir
 
 /* ---- MoE launchers (kernels/moe.hip) ---------------------------------------- */
 uint64_t mfk_moe_workspace_bytes(uint32_t tokens, uint32_t topK, uint32_t experts);
-void mfk_moe_tune(int permuteVariant, int combineVariant);
 int mfk_moe_dispatch(const void *x, const void *topk, uint32_t tokens, uint32_t hidden, uint32_t topK, uint32_t experts,
                      void *out, void *counts, void *offsets, void *rowOf, void *srcOf, void *workspace, void *stream);
 int mfk_moe_combine(const void *rows, const void *rowOf, const void *weights, uint32_t tokens, uint32_t hidden,
@@ -89,9 +86,6 @@ int mfk_moe_combine(const void *rows, const void *rowOf, const void *weights, ui
 
 /* ---- 2-D copy launcher (kernels/copy2d.hip) ----------------------------------- */
 int mfk_copy2d(const void *rectPlan, uint32_t grid, void *stream);
-
-/* ---- yardstick kernels (kernels/probe.hip) ------------------------------------ */
-int mfk_probe(int kind, void *dst, const void *src, uint64_t bytes, uint32_t grid, void *stream);
 
 #ifndef MF_RT_HIDDEN
 #pragma GCC visibility pop

@@ -13,6 +13,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_DIR = os.path.join(_HERE, "lib")
 DATAPLANE_PATH = os.path.join(LIB_DIR, "libmf_hip_dataplane.so")
 PLUGIN_PATH = os.path.join(LIB_DIR, "libmf_hybm_copy_extend.so")
+YARDSTICK_PATH = os.path.join(LIB_DIR, "libmf_hip_yardstick.so")
 
 # ---- enums (values pinned in include/mf_xcopy_types.h) ---------------------
 BM_OK = 0
@@ -182,6 +183,8 @@ _SIGNATURES = {
     "mf_xcopy_batch": (i32, [u64p, u64p, u64p, u32, i32, vp]),
     "mf_xcopy_device_table": (i32, [vp, u32, i32, vp]),
     "mf_xcopy_2d_batch": (i32, [vp, u32, i32, vp]),
+    "mf_copy2d_describe": (None, [u64, ctypes.POINTER(u32), ctypes.POINTER(u32)]),
+    "mf_copy2d_rowcol_mismatches": (u32, [u32, u32, u32, u32]),
     "mf_xcopy_thread_stream": (vp, []),
     "mf_xcopy_tune": (i32, [u32, u32, u32]),
     "mf_xcopy_choose_units": (u32, [u64, u32, i32]),
@@ -216,7 +219,6 @@ _SIGNATURES = {
     "mfrt_memcpy": (ctypes.c_int, [vp, vp, u64]),
     "mfrt_memset": (ctypes.c_int, [vp, ctypes.c_int, u64]),
     "mfrt_memcpy_async": (ctypes.c_int, [vp, vp, u64, vp]),
-    "mf_probe_hbm": (i32, [i32, vp, vp, u64, vp]),
     "mf_va_clear": (None, []),
     "mf_va_add": (i32, [u64, u64, i32, u64, u32]),
     "mf_va_add_external": (i32, [u64, u64, i32, u64, u32, u32]),
@@ -267,11 +269,17 @@ _SIGNATURES = {
 _PLUGIN_SIGNATURES = {
     "hybm_copy_extend": (None, [vp, vp, u64, u32, vp]),
     "hybm_batch_copy_extend": (None, [vp, u32, vp, u32, vp]),
+    "mf_copy_extend_failures": (u64, []),
+}
+
+_YARDSTICK_SIGNATURES = {
+    "mf_probe_hbm": (i32, [i32, vp, vp, u64, vp]),
 }
 
 _lock = threading.Lock()
 _lib = None
 _plugin = None
+_yardstick = None
 
 
 def _bind(handle, table):
@@ -304,6 +312,17 @@ def plugin():
                 raise OSError(f"{PLUGIN_PATH} is missing: build it with `make -C memfabric_hybrid_amd/csrc`")
             _plugin = _bind(ctypes.CDLL(PLUGIN_PATH, mode=ctypes.RTLD_LOCAL), _PLUGIN_SIGNATURES)
         return _plugin
+
+
+def yardstick():
+    """The streaming yardstick kernels (measurement tooling of bench.py and the tests)."""
+    global _yardstick
+    with _lock:
+        if _yardstick is None:
+            if not os.path.exists(YARDSTICK_PATH):
+                raise OSError(f"{YARDSTICK_PATH} is missing: build it with `make -C memfabric_hybrid_amd/csrc`")
+            _yardstick = _bind(ctypes.CDLL(YARDSTICK_PATH, mode=ctypes.RTLD_LOCAL), _YARDSTICK_SIGNATURES)
+        return _yardstick
 
 
 def declared_symbols():

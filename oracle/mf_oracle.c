@@ -710,7 +710,9 @@ static uint16_t f32_to_bf16_rne(float f)
 
 /* combine: y[t][h] = bf16_rne( fma(w[t][K-1], v_{K-1}, ... fma(w[t][0], v_0, 0)) ),
  * v_k = float(rows[rowOf[t*K+k]][h]): fp32 accumulation in slot order with one
- * rounding per step (fmaf), a single final rounding to bf16. */
+ * rounding per step (fmaf), a single final rounding to bf16.  A slot whose
+ * rowOf is negative (an expert id that dispatch flagged as out of range) is
+ * skipped: no row is read for it and the chain goes on with the next slot. */
 void orc_moe_combine(const uint16_t *rows, const int32_t *rowOf, const float *w, uint32_t T, uint32_t H, uint32_t K,
                      uint16_t *y)
 {
@@ -718,6 +720,9 @@ void orc_moe_combine(const uint16_t *rows, const int32_t *rowOf, const float *w,
         for (uint32_t h = 0; h < H; ++h) {
             float acc = 0.0f;
             for (uint32_t k = 0; k < K; ++k) {
+                if (rowOf[(uint64_t)t * K + k] < 0) {
+                    continue;
+                }
                 float v = bf16_to_f32(rows[(uint64_t)rowOf[(uint64_t)t * K + k] * H + h]);
                 acc = fmaf(w[(uint64_t)t * K + k], v, acc);
             }

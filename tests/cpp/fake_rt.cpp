@@ -120,6 +120,9 @@ static void Guard(const char *what)
     }
 }
 uint64_t fake_rt_launches(void) { return g_launches; }
+// The next n xcopy launches fail with a runtime error code instead of running.
+static int g_failLaunches = 0;
+void fake_rt_fail_launches(int n) { g_failLaunches = n; }
 uint64_t fake_rt_chunks(void) { return g_chunksRun; }
 
 int mfrt_init(int device)
@@ -213,6 +216,10 @@ int mfrt_memset(void *dst, int value, uint64_t bytes) { std::memset(dst, value, 
 int mfk_xcopy_inline(const void *inlinePlan, int, uint32_t, void *mask, uint32_t maskValue, void *)
 {
     const mf::InlinePlan &p = *static_cast<const mf::InlinePlan *>(inlinePlan);
+    if (g_failLaunches > 0) {
+        --g_failLaunches;
+        return 719;
+    }
     ++g_launches;
     static const bool skip = std::getenv("FAKE_RT_SKIP_COPY") != nullptr;   // host-path timing: the launch is free
     if (skip) {
@@ -238,6 +245,10 @@ int mfk_xcopy_table(const void *triples, const void *first, const void *nchunkDe
     const uint64_t *t = static_cast<const uint64_t *>(triples);
     const uint32_t *f = static_cast<const uint32_t *>(first);
     const uint32_t total = nchunkDev != nullptr ? *static_cast<const uint32_t *>(nchunkDev) : nchunk;
+    if (g_failLaunches > 0) {
+        --g_failLaunches;
+        return 719;
+    }
     ++g_launches;
     uint32_t s = 0;
     TrackTable(triples, 24ull * nseg);
@@ -301,6 +312,4 @@ uint64_t mfk_moe_workspace_bytes(uint32_t, uint32_t, uint32_t) { return 0; }
 int mfk_moe_dispatch(const void *, const void *, uint32_t, uint32_t, uint32_t, uint32_t, void *, void *, void *, void *, void *,
                      void *, void *) { return -1; }
 int mfk_moe_combine(const void *, const void *, const void *, uint32_t, uint32_t, uint32_t, void *, void *) { return -1; }
-void mfk_moe_tune(int, int) {}
-int mfk_probe(int, void *, const void *, uint64_t, uint32_t, void *) { return -1; }
 }

@@ -20,6 +20,8 @@
 
 extern "C" uint64_t fake_rt_launches(void);
 extern "C" void fake_rt_seal(void);
+extern "C" void fake_rt_fail_launches(int n);
+#include "../../include/mf_hip_copy_extend.h"
 extern "C" uint64_t fake_rt_violations(void);
 extern "C" uint64_t fake_rt_in_flight(void);
 
@@ -249,6 +251,18 @@ static void TestCApi()
     bad = {&cfg, host, 16};
     CHECK(smem_bm_copy(bm, &bad, SMEMB_COPY_L2GH, 0) == SM_INVALID_PARAM);  // L2GH does not override the source
     CHECK(smem_bm_copy(bm, &bad, SMEMB_COPY_BUTT, 0) == SM_INVALID_PARAM);
+    // a size that wraps round the address space is refused, not cut into 2^34 pieces
+    bad = {dev + 4096, host, ~0ull - reinterpret_cast<uint64_t>(dev) - 100};
+    CHECK(smem_bm_copy(bm, &bad, SMEMB_COPY_G2G, 0) == SM_INVALID_PARAM);
+    bad = {dev + 4096, host, ~0ull};
+    CHECK(smem_bm_copy(bm, &bad, SMEMB_COPY_G2G, 0) == SM_INVALID_PARAM);
+    {
+        void *ws[1] = {dev + 4096};
+        void *wd[1] = {host};
+        uint64_t wl[1] = {~0ull - 5};
+        smem_batch_copy_params wrap{ws, wd, wl, 1};
+        CHECK(smem_bm_copy_batch(bm, &wrap, SMEMB_COPY_G2G, 0) != SM_OK);
+    }
     // 2-D copy, aligned and unaligned geometry
     std::memset(dev, 0, pool);
     mf_copy2d_desc rects[2] = {
@@ -706,6 +720,64 @@ static void TestSlotRing()
     hybm_uninit();
 }
 
+// The two-symbol plugin over the same engine: the completion word of a table the CPU can read is
+// stored before the call returns; a failed launch leaves the word alone and is counted.
+static void TestPlugin()
+{
+    CHECK(hybm_init(0, 0) == BM_OK);
+    const uint64_t n = 1u << 20;
+    uint8_t *a = static_cast<uint8_t *>(mfrt_alloc_device(n));
+    uint8_t *b = static_cast<uint8_t *>(mfrt_alloc_device(n));
+    uint64_t *slot = static_cast<uint64_t *>(mfrt_alloc_host(16384 * 24 + 64));
+    uint64_t *devWord = static_cast<uint64_t *>(mfrt_alloc_device(64));
+    CHECK(a != nullptr && b != nullptr && slot != nullptr && devWord != nullptr);
+    std::vector<uint8_t> ref(n);
+    Fill(ref, 21);
+    std::memcpy(a, ref.data(), n);
+    std::memset(b, 0, n);
+    for (uint32_t i = 0; i < 64; ++i) {
+        slot[3 * i] = reinterpret_cast<uint64_t>(a) + i * 4096 + 3;
+        slot[3 * i + 1] = reinterpret_cast<uint64_t>(b) + i * 4096 + 5;
+        slot[3 * i + 2] = 3000;
+    }
+    uint64_t *word = slot + 16384 * 3;
+    *word = 0;
+    const uint64_t failuresBefore = mf_copy_extend_failures();
+    uint64_t launches = fake_rt_launches();
+    hybm_batch_copy_extend(slot, 64, word, 32, nullptr);
+    CHECK(*word == 32);
+    CHECK(fake_rt_launches() - launches == 1);          // no launch of its own for the word
+    bool ok = true;
+    for (uint32_t i = 0; i < 64; ++i) {
+        ok = ok && std::memcmp(b + i * 4096 + 5, ref.data() + i * 4096 + 3, 3000) == 0;
+    }
+    CHECK(ok);
+    CHECK(mf_copy_extend_failures() == failuresBefore);
+    // a word in device memory is stored by the launch path
+    *devWord = 0;
+    hybm_batch_copy_extend(slot, 64, devWord, 32, nullptr);
+    CHECK(*devWord == 32);
+    // a launch that fails: counted, word untouched
+    *word = 0;
+    fake_rt_fail_launches(1);
+    hybm_batch_copy_extend(slot, 64, word, 32, nullptr);
+    CHECK(*word == 0);
+    CHECK(mf_copy_extend_failures() == failuresBefore + 1);
+    fake_rt_fail_launches(1);
+    hybm_copy_extend(a, b, 100, 32, nullptr);
+    CHECK(mf_copy_extend_failures() == failuresBefore + 2);
+    hybm_batch_copy_extend(nullptr, 64, word, 32, nullptr);
+    CHECK(*word == 0 && mf_copy_extend_failures() == failuresBefore + 3);
+    // and the next one works again
+    hybm_batch_copy_extend(slot, 64, word, 32, nullptr);
+    CHECK(*word == 32);
+    mfrt_free_device(a);
+    mfrt_free_device(b);
+    mfrt_free_device(devWord);
+    mfrt_free_host(slot);
+    hybm_uninit();
+}
+
 int main()
 {
     SetLogLevel(3);
@@ -721,6 +793,7 @@ int main()
     TestTrans();
     TestLeases();
     TestMappedWindow();
+    TestPlugin();
     if (g_failed != 0) {
         std::printf("%d check(s) failed\n", g_failed);
         return 1;

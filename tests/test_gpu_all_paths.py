@@ -134,7 +134,7 @@ def test_auto_direction_and_caller_stream(lib, entity, oracle):
     try:
         assert lib.mfrt_memset(gd, 0, 2 * n) == 0
         for _ in range(3):  # producer and consumer back to back on the caller's stream
-            assert lib.mf_probe_hbm(1, local.ptr, None, n, stream) == 0          # fills with 0x5A5A5A5A words
+            assert native.yardstick().mf_probe_hbm(1, local.ptr, None, n, stream) == 0   # fills with the word 0x5A
             params = native.HybmCopyParams(local.ptr, gd + n, n)
             assert lib.hybm_data_copy(entity, ctypes.byref(params), native.HYBM_DIR["AUTO"], stream,
                                       native.ASYNC_COPY_FLAG) == 0, native.last_error()

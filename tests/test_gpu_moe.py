@@ -148,6 +148,27 @@ def test_out_of_range_expert_ids_are_flagged_not_followed(gpu, oracle):
         good = np.delete(np.arange(T * K), [10 * K + 1, 499 * K + 3])
         assert sorted(row_of[good].tolist()) == list(range(T * K - 2))
         assert _fetch(bufs["counts"], np.int32, (E,)).sum() == T * K - 2
+        # combine skips the two slots: with a NaN and an infinity in row 0 of the expert-contiguous
+        # buffer the result still equals the oracle's, and nothing non-finite appears in y
+        rows = _fetch(bufs["out"], np.uint16, (T * K, H)).copy()
+        rows[T * K - 2:] = 0        # the two rows nobody was sent to
+        row_of = row_of.copy()
+        victim = int(np.where(row_of == 0)[0][0])
+        rows[0, 0::2] = 0x7FC0
+        rows[0, 1::2] = 0x7F80
+        row_of[victim] = 1          # nobody reads the poisoned row
+        w = np.random.default_rng(10).random((T, K), dtype=np.float32)
+        rdev, rodev, wdev = _dev(gpu, rows), _dev(gpu, row_of), _dev(gpu, w)
+        y = gpu_util.DeviceBuffer(gpu, T * H * 2)
+        assert gpu.mf_moe_combine(rdev.ptr, rodev.ptr, wdev.ptr, T, H, K, y.ptr, None) == 0
+        assert gpu.mfrt_device_sync() == 0
+        got = _fetch(y, np.uint16, (T, H))
+        exp_y = np.zeros((T, H), dtype=np.uint16)
+        oracle.orc_moe_combine(np_ptr(rows), np_ptr(row_of), np_ptr(w), T, H, K, np_ptr(exp_y))
+        assert np.array_equal(got, exp_y)
+        assert not np.any((got & 0x7F80) == 0x7F80)
+        for b in (rdev, rodev, wdev, y):
+            b.free()
     finally:
         _free(bufs)
     # the same call with valid ids clears the flag again without any reset by the caller

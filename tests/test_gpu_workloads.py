@@ -42,6 +42,8 @@ def _copy2d(gpu, rects, route=native.ROUTE_HBM):
     (4736, 300, 4736, 9472, 0, 4736),      # the down_proj merge geometry, right half
     (16, 1000, 48, 32, 16, 0),             # one unit per row
     (32768, 5, 40000 - 40000 % 16, 65536, 0, 0),  # rows wider than a chunk
+    (2 * MIB + 16, 3, 2 * MIB + 48, 2 * MIB + 16, 32, 0),   # rows wider than 1 MiB: 131 073 units, beyond a 16-bit division trick
+    (1048592, 2, 1048592, 1048608, 0, 16),  # 65 537 units per row
     (100, 77, 160, 300, 5, 11),            # nothing aligned: falls back to one segment per row
     (48, 1, 48, 48, 0, 0),
 ])

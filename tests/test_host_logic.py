@@ -282,3 +282,23 @@ def test_workload_generators():
     assert not np.array_equal(src, src3)
     ids = workloads.page_ids(0xC3, 1310720, 4096)
     assert len(set(ids.tolist())) == 4096
+
+
+# ---- 2-D copy: index arithmetic of the kernel ---------------------------------------------------
+def test_2d_row_and_column_of_every_unit_in_a_chunk(lib):
+    """For every row width the planner can produce, the kernel's (row, column) of each 16-byte unit
+    of a chunk equals u // widthUnits, u % widthUnits.  Chunks of several rows use a multiply-high
+    division; a chunk that holds one row must not (the multiply-high is wrong from 65 537 units on:
+    unit 65 536 of such a row would land in "row 1, column 2^32 - 1")."""
+    widths = list(range(1, 1100)) + [4095, 4096, 4097, 65535, 65536, 65537, (1 << 20) - 1, 1 << 20, (1 << 20) + 1,
+                                     131073, (1 << 24) + 3]
+    rng = np.random.default_rng(5)
+    widths += [int(v) for v in rng.integers(2, 1 << 20, 200)]
+    for wu in widths:
+        rpc, magic = ctypes.c_uint32(0), ctypes.c_uint32(0)
+        lib.mf_copy2d_describe(wu * 16, ctypes.byref(rpc), ctypes.byref(magic))
+        assert rpc.value == max(1, 16384 // (wu * 16))
+        units = rpc.value * wu
+        assert lib.mf_copy2d_rowcol_mismatches(wu, rpc.value, magic.value, units) == 0, wu
+    # the formula the one-row case must not use: the multiply-high alone, on a row of 65 537 units
+    assert lib.mf_copy2d_rowcol_mismatches(65537, 2, (1 << 32) // 65537 + 1, 65537) != 0

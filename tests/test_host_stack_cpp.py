@@ -7,7 +7,7 @@ import subprocess
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 HOST = os.path.join(ROOT, "memfabric_hybrid_amd", "csrc", "host")
 SOURCES = ["mf_log.cpp", "xcopy_engine.cpp", "va_manager.cpp", "hip_data_op.cpp", "compose_data_op.cpp",
-           "mem_entity.cpp", "hybm_api.cpp", "smem_bm_api.cpp", "dataplane_api.cpp", "copy2d_api.cpp", "moe_api.cpp", "trans_entry.cpp", "smem_trans_api.cpp", "host_copy.cpp"]
+           "mem_entity.cpp", "hybm_api.cpp", "smem_bm_api.cpp", "dataplane_api.cpp", "copy2d_api.cpp", "moe_api.cpp", "trans_entry.cpp", "smem_trans_api.cpp", "host_copy.cpp", "copy_extend_plugin.cpp"]
 
 
 def test_host_stack_over_fake_runtime(tmp_path):

@@ -324,6 +324,23 @@ def test_combine_special_cases_and_fp64_check(oracle):
     exact = (vals * w.astype(np.float64)[:, :, None]).sum(axis=1)
     got = bf16_words_to_f32(y).astype(np.float64)
     assert np.all(np.abs(got - exact) <= np.abs(exact) * 2 ** -8 + 1e-6)
+    # a slot without a row is skipped, it is not "row 0 times its weight": the result equals the
+    # combine of the remaining slots alone, even when row 0 holds a NaN and an infinity
+    poisoned = rows.copy()
+    poisoned[0, 0::2] = 0x7FC0      # NaN
+    poisoned[0, 1::2] = 0x7F80      # +inf
+    holes = row_of.reshape(T, K).copy()
+    holes[holes == 0] = 1           # nobody points at the poisoned row ...
+    holes[3, 2] = -1                # ... and two slots point nowhere
+    holes[17, 7] = -1
+    oracle.orc_moe_combine(np_ptr(poisoned), np_ptr(holes), np_ptr(w), T, H, K, np_ptr(y))
+    for t, k in ((3, 2), (17, 7)):
+        keep = [j for j in range(K) if j != k]
+        yk = np.zeros((1, H), dtype=np.uint16)
+        rk, wk = np.ascontiguousarray(holes[t, keep]), np.ascontiguousarray(w[t, keep])   # kept alive across the call
+        oracle.orc_moe_combine(np_ptr(poisoned), np_ptr(rk), np_ptr(wk), 1, H, K - 1, np_ptr(yk))
+        assert np.array_equal(y[t], yk[0])
+    assert not np.any((y & 0x7F80) == 0x7F80)       # nothing infinite or NaN leaked in
 
 
 def test_bf16_rounding_is_nearest_even(oracle):
