@@ -7,7 +7,10 @@ Headline (value / roofline): the 122-segment KV-block batch copy, device to devi
 4 GiB HBM pool, through smem_bm_copy_batch on one stream.  A step is one batch:
 61 x (128 KiB + 16 KiB) = 8 994 816 payload bytes = 17 989 632 bytes of HBM traffic.  Steps
 rotate over 64 segment tables so that the touched set (~1.1 GiB) exceeds the 256 MiB
-last-level cache.  `extras` holds the other workload shapes (host link, large copies, paged
+last-level cache.  Whatever --steps and --warmup say, the GPU is first brought to its steady
+state by an untimed ramp of RAMP_BATCHES batches; then REPETITIONS repetitions of --steps
+batches are timed, each between two synchronisations, and the line reports the median
+repetition (HIP events on the launch stream for the kernel rate, the host clock for `value`).  `extras` holds the other workload shapes (host link, large copies, paged
 gather, MoE dispatch/combine, weight reshard), concurrency and the yardstick kernels.
 Prints ONE JSON line.
 """
@@ -34,6 +37,9 @@ LINK_PEAK_GBPS = 64.0
 POOL_BYTES = 4 << 30
 TABLES = 64
 MIB = 1 << 20
+RAMP_BATCHES = 3000      # untimed, before anything is measured: clocks up, queues and caches in their running state
+REPETITIONS = 21         # timed repetitions of --steps batches each; the median is reported
+MIN_BATCHES = 2000       # the concurrency extras run at least this many batches per configuration
 
 
 class Batch:
@@ -119,44 +125,37 @@ def timed_steps(lib, handle, batches, copy_type, steps, warmup, flags, caller="c
 
 
 def threaded_steps(lib, handle, batches, copy_type, steps, threads):
-    """The same batches submitted by `threads` host threads, each on its own stream (the
-    reference gives every calling thread its own stream as well); wall-clock time."""
-    barrier = threading.Barrier(threads + 1)
-    errors = []
+    """The same batches submitted by `threads` host threads started inside the library (no
+    interpreter in the loop), each on its own stream as the reference gives every calling thread its
+    own; returns the wall-clock seconds from the release of the warmed-up threads to the last wait."""
+    nb = len(batches)
+    table = (ctypes.POINTER(native.BatchCopyParams) * nb)(*[ctypes.pointer(b.params) for b in batches])
+    seconds = ctypes.c_double(0.0)
+    if lib.mf_bm_copy_batch_replay_threads(handle, table, nb, steps, copy_type, threads, ctypes.byref(seconds)) != 0:
+        raise RuntimeError(native.last_error())
+    return seconds.value
 
-    def worker(tid):
-        try:
-            lib.mfrt_bind_thread()
-            nb = len(batches)
-            for i in range(50):
-                lib.smem_bm_copy_batch(handle, batches[(tid * 7 + i) % nb].ref, copy_type, native.ASYNC_COPY_FLAG)
-            lib.smem_bm_wait(handle)
-            barrier.wait()
-            for i in range(tid, steps, threads):
-                if lib.smem_bm_copy_batch(handle, batches[i % nb].ref, copy_type, native.ASYNC_COPY_FLAG) != 0:
-                    raise RuntimeError(native.last_error())
-            if lib.smem_bm_wait(handle) != 0:
-                raise RuntimeError(native.last_error())
-        except Exception as exc:  # noqa: BLE001
-            errors.append(exc)
-            try:
-                barrier.abort()
-            except Exception:  # noqa: BLE001
-                pass
 
-    # the library rewrites the address arrays in place with the same (already normalised) values,
-    # so sharing one set of tables between the threads is harmless
-    pool = [threading.Thread(target=worker, args=(t,)) for t in range(threads)]
-    for t in pool:
-        t.start()
-    barrier.wait()
-    t0 = time.perf_counter()
-    for t in pool:
-        t.join()
-    wall = time.perf_counter() - t0
-    if errors:
-        raise errors[0]
-    return wall
+def median(values):
+    ordered = sorted(values)
+    return ordered[len(ordered) // 2]
+
+
+def steady_state_headline(lib, handle, batches, copy_type, steps, warmup):
+    """Ramp, the caller's warm-up steps, then REPETITIONS timed repetitions of `steps` batches.
+    Returns (median wall seconds per repetition, median event ms per repetition, all event us per batch)."""
+    nb = len(batches)
+    table = (ctypes.POINTER(native.BatchCopyParams) * nb)(*[ctypes.pointer(b.params) for b in batches])
+    stream = lib.mf_xcopy_thread_stream()
+    if lib.mf_bm_copy_batch_replay(handle, table, nb, RAMP_BATCHES + warmup, copy_type, native.ASYNC_COPY_FLAG) != 0:
+        raise RuntimeError(native.last_error())
+    assert lib.mfrt_stream_sync(stream) == 0
+    walls, events = [], []
+    for _ in range(REPETITIONS):
+        wall, ms = timed_steps(lib, handle, batches, copy_type, steps, 0, native.ASYNC_COPY_FLAG)
+        walls.append(wall)
+        events.append(ms)
+    return median(walls), median(events), sorted(ms * 1e3 / steps for ms in events)
 
 
 def cpu_baseline(tables, budget_s=12.0):
@@ -167,13 +166,17 @@ def cpu_baseline(tables, budget_s=12.0):
     ref = oracle_lib.reference()
     fn = ref.ref_batch_copy if ref is not None else oracle_lib.oracle().orc_batch_copy_fast
     kind = "reference" if ref is not None else "port"
-    pool = 1 << 30  # host pools of 1 GiB each; the 4 GiB offsets are folded into them
-    src_pool = np.random.default_rng(1).integers(0, 256, pool, dtype=np.uint8)
-    dst_pool = np.zeros(pool, dtype=np.uint8)
+    pool = POOL_BYTES  # two host pools of 4 GiB, the segment tables used as they are
+    block = np.random.default_rng(1).integers(0, 256, 64 * MIB, dtype=np.uint8)
+    src_pool = np.empty(pool, dtype=np.uint8)
+    dst_pool = np.empty(pool, dtype=np.uint8)
+    for i in range(pool // len(block)):
+        src_pool[i * len(block):(i + 1) * len(block)] = block
+        dst_pool[i * len(block):(i + 1) * len(block)] = 0      # touched before the clock starts
     prepared = []
     for src, dst, lens in tables:
-        s = oracle_lib.ptr_array((src_pool.ctypes.data + (src % np.uint64(pool - MIB))).tolist())
-        d = oracle_lib.ptr_array((dst_pool.ctypes.data + (dst % np.uint64(pool - MIB))).tolist())
+        s = oracle_lib.ptr_array((src_pool.ctypes.data + src).tolist())
+        d = oracle_lib.ptr_array((dst_pool.ctypes.data + dst).tolist())
         prepared.append((d, s, oracle_lib.u64_array(lens.tolist()), len(lens), int(lens.sum())))
     for d, s, l, n, _ in prepared[:8]:
         fn(d, s, l, n)
@@ -212,25 +215,42 @@ def cpu_baseline(tables, budget_s=12.0):
         "unit": "GB/s",
         "cores": 1,
         "kind": kind,
-        "sample": f"{batches} batches of the same 122-segment tables (8994816 B each), host pool to host pool, "
-                  f"{elapsed:.1f} s, single thread as the reference runs it; host has {os.cpu_count()} cores",
+        "sample": f"{batches} batches of the same 122-segment tables (8994816 B each), 4 GiB host pool to 4 GiB "
+                  f"host pool, {elapsed:.1f} s, single thread as the reference runs it; host has {os.cpu_count()} cores",
         "all_cores": {"value": sum(totals) / all_elapsed / GB, "unit": "GB/s", "cores": cores,
                       "sample": f"{cores} threads, each looping over its share of the tables for 3 s "
                                 "(destinations of different tables may coincide: bytes are only timed)"},
     }
 
 
+def kernel_source_digest():
+    """Names the kernel sources a counter summary was measured on."""
+    import hashlib
+    h = hashlib.sha256()
+    for name in ("xcopy.hip", "xcopy_plan.h"):
+        with open(os.path.join(ROOT, "memfabric_hybrid_amd", "csrc", "kernels", name), "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()[:16]
+
+
 def read_traffic():
     """HBM bytes per launch of the headline kernel, from the committed counter summary (rocprofv3
-    --pmc FETCH_SIZE / WRITE_SIZE scaled by the plain copy kernel); None when it is absent."""
+    --pmc FETCH_SIZE / WRITE_SIZE scaled by the plain copy kernel).  The summary names the kernel
+    sources it was measured on; when they have changed since, or the summary is absent, the figure
+    is withheld (None) rather than quoted for a kernel it does not describe."""
     path = os.path.join(ROOT, "profiles", "xcopy_inline_kv122_counters.txt")
+    traffic, digest = None, None
     try:
         for line in open(path):
             if line.startswith("traffic_bytes_per_launch"):
-                return float(line.split("=")[1].split()[0])
+                traffic = float(line.split("=")[1].split()[0])
+            if line.startswith("kernel_source_digest"):
+                digest = line.split("=")[1].split()[0]
     except OSError:
-        pass
-    return None
+        return None, "profiles/xcopy_inline_kv122_counters.txt is absent"
+    if digest != kernel_source_digest():
+        return None, f"counter summary was taken on kernel sources {digest}, these are {kernel_source_digest()}"
+    return traffic, "profiles/xcopy_inline_kv122_counters.txt (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by a plain copy)"
 
 
 def frac(gbps, peak):
@@ -258,22 +278,23 @@ def extras_block(lib, pool, dev, batches, tables, steps):
     copy_ceiling = yard["copy_GBps"]
 
     # ---- KV batch: synchronous calls, concurrency ---------------------------------------------------------
-    k = max(200, steps // 10)
+    k = max(500, steps // 4)
     w, _ = timed_steps(lib, handle, batches, g2g, k, 50, 0)
     out["kv122_d2d_sync_call_us"] = round(w * 1e6 / k, 2)
-    wp, msp = timed_steps(lib, handle, batches, g2g, steps, 100, native.ASYNC_COPY_FLAG, caller="python")
-    out["kv122_python_caller"] = {"us_per_batch_wall": round(wp * 1e6 / steps, 2),
-                                  "us_per_batch_events": round(msp * 1e3 / steps, 2),
+    kp = max(MIN_BATCHES, steps)
+    wp, msp = timed_steps(lib, handle, batches, g2g, kp, 100, native.ASYNC_COPY_FLAG, caller="python")
+    out["kv122_python_caller"] = {"us_per_batch_wall": round(wp * 1e6 / kp, 2),
+                                  "us_per_batch_events": round(msp * 1e3 / kp, 2),
                                   "note": "the headline loop with one ctypes call per batch instead of the C loop"}
-    reps = sorted(timed_steps(lib, handle, batches, g2g, 256, 16, native.ASYNC_COPY_FLAG)[1] * 1e3 / 256 for _ in range(20))
-    out["kv122_d2d_repetitions"] = {"n": 20, "launches_each": 256, "median_us": round(reps[10], 2), "min_us": round(reps[0], 2),
-                                    "max_us": round(reps[-1], 2)}
     conc = {}
-    for threads in (2, 4, 8):
-        wall = threaded_steps(lib, handle, batches, g2g, steps, threads)
-        hbm = 2 * payload * steps / wall / GB
-        conc[f"threads_{threads}"] = {"us_per_batch": round(wall * 1e6 / steps, 2), "hbm_GBps": round(hbm, 1),
+    kc = max(MIN_BATCHES, steps)
+    for threads in (1, 2, 4, 8):
+        wall = median([threaded_steps(lib, handle, batches, g2g, kc, threads) for _ in range(5)])
+        hbm = 2 * payload * kc / wall / GB
+        conc[f"threads_{threads}"] = {"us_per_batch": round(wall * 1e6 / kc, 2), "hbm_GBps": round(hbm, 1),
                                       "frac_of_hbm_peak": frac(hbm, HBM_PEAK_GBPS)}
+    conc["note"] = (f"{kc} batches shared out over C threads inside the library (mf_bm_copy_batch_replay_threads), each thread "
+                    "on its own stream, wall clock from the release of the warmed-up threads to the last wait; median of 5")
     out["kv122_d2d_concurrent_streams"] = conc
 
     # ---- the grid the reference publishes for its transfer benchmark (example/trans/perf/README.md:61-70 there:
@@ -614,10 +635,11 @@ def main():
     payload = batches[0].payload
     g2g = int(bm.BmCopyType.G2G)
 
-    wall, ms = timed_steps(lib, pool.handle, batches, g2g, args.steps, args.warmup, native.ASYNC_COPY_FLAG)
+    wall, ms, rep_us = steady_state_headline(lib, pool.handle, batches, g2g, args.steps, args.warmup)
     per_launch_us = ms * 1e3 / args.steps
     value = payload * args.steps / wall / GB
     achieved = 2 * payload / (per_launch_us * 1e-6) / GB
+    traffic, traffic_source = read_traffic()
 
     result = {
         "metric": "achieved GB/s (payload) for 122-segment KV batch copy, device to device",
@@ -637,6 +659,9 @@ def main():
                         "4 KiB-aligned random offsets in a 4 GiB HBM pool, D2D, 64 rotating tables",
             "api": "smem_bm_copy_batch(SMEMB_COPY_G2G, ASYNC_COPY_FLAG) on one stream + one wait; the K calls are "
                    "issued by a C loop (mf_bm_copy_batch_replay), extras.kv122_python_caller has one ctypes call per batch",
+            "timing": f"untimed ramp of {RAMP_BATCHES} batches + --warmup, then {REPETITIONS} repetitions of --steps batches, "
+                      "each between two synchronisations; ms_per_step / value: median repetition by the host clock "
+                      "(includes one stream wait per repetition), roofline: median repetition by HIP events",
             "payload_bytes": payload,
             "cu_count": lib.mfrt_cu_count(),
         },
@@ -646,10 +671,13 @@ def main():
             "peak": HBM_PEAK_GBPS,
             "unit": "GB/s",
             "frac": achieved / HBM_PEAK_GBPS,
-            "traffic": read_traffic(),
+            "traffic": traffic,
+            "traffic_source": traffic_source,
             "kernel": "XcopyInlineKernel<true, 1> (one launch per batch)",
             "algorithmic_bytes_per_launch": 2 * payload,
             "avg_launch_us": per_launch_us,
+            "repetitions_us_per_launch": {"n": len(rep_us), "min": round(rep_us[0], 3), "median": round(rep_us[len(rep_us) // 2], 3),
+                                          "max": round(rep_us[-1], 3)},
         },
     }
 

@@ -43,7 +43,17 @@ int32_t mf_xcopy_batch(const uint64_t *src, const uint64_t *dst, const uint64_t 
 int32_t mf_bm_copy_batch_replay(smem_bm_t handle, smem_batch_copy_params *const *batches, uint32_t count,
                                 uint32_t steps, smem_bm_copy_type t, uint32_t flags);
 
-/* Same for a {src,dst,len} triple table that already lives in device memory. */
+/* The same `steps` calls shared out over `threads` host threads (call i goes to thread
+ * i % threads), each thread on its own stream as the reference gives every calling thread its
+ * own (src/hybm/csrc/ts_engine/hybm_stream_manager.cpp:73-90), all asynchronous with one
+ * smem_bm_wait per thread at the end.  *seconds receives the wall-clock time from the moment
+ * all threads (already warmed up) are released until the last one has returned from its wait.
+ * The threads share `batches`: the library rewrites the address arrays in place with the same
+ * values, which is harmless.  Returns the first failing call's code. */
+int32_t mf_bm_copy_batch_replay_threads(smem_bm_t handle, smem_batch_copy_params *const *batches, uint32_t count,
+                                        uint32_t steps, smem_bm_copy_type t, uint32_t threads, double *seconds);
+
+/* An enqueue of mf_xcopy_batch for a {src,dst,len} triple table that already lives in device memory. */
 int32_t mf_xcopy_device_table(const void *triples, uint32_t n, int32_t route, void *stream);
 
 /* The stream copies of the calling thread run on when the caller passes none

@@ -1,5 +1,8 @@
 // Native C entry points declared in include/mf_hip_dataplane.h.
+#include <atomic>
+#include <chrono>
 #include <cstring>
+#include <thread>
 #include <vector>
 
 #include "../../../include/mf_hip_dataplane.h"
@@ -48,6 +51,59 @@ MF_EXPORT int32_t mf_bm_copy_batch_replay(smem_bm_t handle, smem_batch_copy_para
         at = at + 1 == count ? 0 : at + 1;
     }
     return 0;
+}
+
+MF_EXPORT int32_t mf_bm_copy_batch_replay_threads(smem_bm_t handle, smem_batch_copy_params *const *batches, uint32_t count,
+                                                  uint32_t steps, smem_bm_copy_type t, uint32_t threads, double *seconds)
+{
+    if (batches == nullptr || count == 0 || threads == 0 || threads > 64 || seconds == nullptr) {
+        MF_FAIL(SM_INVALID_PARAM, "mf_bm_copy_batch_replay_threads: no batches, no result or 0 / more than 64 threads");
+    }
+    std::atomic<uint32_t> ready{0};
+    std::atomic<bool> go{false};
+    std::atomic<int32_t> firstError{0};
+    auto body = [&](uint32_t tid) {
+        auto fail = [&](int32_t ret) {
+            int32_t none = 0;
+            firstError.compare_exchange_strong(none, ret);
+        };
+        // warm-up: the thread's stream and staging exist and have been used before the clock starts
+        for (uint32_t i = 0; i < 64 && firstError.load() == 0; ++i) {
+            const int32_t ret = smem_bm_copy_batch(handle, batches[(tid * 7 + i) % count], t, ASYNC_COPY_FLAG);
+            if (ret != 0) {
+                fail(ret);
+            }
+        }
+        (void)smem_bm_wait(handle);
+        ready.fetch_add(1, std::memory_order_acq_rel);
+        while (!go.load(std::memory_order_acquire)) {
+            std::this_thread::yield();
+        }
+        for (uint32_t i = tid; i < steps && firstError.load(std::memory_order_relaxed) == 0; i += threads) {
+            const int32_t ret = smem_bm_copy_batch(handle, batches[i % count], t, ASYNC_COPY_FLAG);
+            if (ret != 0) {
+                fail(ret);
+            }
+        }
+        const int32_t ret = smem_bm_wait(handle);
+        if (ret != 0) {
+            fail(ret);
+        }
+    };
+    std::vector<std::thread> pool;
+    for (uint32_t tid = 0; tid < threads; ++tid) {
+        pool.emplace_back(body, tid);
+    }
+    while (ready.load(std::memory_order_acquire) < threads) {
+        std::this_thread::yield();
+    }
+    const auto t0 = std::chrono::steady_clock::now();
+    go.store(true, std::memory_order_release);
+    for (auto &th : pool) {
+        th.join();
+    }
+    *seconds = std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count();
+    return firstError.load();
 }
 
 MF_EXPORT void *mf_xcopy_thread_stream(void)
