@@ -56,6 +56,18 @@ int32_t mf_bm_copy_batch_replay_threads(smem_bm_t handle, smem_batch_copy_params
 /* An enqueue of mf_xcopy_batch for a {src,dst,len} triple table that already lives in device memory. */
 int32_t mf_xcopy_device_table(const void *triples, uint32_t n, int32_t route, void *stream);
 
+/* No counterpart in the reference.  mf_xcopy_device_table for callers that cannot allocate: code
+ * under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  The chunk prefix
+ * the kernels need lives in a statically allocated device array (132 KiB per GPU, held until the
+ * process ends) instead of memory the library allocates on demand, and the call creates no stream,
+ * event or staging either: `stream` is used as given (NULL is the null stream).
+ * Limits: n <= MF_XCOPY_STATIC_TABLE_MAX segments (BM_INVALID_PARAM beyond); every call on one GPU
+ * uses the same array, so two calls whose kernels may run at the same time (different streams,
+ * different threads) race: keep them on one stream or order them yourself.  hybm_init must have
+ * run (it looks the array's address up).  Same results as mf_xcopy_device_table. */
+#define MF_XCOPY_STATIC_TABLE_MAX 32768u
+int32_t mf_xcopy_device_table_static(const void *triples, uint32_t n, int32_t route, void *stream);
+
 /* The stream copies of the calling thread run on when the caller passes none
  * (the per-thread stream of the reference's HybmStreamManager,
  * src/hybm/csrc/ts_engine/hybm_stream_manager.cpp:73-90).  NULL before init. */

@@ -36,6 +36,14 @@ MF_EXPORT int32_t mf_xcopy_device_table(const void *triples, uint32_t n, int32_t
     return XcopyEngine::Instance().SubmitDeviceTable(triples, n, route, stream, nullptr, 0);
 }
 
+MF_EXPORT int32_t mf_xcopy_device_table_static(const void *triples, uint32_t n, int32_t route, void *stream)
+{
+    if ((n != 0 && triples == nullptr) || route < 0 || route > MF_ROUTE_FROM_HOST) {
+        MF_FAIL(BM_INVALID_PARAM, "mf_xcopy_device_table_static: null table or unknown route " << route);
+    }
+    return XcopyEngine::Instance().SubmitDeviceTableStatic(triples, n, route, stream);
+}
+
 MF_EXPORT int32_t mf_bm_copy_batch_replay(smem_bm_t handle, smem_batch_copy_params *const *batches, uint32_t count,
                                           uint32_t steps, smem_bm_copy_type t, uint32_t flags)
 {

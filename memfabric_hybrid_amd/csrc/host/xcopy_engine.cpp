@@ -589,6 +589,12 @@ int XcopyEngine::Start(int device)
     if (err != 0) {
         MF_FAIL(BM_ERROR, "GPU runtime start on device " << device << " failed: " << mfrt_error_string(err));
     }
+#ifndef MF_RT_HIDDEN
+    err = mfk_xcopy_static_setup();   // the device is current on this thread: mfrt_init has just selected it
+    if (err != 0) {
+        MF_FAIL(BM_ERROR, "address of the static descriptor scratch not available: " << mfrt_error_string(err));
+    }
+#endif
     started_.store(true, std::memory_order_release);
     return BM_OK;
 }
@@ -859,5 +865,33 @@ int XcopyEngine::SubmitDeviceTable(const void *triples, uint32_t n, int route, v
     g_launches.fetch_add(2, std::memory_order_relaxed);
     return MarkQueued(lease, slot, stream, false);
 }
+
+#ifndef MF_RT_HIDDEN
+int XcopyEngine::SubmitDeviceTableStatic(const void *triples, uint32_t n, int route, void *stream)
+{
+    if (!Started()) {
+        MF_FAIL(BM_NOT_INITIALIZED, "xcopy engine not started");
+    }
+    if (n > MFK_STATIC_TABLE_SEGMENTS) {
+        MF_FAIL(BM_INVALID_PARAM, "table of " << n << " segments exceeds the " << MFK_STATIC_TABLE_SEGMENTS
+                << " the statically allocated scratch holds; split the table or use mf_xcopy_device_table");
+    }
+    if (n == 0) {
+        return BM_OK;
+    }
+    if (mfrt_bind_thread() != 0) {
+        MF_FAIL(BM_ERROR, "cannot make the GPU current on this thread");
+    }
+    const uint32_t cu = mfrt_cu_count();
+    const uint32_t units = ChooseUnits(0, cu, route, tuning_);   // sizes are only known on the GPU
+    const uint32_t grid = GridFor(static_cast<uint64_t>(cu == 0 ? 256 : cu) * 256, cu, route, tuning_);   // surplus workgroups leave at once
+    const int err = mfk_xcopy_table_static(triples, n, units, route, grid, stream);
+    if (err != 0) {
+        MF_FAIL(BM_ERROR, "static-scratch table launch failed (" << err << ")");
+    }
+    g_launches.fetch_add(2, std::memory_order_relaxed);
+    return BM_OK;
+}
+#endif
 
 }  // namespace mf

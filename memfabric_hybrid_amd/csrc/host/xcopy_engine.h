@@ -102,6 +102,11 @@ public:
     // Same for a triple table that lives in device memory the host cannot read.
     int SubmitDeviceTable(const void *triples, uint32_t n, int route, void *stream, void *mask, uint32_t maskValue);
 
+    // The same, with the chunk prefix in the statically allocated device scratch: allocates nothing
+    // (no stream either: `stream` is used as given, NULL being the null stream), at most
+    // MFK_STATIC_TABLE_SEGMENTS segments, calls on one GPU must not overlap.
+    int SubmitDeviceTableStatic(const void *triples, uint32_t n, int route, void *stream);
+
     uint64_t LaunchCount() const;
 
 private:

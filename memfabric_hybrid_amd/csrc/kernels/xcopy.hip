@@ -422,6 +422,65 @@ extern "C" int mfk_xcopy_table(const void *triples, const void *first, const voi
     return err != 0 ? err : mf::Signal(mask, maskValue, s);
 }
 
+#ifndef MF_RT_HIDDEN   // the plugin library has no entry point that needs it
+// Scratch of the entry point that allocates nothing (mfk_xcopy_table_static): the chunk prefix
+// first[0 .. nseg] and, behind it, the chunk count, both written by XcopyPlanKernel and read by
+// XcopyTableKernel of the same call.  One copy per GPU, held until the process ends.  In host code
+// the array's name is only a handle for hipGetSymbolAddress: kernels and copies get the address that
+// call returned for the current device, never the name.
+static __device__ __align__(256) uint32_t scratch[MFK_STATIC_TABLE_SEGMENTS + 64];
+
+namespace {
+constexpr int kMaxDevices = 64;
+uint32_t *g_scratchOf[kMaxDevices] = {};   // device ordinal -> address of that device's copy of `scratch`
+}  // namespace
+
+extern "C" int mfk_xcopy_static_setup(void)
+{
+    int dev = -1;
+    hipError_t err = hipGetDevice(&dev);
+    if (err != hipSuccess) {
+        return static_cast<int>(err);
+    }
+    if (dev < 0 || dev >= kMaxDevices) {
+        return static_cast<int>(hipErrorInvalidDevice);
+    }
+    void *ptr = nullptr;
+    err = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (err != hipSuccess) {
+        return static_cast<int>(err);
+    }
+    g_scratchOf[dev] = static_cast<uint32_t *>(ptr);
+    return 0;
+}
+
+extern "C" int mfk_xcopy_table_static(const void *triples, uint32_t nseg, uint32_t units, int route, uint32_t grid,
+                                      void *stream)
+{
+    if (nseg == 0 || nseg > MFK_STATIC_TABLE_SEGMENTS || grid == 0) {
+        return -1;
+    }
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices || g_scratchOf[dev] == nullptr) {
+        return -2;   // mfk_xcopy_static_setup has not run on this device
+    }
+    uint32_t *first = g_scratchOf[dev];
+    uint32_t *nchunkDev = first + nseg + 1;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    // the plan kernel writes every word the table kernel reads: nothing has to start at zero
+    hipLaunchKernelGGL(mf::XcopyPlanKernel, dim3(1), dim3(mf::kPlanThreads), 0, s, static_cast<const uint64_t *>(triples), nseg,
+                       units, first, nchunkDev);
+    hipError_t err = hipGetLastError();
+    if (err != hipSuccess) {
+        return static_cast<int>(err);
+    }
+    mf::TablePlan plan{static_cast<const uint64_t *>(triples), first, nseg, 0, units, mf::ChunkPattern{}};
+    return mf::WithPolicy(mf::PolicyOf(route), [&](auto ntLoad, auto store) {
+        return mf::LaunchTable<decltype(ntLoad)::value, decltype(store)::value>(plan, nchunkDev, grid, mf::LanesFor(units, route), s);
+    });
+}
+#endif  // MF_RT_HIDDEN
+
 extern "C" int mfk_xcopy_plan(const void *triples, uint32_t nseg, uint32_t units, void *first, void *nchunk,
                               void *stream)
 {

@@ -76,6 +76,13 @@ int mfk_xcopy_table(const void *triples, const void *first, const void *nchunkDe
                     uint32_t units, const void *pattern, int route, uint32_t grid, void *mask, uint32_t maskValue,
                     void *stream);
 int mfk_xcopy_plan(const void *triples, uint32_t nseg, uint32_t units, void *first, void *nchunk, void *stream);
+/* The table form with its chunk prefix in a statically allocated device array instead of memory the
+ * engine allocates: no allocation anywhere, at most MFK_STATIC_TABLE_SEGMENTS segments, one call at a
+ * time per GPU.  mfk_xcopy_static_setup looks the array's address up for the current device (once per
+ * device, at start-up); mfk_xcopy_table_static returns -2 when that has not happened. */
+#define MFK_STATIC_TABLE_SEGMENTS 32768u
+int mfk_xcopy_static_setup(void);
+int mfk_xcopy_table_static(const void *triples, uint32_t nseg, uint32_t units, int route, uint32_t grid, void *stream);
 
 /* ---- MoE launchers (kernels/moe.hip) ---------------------------------------- */
 uint64_t mfk_moe_workspace_bytes(uint32_t tokens, uint32_t topK, uint32_t experts);

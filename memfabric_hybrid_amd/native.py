@@ -184,6 +184,7 @@ _SIGNATURES = {
     # mf_hip_dataplane.h
     "mf_xcopy_batch": (i32, [u64p, u64p, u64p, u32, i32, vp]),
     "mf_xcopy_device_table": (i32, [vp, u32, i32, vp]),
+    "mf_xcopy_device_table_static": (i32, [vp, u32, i32, vp]),
     "mf_xcopy_2d_batch": (i32, [vp, u32, i32, vp]),
     "mf_copy2d_describe": (None, [u64, ctypes.POINTER(u32), ctypes.POINTER(u32)]),
     "mf_copy2d_rowcol_mismatches": (u32, [u32, u32, u32, u32]),

@@ -292,6 +292,17 @@ int mfk_xcopy_plan(const void *triples, uint32_t nseg, uint32_t units, void *fir
     return 0;
 }
 
+int mfk_xcopy_static_setup(void) { return 0; }
+int mfk_xcopy_table_static(const void *triples, uint32_t nseg, uint32_t units, int route, uint32_t grid, void *stream)
+{
+    static uint32_t scratch[MFK_STATIC_TABLE_SEGMENTS + 64];
+    if (nseg == 0 || nseg > MFK_STATIC_TABLE_SEGMENTS) {
+        return -1;
+    }
+    int err = mfk_xcopy_plan(triples, nseg, units, scratch, scratch + nseg + 1, stream);
+    return err != 0 ? err : mfk_xcopy_table(triples, scratch, scratch + nseg + 1, nseg, 0, units, nullptr, route, grid, nullptr, 0, stream);
+}
+
 int mfk_copy2d(const void *rectPlan, uint32_t, void *)
 {
     const mf::RectPlan &p = *static_cast<const mf::RectPlan *>(rectPlan);
