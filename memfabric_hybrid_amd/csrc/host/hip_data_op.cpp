@@ -134,10 +134,13 @@ HipDataOp::Result HipDataOp::Run(void *const *src, void *const *dst, const uint6
             return ret;
         }
         if (!async) {
-            int err = mfrt_stream_sync(stream);
-            if (err != 0) {
-                MF_FAIL(BM_ERROR, "copy failed on the GPU: " << mfrt_error_string(err));
+            uint64_t bytes = 0;
+            if (n <= 4096) {   // a long table is not worth adding up: such a batch waits on the stream
+                for (uint32_t i = 0; i < n; ++i) {
+                    bytes += len[i];
+                }
             }
+            return engine.WaitStream(stream, bytes);
         }
         return BM_OK;
     }

@@ -92,6 +92,13 @@ public:
     void *ThreadBounceEvent(uint32_t index);
     // Wait for everything this thread enqueued on its own stream.
     int DrainThread();
+    // Wait for everything queued on `stream` so far: what a blocking copy does after its launch.
+    // Work expected to be short (`bytes` moved, 0 = unknown) is awaited by polling a word in pinned
+    // memory that a one-lane launch behind the copy stores, for at most kSpinMicros; anything else,
+    // and a poll that runs out of time, waits on the stream.
+    static constexpr uint64_t kSpinBytes = 256ull << 20;
+    static constexpr uint32_t kSpinMicros = 200;
+    int WaitStream(void *stream, uint64_t bytes);
 
     // Enqueue one batch.  Addresses must be device-accessible.  stream may be
     // NULL (thread stream).  mask/maskValue: plugin completion word or NULL.

@@ -203,7 +203,8 @@ __global__ __launch_bounds__(kXcopyThreads) void XcopySingleKernel(uint64_t src,
     } while (c < nchunk);
 }
 
-// Completion word of the plugin ABI.  It is written by a launch of its own right behind the copy
+// Completion word (of the plugin ABI for tables and words in device memory, and of blocking calls,
+// whose host thread polls it).  It is written by a launch of its own right behind the copy
 // launch on the same stream: the copy kernel's end-of-kernel release makes every store visible once
 // for the whole grid.  (Signalling from inside the copy kernel needs a system-scope release in
 // every workgroup before it may count itself done, an L2 write-back each: 77 us instead of 5.5 us
@@ -395,6 +396,11 @@ extern "C" int mfk_xcopy_inline(const void *inlinePlan, int route, uint32_t grid
         return mf::LaunchInline<decltype(ntLoad)::value, decltype(store)::value>(plan, grid, mf::LanesFor(plan.units, route), s);
     });
     return err != 0 ? err : mf::Signal(mask, maskValue, s);
+}
+
+extern "C" int mfk_xcopy_signal(void *word, uint32_t value, void *stream)
+{
+    return mf::Signal(word, value, static_cast<hipStream_t>(stream));
 }
 
 extern "C" int mfk_xcopy_table(const void *triples, const void *first, const void *nchunkDev, uint32_t nseg,

@@ -75,6 +75,9 @@ int mfk_xcopy_inline(const void *inlinePlan, int route, uint32_t grid, void *mas
 int mfk_xcopy_table(const void *triples, const void *first, const void *nchunkDev, uint32_t nseg, uint32_t nchunk,
                     uint32_t units, const void *pattern, int route, uint32_t grid, void *mask, uint32_t maskValue,
                     void *stream);
+/* One lane stores `value` (as a 64-bit word, released at system scope) into `word` once everything queued on
+ * `stream` before it has finished. */
+int mfk_xcopy_signal(void *word, uint32_t value, void *stream);
 int mfk_xcopy_plan(const void *triples, uint32_t nseg, uint32_t units, void *first, void *nchunk, void *stream);
 /* The table form with its chunk prefix in a statically allocated device array instead of memory the
  * engine allocates: no allocation anywhere, at most MFK_STATIC_TABLE_SEGMENTS segments, one call at a

@@ -179,6 +179,32 @@ def test_out_of_range_expert_ids_are_flagged_not_followed(gpu, oracle):
         _free(bufs)
 
 
+def test_same_workspace_reused_by_calls_of_different_sizes(gpu, oracle):
+    """Histograms and status of one call must not leak into the next call on the same workspace."""
+    E, K, H = 64, 4, 64
+    sizes = [5000, 700, 5000, 33]
+    ws_bytes = gpu.mf_moe_workspace_bytes(max(sizes), K, E)
+    ws = gpu_util.DeviceBuffer(gpu, ws_bytes)
+    ws.fill(0xFF)
+    try:
+        for i, T in enumerate(sizes):
+            x, topk, _ = _inputs(oracle, 0xB0 + i, T, H, K, E)
+            _, exp_counts, exp_offsets, exp_row, _ = _oracle_dispatch(oracle, x, topk, E)
+            dt = _dev(gpu, topk)
+            counts, offsets = gpu_util.DeviceBuffer(gpu, E * 4), gpu_util.DeviceBuffer(gpu, E * 4)
+            row_of = gpu_util.DeviceBuffer(gpu, T * K * 4)
+            assert gpu.mf_moe_dispatch(None, dt.ptr, T, H, K, E, None, counts.ptr, offsets.ptr, row_of.ptr, None, ws.ptr,
+                                       ws_bytes, None) == 0, native.last_error()
+            assert gpu.mfrt_device_sync() == 0
+            assert np.array_equal(_fetch(counts, np.int32, (E,)), exp_counts)
+            assert np.array_equal(_fetch(offsets, np.int32, (E,)), exp_offsets)
+            assert np.array_equal(_fetch(row_of, np.int32, (T * K,)), exp_row)
+            for b in (dt, counts, offsets, row_of):
+                b.free()
+    finally:
+        ws.free()
+
+
 def test_argument_errors(gpu):
     p = ctypes.c_void_p(0x1000)
     assert gpu.mf_moe_dispatch(p, None, 4, 8, 2, 4, p, p, p, p, None, p, 1 << 20, None) == native.BM_INVALID_PARAM
