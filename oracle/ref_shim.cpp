@@ -1,7 +1,8 @@
 // TEST INFRASTRUCTURE ONLY.  extern "C" doorway into pieces of the reference
 // that compile from their own sources with g++ alone: the address registry
-// (src/hybm/csrc/mm/hybm_va_manager.cpp) and the host branch of
-// DlHybridApi::Memcpy (src/hybm/csrc/under_api/dl_hybrid_api.h:150-169).
+// (src/hybm/csrc/mm/hybm_va_manager.cpp), the host branch of
+// DlHybridApi::Memcpy (src/hybm/csrc/under_api/dl_hybrid_api.h:150-169) and the
+// loader of the copy plugin (src/hybm/csrc/under_api/dl_hybm_copy_extend.cpp).
 // Built by oracle/Makefile into oracle/_ref/libmf_ref.so from the sources
 // where they lie; nothing of the reference is copied into this repository.
 // Used to validate oracle/mf_oracle.c and as the "reference" CPU baseline.
@@ -114,5 +115,33 @@ int32_t ref_batch_copy(void *const *dsts, void *const *srcs, const uint64_t *cou
         }
     }
     return 0;
+}
+}
+
+// The reference's plugin loader as it is (src/hybm/csrc/under_api/dl_hybm_copy_extend.cpp:25-86:
+// directory from MEMFABRIC_HYBRID_EXTEND_LIB_PATH, dlopen(RTLD_NOW | RTLD_NODELETE), both symbols
+// or unload) and the thunks HostDataOpSDMA calls through (dl_hybm_copy_extend.h:29-51).
+#include "dl_hybm_copy_extend.h"
+
+extern "C" {
+
+int32_t ref_extend_try_load(void)
+{
+    return DlHybmExtendApi::TryLoadLibrary();
+}
+
+void ref_extend_cleanup(void)
+{
+    DlHybmExtendApi::CleanupLibrary();
+}
+
+int32_t ref_extend_copy(const void *src, void *dst, uint64_t len, uint32_t concurrent, void *stream)
+{
+    return DlHybmExtendApi::HybmCopyExtend(src, dst, len, concurrent, stream);
+}
+
+int32_t ref_extend_batch_copy(void *param, uint32_t count, void *mask, uint32_t concurrent, void *stream)
+{
+    return DlHybmExtendApi::HybmBatchCopyExtend(param, count, mask, concurrent, stream);
 }
 }

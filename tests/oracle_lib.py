@@ -79,6 +79,10 @@ _REF_SIG = {
     "ref_mask48": (u64, [u64]),
     "ref_memcpy": (i32, [vp, u64, vp, u64, u32]),
     "ref_batch_copy": (i32, [vpp, vpp, u64p, u32]),
+    "ref_extend_try_load": (i32, []),
+    "ref_extend_cleanup": (None, []),
+    "ref_extend_copy": (i32, [vp, vp, u64, u32, vp]),
+    "ref_extend_batch_copy": (i32, [vp, u32, vp, u32, vp]),
 }
 
 _oracle = None

@@ -1,0 +1,122 @@
+"""Size-independent properties at the full sizes of the benchmark configurations that the byte-for-byte
+oracle comparisons (run at sizes the CPU finishes in seconds) do not reach: 1 GiB and 2 GiB single
+copies host -> device -> device -> host through smem_bm_copy, and the paged KV gather / scatter on a
+40 GiB pool.  Sources are built from one random block XORed with a per-block constant, so every
+64 MiB of a large buffer differs and a piece that lands at a wrong offset cannot go unnoticed."""
+
+import numpy as np
+import pytest
+
+from memfabric_hybrid_amd import bm, native, workloads
+from tests import gpu_util
+from tests.oracle_lib import np_ptr
+
+pytestmark = pytest.mark.gpu
+
+MIB = 1 << 20
+GIB = 1 << 30
+GUARD = 2 * MIB
+
+
+def _pattern_block(oracle):
+    block = np.empty(64 * MIB, dtype=np.uint8)
+    oracle.orc_fill_random(np_ptr(block), len(block), 0xF5)
+    return block
+
+
+def _fill_pattern(view, block):
+    for i in range(0, len(view), len(block)):
+        m = min(len(block), len(view) - i)
+        np.bitwise_xor(block[:m], np.uint8((i // len(block) * 29 + 3) & 0xFF), out=view[i:i + m])
+
+
+def _same_as_pattern(view, block):
+    for i in range(0, len(view), len(block)):
+        m = min(len(block), len(view) - i)
+        if not np.array_equal(view[i:i + m], block[:m] ^ np.uint8((i // len(block) * 29 + 3) & 0xFF)):
+            return False
+    return True
+
+
+@pytest.fixture(scope="module")
+def pool(lib):
+    assert bm.initialize("tcp://127.0.0.1:0", 1, 0) == 0, native.last_error()
+    p = bm.create(7, 2 * (2 * GIB + GUARD) + GUARD, 2 * (2 * GIB + GUARD) + GUARD)
+    yield p
+    p.destroy()
+    bm.uninitialize()
+
+
+@pytest.mark.parametrize("nbytes", [GIB, 2 * GIB], ids=["1GiB", "2GiB"])
+def test_single_copies_at_full_size_host_device_device_host(pool, lib, oracle, nbytes):
+    """smem_bm_copy of 1 GiB / 2 GiB: pinned host pool -> HBM pool (host link), HBM -> HBM, HBM ->
+    pinned host pool (host link); what arrives back equals what left, and the guard bytes round
+    every destination are untouched."""
+    dev = pool.peer_rank_ptr(0, bm.BmMemType.DEVICE)
+    host = pool.peer_rank_ptr(0, bm.BmMemType.HOST)
+    span = 2 * GIB + GUARD
+    host_all = gpu_util.host_view(host, 2 * span + GUARD)
+    block = _pattern_block(oracle)
+    src_off, back_off = GUARD, span + GUARD                  # two host regions, guards in front, between and behind
+    dev_a, dev_b = GUARD, span + GUARD
+    host_all[:] = 0xA5
+    _fill_pattern(host_all[src_off:src_off + nbytes], block)
+    assert lib.mfrt_memset(dev, 0x5A, 2 * span + GUARD) == 0
+    g2g = bm.BmCopyType.G2G
+    assert pool.copy_data(host + src_off, dev + dev_a, nbytes, g2g) == 0, native.last_error()          # H2D
+    assert pool.copy_data(dev + dev_a, dev + dev_b, nbytes, g2g) == 0, native.last_error()              # D2D
+    assert pool.copy_data(dev + dev_b, host + back_off, nbytes, g2g) == 0, native.last_error()          # D2H
+    assert _same_as_pattern(host_all[back_off:back_off + nbytes], block)
+    assert np.all(host_all[back_off - GUARD:back_off] == 0xA5)
+    assert np.all(host_all[back_off + nbytes:back_off + nbytes + GUARD] == 0xA5)
+    edge = np.empty(GUARD, dtype=np.uint8)
+    for at in (dev_a - GUARD, dev_a + nbytes, dev_b - GUARD, dev_b + nbytes):
+        if at + GUARD <= 2 * span + GUARD and not (dev_a <= at < dev_a + nbytes) and not (dev_b <= at < dev_b + nbytes):
+            assert lib.mfrt_memcpy(np_ptr(edge), dev + at, GUARD) == 0
+            assert np.all(edge == 0x5A), at
+    # idempotence: the same device -> device copy once more changes nothing
+    assert pool.copy_data(dev + dev_a, dev + dev_b, nbytes, g2g) == 0, native.last_error()
+    assert pool.copy_data(dev + dev_b, host + back_off, nbytes, g2g) == 0, native.last_error()
+    assert _same_as_pattern(host_all[back_off:back_off + nbytes], block)
+
+
+def test_paged_gather_and_scatter_on_a_40_gib_pool(lib, oracle):
+    """4096 distinct 32 KiB pages sampled from a 40 GiB HBM pool (offsets far beyond 32 bits):
+    gather equals the sampled pages in order; scattering them to 4096 other pages and gathering
+    those returns the same bytes; pages next to the targets are untouched."""
+    assert lib.hybm_init(0, 0) == 0, native.last_error()
+    page, count = 32768, 4096
+    pool_bytes = 40 * GIB
+    pool = lib.mfrt_alloc_device(pool_bytes)
+    if not pool:
+        lib.hybm_uninit()
+        pytest.skip("a 40 GiB device allocation is not available on this GPU right now")
+    flat = gpu_util.DeviceBuffer(lib, count * page)
+    again = gpu_util.DeviceBuffer(lib, count * page)
+    try:
+        total_pages = pool_bytes // page
+        picks = workloads.page_ids(0xC3, total_pages, 2 * count)
+        ids, fresh = picks[:count], picks[count:]
+        assert int(ids.max()) * page > (1 << 35)             # the sample really reaches the far end
+        pages = np.empty((count, page), dtype=np.uint8)
+        oracle.orc_fill_random(np_ptr(pages), pages.size, 0xC3)
+        filler = np.full(page, 0x77, dtype=np.uint8)
+        for i in range(count):                               # only the sampled pages and the scatter targets are initialised
+            assert lib.mfrt_memcpy(pool + int(ids[i]) * page, pages[i].ctypes.data, page) == 0
+            assert lib.mfrt_memcpy(pool + int(fresh[i]) * page, filler.ctypes.data, page) == 0
+        lanes = np.arange(count, dtype=np.uint64) * page
+        gpu_util.xcopy(lib, pool + ids * page, flat.ptr + lanes, [page] * count, native.ROUTE_HBM)
+        assert np.array_equal(flat.download().reshape(count, page), pages)
+        gpu_util.xcopy(lib, flat.ptr + lanes, pool + fresh * page, [page] * count, native.ROUTE_HBM)
+        gpu_util.xcopy(lib, pool + fresh * page, again.ptr + lanes, [page] * count, native.ROUTE_HBM)
+        assert np.array_equal(again.download().reshape(count, page), pages)
+        # the originals are still in place (the scatter went elsewhere)
+        probe = np.empty(page, dtype=np.uint8)
+        for i in range(0, count, 257):
+            assert lib.mfrt_memcpy(np_ptr(probe), pool + int(ids[i]) * page, page) == 0
+            assert np.array_equal(probe, pages[i])
+    finally:
+        flat.free()
+        again.free()
+        lib.mfrt_free_device(pool)
+        lib.hybm_uninit()
