@@ -41,6 +41,7 @@ struct StagingSlot {
 // runtime, or a tool hooked into it, may already have torn down its own per-thread state).  The
 // next new thread takes an idle lease over; Stop() releases all of them.
 struct ThreadLease {
+    uint32_t ordinal = 0;           // position in creation order
     void *stream = nullptr;
     StagingSlot slots[kSlots];
     uint32_t cursor = 0;
@@ -114,12 +115,24 @@ struct LeasePool {
         std::lock_guard<std::mutex> guard(lock);
         epochOut = epoch;
         if (!idle.empty()) {
-            ThreadLease *lease = idle.back();
-            idle.pop_back();
+            // The oldest idle lease, not the one handed back last: the runtime spreads streams over its
+            // few hardware queues in creation order, and two streams on one hardware queue do not overlap
+            // (two submitting threads whose streams share a queue measured 4.9 us per 9 MB batch, the same
+            // as one thread; on different queues 4.1 us).  N threads alive at a time then hold the N
+            // oldest streams, which sit on different queues as far as there are queues.
+            size_t best = 0;
+            for (size_t i = 1; i < idle.size(); ++i) {
+                if (idle[i]->ordinal < idle[best]->ordinal) {
+                    best = i;
+                }
+            }
+            ThreadLease *lease = idle[best];
+            idle.erase(idle.begin() + static_cast<std::ptrdiff_t>(best));
             lease->adopted = true;
             return lease;
         }
         all.emplace_back(new ThreadLease());
+        all.back()->ordinal = static_cast<uint32_t>(all.size() - 1);
         return all.back().get();
     }
     void GiveBack(ThreadLease *lease, uint64_t leaseEpoch)
