@@ -87,7 +87,7 @@ MF_EXPORT int32_t mf_bm_copy_batch_replay_threads(smem_bm_t handle, smem_batch_c
         while (!go.load(std::memory_order_acquire)) {
             std::this_thread::yield();
         }
-        for (uint32_t i = tid; i < steps && firstError.load(std::memory_order_relaxed) == 0; i += threads) {
+        for (uint32_t i = tid; i < steps && firstError.load(std::memory_order_relaxed) == 0; i += threads) {   // nothing is submitted once anything failed
             const int32_t ret = smem_bm_copy_batch(handle, batches[i % count], t, ASYNC_COPY_FLAG);
             if (ret != 0) {
                 fail(ret);
@@ -99,10 +99,15 @@ MF_EXPORT int32_t mf_bm_copy_batch_replay_threads(smem_bm_t handle, smem_batch_c
         }
     };
     std::vector<std::thread> pool;
-    for (uint32_t tid = 0; tid < threads; ++tid) {
-        pool.emplace_back(body, tid);
+    uint32_t started = 0;
+    try {
+        for (; started < threads; ++started) {
+            pool.emplace_back(body, started);
+        }
+    } catch (...) {   // the system refused another thread: let the ones that run finish, then report
+        firstError.store(SM_ERROR);
     }
-    while (ready.load(std::memory_order_acquire) < threads) {
+    while (ready.load(std::memory_order_acquire) < started) {
         std::this_thread::yield();
     }
     const auto t0 = std::chrono::steady_clock::now();

@@ -698,7 +698,8 @@ int XcopyEngine::DrainThread()
 // completion signal behind the kernel and then takes 7 us to see it fire, whatever the wait policy
 // of the device (measured: 16.1 us per blocking 9 MB batch with the default policy and with
 // hipDeviceScheduleSpin alike; an event recorded behind the launch and polled or waited for:
-// 15.5 us; hipStreamWriteValue64 polled: 13.1 us).  A one-lane launch that stores a sequence number
+// 15.5 us; hipStreamWriteValue64 polled: 13.1 us; the kernel launched with a stop event of its own
+// and that event polled: 13.3 us).  A one-lane launch that stores a sequence number
 // into pinned memory, polled by the caller, is the shortest way round: 11.8 us.  It starts after
 // the copy kernel has ended, so it carries the same guarantee as the stream wait: the copy's
 // end-of-kernel release has made its stores visible to the device, and stores to host memory were
