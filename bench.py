@@ -286,6 +286,14 @@ def extras_block(lib, pool, dev, batches, tables, steps):
     out["kv122_python_caller"] = {"us_per_batch_wall": round(wp * 1e6 / kp, 2),
                                   "us_per_batch_events": round(msp * 1e3 / kp, 2),
                                   "note": "the headline loop with one ctypes call per batch instead of the C loop"}
+    unordered = native.ASYNC_COPY_FLAG | native.MF_COPY_UNORDERED_FLAG
+    ku = max(MIN_BATCHES, steps)
+    reps_u = sorted(timed_steps(lib, handle, batches, g2g, ku, 0, unordered)[1] * 1e3 / ku for _ in range(5))
+    out["kv122_unordered_one_stream"] = {
+        "us_per_batch": round(reps_u[2], 2), "hbm_GBps": round(2 * payload / reps_u[2] / 1e3, 1),
+        "frac_of_hbm_peak": frac(2 * payload / reps_u[2] / 1e3, HBM_PEAK_GBPS),
+        "note": "the headline loop with MF_COPY_UNORDERED_FLAG: the caller declares its batches independent and they are "
+                "launched without a barrier, so start-up and drain of consecutive batches overlap; one thread, one stream"}
     conc = {}
     kc = max(MIN_BATCHES, steps)
     for threads in (1, 2, 4, 8):

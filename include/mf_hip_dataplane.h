@@ -21,6 +21,17 @@
 extern "C" {
 #endif
 
+/* A flag of this build for the `flags` argument of smem_bm_copy[_batch] / hybm_data_[batch_]copy, beside the
+ * reference's ASYNC_COPY_FLAG and COPY_EXTEND_FLAG (no counterpart in the reference; a bit far from theirs).
+ * Together with ASYNC_COPY_FLAG it declares that the copy is independent of everything the caller has
+ * submitted on the same stream and not yet waited for: it may run while earlier copies still run and
+ * later unordered copies may run beside it.  A copy WITHOUT the flag submitted afterwards still waits for
+ * it, and so do smem_bm_wait / hybm_wait and a stream synchronisation.  KV blocks of different requests
+ * are such copies.  What it buys: consecutive batches of up to 128 segments from one thread overlap their
+ * start-up and drain on the GPU (a 9 MB batch: 5.3 instead of 5.9 us per batch on one stream).  Copies the
+ * flag cannot help (more than 128 segments, pageable memory, blocking calls) ignore it. */
+#define MF_COPY_UNORDERED_FLAG (1UL << 16)
+
 /* ---- which memory a copy touches (selects the kernel's cache policy) ---- */
 #define MF_ROUTE_HBM 0
 #define MF_ROUTE_TO_HOST 1

@@ -4,6 +4,7 @@
 #include <cstring>
 #include <vector>
 
+#include "../../../include/mf_hip_dataplane.h"
 #include "../rt/mf_rt.h"
 #include "copy_direction.h"
 #include "mf_log.h"
@@ -128,8 +129,9 @@ HipDataOp::Result HipDataOp::Run(void *const *src, void *const *dst, const uint6
 
     if (!srcPageable && !dstPageable) {
         static_assert(sizeof(void *) == sizeof(uint64_t), "64-bit addresses expected");
+        const bool unordered = async && (options.flags & MF_COPY_UNORDERED_FLAG) != 0;
         int ret = engine.Submit(reinterpret_cast<const uint64_t *>(src), reinterpret_cast<const uint64_t *>(dst), len, n,
-                                RouteOf(srcOnHost, dstOnHost), stream, nullptr, 0);
+                                RouteOf(srcOnHost, dstOnHost), stream, nullptr, 0, unordered);
         if (ret != BM_OK) {
             return ret;
         }

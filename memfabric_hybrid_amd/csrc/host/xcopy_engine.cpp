@@ -744,7 +744,7 @@ uint64_t XcopyEngine::LaunchCount() const
 }
 
 int XcopyEngine::Submit(const uint64_t *src, const uint64_t *dst, const uint64_t *len, uint32_t n, int route,
-                        void *stream, void *mask, uint32_t maskValue)
+                        void *stream, void *mask, uint32_t maskValue, bool unordered)
 {
     if (!Started()) {
         MF_FAIL(BM_NOT_INITIALIZED, "xcopy engine not started");
@@ -781,7 +781,8 @@ int XcopyEngine::Submit(const uint64_t *src, const uint64_t *dst, const uint64_t
     }
     if (inlined) {
         const uint32_t grid = GridFor(plan.nchunk, cu, route, tuning_);
-        int err = mfk_xcopy_inline(&plan, route, grid, mask, maskValue, stream);
+        // a completion word is stored by a launch of its own behind the copy, which an unordered copy would not hold back
+        int err = mfk_xcopy_inline(&plan, route, grid, mask, maskValue, stream, unordered && mask == nullptr ? 1 : 0);
         if (err != 0) {
             MF_FAIL(BM_ERROR, "xcopy launch failed: " << mfrt_error_string(err));
         }
@@ -831,7 +832,7 @@ int XcopyEngine::Submit(const uint64_t *src, const uint64_t *dst, const uint64_t
         InlinePlan empty;
         SegList none;
         (void)BuildInlinePlan(none, kXcopyThreads, empty);
-        int err = mfk_xcopy_inline(&empty, route, 1, mask, maskValue, stream);
+        int err = mfk_xcopy_inline(&empty, route, 1, mask, maskValue, stream, 0);
         return err == 0 ? BM_OK : BM_ERROR;
     }
 
@@ -861,7 +862,7 @@ int XcopyEngine::Submit(const uint64_t *src, const uint64_t *dst, const uint64_t
         }
         // (Uploading on a stream of its own, with the copy stream waiting for an event, was measured: the
         // two extra queue operations cost what the overlap gains, 56 us per 4096-page gather either way.)
-        err = mfk_xcopy_inline(&stagePlan, MFRT_ROUTE_FROM_HOST, stagePlan.nchunk, nullptr, 0, stream);
+        err = mfk_xcopy_inline(&stagePlan, MFRT_ROUTE_FROM_HOST, stagePlan.nchunk, nullptr, 0, stream, 0);
         if (err != 0) {
             MF_FAIL(BM_ERROR, "descriptor staging launch failed: " << mfrt_error_string(err));
         }
@@ -897,7 +898,7 @@ int XcopyEngine::SubmitDeviceTable(const void *triples, uint32_t n, int route, v
         InlinePlan empty;
         SegList none;
         (void)BuildInlinePlan(none, kXcopyThreads, empty);
-        int err = mfk_xcopy_inline(&empty, route, 1, mask, maskValue, stream);
+        int err = mfk_xcopy_inline(&empty, route, 1, mask, maskValue, stream, 0);
         return err == 0 ? BM_OK : BM_ERROR;
     }
     // The prefix is computed on the GPU; its slot is only ever touched by kernels of this stream.

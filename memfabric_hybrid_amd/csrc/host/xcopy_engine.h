@@ -103,8 +103,10 @@ public:
     // Enqueue one batch.  Addresses must be device-accessible.  stream may be
     // NULL (thread stream).  mask/maskValue: plugin completion word or NULL.
     // Returns 0 or a negative BM_* code; never waits for the copy itself.
+    // unordered: the caller vouches that the batch is independent of everything still in flight on
+    // `stream`; a batch that fits the kernel-argument form is then launched without a barrier.
     int Submit(const uint64_t *src, const uint64_t *dst, const uint64_t *len, uint32_t n, int route, void *stream,
-               void *mask, uint32_t maskValue);
+               void *mask, uint32_t maskValue, bool unordered = false);
 
     // Same for a triple table that lives in device memory the host cannot read.
     int SubmitDeviceTable(const void *triples, uint32_t n, int route, void *stream, void *mask, uint32_t maskValue);

@@ -14,6 +14,7 @@
 // device, the host link (1 byte per payload byte) when one side is pinned
 // host memory.  No LDS, no MFMA: nothing here is reused or contracted.
 #include <hip/hip_runtime.h>
+#include <hip/hip_ext.h>
 #include <stdint.h>
 
 #include <type_traits>
@@ -346,15 +347,28 @@ uint32_t LanesFor(uint32_t units, int route)
     return lanes <= 64 ? 64u : (lanes <= 128 ? 128u : kXcopyThreads);
 }
 
+// anyOrder: the launch carries no barrier, so the command processor may start it while launches queued
+// before it on the same stream still run (hipExtAnyOrderLaunch).  Measured on the 9 MB batch, one stream:
+// 5.3 us per launch against 5.9 us with the barrier.
 template <bool kNtLoad, int kStore>
-int LaunchInline(const InlinePlan &plan, uint32_t grid, uint32_t lanes, hipStream_t stream)
+int LaunchInline(const InlinePlan &plan, uint32_t grid, uint32_t lanes, hipStream_t stream, bool anyOrder)
 {
+    const uint32_t flags = anyOrder ? hipExtAnyOrderLaunch : 0u;
     if (plan.first[1] == kNoChunk && plan.nchunk <= kSingleMaxChunks) {
-        hipLaunchKernelGGL((XcopySingleKernel<kNtLoad, kStore>), dim3(grid), dim3(lanes), 0, stream, plan.src[0], plan.dst[0],
-                           plan.len[0], plan.nchunk, plan.units);
+        if (anyOrder) {
+            hipExtLaunchKernelGGL((XcopySingleKernel<kNtLoad, kStore>), dim3(grid), dim3(lanes), 0, stream, nullptr, nullptr, flags,
+                                  plan.src[0], plan.dst[0], plan.len[0], plan.nchunk, plan.units);
+        } else {
+            hipLaunchKernelGGL((XcopySingleKernel<kNtLoad, kStore>), dim3(grid), dim3(lanes), 0, stream, plan.src[0], plan.dst[0],
+                               plan.len[0], plan.nchunk, plan.units);
+        }
         return static_cast<int>(hipGetLastError());
     }
-    hipLaunchKernelGGL((XcopyInlineKernel<kNtLoad, kStore>), dim3(grid), dim3(lanes), 0, stream, plan);
+    if (anyOrder) {
+        hipExtLaunchKernelGGL((XcopyInlineKernel<kNtLoad, kStore>), dim3(grid), dim3(lanes), 0, stream, nullptr, nullptr, flags, plan);
+    } else {
+        hipLaunchKernelGGL((XcopyInlineKernel<kNtLoad, kStore>), dim3(grid), dim3(lanes), 0, stream, plan);
+    }
     return static_cast<int>(hipGetLastError());
 }
 
@@ -379,7 +393,7 @@ int Signal(void *mask, uint32_t maskValue, hipStream_t stream)
 }  // namespace mf
 
 extern "C" int mfk_xcopy_inline(const void *inlinePlan, int route, uint32_t grid, void *mask, uint32_t maskValue,
-                                void *stream)
+                                void *stream, int anyOrder)
 {
     const mf::InlinePlan &plan = *static_cast<const mf::InlinePlan *>(inlinePlan);
     hipStream_t s = static_cast<hipStream_t>(stream);
@@ -393,7 +407,8 @@ extern "C" int mfk_xcopy_inline(const void *inlinePlan, int route, uint32_t grid
         grid = (1u << 24) - 1;   // the grid size in lanes must stay below 2^32; workgroups loop over the rest
     }
     const int err = mf::WithPolicy(mf::PolicyOf(route), [&](auto ntLoad, auto store) {
-        return mf::LaunchInline<decltype(ntLoad)::value, decltype(store)::value>(plan, grid, mf::LanesFor(plan.units, route), s);
+        return mf::LaunchInline<decltype(ntLoad)::value, decltype(store)::value>(plan, grid, mf::LanesFor(plan.units, route), s,
+                                                                                 anyOrder != 0);
     });
     return err != 0 ? err : mf::Signal(mask, maskValue, s);
 }

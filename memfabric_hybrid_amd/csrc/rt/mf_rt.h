@@ -69,7 +69,10 @@ int mfrt_memset(void *dst, int value, uint64_t bytes);
 int mfrt_memcpy_async(void *dst, const void *src, uint64_t bytes, void *stream);  /* the runtime's own DMA path */
 
 /* ---- xcopy launchers (kernels/xcopy.hip) --------------------------------- */
-int mfk_xcopy_inline(const void *inlinePlan, int route, uint32_t grid, void *mask, uint32_t maskValue, void *stream);
+/* anyOrder != 0: the launch does not wait for launches queued before it on `stream` (it carries no barrier);
+ * launches queued after it without that option still wait for it. */
+int mfk_xcopy_inline(const void *inlinePlan, int route, uint32_t grid, void *mask, uint32_t maskValue, void *stream,
+                     int anyOrder);
 /* pattern: NULL, or a mf::ChunkPattern (kernels/xcopy_plan.h) that the chunk counts of the segments follow;
  * then `first` is not read (may be NULL) and `triples` may live in pinned host memory. */
 int mfk_xcopy_table(const void *triples, const void *first, const void *nchunkDev, uint32_t nseg, uint32_t nchunk,

@@ -25,6 +25,7 @@ SM_ERROR = -1
 SM_INVALID_PARAM = -2000
 SM_NOT_INITIALIZED = -2008
 
+MF_COPY_UNORDERED_FLAG = 1 << 16
 ASYNC_COPY_FLAG = 1
 COPY_EXTEND_FLAG = 2
 

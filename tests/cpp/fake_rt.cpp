@@ -213,7 +213,7 @@ int mfrt_memcpy(void *dst, const void *src, uint64_t bytes) { std::memmove(dst, 
 int mfrt_memcpy_async(void *dst, const void *src, uint64_t bytes, void *) { std::memmove(dst, src, bytes); return 0; }
 int mfrt_memset(void *dst, int value, uint64_t bytes) { std::memset(dst, value, bytes); return 0; }
 
-int mfk_xcopy_inline(const void *inlinePlan, int, uint32_t, void *mask, uint32_t maskValue, void *)
+int mfk_xcopy_inline(const void *inlinePlan, int, uint32_t, void *mask, uint32_t maskValue, void *, int)
 {
     const mf::InlinePlan &p = *static_cast<const mf::InlinePlan *>(inlinePlan);
     if (g_failLaunches > 0) {

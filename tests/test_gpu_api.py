@@ -194,6 +194,40 @@ def test_async_copy_completes_on_wait(pool, lib, oracle):
     assert np.array_equal(got, block)
 
 
+def test_unordered_batches_and_the_ordered_copy_behind_them(pool, lib, oracle):
+    """MF_COPY_UNORDERED_FLAG: batches the caller declares independent are launched without a barrier.
+    Sixty such batches of up to 100 ragged pieces, all with destinations of their own, then ONE ordinary
+    asynchronous copy that reads what they wrote: it has to wait for all of them.  Compared with the
+    oracle applied in order; repeated so that an ordering slip has many chances to show."""
+    dev = pool.peer_rank_ptr(0, bm.BmMemType.DEVICE)
+    half = 40 * MIB
+    init = _rand(oracle, half, 0xD8)
+    g2g = bm.BmCopyType.G2G
+    flags = native.ASYNC_COPY_FLAG | native.MF_COPY_UNORDERED_FLAG
+    rng = np.random.default_rng(12)
+    got = np.empty(half, dtype=np.uint8)
+    for rep in range(4):
+        assert lib.mfrt_memcpy(dev, np_ptr(init), half) == 0
+        assert lib.mfrt_memset(dev + half, 0x11 + rep, 2 * half) == 0
+        expect = np.full(half, 0x11 + rep, dtype=np.uint8)
+        cursor = 0
+        for b in range(60):
+            count = int(rng.integers(1, 101))
+            lens = rng.integers(0, 20000, count)
+            src = rng.integers(0, half - 20000, count)
+            dst = cursor + np.cumsum(lens + 13) - lens - 13          # disjoint destinations, 13 bytes apart, any alignment
+            cursor = int(dst[-1] + lens[-1] + 13)
+            assert cursor < half
+            assert pool.copy_data_batch((dev + src).tolist(), (dev + half + dst).tolist(), lens.tolist(), count, g2g, flags) == 0, \
+                native.last_error()
+            gpu_util.oracle_batch(oracle, init, expect, src, dst, lens)
+        # ordinary (ordered) copy of everything the unordered batches wrote
+        assert pool.copy_data(dev + half, dev + 2 * half, half, g2g, native.ASYNC_COPY_FLAG) == 0, native.last_error()
+        assert pool.wait() == 0
+        assert lib.mfrt_memcpy(np_ptr(got), dev + 2 * half, half) == 0
+        assert np.array_equal(got, expect), rep
+
+
 def test_replayed_batches_keep_stream_order(pool, lib, oracle):
     """mf_bm_copy_batch_replay issues the same calls a loop would: three batches, each reading what
     the one before wrote, cycled for seven steps on one stream, against the oracle applied in order."""
