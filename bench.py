@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the MemFabric xcopy hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-extras] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-extras] [--no-cpu] | --calibrate | --phases
 
 Headline (value / roofline): the 122-segment KV-block batch copy, device to device inside a
 4 GiB HBM pool, through smem_bm_copy_batch on one stream.  A step is one batch:
@@ -616,9 +616,19 @@ def main():
     ap.add_argument("--no-extras", action="store_true", help="headline only")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--calibrate", action="store_true", help="only run the plain copy kernel (counter calibration)")
+    ap.add_argument("--phases", action="store_true",
+                    help="only run the stand-alone program that takes the KV batch apart (lib/mf_batch_phases) and print its JSON")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build is a single-GPU data plane (no collectives, no sharding); run with --gpus 1")
+
+    if args.phases:
+        # a child process of its own, started before this one touches the GPU
+        import subprocess
+        exe = os.path.join(ROOT, "memfabric_hybrid_amd", "lib", "mf_batch_phases")
+        done = subprocess.run([exe], stdout=subprocess.PIPE, text=True, timeout=300)
+        sys.stdout.write(done.stdout)
+        sys.exit(done.returncode)
 
     lib = native.lib()
     if args.calibrate:

@@ -50,6 +50,11 @@ def test_yardstick_library_exports_its_one_symbol():
     native.yardstick()
 
 
+def test_measurement_program_is_built():
+    exe = os.path.join(native.LIB_DIR, "mf_batch_phases")
+    assert os.path.exists(exe) and os.access(exe, os.X_OK)      # bench.py --phases runs it
+
+
 def test_libraries_load_and_bind():
     lib = native.lib()
     assert lib.hybm_get_error_string(0) == b"success"
