@@ -294,6 +294,17 @@ def extras_block(lib, pool, dev, batches, tables, steps):
         "frac_of_hbm_peak": frac(2 * payload / reps_u[2] / 1e3, HBM_PEAK_GBPS),
         "note": "the headline loop with MF_COPY_UNORDERED_FLAG: the caller declares its batches independent and they are "
                 "launched without a barrier, so start-up and drain of consecutive batches overlap; one thread, one stream"}
+    # the headline loop with the held stores switched off and on in turn, in this process
+    held, not_held = [], []
+    for _ in range(5):
+        assert lib.mf_xcopy_hold_stores(0) == 0
+        not_held.append(timed_steps(lib, handle, batches, g2g, ku, 0, native.ASYNC_COPY_FLAG)[1] * 1e3 / ku)
+        assert lib.mf_xcopy_hold_stores(-1) == 0
+        held.append(timed_steps(lib, handle, batches, g2g, ku, 0, native.ASYNC_COPY_FLAG)[1] * 1e3 / ku)
+    out["kv122_held_stores"] = {
+        "us_per_batch_not_held": round(median(not_held), 2), "us_per_batch_held": round(median(held), 2),
+        "note": "mf_xcopy_hold_stores(0) against the default (every wave of a 960 to 5632 chunk launch keeps its data until the "
+                "loads of the whole launch are out, so HBM sees a read burst and then a write burst); 5 alternations, medians"}
     conc = {}
     kc = max(MIN_BATCHES, steps)
     for threads in (1, 2, 4, 8):
@@ -691,7 +702,7 @@ def main():
             "frac": achieved / HBM_PEAK_GBPS,
             "traffic": traffic,
             "traffic_source": traffic_source,
-            "kernel": "XcopyInlineKernel<true, 1> (one launch per batch)",
+            "kernel": "XcopyInlineKernel<true, 1, true> (one launch per batch; stores held back until the loads of the launch are out)",
             "algorithmic_bytes_per_launch": 2 * payload,
             "avg_launch_us": per_launch_us,
             "repetitions_us_per_launch": {"n": len(rep_us), "min": round(rep_us[0], 3), "median": round(rep_us[len(rep_us) // 2], 3),

@@ -134,6 +134,15 @@ MF_EXPORT int32_t mf_xcopy_tune(uint32_t units, uint32_t wgPerCu, uint32_t wgPer
     return BM_OK;
 }
 
+MF_EXPORT int32_t mf_xcopy_hold_stores(int32_t nanos)
+{
+    if (nanos < -1) {
+        MF_FAIL(BM_INVALID_PARAM, "hold: -1 (the rule), 0 (never) or a time in ns, got " << nanos);
+    }
+    XcopyEngine::Instance().Tuning().holdNanos = nanos;
+    return BM_OK;
+}
+
 MF_EXPORT uint32_t mf_xcopy_choose_units(uint64_t totalBytes, uint32_t cuCount, int32_t route)
 {
     return ChooseUnits(totalBytes, cuCount, route, XcopyEngine::Instance().Tuning());

@@ -104,6 +104,8 @@ struct ThreadLease {
     }
 };
 
+std::atomic<uint32_t> g_leasesOut{0};   // leases held by live threads: more than one means launches of several streams may overlap
+
 struct LeasePool {
     std::mutex lock;
     std::vector<std::unique_ptr<ThreadLease>> all;
@@ -129,10 +131,12 @@ struct LeasePool {
             ThreadLease *lease = idle[best];
             idle.erase(idle.begin() + static_cast<std::ptrdiff_t>(best));
             lease->adopted = true;
+            g_leasesOut.store(static_cast<uint32_t>(all.size() - idle.size()), std::memory_order_relaxed);
             return lease;
         }
         all.emplace_back(new ThreadLease());
         all.back()->ordinal = static_cast<uint32_t>(all.size() - 1);
+        g_leasesOut.store(static_cast<uint32_t>(all.size() - idle.size()), std::memory_order_relaxed);
         return all.back().get();
     }
     void GiveBack(ThreadLease *lease, uint64_t leaseEpoch)
@@ -140,6 +144,7 @@ struct LeasePool {
         std::lock_guard<std::mutex> guard(lock);
         if (leaseEpoch == epoch) {
             idle.push_back(lease);
+            g_leasesOut.store(static_cast<uint32_t>(all.size() - idle.size()), std::memory_order_relaxed);
         }
     }
     void DestroyAll()
@@ -150,6 +155,7 @@ struct LeasePool {
         }
         all.clear();
         idle.clear();
+        g_leasesOut.store(0, std::memory_order_relaxed);
         ++epoch;
     }
     uint64_t Epoch()
@@ -743,6 +749,23 @@ uint64_t XcopyEngine::LaunchCount() const
     return g_launches.load();
 }
 
+// How long the waves of a launch keep their data before they store (0: not at all): the tuning knob over
+// HoldNanosFor's rule, for HBM routes and ordered launches only.
+uint32_t XcopyEngine::HoldFor(const InlinePlan &plan, uint32_t grid, int route, bool unordered) const
+{
+    if (route != MFRT_ROUTE_HBM || unordered || tuning_.holdNanos == 0) {
+        return 0;
+    }
+    // With launches of another thread's stream on the chip at the same time not every wave of a large launch is
+    // resident at once, and the wait costs instead of gaining (two submitting threads, 24 MiB copies: 8.2 us per
+    // copy without, 9.0 us with; 21 MB batches 7.9 / 8.2 us; 16 MB and below: the same or better with the wait).
+    if (plan.nchunk > kHoldSharedMaxChunks && g_leasesOut.load(std::memory_order_relaxed) > 1) {
+        return 0;
+    }
+    const uint32_t rule = HoldNanosFor(plan.nchunk, grid, plan.units, plan.first[1] == kNoChunk);
+    return rule != 0 && tuning_.holdNanos > 0 ? static_cast<uint32_t>(tuning_.holdNanos) : rule;
+}
+
 int XcopyEngine::Submit(const uint64_t *src, const uint64_t *dst, const uint64_t *len, uint32_t n, int route,
                         void *stream, void *mask, uint32_t maskValue, bool unordered)
 {
@@ -782,7 +805,8 @@ int XcopyEngine::Submit(const uint64_t *src, const uint64_t *dst, const uint64_t
     if (inlined) {
         const uint32_t grid = GridFor(plan.nchunk, cu, route, tuning_);
         // a completion word is stored by a launch of its own behind the copy, which an unordered copy would not hold back
-        int err = mfk_xcopy_inline(&plan, route, grid, mask, maskValue, stream, unordered && mask == nullptr ? 1 : 0);
+        int err = mfk_xcopy_inline(&plan, route, grid, mask, maskValue, stream, unordered && mask == nullptr ? 1 : 0,
+                                   HoldFor(plan, grid, route, unordered));
         if (err != 0) {
             MF_FAIL(BM_ERROR, "xcopy launch failed: " << mfrt_error_string(err));
         }
@@ -832,7 +856,7 @@ int XcopyEngine::Submit(const uint64_t *src, const uint64_t *dst, const uint64_t
         InlinePlan empty;
         SegList none;
         (void)BuildInlinePlan(none, kXcopyThreads, empty);
-        int err = mfk_xcopy_inline(&empty, route, 1, mask, maskValue, stream, 0);
+        int err = mfk_xcopy_inline(&empty, route, 1, mask, maskValue, stream, 0, 0);
         return err == 0 ? BM_OK : BM_ERROR;
     }
 
@@ -862,7 +886,7 @@ int XcopyEngine::Submit(const uint64_t *src, const uint64_t *dst, const uint64_t
         }
         // (Uploading on a stream of its own, with the copy stream waiting for an event, was measured: the
         // two extra queue operations cost what the overlap gains, 56 us per 4096-page gather either way.)
-        err = mfk_xcopy_inline(&stagePlan, MFRT_ROUTE_FROM_HOST, stagePlan.nchunk, nullptr, 0, stream, 0);
+        err = mfk_xcopy_inline(&stagePlan, MFRT_ROUTE_FROM_HOST, stagePlan.nchunk, nullptr, 0, stream, 0, 0);
         if (err != 0) {
             MF_FAIL(BM_ERROR, "descriptor staging launch failed: " << mfrt_error_string(err));
         }
@@ -898,7 +922,7 @@ int XcopyEngine::SubmitDeviceTable(const void *triples, uint32_t n, int route, v
         InlinePlan empty;
         SegList none;
         (void)BuildInlinePlan(none, kXcopyThreads, empty);
-        int err = mfk_xcopy_inline(&empty, route, 1, mask, maskValue, stream, 0);
+        int err = mfk_xcopy_inline(&empty, route, 1, mask, maskValue, stream, 0, 0);
         return err == 0 ? BM_OK : BM_ERROR;
     }
     // The prefix is computed on the GPU; its slot is only ever touched by kernels of this stream.

@@ -46,6 +46,7 @@ struct XcopyTuning {
     uint32_t wgPerCu = 0;        // HBM routes: grid cap in workgroups per CU, 0 = one workgroup per chunk
     uint32_t wgPerCuLink = 1;    // routes bound by the host link: workgroups per CU
     uint32_t minUnits = kXcopyThreads;   // 4 KiB: the chunk of HBM routes
+    int32_t holdNanos = -1;      // stores held back in inline launches: -1 = HoldNanosFor's rule, 0 = never, else that long
 };
 
 uint32_t ChooseUnits(uint64_t totalBytes, uint32_t cuCount, int route, const XcopyTuning &tuning);
@@ -121,6 +122,7 @@ public:
 private:
     XcopyEngine() = default;
 
+    uint32_t HoldFor(const InlinePlan &plan, uint32_t grid, int route, bool unordered) const;
     XcopyTuning tuning_;
     std::atomic<bool> started_{false};   // read by every calling thread, flipped by Start / Stop
 };

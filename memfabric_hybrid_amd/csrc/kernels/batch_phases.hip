@@ -1,7 +1,8 @@
 // mf_batch_phases: a stand-alone measurement program (not part of the data plane, nothing links it).
 // It takes the 122-segment KV batch apart on one GPU: what a launch that waits for its predecessor costs,
 // what the descriptor lookup, the loads and the stores of a 9 MB batch add, and what the product kernel
-// needs, each as the period per launch of dependent launches on one stream.  Every kernel is first run
+// needs (with its stores held back until the loads of the launch are out, as the library launches this
+// batch, and without), each as the period per launch of dependent launches on one stream.  Every kernel is first run
 // from the host loop (period by HIP events; cheap kernels are bound by the host there) and then
 // replayed from a HIP graph of the same launches, where the host does not set the pace.
 // Prints one JSON object.  The product kernel is compiled in from its source, so what is timed is the
@@ -104,7 +105,13 @@ void LaunchPhase(const InlinePlan &plan, uint32_t grid, hipStream_t s)
 }
 void LaunchProduct(const InlinePlan &plan, uint32_t grid, hipStream_t s)
 {
-    hipLaunchKernelGGL((XcopyInlineKernel<true, kStoreStream>), dim3(grid != 0 ? grid : plan.nchunk), dim3(64), 0, s, plan);
+    hipLaunchKernelGGL((XcopyInlineKernel<true, kStoreStream>), dim3(grid != 0 ? grid : plan.nchunk), dim3(64), 0, s, plan, 0u);
+}
+// the same with the stores held back for as long as the library's rule says for this grid
+void LaunchProductHeld(const InlinePlan &plan, uint32_t grid, hipStream_t s)
+{
+    const uint32_t ticks = HoldTicks(HoldNanosFor(plan.nchunk, plan.nchunk, plan.units, false));
+    hipLaunchKernelGGL((XcopyInlineKernel<true, kStoreStream, true>), dim3(grid != 0 ? grid : plan.nchunk), dim3(64), 0, s, plan, ticks);
 }
 
 double Median(std::vector<double> v)
@@ -241,7 +248,8 @@ int main()
     const Row rows[] = {
         {"empty_kernel_one_workgroup", LaunchPhase<0>, 1},   {"empty_kernel", LaunchPhase<0>, 0},
         {"descriptor_lookup", LaunchPhase<1>, 0},            {"lookup_and_loads", LaunchPhase<2>, 0},
-        {"lookup_and_stores", LaunchPhase<3>, 0},            {"product_kernel", LaunchProduct, 0},
+        {"lookup_and_stores", LaunchPhase<3>, 0},            {"product_kernel_stores_not_held", LaunchProduct, 0},
+        {"product_kernel", LaunchProductHeld, 0},
     };
     std::printf("{\"workload\": \"122-segment KV batch, 64 tables in a 4 GiB pool, grid %u single-wave workgroups\", "
                 "\"unit\": \"us per launch, dependent launches on one stream\", \"phases\": {", plans[0].nchunk);

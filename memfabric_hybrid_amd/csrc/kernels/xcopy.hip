@@ -17,6 +17,7 @@
 #include <hip/hip_ext.h>
 #include <stdint.h>
 
+#include <atomic>
 #include <type_traits>
 
 #include <cstdlib>
@@ -80,9 +81,21 @@ __device__ __forceinline__ void CopyByte(uint64_t src, uint64_t dst)
 
 constexpr uint32_t kDepth = 4;                          // 128-bit loads in flight per lane
 
-// Copy chunk k of one segment.  All arguments are wave-uniform.
-template <bool kNtLoad, int kStore>
-__device__ __forceinline__ void CopyChunk(uint64_t src, uint64_t dst, uint64_t len, uint64_t k, uint32_t units)
+// Wait until `ticks` of the constant-rate clock have passed since t0, after the loads have landed (so
+// that the wait runs concurrently with the load latency instead of on top of it).
+__device__ __forceinline__ void HoldStores(uint64_t t0, uint32_t ticks)
+{
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    while (wall_clock64() - t0 < ticks) {
+        __builtin_amdgcn_s_sleep(1);
+    }
+}
+
+// Copy chunk k of one segment.  All arguments are wave-uniform.  kHold: the stores of the first step wait
+// for HoldStores(t0, ticks).
+template <bool kNtLoad, int kStore, bool kHold = false>
+__device__ __forceinline__ void CopyChunk(uint64_t src, uint64_t dst, uint64_t len, uint64_t k, uint32_t units, uint64_t t0 = 0,
+                                          uint32_t ticks = 0)
 {
     const SegGeom g = SegmentGeometry(dst, len);
     const uint64_t u0 = k * units;
@@ -101,6 +114,9 @@ __device__ __forceinline__ void CopyChunk(uint64_t src, uint64_t dst, uint64_t l
         for (uint32_t j = 0; j < kDepth; ++j) {
             v[j] = LoadUnit<kNtLoad>(s + static_cast<uint64_t>(i + j * lanes + tid) * kUnitBytes);
         }
+        if (kHold && i == 0) {
+            HoldStores(t0, ticks);
+        }
 #pragma unroll
         for (uint32_t j = 0; j < kDepth; ++j) {
             StoreUnit<kStore>(d + static_cast<uint64_t>(i + j * lanes + tid) * kUnitBytes, v[j]);
@@ -114,6 +130,9 @@ __device__ __forceinline__ void CopyChunk(uint64_t src, uint64_t dst, uint64_t l
             if (u < n) {
                 v[j] = LoadUnit<kNtLoad>(s + static_cast<uint64_t>(u) * kUnitBytes);
             }
+        }
+        if (kHold && i == 0) {
+            HoldStores(t0, ticks);
         }
 #pragma unroll
         for (uint32_t j = 0; j < kDepth; ++j) {
@@ -145,9 +164,14 @@ __device__ __forceinline__ uint64_t ReadLane64(uint64_t v, uint32_t lane)
 // trip; the owner of a chunk is then found with two ballots and read out of
 // the owning lane.  (A scalar search would chain three dependent loads, each
 // a full L2 round trip, before the first byte of payload is requested.)
-template <bool kNtLoad, int kStore>
-__global__ __launch_bounds__(kXcopyThreads) void XcopyInlineKernel(const InlinePlan p)
+//
+// kHold: every wave keeps its loaded data until `holdTicks` of the constant-rate clock after its own
+// start, which separates the read burst of the launch from its write burst (HoldNanosFor has the
+// measurements); such a launch has one chunk per workgroup.
+template <bool kNtLoad, int kStore, bool kHold = false>
+__global__ __launch_bounds__(kXcopyThreads) void XcopyInlineKernel(const InlinePlan p, uint32_t holdTicks)
 {
+    const uint64_t t0 = kHold ? wall_clock64() : 0;
     const uint32_t lane = threadIdx.x & 63u;
     const uint32_t f0 = p.first[lane];
     const uint32_t f1 = p.first[lane + 64];
@@ -182,7 +206,7 @@ __global__ __launch_bounds__(kXcopyThreads) void XcopyInlineKernel(const InlineP
             len = __builtin_amdgcn_readlane(l1, row);
             first = __builtin_amdgcn_readlane(f1, row);
         }
-        CopyChunk<kNtLoad, kStore>(src, dst, len, c - first, units);
+        CopyChunk<kNtLoad, kStore, kHold>(src, dst, len, c - first, units, t0, holdTicks);
         c += gridDim.x;
     } while (c < nchunk);
 }
@@ -193,13 +217,14 @@ __global__ __launch_bounds__(kXcopyThreads) void XcopyInlineKernel(const InlineP
 // of 15.4 us per blocking call, back-to-back 32 MiB copies 10.8 us instead of 11.5 us each; from
 // about 200 MiB on the table form is 1 % faster (512 MiB: 166.4 us against 168.8 us), hence the limit.
 constexpr uint32_t kSingleMaxChunks = 49152;
-template <bool kNtLoad, int kStore>
+template <bool kNtLoad, int kStore, bool kHold = false>
 __global__ __launch_bounds__(kXcopyThreads) void XcopySingleKernel(uint64_t src, uint64_t dst, uint32_t len, uint32_t nchunk,
-                                                                   uint32_t units)
+                                                                   uint32_t units, uint32_t holdTicks)
 {
+    const uint64_t t0 = kHold ? wall_clock64() : 0;
     uint32_t c = blockIdx.x;
     do {
-        CopyChunk<kNtLoad, kStore>(src, dst, len, c, units);
+        CopyChunk<kNtLoad, kStore, kHold>(src, dst, len, c, units, t0, holdTicks);
         c += gridDim.x;
     } while (c < nchunk);
 }
@@ -347,27 +372,62 @@ uint32_t LanesFor(uint32_t units, int route)
     return lanes <= 64 ? 64u : (lanes <= 128 ? 128u : kXcopyThreads);
 }
 
+// Ticks of the device's constant-rate clock (the one wall_clock64() reads) in `nanos`.
+uint32_t HoldTicks(uint32_t nanos)
+{
+    static std::atomic<int> khzOf[64];
+    int dev = 0;
+    if (nanos == 0 || hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) {
+        return 0;
+    }
+    int khz = khzOf[dev].load(std::memory_order_relaxed);
+    if (khz == 0) {
+        if (hipDeviceGetAttribute(&khz, hipDeviceAttributeWallClockRate, dev) != hipSuccess || khz <= 0) {
+            khz = -1;   // unknown clock: no hold on this device
+        }
+        khzOf[dev].store(khz, std::memory_order_relaxed);
+    }
+    if (khz < 0) {
+        return 0;
+    }
+    const uint64_t capped = nanos < 10000 ? nanos : 10000;   // no wave ever waits longer than 10 us
+    return static_cast<uint32_t>(capped * static_cast<uint64_t>(khz) / 1000000u);
+}
+
 // anyOrder: the launch carries no barrier, so the command processor may start it while launches queued
 // before it on the same stream still run (hipExtAnyOrderLaunch).  Measured on the 9 MB batch, one stream:
 // 5.3 us per launch against 5.9 us with the barrier.
+// holdNanos: the caller's HoldNanosFor(); the launch qualifies only if it still has one chunk per workgroup.
 template <bool kNtLoad, int kStore>
-int LaunchInline(const InlinePlan &plan, uint32_t grid, uint32_t lanes, hipStream_t stream, bool anyOrder)
+int LaunchInline(const InlinePlan &plan, uint32_t grid, uint32_t lanes, hipStream_t stream, bool anyOrder, uint32_t holdNanos)
 {
     const uint32_t flags = anyOrder ? hipExtAnyOrderLaunch : 0u;
+    const uint32_t ticks = grid == plan.nchunk && lanes == 64 ? HoldTicks(holdNanos) : 0;
     if (plan.first[1] == kNoChunk && plan.nchunk <= kSingleMaxChunks) {
         if (anyOrder) {
             hipExtLaunchKernelGGL((XcopySingleKernel<kNtLoad, kStore>), dim3(grid), dim3(lanes), 0, stream, nullptr, nullptr, flags,
-                                  plan.src[0], plan.dst[0], plan.len[0], plan.nchunk, plan.units);
+                                  plan.src[0], plan.dst[0], plan.len[0], plan.nchunk, plan.units, 0u);
+        } else if (ticks != 0) {
+            hipLaunchKernelGGL((XcopySingleKernel<kNtLoad, kStore, true>), dim3(grid), dim3(lanes), 0, stream, plan.src[0],
+                               plan.dst[0], plan.len[0], plan.nchunk, plan.units, ticks);
         } else {
             hipLaunchKernelGGL((XcopySingleKernel<kNtLoad, kStore>), dim3(grid), dim3(lanes), 0, stream, plan.src[0], plan.dst[0],
-                               plan.len[0], plan.nchunk, plan.units);
+                               plan.len[0], plan.nchunk, plan.units, 0u);
         }
         return static_cast<int>(hipGetLastError());
     }
-    if (anyOrder) {
-        hipExtLaunchKernelGGL((XcopyInlineKernel<kNtLoad, kStore>), dim3(grid), dim3(lanes), 0, stream, nullptr, nullptr, flags, plan);
+    if (ticks != 0) {
+        if (anyOrder) {
+            hipExtLaunchKernelGGL((XcopyInlineKernel<kNtLoad, kStore, true>), dim3(grid), dim3(lanes), 0, stream, nullptr, nullptr,
+                                  flags, plan, ticks);
+        } else {
+            hipLaunchKernelGGL((XcopyInlineKernel<kNtLoad, kStore, true>), dim3(grid), dim3(lanes), 0, stream, plan, ticks);
+        }
+    } else if (anyOrder) {
+        hipExtLaunchKernelGGL((XcopyInlineKernel<kNtLoad, kStore>), dim3(grid), dim3(lanes), 0, stream, nullptr, nullptr, flags, plan,
+                              0u);
     } else {
-        hipLaunchKernelGGL((XcopyInlineKernel<kNtLoad, kStore>), dim3(grid), dim3(lanes), 0, stream, plan);
+        hipLaunchKernelGGL((XcopyInlineKernel<kNtLoad, kStore>), dim3(grid), dim3(lanes), 0, stream, plan, 0u);
     }
     return static_cast<int>(hipGetLastError());
 }
@@ -393,7 +453,7 @@ int Signal(void *mask, uint32_t maskValue, hipStream_t stream)
 }  // namespace mf
 
 extern "C" int mfk_xcopy_inline(const void *inlinePlan, int route, uint32_t grid, void *mask, uint32_t maskValue,
-                                void *stream, int anyOrder)
+                                void *stream, int anyOrder, uint32_t holdNanos)
 {
     const mf::InlinePlan &plan = *static_cast<const mf::InlinePlan *>(inlinePlan);
     hipStream_t s = static_cast<hipStream_t>(stream);
@@ -408,7 +468,7 @@ extern "C" int mfk_xcopy_inline(const void *inlinePlan, int route, uint32_t grid
     }
     const int err = mf::WithPolicy(mf::PolicyOf(route), [&](auto ntLoad, auto store) {
         return mf::LaunchInline<decltype(ntLoad)::value, decltype(store)::value>(plan, grid, mf::LanesFor(plan.units, route), s,
-                                                                                 anyOrder != 0);
+                                                                                 anyOrder != 0, holdNanos);
     });
     return err != 0 ? err : mf::Signal(mask, maskValue, s);
 }

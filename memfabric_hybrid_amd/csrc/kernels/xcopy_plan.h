@@ -77,6 +77,61 @@ struct InlinePlan {
     uint32_t units;                     // 16-byte units per chunk, a multiple of 64
 };
 
+// Stores held back: how long after its start a wave of the inline kernel waits before it stores.
+//
+// A launch of a few thousand single-chunk waves has every load in flight within the first two
+// microseconds and would issue its stores as the data trickle in, so HBM sees reads and writes mixed
+// for most of the kernel.  When every wave instead keeps its four loaded registers until the loads
+// of the whole launch are out, the reads run as one burst and the writes as another, and the kernel
+// is shorter.  Measured through smem_bm_copy_batch, batches back to back on one stream, K and V
+// blocks in turn (61 of each, V blocks of 16 KiB), period per batch without the wait / at the best wait:
+//    976 chunks 3.79 / 3.24 us (1300 ns)     2684 chunks 6.45 / 5.11 us (2200 ns)
+//   1220 chunks 4.11 / 3.47 us (1400 ns)     3172 chunks 6.86 / 5.78 us (2600 ns)
+//   1708 chunks 4.76 / 4.32 us (1500-1900)   3904 chunks 8.02 / 6.54 us (3000 ns)
+//   2196 chunks 5.29 / 4.56 us (1900 ns)     5124 chunks 9.72 / 8.79 us (3400 ns)
+// and for other mixes of about 2048 chunks: 64 x 128 KiB 5.05 / 4.64, 32 x 256 KiB 4.99 / 4.38,
+// 128 x 64 KiB 5.07 / 4.61, 8 x 1 MiB + 100 x 20 KiB 6.12 / 5.07 us; 128 ragged segments of about
+// 70000 bytes gain nothing and lose nothing (6.5 us either way).  The wait is counted from the start of
+// the wave, which absorbs the spread of the table fetch (counted from the issue of the loads the same
+// wait gains nothing), and it is the same for every wave: shortening it for waves that start later did
+// not help.  The best wait grows with the number of waves the dispatcher has to start.  100 to 200 ns
+// short of it the gain is lost (2196 chunks: 1700 ns 4.87 us, 1600 ns 5.09 us), each 100 ns beyond it
+// costs 0.1 us, so the rule aims a little long.  From about 7000 chunks on the gain is below 5 % and the
+// best wait no longer follows the line: not every wave of such a launch is resident at once, and a wait
+// only delays the ones behind (11956 chunks: 19.3 us without, 20.2 us with).  Below about
+// 1000 chunks the period is the cost of a dependent launch and no wait changes it.
+// Launches that overlap on purpose (no barrier between them) lose with a wait: 4.53 us without, 4.81 with.
+//
+// A single segment (its three words are plain kernel arguments, no table to fetch) has its loads out
+// about 0.6 us earlier, and its best wait is shorter by as much; copies back to back on one stream,
+// without / at the best wait:
+//   1536 chunks (6 MiB) 3.64 / 3.39 us (1000 ns)     4096 chunks (16 MiB) 7.06 / 5.97 us (2300 ns)
+//   2048 chunks (8 MiB) 4.08 / 3.83 us (1300 ns)     5120 chunks (20 MiB) 8.74 / 7.07 us (2900 ns)
+//   3072 chunks (12 MiB) 5.71 / 4.90 us (1800 ns)    6144 chunks (24 MiB) 10.03 / 8.18 us (3400 ns)
+// 1024 chunks gain nothing (3.1 us either way); 7168 chunks gain 5 %, 8192 and more 3 % and less: past
+// 6144 single-wave workgroups (24 per CU) not every wave of the launch is resident at once.
+constexpr uint32_t kHoldMinChunks = 960;        // table in the kernel arguments
+constexpr uint32_t kHoldKneeChunks = 3904;
+constexpr uint32_t kHoldMinChunksSingle = 1400; // one segment
+constexpr uint32_t kHoldMaxChunks = 6144;
+constexpr uint32_t kHoldSharedMaxChunks = 4096; // the limit while several threads submit on streams of their own
+inline uint32_t HoldNanosFor(uint32_t nchunk, uint32_t grid, uint32_t units, bool single)
+{
+    if (units != kXcopyThreads || grid != nchunk || nchunk > kHoldMaxChunks) {
+        return 0;   // only launches of one 4 KiB chunk per single-wave workgroup were measured
+    }
+    if (single) {
+        return nchunk < kHoldMinChunksSingle ? 0 : 100 + nchunk * 57 / 100;
+    }
+    if (nchunk < kHoldMinChunks) {
+        return 0;
+    }
+    if (nchunk <= kHoldKneeChunks) {
+        return 700 + nchunk * 6 / 10;
+    }
+    return 700 + kHoldKneeChunks * 6 / 10 + (nchunk - kHoldKneeChunks) * 33 / 100;
+}
+
 // Chunk counts that repeat with a short period: pages of one size (period 1), K and V blocks
 // taking turns (period 2), ...  With such a pattern the owner of a chunk follows from a division
 // and at most kMaxPeriod comparisons, and no chunk prefix is needed.

@@ -71,8 +71,10 @@ int mfrt_memcpy_async(void *dst, const void *src, uint64_t bytes, void *stream);
 /* ---- xcopy launchers (kernels/xcopy.hip) --------------------------------- */
 /* anyOrder != 0: the launch does not wait for launches queued before it on `stream` (it carries no barrier);
  * launches queued after it without that option still wait for it. */
+/* holdNanos != 0: every wave keeps its loaded data until that long after its own start (see HoldNanosFor in
+ * kernels/xcopy_plan.h); honoured only by a launch of one 4 KiB chunk per workgroup. */
 int mfk_xcopy_inline(const void *inlinePlan, int route, uint32_t grid, void *mask, uint32_t maskValue, void *stream,
-                     int anyOrder);
+                     int anyOrder, uint32_t holdNanos);
 /* pattern: NULL, or a mf::ChunkPattern (kernels/xcopy_plan.h) that the chunk counts of the segments follow;
  * then `first` is not read (may be NULL) and `triples` may live in pinned host memory. */
 int mfk_xcopy_table(const void *triples, const void *first, const void *nchunkDev, uint32_t nseg, uint32_t nchunk,

@@ -23,6 +23,7 @@ std::mutex g_lock;
 std::map<uint64_t, std::pair<uint64_t, int>> g_allocs;  // base -> (size, kind)
 int g_device = -1;
 uint64_t g_launches = 0;
+uint32_t g_lastHold = 0;     // holdNanos of the latest inline launch
 uint64_t g_chunksRun = 0;
 
 void *Track(uint64_t bytes, int kind)
@@ -120,6 +121,7 @@ static void Guard(const char *what)
     }
 }
 uint64_t fake_rt_launches(void) { return g_launches; }
+uint32_t fake_rt_last_hold(void) { return g_lastHold; }
 // The next n xcopy launches fail with a runtime error code instead of running.
 static int g_failLaunches = 0;
 void fake_rt_fail_launches(int n) { g_failLaunches = n; }
@@ -213,9 +215,10 @@ int mfrt_memcpy(void *dst, const void *src, uint64_t bytes) { std::memmove(dst, 
 int mfrt_memcpy_async(void *dst, const void *src, uint64_t bytes, void *) { std::memmove(dst, src, bytes); return 0; }
 int mfrt_memset(void *dst, int value, uint64_t bytes) { std::memset(dst, value, bytes); return 0; }
 
-int mfk_xcopy_inline(const void *inlinePlan, int, uint32_t, void *mask, uint32_t maskValue, void *, int)
+int mfk_xcopy_inline(const void *inlinePlan, int, uint32_t, void *mask, uint32_t maskValue, void *, int, uint32_t holdNanos)
 {
     const mf::InlinePlan &p = *static_cast<const mf::InlinePlan *>(inlinePlan);
+    g_lastHold = holdNanos;
     if (g_failLaunches > 0) {
         --g_failLaunches;
         return 719;

@@ -8,6 +8,7 @@
 #include <cstdlib>
 #include <cstring>
 #include <random>
+#include <atomic>
 #include <thread>
 #include <vector>
 
@@ -19,6 +20,7 @@
 #include "../../memfabric_hybrid_amd/csrc/host/host_copy.h"
 
 extern "C" uint64_t fake_rt_launches(void);
+extern "C" uint32_t fake_rt_last_hold(void);
 extern "C" void fake_rt_seal(void);
 extern "C" void fake_rt_fail_launches(int n);
 #include "../../include/mf_hip_copy_extend.h"
@@ -778,6 +780,112 @@ static void TestPlugin()
     hybm_uninit();
 }
 
+// Which launches are told to hold their stores back, and for how long.
+static void TestHeldStores()
+{
+    CHECK(HoldNanosFor(959, 959, 256, false) == 0 && HoldNanosFor(960, 960, 256, false) == 700 + 576);
+    CHECK(HoldNanosFor(2196, 2196, 256, false) == 700 + 1317);
+    CHECK(HoldNanosFor(3904, 3904, 256, false) == 3042 && HoldNanosFor(3905, 3905, 256, false) == 3042);
+    CHECK(HoldNanosFor(6144, 6144, 256, false) == 3042 + 739 && HoldNanosFor(6145, 6145, 256, false) == 0);
+    CHECK(HoldNanosFor(2196, 2195, 256, false) == 0);    // a workgroup with two chunks
+    CHECK(HoldNanosFor(2196, 2196, 512, false) == 0);    // chunks of 8 KiB
+    CHECK(HoldNanosFor(1399, 1399, 256, true) == 0 && HoldNanosFor(1400, 1400, 256, true) == 100 + 798);
+    CHECK(HoldNanosFor(6144, 6144, 256, true) == 100 + 3502 && HoldNanosFor(6145, 6145, 256, true) == 0);
+    for (int single = 0; single < 2; ++single) {  // never shorter for more chunks, and one segment never waits longer than many
+        uint32_t last = 0;
+        for (uint32_t n = 960; n <= 6144; ++n) {
+            const uint32_t h = HoldNanosFor(n, n, 256, single != 0);
+            CHECK(h >= last && h < 4000);
+            CHECK(single == 0 || h < HoldNanosFor(n, n, 256, false));
+            last = h;
+        }
+    }
+
+    CHECK(hybm_init(0, 0) == BM_OK);
+    const uint64_t seg = 128u << 10;
+    const uint32_t count = 32;                    // 32 x 128 KiB = 1024 chunks of 4 KiB
+    std::vector<uint8_t> from(seg * count), to(seg * count, 0);
+    for (size_t i = 0; i < from.size(); ++i) {
+        from[i] = static_cast<uint8_t>(i * 31 + (i >> 12));
+    }
+    std::vector<uint64_t> src(count), dst(count), len(count, seg);
+    for (uint32_t i = 0; i < count; ++i) {
+        src[i] = reinterpret_cast<uint64_t>(from.data()) + i * seg;
+        dst[i] = reinterpret_cast<uint64_t>(to.data()) + (count - 1 - i) * seg;
+    }
+    XcopyEngine &engine = XcopyEngine::Instance();
+    void *stream = mf_xcopy_thread_stream();
+    CHECK(engine.Submit(src.data(), dst.data(), len.data(), count, MF_ROUTE_HBM, stream, nullptr, 0) == BM_OK);
+    CHECK(fake_rt_last_hold() == HoldNanosFor(1024, 1024, 256, false));
+    CHECK(engine.Submit(src.data(), dst.data(), len.data(), count, MF_ROUTE_HBM, stream, nullptr, 0, true) == BM_OK);
+    CHECK(fake_rt_last_hold() == 0);              // unordered launches overlap on purpose
+    CHECK(engine.Submit(src.data(), dst.data(), len.data(), count, MF_ROUTE_TO_HOST, stream, nullptr, 0) == BM_OK);
+    CHECK(fake_rt_last_hold() == 0);              // the host link is the bound there, not HBM
+    {
+        const uint64_t one = seg * count;          // the same bytes as one segment of 1024 chunks, then as one of 2048
+        uint64_t s1 = src[0], d1 = reinterpret_cast<uint64_t>(to.data()), l1 = one;
+        CHECK(engine.Submit(&s1, &d1, &l1, 1, MF_ROUTE_HBM, stream, nullptr, 0) == BM_OK);
+        CHECK(fake_rt_last_hold() == 0);          // below the 1400 chunks from which a single segment gains
+        std::vector<uint8_t> wider(4 * one);
+        s1 = reinterpret_cast<uint64_t>(wider.data());
+        d1 = s1 + 2 * one;
+        l1 = 2 * one;
+        CHECK(engine.Submit(&s1, &d1, &l1, 1, MF_ROUTE_HBM, stream, nullptr, 0) == BM_OK);
+        CHECK(fake_rt_last_hold() == HoldNanosFor(2048, 2048, 256, true));
+        CHECK(engine.DrainThread() == BM_OK);
+    }
+    {
+        // 5120 chunks: held while this thread is the only submitter, not while a second thread has a stream
+        std::vector<uint8_t> big(40u << 20);
+        uint64_t s5[2], d5[2], l5[2] = {10u << 20, 10u << 20};
+        for (int i = 0; i < 2; ++i) {
+            s5[i] = reinterpret_cast<uint64_t>(big.data()) + (static_cast<uint64_t>(i) << 20) * 10;
+            d5[i] = s5[i] + (20u << 20);
+        }
+        std::swap(d5[0], d5[1]);   // not one run
+        CHECK(engine.Submit(s5, d5, l5, 2, MF_ROUTE_HBM, stream, nullptr, 0) == BM_OK);
+        CHECK(fake_rt_last_hold() == HoldNanosFor(5120, 5120, 256, false));
+        std::atomic<int> phase{0};
+        std::thread other([&] {
+            (void)mf_xcopy_thread_stream();
+            phase.store(1);
+            while (phase.load() != 2) {
+                std::this_thread::yield();
+            }
+        });
+        while (phase.load() != 1) {
+            std::this_thread::yield();
+        }
+        CHECK(engine.Submit(s5, d5, l5, 2, MF_ROUTE_HBM, stream, nullptr, 0) == BM_OK);
+        CHECK(fake_rt_last_hold() == 0);
+        CHECK(engine.Submit(src.data(), dst.data(), len.data(), count, MF_ROUTE_HBM, stream, nullptr, 0) == BM_OK);
+        CHECK(fake_rt_last_hold() == HoldNanosFor(1024, 1024, 256, false));   // small launches keep the wait
+        phase.store(2);
+        other.join();
+        CHECK(engine.Submit(s5, d5, l5, 2, MF_ROUTE_HBM, stream, nullptr, 0) == BM_OK);
+        CHECK(fake_rt_last_hold() == HoldNanosFor(5120, 5120, 256, false));
+        CHECK(engine.DrainThread() == BM_OK);
+    }
+    CHECK(engine.Submit(src.data(), dst.data(), len.data(), count, MF_ROUTE_HBM, stream, nullptr, 0) == BM_OK);
+    CHECK(mf_xcopy_hold_stores(2500) == BM_OK);
+    CHECK(engine.Submit(src.data(), dst.data(), len.data(), count, MF_ROUTE_HBM, stream, nullptr, 0) == BM_OK);
+    CHECK(fake_rt_last_hold() == 2500);
+    CHECK(engine.Submit(src.data(), dst.data(), len.data(), 4, MF_ROUTE_HBM, stream, nullptr, 0) == BM_OK);
+    CHECK(fake_rt_last_hold() == 0);              // 128 chunks: the fixed time applies only where the rule does
+    CHECK(mf_xcopy_hold_stores(0) == BM_OK);
+    CHECK(engine.Submit(src.data(), dst.data(), len.data(), count, MF_ROUTE_HBM, stream, nullptr, 0) == BM_OK);
+    CHECK(fake_rt_last_hold() == 0);
+    CHECK(mf_xcopy_hold_stores(-2) == BM_INVALID_PARAM);
+    CHECK(mf_xcopy_hold_stores(-1) == BM_OK);
+    CHECK(engine.DrainThread() == BM_OK);
+    bool ok = true;
+    for (uint32_t i = 0; i < count; ++i) {
+        ok = ok && std::memcmp(to.data() + (count - 1 - i) * seg, from.data() + i * seg, seg) == 0;
+    }
+    CHECK(ok);
+    hybm_uninit();
+}
+
 int main()
 {
     SetLogLevel(3);
@@ -794,6 +902,7 @@ int main()
     TestLeases();
     TestMappedWindow();
     TestPlugin();
+    TestHeldStores();
     if (g_failed != 0) {
         std::printf("%d check(s) failed\n", g_failed);
         return 1;

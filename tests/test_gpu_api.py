@@ -228,6 +228,44 @@ def test_unordered_batches_and_the_ordered_copy_behind_them(pool, lib, oracle):
         assert np.array_equal(got, expect), rep
 
 
+def test_held_stores_copy_the_same_bytes(pool, lib, oracle):
+    """Batches of 1000 to 5600 chunks wait with their stores (mf_xcopy_hold_stores).  Three ragged batches
+    of that size, each reading what the one before wrote, cycled on one stream, with the library's rule,
+    with no wait and with a wait far longer than any load takes: the same bytes as the oracle applied in
+    order every time (pieces start and end at any byte, so waves with partial chunks wait too)."""
+    dev = pool.peer_rank_ptr(0, bm.BmMemType.DEVICE)
+    region = 12 * MIB
+    n = 3 * region
+    init = _rand(oracle, n, 0xD9)
+    rng = np.random.default_rng(13)
+    tables = []
+    for b in range(3):   # batch b moves 48 ragged pieces (about 7 MB, 1800 chunks) from region b to region (b + 1) % 3
+        lens = rng.integers(100000, 200000, 48)
+        src = b * region + np.cumsum(lens) - lens + rng.integers(0, 7)
+        dst = ((b + 1) % 3) * region + np.cumsum(lens) - lens + rng.integers(0, 7)
+        assert int(lens.sum()) + 7 < region
+        tables.append((src, dst, lens))
+    g2g = bm.BmCopyType.G2G
+    got = np.empty(n, dtype=np.uint8)
+    try:
+        for nanos in (-1, 0, 9000):
+            assert lib.mf_xcopy_hold_stores(nanos) == 0
+            assert lib.mfrt_memcpy(dev, np_ptr(init), n) == 0
+            expect = init.copy()
+            for step in range(7):
+                src, dst, lens = tables[step % 3]
+                assert pool.copy_data_batch((dev + src).tolist(), (dev + dst).tolist(), lens.tolist(), len(lens), g2g,
+                                            native.ASYNC_COPY_FLAG) == 0, native.last_error()
+                before = expect.copy()
+                gpu_util.oracle_batch(oracle, before, expect, src, dst, lens)
+            assert pool.wait() == 0
+            assert lib.mfrt_memcpy(np_ptr(got), dev, n) == 0
+            assert np.array_equal(got, expect), nanos
+    finally:
+        assert lib.mf_xcopy_hold_stores(-1) == 0
+    assert lib.mf_xcopy_hold_stores(-2) != 0
+
+
 def test_replayed_batches_keep_stream_order(pool, lib, oracle):
     """mf_bm_copy_batch_replay issues the same calls a loop would: three batches, each reading what
     the one before wrote, cycled for seven steps on one stream, against the oracle applied in order."""
