@@ -118,6 +118,15 @@ int32_t mf_xcopy_tune(uint32_t units, uint32_t wgPerCu, uint32_t wgPerCuLink);
  * 0 = never wait, otherwise that many ns for every launch the rule would pick.  Other launches, and
  * batches submitted with MF_COPY_UNORDERED_FLAG, never wait. */
 int32_t mf_xcopy_hold_stores(int32_t nanos);
+/* Read and write windows.  A batch of up to 128 segments and 512 MiB or more between HBM addresses is copied
+ * by 4096 waves that alternate, all together and by the GPU's constant-rate clock, between a read half and a
+ * write half of a period, so that HBM sees long bursts of one direction: 6.65-6.75 TB/s instead of 6.1-6.35 on
+ * aligned copies of 512 MiB to 2 GiB, 6.05-6.3 instead of 5.75-5.85 when sources sit at odd addresses.  The
+ * period is cut for a rate of HBM traffic (read + written) in MB/s, 6 800 000 by default; at 7 000 000 the waves
+ * of a 2 GiB copy now and then no longer keep up, the windows dissolve and the copy runs at about the rate it
+ * has without them; at 7 200 000 and above most launches do.  0 switches the form off.  While several threads
+ * submit on streams of their own it is not used. */
+int32_t mf_xcopy_windows(uint32_t megabytesPerSecond);
 uint32_t mf_xcopy_choose_units(uint64_t totalBytes, uint32_t cuCount, int32_t route);
 uint64_t mf_xcopy_launch_count(void);
 

@@ -143,6 +143,15 @@ MF_EXPORT int32_t mf_xcopy_hold_stores(int32_t nanos)
     return BM_OK;
 }
 
+MF_EXPORT int32_t mf_xcopy_windows(uint32_t megabytesPerSecond)
+{
+    if (megabytesPerSecond != 0 && (megabytesPerSecond < 1000000 || megabytesPerSecond > 16000000)) {
+        MF_FAIL(BM_INVALID_PARAM, "windows: 0 (never) or a rate between 1 000 000 and 16 000 000 MB/s, got " << megabytesPerSecond);
+    }
+    XcopyEngine::Instance().Tuning().windowMBps = megabytesPerSecond;
+    return BM_OK;
+}
+
 MF_EXPORT uint32_t mf_xcopy_choose_units(uint64_t totalBytes, uint32_t cuCount, int32_t route)
 {
     return ChooseUnits(totalBytes, cuCount, route, XcopyEngine::Instance().Tuning());

@@ -787,6 +787,7 @@ int XcopyEngine::Submit(const uint64_t *src, const uint64_t *dst, const uint64_t
     bool inlined = false;
     uint32_t units = 0;
     bool oversized = false;      // a run the 32-bit length of the inline table cannot hold is possible
+    bool windowed = false;
     if (n <= 4 * kInlineSegs) {  // small enough that a failed attempt costs next to nothing
         uint64_t total = 0;
         for (uint32_t i = 0; i < n; ++i) {
@@ -794,13 +795,29 @@ int XcopyEngine::Submit(const uint64_t *src, const uint64_t *dst, const uint64_t
         }
         oversized = total > 0xFFFFFFFFull;
         units = ChooseUnits(total, cu, route, tuning_);
+        // Large HBM copies of one submitter: 16 KiB chunks for the kernel that alternates between read and write
+        // windows.  Two such launches at a time would each cut their periods for the whole chip's rate, so a
+        // second thread with a stream of its own switches the form off, as it does for the largest held launches.
+        windowed = route == MFRT_ROUTE_HBM && !unordered && total >= kWindowMinBytes && tuning_.windowMBps != 0 &&
+                   tuning_.unitsOverride == 0 && g_leasesOut.load(std::memory_order_relaxed) <= 1;
+        if (windowed) {
+            units = mfk_xcopy_window_units();
+        }
         inlined = BuildInlineDirect(src, dst, len, n, units, plan);
     }
     if (!inlined && oversized) {
         // a run of 4 GiB and more may have made the one-pass attempt give up: the general inline path cuts it into pieces
         NormalizeSegments(src, dst, len, n, kInlinePiece, ctx.segs);
-        units = ChooseUnits(ctx.segs.totalBytes, cu, route, tuning_);
+        units = windowed ? mfk_xcopy_window_units() : ChooseUnits(ctx.segs.totalBytes, cu, route, tuning_);
         inlined = BuildInlinePlan(ctx.segs, units, plan);
+    }
+    if (inlined && windowed) {
+        int err = mfk_xcopy_windowed(&plan, tuning_.windowMBps, mask, maskValue, stream);
+        if (err != 0) {
+            MF_FAIL(BM_ERROR, "xcopy launch failed: " << mfrt_error_string(err));
+        }
+        g_launches.fetch_add(1, std::memory_order_relaxed);
+        return BM_OK;
     }
     if (inlined) {
         const uint32_t grid = GridFor(plan.nchunk, cu, route, tuning_);

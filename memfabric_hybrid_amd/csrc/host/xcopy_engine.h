@@ -47,7 +47,12 @@ struct XcopyTuning {
     uint32_t wgPerCuLink = 1;    // routes bound by the host link: workgroups per CU
     uint32_t minUnits = kXcopyThreads;   // 4 KiB: the chunk of HBM routes
     int32_t holdNanos = -1;      // stores held back in inline launches: -1 = HoldNanosFor's rule, 0 = never, else that long
+    uint32_t windowMBps = 6800000;   // HBM copies of kWindowMinBytes and more alternate between read and write windows cut for this rate; 0 = never
 };
+
+// From this total on a batch of up to 128 segments between HBM addresses is copied in read and write windows
+// (XcopyWindowKernel has the measurements; 512 MiB gains 2 %, 256 MiB nothing).
+constexpr uint64_t kWindowMinBytes = 512ull << 20;
 
 uint32_t ChooseUnits(uint64_t totalBytes, uint32_t cuCount, int route, const XcopyTuning &tuning);
 

@@ -211,6 +211,164 @@ __global__ __launch_bounds__(kXcopyThreads) void XcopyInlineKernel(const InlineP
     } while (c < nchunk);
 }
 
+// Read and write windows.  A copy that runs for hundreds of microseconds streams faster when the whole chip
+// alternates between reading and writing than when every wave stores as soon as its loads have landed:
+// HBM then sees long bursts of one direction instead of a mix.  The waves need no communication for
+// that, only the constant-rate clock every wave can read: a period is cut into a read half and a write
+// half, wave i of a launch of G waves issues the 16 loads per lane of its next 16 KiB chunk at
+// offset i * (period / 2) / G into the read half, waits for them, and issues the stores at the same
+// offset into the write half.  The period is the time the launch's 2 * G * 16 KiB per round need at a
+// target rate; up to a target the part sustains, the copy simply runs at the pace the clock sets.
+// Measured with a stand-alone kernel of this shape on 1 and 2 GiB (4096 waves: 64 MiB read and 64 MiB
+// written per 18 to 20 us period): target 6.6 / 6.8 / 7.0 / 7.2 / 7.4 TB/s -> 6.39 / 6.59 / 6.7 / 6.97 / 7.15 TB/s
+// achieved, against 6.1-6.2 TB/s for one wave per 4 KiB chunk that stores at once; at 7.6 TB/s the waves no
+// longer keep up, the windows dissolve and the copy falls back to 5.8-6.1 TB/s.  This kernel, which also
+// looks its chunk up in the plan, through smem_bm_copy_batch on a pool, target 6.8 against no windows:
+// 512 MiB 6.65 / 6.34 TB/s, 1 GiB 6.73 / 6.23, 2 GiB 6.6-6.7 / 6.12, 100 segments of about 10 MB at odd addresses
+// 6.28 / 5.84, 3 x 700 MB at odd addresses 6.05 / 5.73; at 6.6 it measures 6.47 / 6.54 / 6.57 / 6.09 / 6.1-6.2, at
+// 7.0 the 2 GiB copy dissolves now and then (6.2-6.3), at 7.2 and above most launches do.  256 MiB gains nothing
+// (the first and the last half period, in which the chip only reads or only writes, cost what the windows
+// gain), 128 MiB loses.  Memory that has never been written copies erratically under windows (6.0 to 6.8 TB/s
+// from one launch to the next); initialised memory does not.  2048 waves dissolve one step earlier than 4096;
+// 4, 8 or 32 loads per lane and windows that are not spread over their half were slower or less stable.  A wave
+// that is late proceeds at once: letting it skip to its slot in a later period made a dissolved launch slower
+// (4.4 instead of 5.7 TB/s).
+constexpr uint32_t kWindowDepth = 16;                       // 128-bit loads per lane and round
+constexpr uint32_t kWindowUnits = 64 * kWindowDepth;        // 16 KiB chunks, one wave each
+constexpr uint32_t kWindowWaves = 4096;                     // 16 per CU
+
+__device__ __forceinline__ void WaitForClock(uint64_t t)
+{
+    while (wall_clock64() < t) {
+        __builtin_amdgcn_s_sleep(1);
+    }
+}
+
+// Copy chunk k (kWindowUnits units) of one segment: loads at `slot`, stores at `slot + half`.  A chunk that is
+// not whole (the last one of a segment, or one with head or tail bytes) goes through CopyChunk in the
+// write half: there are at most two such chunks per segment.
+template <bool kNtLoad, int kStore>
+__device__ __forceinline__ void CopyChunkWindowed(uint64_t src, uint64_t dst, uint64_t len, uint64_t k, uint64_t slot, uint32_t half)
+{
+    const SegGeom g = SegmentGeometry(dst, len);
+    const uint64_t u0 = k * kWindowUnits;
+    const bool whole = u0 + kWindowUnits <= g.body && (k != 0 || g.head == 0) && (u0 + kWindowUnits < g.body || g.tail == 0);
+    WaitForClock(slot);
+    if (!whole) {
+        WaitForClock(slot + half);
+        CopyChunk<kNtLoad, kStore>(src, dst, len, k, kWindowUnits);
+        return;
+    }
+    const uint64_t s = src + g.head + u0 * kUnitBytes + threadIdx.x * kUnitBytes;
+    const uint64_t d = dst + g.head + u0 * kUnitBytes + threadIdx.x * kUnitBytes;
+    u32x4 v[kWindowDepth];
+#pragma unroll
+    for (uint32_t j = 0; j < kWindowDepth; ++j) {
+        v[j] = LoadUnit<kNtLoad>(s + j * 64 * kUnitBytes);
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    WaitForClock(slot + half);
+#pragma unroll
+    for (uint32_t j = 0; j < kWindowDepth; ++j) {
+        StoreUnit<kStore>(d + j * 64 * kUnitBytes, v[j]);
+    }
+}
+
+// Where the waves of a windowed launch agree on the start of their first period: workgroup 0, which the
+// dispatcher starts first, publishes its clock under the launch's sequence number, the others read it.
+// (Deriving the start from the clock alone, as the next multiple of the period, costs every launch half a
+// period on average: 10 us, 3 % of a 1 GiB copy.  Letting whichever wave comes first publish with a
+// compare-and-swap serialises 4096 same-address atomics across the XCDs: 1.2 ms.)  A wave that does not see
+// the value within a few microseconds goes by its own clock, so no wave waits on another for long.  One slot
+// per launch in flight; a slot is reused after kEpochSlots launches.
+constexpr uint32_t kEpochSlots = 64;
+constexpr uint32_t kEpochClockBits = 40;                    // 2^40 ticks of 10 ns: three hours, compared modulo
+constexpr uint32_t kEpochPolls = 64;
+__device__ unsigned long long g_windowEpoch[kEpochSlots];
+#ifdef MF_WINDOW_DEBUG
+__device__ long long g_windowDebug[4096 * 3];
+#endif
+
+__device__ __forceinline__ uint64_t AgreedStart(uint32_t seq)
+{
+    unsigned long long *slot = &g_windowEpoch[seq % kEpochSlots];
+    const unsigned long long tag = static_cast<unsigned long long>(seq & 0xFFFFFFu) << kEpochClockBits;
+    const unsigned long long mask = (1ull << kEpochClockBits) - 1;
+    unsigned long long low = (wall_clock64() + 64) & mask;   // 0.6 us ahead: the first slots of the first waves do not lie in the past
+    if (blockIdx.x == 0) {
+        __hip_atomic_store(slot, tag | low, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    } else {
+        for (uint32_t poll = 0; poll < kEpochPolls; ++poll) {
+            const unsigned long long seen = __hip_atomic_load(slot, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if ((seen & ~mask) == tag) {
+                low = seen & mask;
+                break;
+            }
+            __builtin_amdgcn_s_sleep(4);
+        }
+    }
+    // back to a full clock value near now
+    const uint64_t now = wall_clock64();
+    uint64_t start = (now & ~mask) | low;
+    if (start > now + (mask >> 1)) {
+        start -= mask + 1;
+    } else if (start + (mask >> 1) < now) {
+        start += mask + 1;
+    }
+    return start;
+}
+
+// The inline plan (chunks of kWindowUnits units) copied by gridDim.x single-wave workgroups that walk
+// the chunks with stride gridDim.x, one chunk per period each.
+template <bool kNtLoad, int kStore>
+__global__ __launch_bounds__(64) void XcopyWindowKernel(const InlinePlan p, uint32_t period, uint32_t seq)
+{
+    const uint32_t lane = threadIdx.x & 63u;
+    const uint32_t f0 = p.first[lane];
+    const uint32_t f1 = p.first[lane + 64];
+    const uint64_t s0 = p.src[lane];
+    const uint64_t s1 = p.src[lane + 64];
+    const uint64_t d0 = p.dst[lane];
+    const uint64_t d1 = p.dst[lane + 64];
+    const uint32_t l0 = p.len[lane];
+    const uint32_t l1 = p.len[lane + 64];
+    const uint32_t nchunk = p.nchunk;
+    const uint32_t half = period / 2;
+#ifdef MF_WINDOW_DEBUG
+    const uint64_t dbgT0 = wall_clock64();
+#endif
+    uint64_t slot = AgreedStart(seq) + static_cast<uint64_t>(blockIdx.x) * half / gridDim.x;
+#ifdef MF_WINDOW_DEBUG
+    if (lane == 0 && blockIdx.x < 4096) {
+        g_windowDebug[blockIdx.x * 3] = static_cast<long long>(slot - static_cast<uint64_t>(blockIdx.x) * half / gridDim.x);
+        g_windowDebug[blockIdx.x * 3 + 1] = static_cast<long long>(dbgT0);
+        g_windowDebug[blockIdx.x * 3 + 2] = static_cast<long long>(wall_clock64());
+    }
+#endif
+    for (uint32_t c = blockIdx.x; c < nchunk; c += gridDim.x) {
+        const uint32_t below = __popcll(__ballot(f0 <= c)) + __popcll(__ballot(f1 <= c));
+        const uint32_t s = below - 1;
+        const uint32_t row = s & 63u;
+        uint64_t src;
+        uint64_t dst;
+        uint32_t len;
+        uint32_t first;
+        if (s < 64) {
+            src = ReadLane64(s0, row);
+            dst = ReadLane64(d0, row);
+            len = __builtin_amdgcn_readlane(l0, row);
+            first = __builtin_amdgcn_readlane(f0, row);
+        } else {
+            src = ReadLane64(s1, row);
+            dst = ReadLane64(d1, row);
+            len = __builtin_amdgcn_readlane(l1, row);
+            first = __builtin_amdgcn_readlane(f1, row);
+        }
+        CopyChunkWindowed<kNtLoad, kStore>(src, dst, len, c - first, slot, half);
+        slot += period;
+    }
+}
+
 // A single segment needs no table: its three words travel as plain kernel arguments (28 bytes
 // instead of the 3080-byte plan), which is cheaper for the host to hand over and spares every
 // wave the table fetch.  Measured against the table form on one box: an 8 MiB copy 13.7 us instead
@@ -432,6 +590,30 @@ int LaunchInline(const InlinePlan &plan, uint32_t grid, uint32_t lanes, hipStrea
     return static_cast<int>(hipGetLastError());
 }
 
+// windowMBps: the rate (MB/s of HBM traffic, read + written) the period of a windowed launch is cut for.
+template <bool kNtLoad, int kStore>
+int LaunchWindowed(const InlinePlan &plan, uint32_t grid, uint32_t windowMBps, hipStream_t stream)
+{
+    int dev = 0;
+    int khz = 0;
+    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&khz, hipDeviceAttributeWallClockRate, dev) != hipSuccess || khz <= 0) {
+        return static_cast<int>(hipErrorInvalidDevice);
+    }
+    // bytes per round / (MB/s) = microseconds; ticks = microseconds * kHz / 1000
+    const uint64_t bytes = 2ull * grid * kWindowUnits * kUnitBytes;
+    const uint64_t ticks = bytes * static_cast<uint64_t>(khz) / (static_cast<uint64_t>(windowMBps) * 1000u);
+    if (ticks < 16 || ticks > 1000000) {
+        return static_cast<int>(hipErrorInvalidValue);
+    }
+    static std::atomic<uint32_t> launches{0};
+    uint32_t seq;
+    do {
+        seq = launches.fetch_add(1, std::memory_order_relaxed) + 1;
+    } while ((seq & 0xFFFFFFu) == 0);   // the 24 bits the kernel compares are never 0, which is what an untouched slot holds
+    hipLaunchKernelGGL((XcopyWindowKernel<kNtLoad, kStore>), dim3(grid), dim3(64), 0, stream, plan, static_cast<uint32_t>(ticks), seq);
+    return static_cast<int>(hipGetLastError());
+}
+
 template <bool kNtLoad, int kStore>
 int LaunchTable(const TablePlan &plan, const uint32_t *nchunkDev, uint32_t grid, uint32_t lanes, hipStream_t stream)
 {
@@ -469,6 +651,30 @@ extern "C" int mfk_xcopy_inline(const void *inlinePlan, int route, uint32_t grid
     const int err = mf::WithPolicy(mf::PolicyOf(route), [&](auto ntLoad, auto store) {
         return mf::LaunchInline<decltype(ntLoad)::value, decltype(store)::value>(plan, grid, mf::LanesFor(plan.units, route), s,
                                                                                  anyOrder != 0, holdNanos);
+    });
+    return err != 0 ? err : mf::Signal(mask, maskValue, s);
+}
+
+extern "C" uint32_t mfk_xcopy_window_units(void)
+{
+    return mf::kWindowUnits;
+}
+
+extern "C" uint32_t mfk_xcopy_window_waves(void)
+{
+    return mf::kWindowWaves;
+}
+
+extern "C" int mfk_xcopy_windowed(const void *inlinePlan, uint32_t windowMBps, void *mask, uint32_t maskValue, void *stream)
+{
+    const mf::InlinePlan &plan = *static_cast<const mf::InlinePlan *>(inlinePlan);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (plan.units != mf::kWindowUnits || plan.nchunk == 0 || windowMBps == 0) {
+        return -1;
+    }
+    const uint32_t grid = plan.nchunk < mf::kWindowWaves ? plan.nchunk : mf::kWindowWaves;
+    const int err = mf::WithPolicy(mf::PolicyOf(MFRT_ROUTE_HBM), [&](auto ntLoad, auto store) {
+        return mf::LaunchWindowed<decltype(ntLoad)::value, decltype(store)::value>(plan, grid, windowMBps, s);
     });
     return err != 0 ? err : mf::Signal(mask, maskValue, s);
 }

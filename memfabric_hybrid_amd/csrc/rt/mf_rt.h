@@ -75,6 +75,12 @@ int mfrt_memcpy_async(void *dst, const void *src, uint64_t bytes, void *stream);
  * kernels/xcopy_plan.h); honoured only by a launch of one 4 KiB chunk per workgroup. */
 int mfk_xcopy_inline(const void *inlinePlan, int route, uint32_t grid, void *mask, uint32_t maskValue, void *stream,
                      int anyOrder, uint32_t holdNanos);
+/* HBM to HBM copies of hundreds of MiB: the plan's chunks are mfk_xcopy_window_units() units (16 KiB), copied by up to
+ * mfk_xcopy_window_waves() single-wave workgroups that alternate, chip-wide and by the clock, between a read half and a
+ * write half of a period cut for `windowMBps` MB/s of HBM traffic (see XcopyWindowKernel). */
+uint32_t mfk_xcopy_window_units(void);
+uint32_t mfk_xcopy_window_waves(void);
+int mfk_xcopy_windowed(const void *inlinePlan, uint32_t windowMBps, void *mask, uint32_t maskValue, void *stream);
 /* pattern: NULL, or a mf::ChunkPattern (kernels/xcopy_plan.h) that the chunk counts of the segments follow;
  * then `first` is not read (may be NULL) and `triples` may live in pinned host memory. */
 int mfk_xcopy_table(const void *triples, const void *first, const void *nchunkDev, uint32_t nseg, uint32_t nchunk,

@@ -192,6 +192,7 @@ _SIGNATURES = {
     "mf_xcopy_thread_stream": (vp, []),
     "mf_xcopy_tune": (i32, [u32, u32, u32]),
     "mf_xcopy_hold_stores": (i32, [i32]),
+    "mf_xcopy_windows": (i32, [u32]),
     "mf_xcopy_choose_units": (u32, [u64, u32, i32]),
     "mf_xcopy_launch_count": (u64, []),
     "mf_xcopy_describe_plan": (i64, [u64p, u64p, u64p, u32, u32, u64p, u64, ctypes.POINTER(i32)]),

@@ -23,7 +23,8 @@ std::mutex g_lock;
 std::map<uint64_t, std::pair<uint64_t, int>> g_allocs;  // base -> (size, kind)
 int g_device = -1;
 uint64_t g_launches = 0;
-uint32_t g_lastHold = 0;     // holdNanos of the latest inline launch
+uint32_t g_lastHold = 0;
+uint32_t g_lastWindow = 0;   // rate of the latest windowed launch, cleared by fake_rt_last_window()     // holdNanos of the latest inline launch
 uint64_t g_chunksRun = 0;
 
 void *Track(uint64_t bytes, int kind)
@@ -122,6 +123,7 @@ static void Guard(const char *what)
 }
 uint64_t fake_rt_launches(void) { return g_launches; }
 uint32_t fake_rt_last_hold(void) { return g_lastHold; }
+uint32_t fake_rt_last_window(void) { const uint32_t w = g_lastWindow; g_lastWindow = 0; return w; }
 // The next n xcopy launches fail with a runtime error code instead of running.
 static int g_failLaunches = 0;
 void fake_rt_fail_launches(int n) { g_failLaunches = n; }
@@ -240,6 +242,18 @@ int mfk_xcopy_inline(const void *inlinePlan, int, uint32_t, void *mask, uint32_t
         *static_cast<uint64_t *>(mask) = maskValue;
     }
     return 0;
+}
+
+uint32_t mfk_xcopy_window_units(void) { return 1024; }
+uint32_t mfk_xcopy_window_waves(void) { return 4096; }
+int mfk_xcopy_windowed(const void *inlinePlan, uint32_t windowMBps, void *mask, uint32_t maskValue, void *stream)
+{
+    const mf::InlinePlan &p = *static_cast<const mf::InlinePlan *>(inlinePlan);
+    if (p.units != 1024 || p.nchunk == 0 || windowMBps == 0) {
+        return -1;
+    }
+    g_lastWindow = windowMBps;
+    return mfk_xcopy_inline(inlinePlan, 0, p.nchunk, mask, maskValue, stream, 0, 0);
 }
 
 int mfk_xcopy_table(const void *triples, const void *first, const void *nchunkDev, uint32_t nseg, uint32_t nchunk,

@@ -21,6 +21,7 @@
 
 extern "C" uint64_t fake_rt_launches(void);
 extern "C" uint32_t fake_rt_last_hold(void);
+extern "C" uint32_t fake_rt_last_window(void);
 extern "C" void fake_rt_seal(void);
 extern "C" void fake_rt_fail_launches(int n);
 #include "../../include/mf_hip_copy_extend.h"
@@ -886,6 +887,63 @@ static void TestHeldStores()
     hybm_uninit();
 }
 
+// Which batches take the form with read and write windows.
+static void TestWindows()
+{
+    CHECK(hybm_init(0, 0) == BM_OK);
+    const uint64_t gib = 1ull << 30;
+    std::vector<uint8_t> mem(2 * gib + 64);
+    for (uint64_t i = 0; i < gib; i += 4093) {
+        mem[i] = static_cast<uint8_t>(i * 7 + 1);
+    }
+    XcopyEngine &engine = XcopyEngine::Instance();
+    void *stream = mf_xcopy_thread_stream();
+    uint64_t s1 = reinterpret_cast<uint64_t>(mem.data());
+    uint64_t d1 = s1 + gib + 3;                    // an odd destination: head and tail bytes
+    uint64_t l1 = gib;
+    (void)fake_rt_last_window();
+    CHECK(engine.Submit(&s1, &d1, &l1, 1, MF_ROUTE_HBM, stream, nullptr, 0) == BM_OK);
+    CHECK(fake_rt_last_window() == 6800000);
+    CHECK(engine.DrainThread() == BM_OK);
+    bool ok = true;
+    for (uint64_t i = 0; i < gib; i += 4093) {
+        ok = ok && mem[gib + 3 + i] == static_cast<uint8_t>(i * 7 + 1);
+    }
+    CHECK(ok && mem[gib + 3 + gib - 1] == mem[gib - 1]);
+    l1 = (gib >> 1) - 1;                           // one byte below the limit: the ordinary form
+    CHECK(engine.Submit(&s1, &d1, &l1, 1, MF_ROUTE_HBM, stream, nullptr, 0) == BM_OK);
+    CHECK(fake_rt_last_window() == 0);
+    l1 = gib;
+    CHECK(engine.Submit(&s1, &d1, &l1, 1, MF_ROUTE_HBM, stream, nullptr, 0, true) == BM_OK);
+    CHECK(fake_rt_last_window() == 0);             // unordered launches overlap on purpose
+    CHECK(mf_xcopy_windows(0) == BM_OK);
+    CHECK(engine.Submit(&s1, &d1, &l1, 1, MF_ROUTE_HBM, stream, nullptr, 0) == BM_OK);
+    CHECK(fake_rt_last_window() == 0);
+    CHECK(mf_xcopy_windows(999) == BM_INVALID_PARAM && mf_xcopy_windows(6400000) == BM_OK);
+    {
+        std::atomic<int> phase{0};
+        std::thread other([&] {
+            (void)mf_xcopy_thread_stream();
+            phase.store(1);
+            while (phase.load() != 2) {
+                std::this_thread::yield();
+            }
+        });
+        while (phase.load() != 1) {
+            std::this_thread::yield();
+        }
+        CHECK(engine.Submit(&s1, &d1, &l1, 1, MF_ROUTE_HBM, stream, nullptr, 0) == BM_OK);
+        CHECK(fake_rt_last_window() == 0);         // a second submitter with a stream of its own
+        phase.store(2);
+        other.join();
+    }
+    CHECK(engine.Submit(&s1, &d1, &l1, 1, MF_ROUTE_HBM, stream, nullptr, 0) == BM_OK);
+    CHECK(fake_rt_last_window() == 6400000);
+    CHECK(mf_xcopy_windows(6800000) == BM_OK);
+    CHECK(engine.DrainThread() == BM_OK);
+    hybm_uninit();
+}
+
 int main()
 {
     SetLogLevel(3);
@@ -903,6 +961,7 @@ int main()
     TestMappedWindow();
     TestPlugin();
     TestHeldStores();
+    TestWindows();
     if (g_failed != 0) {
         std::printf("%d check(s) failed\n", g_failed);
         return 1;

@@ -80,6 +80,52 @@ def test_single_copies_at_full_size_host_device_device_host(pool, lib, oracle, n
     assert _same_as_pattern(host_all[back_off:back_off + nbytes], block)
 
 
+@pytest.mark.parametrize("rate", [-1, 7400000, 0], ids=["default-windows", "short-periods", "no-windows"])
+def test_ragged_batch_above_one_gib_in_read_and_write_windows(pool, lib, oracle, rate):
+    """A device-to-device batch of 1 GiB and more goes through the kernel that alternates between read and
+    write windows.  Seven pieces of about 170 MB with odd lengths at odd source and destination addresses
+    (partial first and last chunks, head and tail bytes), with the default period, with a period too short
+    for the waves to keep up (they then proceed late; the result must not depend on timing) and with the
+    form switched off: what comes back equals the same slices cut on the CPU, and the bytes between and
+    round the destinations are untouched."""
+    dev = pool.peer_rank_ptr(0, bm.BmMemType.DEVICE)
+    host = pool.peer_rank_ptr(0, bm.BmMemType.HOST)
+    span = 2 * GIB + GUARD
+    host_all = gpu_util.host_view(host, 2 * span + GUARD)
+    block = _pattern_block(oracle)
+    total = GIB + 256 * MIB
+    _fill_pattern(host_all[GUARD:GUARD + total], block)
+    g2g = bm.BmCopyType.G2G
+    assert pool.copy_data(host + GUARD, dev + GUARD, total, g2g) == 0, native.last_error()
+    assert lib.mfrt_memset(dev + span, 0x5A, span) == 0
+    rng = np.random.default_rng(21)
+    lens = rng.integers(160 * MIB, 175 * MIB, 7) | 1                       # odd lengths
+    gaps = rng.integers(1, 4096, 7) | 1
+    src = GUARD + np.cumsum(lens + gaps) - lens                            # odd addresses
+    dst = span + GUARD + np.cumsum(lens + 2 * gaps + 1) - lens
+    assert int(lens.sum()) >= GIB and int(src[-1] + lens[-1]) <= GUARD + total
+    assert int(dst[-1] + lens[-1]) + GUARD <= 2 * span + GUARD
+    try:
+        if rate >= 0:
+            assert lib.mf_xcopy_windows(rate) == 0
+        assert pool.copy_data_batch((dev + src).tolist(), (dev + dst).tolist(), lens.tolist(), len(lens), g2g, 0) == 0, \
+            native.last_error()
+    finally:
+        assert lib.mf_xcopy_windows(6800000) == 0
+    assert lib.mf_xcopy_windows(999) != 0
+    lo, hi = int(dst[0]) - GUARD, int(dst[-1] + lens[-1]) + GUARD
+    back = span + GUARD                                                    # the second host region
+    assert hi - lo <= span
+    assert pool.copy_data(dev + lo, host + back, hi - lo, g2g) == 0, native.last_error()
+    got = host_all[back:back + hi - lo]
+    cursor = lo
+    for s_off, d_off, n in zip(src.tolist(), dst.tolist(), lens.tolist()):
+        assert np.all(got[cursor - lo:d_off - lo] == 0x5A), d_off          # the gap in front of the piece
+        assert np.array_equal(got[d_off - lo:d_off - lo + n], host_all[s_off:s_off + n]), d_off
+        cursor = d_off + n
+    assert np.all(got[cursor - lo:] == 0x5A)
+
+
 def test_paged_gather_and_scatter_on_a_40_gib_pool(lib, oracle):
     """4096 distinct 32 KiB pages sampled from a 40 GiB HBM pool (offsets far beyond 32 bits):
     gather equals the sampled pages in order; scattering them to 4096 other pages and gathering
