@@ -595,6 +595,7 @@ def extras_reshard(lib):
     sp, dp = lib.mfrt_alloc_device(s_bytes), lib.mfrt_alloc_device(d_bytes)
     if not sp or not dp:
         return {"error": "allocation failed"}
+    lib.mfrt_memset(sp, 0x5A, s_bytes)   # weights that were written at some point, as a checkpoint in HBM is
     segments, rects = workloads.reshard_plan(tensors, layers, sp, dp)
     s_arr = native.u64_array([s for s, _, _ in segments])
     d_arr = native.u64_array([d for _, d, _ in segments])

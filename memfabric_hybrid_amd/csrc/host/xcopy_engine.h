@@ -53,6 +53,7 @@ struct XcopyTuning {
 // From this total on a batch of up to 128 segments between HBM addresses is copied in read and write windows
 // (XcopyWindowKernel has the measurements; 512 MiB gains 2 %, 256 MiB nothing).
 constexpr uint64_t kWindowMinBytes = 512ull << 20;
+constexpr uint64_t kWindowSliceMinSegmentBytes = 4ull << 20;   // tables of segments this long on average are cut into windowed launches
 
 uint32_t ChooseUnits(uint64_t totalBytes, uint32_t cuCount, int route, const XcopyTuning &tuning);
 

@@ -941,6 +941,24 @@ static void TestWindows()
     CHECK(fake_rt_last_window() == 6400000);
     CHECK(mf_xcopy_windows(6800000) == BM_OK);
     CHECK(engine.DrainThread() == BM_OK);
+    {
+        // a table of long segments is cut into launches of 128 segments, each in windows: 300 x 4 MiB -> 128 + 128 + 44
+        const uint32_t count = 300;
+        const uint64_t seg = 4ull << 20;
+        std::vector<uint64_t> src(count), dst(count), len(count, seg);
+        for (uint32_t i = 0; i < count; ++i) {
+            src[i] = reinterpret_cast<uint64_t>(mem.data()) + (i % 200) * seg + i;     // not adjacent: no merging
+            dst[i] = reinterpret_cast<uint64_t>(mem.data()) + gib + ((i * 7) % 200) * seg + 2 * i;
+        }
+        const uint64_t before = mf_xcopy_launch_count();
+        (void)fake_rt_last_window();
+        uint64_t word = 0;
+        CHECK(engine.Submit(src.data(), dst.data(), len.data(), count, MF_ROUTE_HBM, stream, &word, 32) == BM_OK);
+        CHECK(mf_xcopy_launch_count() - before == 3);
+        CHECK(fake_rt_last_window() == 6800000);   // the two full slices (512 MiB each) went in windows; the last one (176 MiB) is below the limit
+        CHECK(word == 32);
+        CHECK(engine.DrainThread() == BM_OK);
+    }
     hybm_uninit();
 }
 

@@ -80,14 +80,16 @@ def test_single_copies_at_full_size_host_device_device_host(pool, lib, oracle, n
     assert _same_as_pattern(host_all[back_off:back_off + nbytes], block)
 
 
+@pytest.mark.parametrize("pieces", [7, 200], ids=["7-pieces", "200-pieces"])
 @pytest.mark.parametrize("rate", [-1, 7400000, 0], ids=["default-windows", "short-periods", "no-windows"])
-def test_ragged_batch_above_one_gib_in_read_and_write_windows(pool, lib, oracle, rate):
+def test_ragged_batch_above_one_gib_in_read_and_write_windows(pool, lib, oracle, rate, pieces):
     """A device-to-device batch of 1 GiB and more goes through the kernel that alternates between read and
-    write windows.  Seven pieces of about 170 MB with odd lengths at odd source and destination addresses
-    (partial first and last chunks, head and tail bytes), with the default period, with a period too short
-    for the waves to keep up (they then proceed late; the result must not depend on timing) and with the
-    form switched off: what comes back equals the same slices cut on the CPU, and the bytes between and
-    round the destinations are untouched."""
+    write windows.  Seven pieces of about 170 MB, or 200 of about 6 MB (a table that the engine cuts into
+    launches of 128 segments), with odd lengths at odd source and destination addresses (partial first and
+    last chunks, head and tail bytes), with the default period, with a period too short for the waves to
+    keep up (they then proceed late; the result must not depend on timing) and with the form switched off:
+    what comes back equals the same slices cut on the CPU, and the bytes between and round the destinations
+    are untouched."""
     dev = pool.peer_rank_ptr(0, bm.BmMemType.DEVICE)
     host = pool.peer_rank_ptr(0, bm.BmMemType.HOST)
     span = 2 * GIB + GUARD
@@ -99,8 +101,9 @@ def test_ragged_batch_above_one_gib_in_read_and_write_windows(pool, lib, oracle,
     assert pool.copy_data(host + GUARD, dev + GUARD, total, g2g) == 0, native.last_error()
     assert lib.mfrt_memset(dev + span, 0x5A, span) == 0
     rng = np.random.default_rng(21)
-    lens = rng.integers(160 * MIB, 175 * MIB, 7) | 1                       # odd lengths
-    gaps = rng.integers(1, 4096, 7) | 1
+    each = (GIB + 100 * MIB) // pieces
+    lens = rng.integers(each - each // 20, each + each // 25, pieces) | 1  # odd lengths
+    gaps = rng.integers(1, 4096, pieces) | 1
     src = GUARD + np.cumsum(lens + gaps) - lens                            # odd addresses
     dst = span + GUARD + np.cumsum(lens + 2 * gaps + 1) - lens
     assert int(lens.sum()) >= GIB and int(src[-1] + lens[-1]) <= GUARD + total
