@@ -227,7 +227,7 @@ def kernel_source_digest():
     """Names the kernel sources a counter summary was measured on."""
     import hashlib
     h = hashlib.sha256()
-    for name in ("xcopy.hip", "xcopy_plan.h"):
+    for name in ("xcopy.hip", "xcopy_plan.h", "window_clock.h"):
         with open(os.path.join(ROOT, "memfabric_hybrid_amd", "csrc", "kernels", name), "rb") as f:
             h.update(f.read())
     return h.hexdigest()[:16]

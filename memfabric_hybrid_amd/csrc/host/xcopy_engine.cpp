@@ -766,6 +766,14 @@ uint32_t XcopyEngine::HoldFor(const InlinePlan &plan, uint32_t grid, int route, 
     return rule != 0 && tuning_.holdNanos > 0 ? static_cast<uint32_t>(tuning_.holdNanos) : rule;
 }
 
+bool XcopyEngine::WindowsApply(uint64_t bytes, int route) const
+{
+    // Two such launches at a time would each cut their periods for the whole chip's rate, so a second thread with a
+    // stream of its own switches the form off, as it does for the largest held launches.
+    return route == MFRT_ROUTE_HBM && bytes >= kWindowMinBytes && tuning_.windowMBps != 0 && tuning_.unitsOverride == 0 &&
+           g_leasesOut.load(std::memory_order_relaxed) <= 1;
+}
+
 int XcopyEngine::Submit(const uint64_t *src, const uint64_t *dst, const uint64_t *len, uint32_t n, int route,
                         void *stream, void *mask, uint32_t maskValue, bool unordered)
 {
@@ -795,11 +803,8 @@ int XcopyEngine::Submit(const uint64_t *src, const uint64_t *dst, const uint64_t
         }
         oversized = total > 0xFFFFFFFFull;
         units = ChooseUnits(total, cu, route, tuning_);
-        // Large HBM copies of one submitter: 16 KiB chunks for the kernel that alternates between read and write
-        // windows.  Two such launches at a time would each cut their periods for the whole chip's rate, so a
-        // second thread with a stream of its own switches the form off, as it does for the largest held launches.
-        windowed = route == MFRT_ROUTE_HBM && !unordered && total >= kWindowMinBytes && tuning_.windowMBps != 0 &&
-                   tuning_.unitsOverride == 0 && g_leasesOut.load(std::memory_order_relaxed) <= 1;
+        // Large HBM copies of one submitter: 16 KiB chunks for the kernel that alternates between read and write windows.
+        windowed = !unordered && WindowsApply(total, route);
         if (windowed) {
             units = mfk_xcopy_window_units();
         }

@@ -89,6 +89,9 @@ public:
         return tuning_;
     }
 
+    // Whether an ordered launch that moves `bytes` on `route` takes the form with read and write windows.
+    bool WindowsApply(uint64_t bytes, int route) const;
+
     // The calling thread's own stream (created on first use).
     void *ThreadStream();
     // Pinned, device-mapped staging memory of the calling thread, at least `bytes` long; it lives
@@ -129,6 +132,7 @@ private:
     XcopyEngine() = default;
 
     uint32_t HoldFor(const InlinePlan &plan, uint32_t grid, int route, bool unordered) const;
+
     XcopyTuning tuning_;
     std::atomic<bool> started_{false};   // read by every calling thread, flipped by Start / Stop
 };

@@ -23,6 +23,7 @@
 #include <cstdlib>
 
 #include "xcopy_plan.h"
+#include "window_clock.h"
 #include "../rt/mf_rt.h"
 
 namespace mf {
@@ -237,13 +238,6 @@ constexpr uint32_t kWindowDepth = 16;                       // 128-bit loads per
 constexpr uint32_t kWindowUnits = 64 * kWindowDepth;        // 16 KiB chunks, one wave each
 constexpr uint32_t kWindowWaves = 4096;                     // 16 per CU
 
-__device__ __forceinline__ void WaitForClock(uint64_t t)
-{
-    while (wall_clock64() < t) {
-        __builtin_amdgcn_s_sleep(1);
-    }
-}
-
 // Copy chunk k (kWindowUnits units) of one segment: loads at `slot`, stores at `slot + half`.  A chunk that is
 // not whole (the last one of a segment, or one with head or tail bytes) goes through CopyChunk in the
 // write half: there are at most two such chunks per segment.
@@ -274,50 +268,6 @@ __device__ __forceinline__ void CopyChunkWindowed(uint64_t src, uint64_t dst, ui
     }
 }
 
-// Where the waves of a windowed launch agree on the start of their first period: workgroup 0, which the
-// dispatcher starts first, publishes its clock under the launch's sequence number, the others read it.
-// (Deriving the start from the clock alone, as the next multiple of the period, costs every launch half a
-// period on average: 10 us, 3 % of a 1 GiB copy.  Letting whichever wave comes first publish with a
-// compare-and-swap serialises 4096 same-address atomics across the XCDs: 1.2 ms.)  A wave that does not see
-// the value within a few microseconds goes by its own clock, so no wave waits on another for long.  One slot
-// per launch in flight; a slot is reused after kEpochSlots launches.
-constexpr uint32_t kEpochSlots = 64;
-constexpr uint32_t kEpochClockBits = 40;                    // 2^40 ticks of 10 ns: three hours, compared modulo
-constexpr uint32_t kEpochPolls = 64;
-__device__ unsigned long long g_windowEpoch[kEpochSlots];
-#ifdef MF_WINDOW_DEBUG
-__device__ long long g_windowDebug[4096 * 3];
-#endif
-
-__device__ __forceinline__ uint64_t AgreedStart(uint32_t seq)
-{
-    unsigned long long *slot = &g_windowEpoch[seq % kEpochSlots];
-    const unsigned long long tag = static_cast<unsigned long long>(seq & 0xFFFFFFu) << kEpochClockBits;
-    const unsigned long long mask = (1ull << kEpochClockBits) - 1;
-    unsigned long long low = (wall_clock64() + 64) & mask;   // 0.6 us ahead: the first slots of the first waves do not lie in the past
-    if (blockIdx.x == 0) {
-        __hip_atomic_store(slot, tag | low, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    } else {
-        for (uint32_t poll = 0; poll < kEpochPolls; ++poll) {
-            const unsigned long long seen = __hip_atomic_load(slot, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            if ((seen & ~mask) == tag) {
-                low = seen & mask;
-                break;
-            }
-            __builtin_amdgcn_s_sleep(4);
-        }
-    }
-    // back to a full clock value near now
-    const uint64_t now = wall_clock64();
-    uint64_t start = (now & ~mask) | low;
-    if (start > now + (mask >> 1)) {
-        start -= mask + 1;
-    } else if (start + (mask >> 1) < now) {
-        start += mask + 1;
-    }
-    return start;
-}
-
 // The inline plan (chunks of kWindowUnits units) copied by gridDim.x single-wave workgroups that walk
 // the chunks with stride gridDim.x, one chunk per period each.
 template <bool kNtLoad, int kStore>
@@ -334,17 +284,7 @@ __global__ __launch_bounds__(64) void XcopyWindowKernel(const InlinePlan p, uint
     const uint32_t l1 = p.len[lane + 64];
     const uint32_t nchunk = p.nchunk;
     const uint32_t half = period / 2;
-#ifdef MF_WINDOW_DEBUG
-    const uint64_t dbgT0 = wall_clock64();
-#endif
     uint64_t slot = AgreedStart(seq) + static_cast<uint64_t>(blockIdx.x) * half / gridDim.x;
-#ifdef MF_WINDOW_DEBUG
-    if (lane == 0 && blockIdx.x < 4096) {
-        g_windowDebug[blockIdx.x * 3] = static_cast<long long>(slot - static_cast<uint64_t>(blockIdx.x) * half / gridDim.x);
-        g_windowDebug[blockIdx.x * 3 + 1] = static_cast<long long>(dbgT0);
-        g_windowDebug[blockIdx.x * 3 + 2] = static_cast<long long>(wall_clock64());
-    }
-#endif
     for (uint32_t c = blockIdx.x; c < nchunk; c += gridDim.x) {
         const uint32_t below = __popcll(__ballot(f0 <= c)) + __popcll(__ballot(f1 <= c));
         const uint32_t s = below - 1;
@@ -594,23 +534,11 @@ int LaunchInline(const InlinePlan &plan, uint32_t grid, uint32_t lanes, hipStrea
 template <bool kNtLoad, int kStore>
 int LaunchWindowed(const InlinePlan &plan, uint32_t grid, uint32_t windowMBps, hipStream_t stream)
 {
-    int dev = 0;
-    int khz = 0;
-    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&khz, hipDeviceAttributeWallClockRate, dev) != hipSuccess || khz <= 0) {
-        return static_cast<int>(hipErrorInvalidDevice);
-    }
-    // bytes per round / (MB/s) = microseconds; ticks = microseconds * kHz / 1000
-    const uint64_t bytes = 2ull * grid * kWindowUnits * kUnitBytes;
-    const uint64_t ticks = bytes * static_cast<uint64_t>(khz) / (static_cast<uint64_t>(windowMBps) * 1000u);
-    if (ticks < 16 || ticks > 1000000) {
+    const uint32_t ticks = WindowPeriodTicks(2ull * grid * kWindowUnits * kUnitBytes, windowMBps);
+    if (ticks == 0) {
         return static_cast<int>(hipErrorInvalidValue);
     }
-    static std::atomic<uint32_t> launches{0};
-    uint32_t seq;
-    do {
-        seq = launches.fetch_add(1, std::memory_order_relaxed) + 1;
-    } while ((seq & 0xFFFFFFu) == 0);   // the 24 bits the kernel compares are never 0, which is what an untouched slot holds
-    hipLaunchKernelGGL((XcopyWindowKernel<kNtLoad, kStore>), dim3(grid), dim3(64), 0, stream, plan, static_cast<uint32_t>(ticks), seq);
+    hipLaunchKernelGGL((XcopyWindowKernel<kNtLoad, kStore>), dim3(grid), dim3(64), 0, stream, plan, ticks, NextWindowSeq());
     return static_cast<int>(hipGetLastError());
 }
 
