@@ -30,35 +30,45 @@ __device__ __forceinline__ void WaitForClock(uint64_t t)
 constexpr uint32_t kEpochSlots = 64;
 constexpr uint32_t kEpochClockBits = 40;                    // 2^40 ticks of 10 ns: three hours, compared modulo
 constexpr uint32_t kEpochPolls = 64;
+constexpr uint32_t kEpochFreshTicks = 2000;                 // workgroup 0 starts at most 20 us before any other wave of its launch
 __device__ unsigned long long g_windowEpoch[kEpochSlots];
+
+// A clock value whose low kEpochClockBits bits are `low`, the one nearest to `now`.
+__device__ __forceinline__ uint64_t NearClock(uint64_t now, unsigned long long low)
+{
+    const unsigned long long mask = (1ull << kEpochClockBits) - 1;
+    uint64_t t = (now & ~mask) | low;
+    if (t > now + (mask >> 1)) {
+        t -= mask + 1;
+    } else if (t + (mask >> 1) < now) {
+        t += mask + 1;
+    }
+    return t;
+}
 
 __device__ __forceinline__ uint64_t AgreedStart(uint32_t seq)
 {
     unsigned long long *slot = &g_windowEpoch[seq % kEpochSlots];
     const unsigned long long tag = static_cast<unsigned long long>(seq & 0xFFFFFFu) << kEpochClockBits;
     const unsigned long long mask = (1ull << kEpochClockBits) - 1;
-    unsigned long long low = (wall_clock64() + 64) & mask;   // 0.6 us ahead: the first slots of the first waves do not lie in the past
+    const uint64_t mine = wall_clock64() + 64;   // 0.6 us ahead: the first slots of the first waves do not lie in the past
     if (blockIdx.x == 0) {
-        __hip_atomic_store(slot, tag | low, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    } else {
-        for (uint32_t poll = 0; poll < kEpochPolls; ++poll) {
-            const unsigned long long seen = __hip_atomic_load(slot, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            if ((seen & ~mask) == tag) {
-                low = seen & mask;
-                break;
+        __hip_atomic_store(slot, tag | (mine & mask), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        return mine;
+    }
+    for (uint32_t poll = 0; poll < kEpochPolls; ++poll) {
+        const unsigned long long seen = __hip_atomic_load(slot, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if ((seen & ~mask) == tag) {
+            // A start that lies long before this wave's own is not this launch's: a launch replayed from a HIP graph
+            // carries the sequence number it was captured with and finds the start of the replay before.
+            const uint64_t start = NearClock(mine, seen & mask);
+            if (start + kEpochFreshTicks >= mine) {
+                return start;
             }
-            __builtin_amdgcn_s_sleep(4);
         }
+        __builtin_amdgcn_s_sleep(4);
     }
-    // back to a full clock value near now
-    const uint64_t now = wall_clock64();
-    uint64_t start = (now & ~mask) | low;
-    if (start > now + (mask >> 1)) {
-        start -= mask + 1;
-    } else if (start + (mask >> 1) < now) {
-        start += mask + 1;
-    }
-    return start;
+    return mine;
 }
 
 // Period (ticks of the constant-rate clock) in which `bytes` of HBM traffic, read + written, pass at windowMBps
