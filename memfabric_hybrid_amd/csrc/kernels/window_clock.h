@@ -10,6 +10,8 @@
 
 #include <atomic>
 
+#include "xcopy_plan.h"
+
 namespace mf {
 namespace {
 
@@ -28,23 +30,9 @@ __device__ __forceinline__ void WaitForClock(uint64_t t)
 // the value within a few microseconds goes by its own clock, so no wave waits on another for long.  One slot
 // per launch in flight; a slot is reused after kEpochSlots launches.
 constexpr uint32_t kEpochSlots = 64;
-constexpr uint32_t kEpochClockBits = 40;                    // 2^40 ticks of 10 ns: three hours, compared modulo
 constexpr uint32_t kEpochPolls = 64;
 constexpr uint32_t kEpochFreshTicks = 2000;                 // workgroup 0 starts at most 20 us before any other wave of its launch
 __device__ unsigned long long g_windowEpoch[kEpochSlots];
-
-// A clock value whose low kEpochClockBits bits are `low`, the one nearest to `now`.
-__device__ __forceinline__ uint64_t NearClock(uint64_t now, unsigned long long low)
-{
-    const unsigned long long mask = (1ull << kEpochClockBits) - 1;
-    uint64_t t = (now & ~mask) | low;
-    if (t > now + (mask >> 1)) {
-        t -= mask + 1;
-    } else if (t + (mask >> 1) < now) {
-        t += mask + 1;
-    }
-    return t;
-}
 
 __device__ __forceinline__ uint64_t AgreedStart(uint32_t seq)
 {

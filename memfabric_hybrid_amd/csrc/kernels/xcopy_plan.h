@@ -132,6 +132,22 @@ inline uint32_t HoldNanosFor(uint32_t nchunk, uint32_t grid, uint32_t units, boo
     return 700 + kHoldKneeChunks * 6 / 10 + (nchunk - kHoldKneeChunks) * 33 / 100;
 }
 
+// The start of a windowed launch's first period travels between its waves as the low kEpochClockBits bits of a
+// clock value (2^40 ticks of 10 ns: three hours) under a sequence number; NearClock restores the full value: the
+// one with those low bits that is nearest to `now`.
+constexpr uint32_t kEpochClockBits = 40;
+MF_HD inline uint64_t NearClock(uint64_t now, uint64_t low)
+{
+    const uint64_t mask = (1ull << kEpochClockBits) - 1;
+    uint64_t t = (now & ~mask) | low;
+    if (t > now && t - now > (mask >> 1)) {
+        t -= mask + 1;
+    } else if (t < now && now - t > (mask >> 1)) {
+        t += mask + 1;
+    }
+    return t;
+}
+
 // Chunk counts that repeat with a short period: pages of one size (period 1), K and V blocks
 // taking turns (period 2), ...  With such a pattern the owner of a chunk follows from a division
 // and at most kMaxPeriod comparisons, and no chunk prefix is needed.

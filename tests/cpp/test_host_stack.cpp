@@ -890,6 +890,20 @@ static void TestHeldStores()
 // Which batches take the form with read and write windows.
 static void TestWindows()
 {
+    {
+        // the clock value a wave restores from the 40 published bits is the one nearest to its own clock, across a wrap of those bits
+        const uint64_t span = 1ull << 40;
+        const uint64_t nows[] = {5, span - 3, span + 7, 3 * span + 11, 7 * span - 1, (1ull << 63) + 12345};
+        for (uint64_t now : nows) {
+            for (int64_t off : {-2000ll, -64ll, 0ll, 64ll, 250000ll, -250000ll}) {
+                if (off < 0 && static_cast<uint64_t>(-off) > now) {
+                    continue;
+                }
+                const uint64_t start = now + static_cast<uint64_t>(off);
+                CHECK(NearClock(now, start & (span - 1)) == start);
+            }
+        }
+    }
     CHECK(hybm_init(0, 0) == BM_OK);
     const uint64_t gib = 1ull << 30;
     std::vector<uint8_t> mem(2 * gib + 64);
