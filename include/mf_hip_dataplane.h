@@ -54,6 +54,12 @@ int32_t mf_xcopy_batch(const uint64_t *src, const uint64_t *dst, const uint64_t 
 int32_t mf_bm_copy_batch_replay(smem_bm_t handle, smem_batch_copy_params *const *batches, uint32_t count,
                                 uint32_t steps, smem_bm_copy_type t, uint32_t flags);
 
+/* The same for the transfer front-end: `steps` calls of smem_trans_batch_write_submit(handle, sources, remoteUniqueId,
+ * destinations, dataSizes, batchSize, stream, 0) with the arrays of batches[i % count] (sources = local addresses,
+ * destinations = addresses in the peer's registered memory). */
+int32_t mf_trans_batch_write_replay(smem_trans_t handle, smem_batch_copy_params *const *batches, uint32_t count, uint32_t steps,
+                                    const char *remoteUniqueId, void *stream);
+
 /* The same `steps` calls shared out over `threads` host threads (call i goes to thread
  * i % threads), each thread on its own stream as the reference gives every calling thread its
  * own (src/hybm/csrc/ts_engine/hybm_stream_manager.cpp:73-90), all asynchronous with one

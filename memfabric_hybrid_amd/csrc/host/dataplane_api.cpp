@@ -61,6 +61,26 @@ MF_EXPORT int32_t mf_bm_copy_batch_replay(smem_bm_t handle, smem_batch_copy_para
     return 0;
 }
 
+MF_EXPORT int32_t mf_trans_batch_write_replay(smem_trans_t handle, smem_batch_copy_params *const *batches, uint32_t count,
+                                              uint32_t steps, const char *remoteUniqueId, void *stream)
+{
+    if (batches == nullptr || count == 0) {
+        MF_FAIL(SM_INVALID_PARAM, "mf_trans_batch_write_replay: no batches");
+    }
+    uint32_t at = 0;
+    for (uint32_t i = 0; i < steps; ++i) {
+        smem_batch_copy_params *b = batches[at];
+        const int32_t ret = smem_trans_batch_write_submit(handle, const_cast<const void **>(b->sources), remoteUniqueId, b->destinations,
+                                                          const_cast<size_t *>(reinterpret_cast<const size_t *>(b->dataSizes)), b->batchSize,
+                                                          stream, 0);
+        if (ret != 0) {
+            return ret;
+        }
+        at = at + 1 == count ? 0 : at + 1;
+    }
+    return 0;
+}
+
 MF_EXPORT int32_t mf_bm_copy_batch_replay_threads(smem_bm_t handle, smem_batch_copy_params *const *batches, uint32_t count,
                                                   uint32_t steps, smem_bm_copy_type t, uint32_t threads, double *seconds)
 {

@@ -173,6 +173,7 @@ _SIGNATURES = {
     "smem_bm_copy": (i32, [vp, ctypes.POINTER(SmemCopyParams), ctypes.c_int, u32]),
     "smem_bm_copy_batch": (i32, [vp, ctypes.POINTER(BatchCopyParams), ctypes.c_int, u32]),
     "mf_bm_copy_batch_replay": (i32, [vp, ctypes.POINTER(ctypes.POINTER(BatchCopyParams)), u32, u32, ctypes.c_int, u32]),
+    "mf_trans_batch_write_replay": (i32, [vp, ctypes.POINTER(ctypes.POINTER(BatchCopyParams)), u32, u32, ctypes.c_char_p, vp]),
     "mf_bm_copy_batch_replay_threads": (i32, [vp, ctypes.POINTER(ctypes.POINTER(BatchCopyParams)), u32, u32, ctypes.c_int, u32,
                                         ctypes.POINTER(ctypes.c_double)]),
     "smem_bm_wait": (i32, [vp]),
