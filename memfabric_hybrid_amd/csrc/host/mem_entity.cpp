@@ -408,7 +408,7 @@ int MemEntity::RemoveRange(uint64_t base)
     return BM_OK;
 }
 
-bool MemEntity::InRanges(uint64_t a, uint64_t length) const
+bool MemEntity::InRanges(uint64_t a, uint64_t length, uint64_t *rangeBase, uint64_t *rangeEnd) const
 {
     // Batches walk one or two ranges; the last hit of this thread answers most calls without
     // the lock.  The epoch makes a hit from before any change of the range set worthless.
@@ -421,6 +421,10 @@ bool MemEntity::InRanges(uint64_t a, uint64_t length) const
     thread_local Hit hit;
     const uint64_t epoch = rangeEpoch_.load(std::memory_order_acquire);
     if (hit.owner == this && hit.epoch == epoch && a >= hit.base && a + length <= hit.end && a + length >= a) {
+        if (rangeBase != nullptr) {
+            *rangeBase = hit.base;
+            *rangeEnd = hit.end;
+        }
         return true;
     }
     std::shared_lock<std::shared_mutex> guard(rangeLock_);
@@ -429,6 +433,10 @@ bool MemEntity::InRanges(uint64_t a, uint64_t length) const
         return false;
     }
     hit = Hit{this, rangeEpoch_.load(std::memory_order_acquire), it->first, it->first + it->second.size};
+    if (rangeBase != nullptr) {
+        *rangeBase = hit.base;
+        *rangeEnd = hit.end;
+    }
     return true;
 }
 
@@ -511,15 +519,18 @@ uint32_t MemEntity::FirstOutside(void *const *ptrs, const uint64_t *lengths, uin
     const uint64_t hostLo = host_.base;
     const uint64_t hostHi = host_.base == 0 ? 0 : host_.base + (hostBacked < host_.Span() ? hostBacked : host_.Span());
     const bool haveRanges = rangeCount_.load(std::memory_order_acquire) != 0;
+    uint64_t rangeLo = 1;   // the registered range the element before lay in (none yet): most of a batch lies in one
+    uint64_t rangeHi = 0;
     for (uint32_t i = 0; i < n; ++i) {
         const uint64_t a = reinterpret_cast<uint64_t>(ptrs[i]);
         const uint64_t end = a + lengths[i];
         const bool inDevice = a >= devLo && end <= devHi;
         const bool inHost = a >= hostLo && end <= hostHi;
-        if (a != 0 && end >= a && (inDevice || inHost)) {
+        const bool inRange = a >= rangeLo && end <= rangeHi;
+        if (a != 0 && end >= a && (inDevice || inHost || inRange)) {
             continue;
         }
-        if (a == 0 || !haveRanges || !InRanges(a, lengths[i])) {
+        if (a == 0 || !haveRanges || !InRanges(a, lengths[i], &rangeLo, &rangeHi)) {
             return i;
         }
     }

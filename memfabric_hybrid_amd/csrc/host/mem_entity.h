@@ -111,7 +111,7 @@ private:
         hybm_mem_type type;
         uint32_t uses;
     };
-    bool InRanges(uint64_t a, uint64_t length) const;
+    bool InRanges(uint64_t a, uint64_t length, uint64_t *rangeBase = nullptr, uint64_t *rangeEnd = nullptr) const;
     mutable std::shared_mutex rangeLock_;
     std::map<uint64_t, Range, std::greater<uint64_t>> ranges_;   // by start, descending: lower_bound = covering candidate
     std::atomic<uint32_t> rangeCount_{0};
