@@ -92,3 +92,15 @@ MF_EXPORT int32_t mf_moe_combine(const void *rows, const int32_t *rowOf, const f
     }
     return BM_OK;
 }
+
+MF_EXPORT int32_t mf_moe_combine_windows(uint32_t readMBps, uint32_t writeMBps)
+{
+    const bool off = readMBps == 0 && writeMBps == 0;
+    const bool inRange = readMBps >= 1000000u && readMBps <= 16000000u && writeMBps >= 1000000u && writeMBps <= 16000000u;
+    if (!off && !inRange) {
+        MF_FAIL(BM_INVALID_PARAM, "mf_moe_combine_windows: rates are 0, 0 (off) or 1000000 ... 16000000 MB/s, got "
+                                      << readMBps << ", " << writeMBps);
+    }
+    mfk_moe_combine_windows(readMBps, writeMBps);
+    return BM_OK;
+}

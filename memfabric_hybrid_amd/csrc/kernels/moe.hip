@@ -14,12 +14,18 @@
 //                    stored to its K destination rows (HBM bound: H*2*(1+K) bytes per token)
 //   MoeCombineKernel one workgroup per token: K rows gathered, fp32 FMA chain in slot
 //                    order, one rounding to bf16 (HBM bound: H*2*(K+1) bytes per token)
+//   MoeCombineWindowKernel  the same arithmetic for wide rows and many tokens, by waves that
+//                    stay for the whole launch and, chip-wide and by the clock, read for
+//                    most of a period and write at its end
 // Ranks come from ballots and prefix sums, never from atomics on a shared
 // cursor, so the permutation is the same on every run and equals the CPU sort.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
+
 #include "../rt/mf_rt.h"
+#include "window_clock.h"
 
 namespace mf {
 namespace {
@@ -469,6 +475,137 @@ __global__ __launch_bounds__(kThreads) void MoeCombineKernel(const u32x4 *__rest
     }
 }
 
+// The combine of wide rows when there are many tokens: gridDim.x single-wave workgroups, all
+// resident at once, walk the items (token, 128-unit slice of the row) with stride gridDim.x.
+// HBM streams reads at 7.0 TB/s and the combine's mix of eight reads to one write at 6.0, so
+// the two are kept apart in time: a period is kItems read parts and one write part.  In read
+// part j a wave requests the 16 pieces of its j-th item of the period (eight rows, two column
+// positions per lane) at its own offset of the part, reduces them when they have arrived and
+// keeps the result, 8 registers per item; in the write part it stores the kItems results at
+// its own offset of that part.  The start of the first period is agreed through
+// AgreedStart(); after that every wave goes by the constant-rate clock alone.  Measured on
+// 8192 tokens of 7168 elements: 164-168 us against 177-181 us for one workgroup per item, on
+// 16 384 tokens 323-330 against 359-365 us (read parts paced at 6.6-6.8 TB/s, write parts at
+// 6.0-6.5; at 7.0 the waves fall behind now and then, and on some boxes already at 6.8 when the
+// launch runs for seven periods).  From about six items per wave on it is the faster form.
+// Arithmetic and the rule for slots without a row are MoeCombineKernel's.
+constexpr uint32_t kCombineItems = 4;                  // 32 result registers, 116 in all: sixteen waves per CU
+constexpr uint32_t kCombineWavesPerCu = 16;
+constexpr uint32_t kCombineSliceUnits = 128;           // two column positions per lane
+constexpr uint32_t kCombineMinItemsPerWave = 6;
+
+template <uint32_t kItems>
+__global__ __launch_bounds__(64) void MoeCombineWindowKernel(const u32x4 *__restrict__ rowsIn,
+                                                             const int32_t *__restrict__ rowOf,
+                                                             const float *__restrict__ weights, uint32_t unitsPerRow,
+                                                             uint32_t parts, uint32_t items, u32x4 *__restrict__ y,
+                                                             uint32_t readTicks, uint32_t writeTicks, uint32_t seq)
+{
+    constexpr uint32_t kSlots = 8;
+    constexpr uint32_t kBatch = kCombineSliceUnits / 64;
+    const uint64_t start = AgreedStart(seq);
+    const uint32_t period = kItems * readTicks + writeTicks;
+    const uint32_t readOffset = static_cast<uint32_t>(static_cast<uint64_t>(blockIdx.x) * readTicks / gridDim.x);
+    const uint32_t writeOffset = static_cast<uint32_t>(static_cast<uint64_t>(blockIdx.x) * writeTicks / gridDim.x);
+    const uint32_t perPart = (unitsPerRow + parts - 1) / parts;
+    const MF_GLOBAL u32x4 *in = reinterpret_cast<const MF_GLOBAL u32x4 *>(reinterpret_cast<uint64_t>(rowsIn));
+    MF_GLOBAL u32x4 *out = reinterpret_cast<MF_GLOBAL u32x4 *>(reinterpret_cast<uint64_t>(y));
+    uint64_t t0 = start;
+    for (uint32_t base = 0; base < items; base += kItems * gridDim.x, t0 += period) {
+        if (base + blockIdx.x >= items) {
+            break;                                     // nothing left for this wave
+        }
+        // The last period holds as many read parts as it has items per wave, and its last read part lasts as long
+        // as the waves that still have an item need to request it (both the same for every wave).
+        const uint32_t remaining = items - base;
+        const uint32_t left = (remaining + gridDim.x - 1) / gridDim.x;
+        const uint32_t readParts = left < kItems ? left : kItems;
+        const uint32_t inLastPart = remaining - (readParts - 1) * gridDim.x;       // >= 1
+        const uint32_t lastPartTicks = inLastPart >= gridDim.x ? readTicks
+            : static_cast<uint32_t>(static_cast<uint64_t>(inLastPart) * readTicks / gridDim.x);
+        const uint32_t readEnd = (readParts - 1) * readTicks + lastPartTicks;
+        u32x4 o[kItems][kBatch];
+#pragma unroll
+        for (uint32_t j = 0; j < kItems; ++j) {
+            const uint32_t item = base + j * gridDim.x + blockIdx.x;
+            if (j < readParts && item < items) {
+                const uint32_t token = item / parts;
+                const uint32_t begin = (item - token * parts) * perPart;
+                const uint32_t end = begin + perPart < unitsPerRow ? begin + perPart : unitsPerRow;
+                // No branch on a slot without a row (rowOf < 0): its pieces are read from the token's own row
+                // of y, which is memory this launch owns, masked to zero and multiplied by -0.0f, and
+                // fma(-0.0f, 0.0f, acc) is acc for every acc, so the slot contributes nothing, as if skipped.
+                const MF_GLOBAL u32x4 *rowPtr[kSlots];
+                float w[kSlots];
+                uint32_t keep[kSlots];
+#pragma unroll
+                for (uint32_t k = 0; k < kSlots; ++k) {
+                    const int32_t row = rowOf[static_cast<uint64_t>(token) * kSlots + k];
+                    const float weight = weights[static_cast<uint64_t>(token) * kSlots + k];
+                    rowPtr[k] = row < 0 ? out + static_cast<uint64_t>(token) * unitsPerRow
+                                        : in + static_cast<uint64_t>(row) * unitsPerRow;
+                    w[k] = row < 0 ? -0.0f : weight;
+                    keep[k] = row < 0 ? 0u : 0xFFFFFFFFu;
+                }
+                WaitForClock(t0 + j * readTicks + readOffset);
+                u32x4 v[kBatch][kSlots];
+#pragma unroll
+                for (uint32_t b = 0; b < kBatch; ++b) {
+                    const uint32_t u = begin + b * 64 + threadIdx.x;
+                    if (u < end) {
+#pragma unroll
+                        for (uint32_t k = 0; k < kSlots; ++k) {
+                            v[b][k] = __builtin_nontemporal_load(rowPtr[k] + u);
+                        }
+                    }
+                }
+#pragma unroll
+                for (uint32_t b = 0; b < kBatch; ++b) {
+                    float acc[8];
+#pragma unroll
+                    for (uint32_t i = 0; i < 8; ++i) {
+                        acc[i] = 0.0f;
+                    }
+#pragma unroll
+                    for (uint32_t k = 0; k < kSlots; ++k) {
+#pragma unroll
+                        for (uint32_t i = 0; i < 4; ++i) {
+                            const uint32_t word = v[b][k][i] & keep[k];
+                            acc[2 * i] = __builtin_fmaf(w[k], Bf16Lo(word), acc[2 * i]);
+                            acc[2 * i + 1] = __builtin_fmaf(w[k], Bf16Hi(word), acc[2 * i + 1]);
+                        }
+                    }
+#pragma unroll
+                    for (uint32_t i = 0; i < 4; ++i) {
+                        o[j][b][i] = ToBf16(acc[2 * i]) | (ToBf16(acc[2 * i + 1]) << 16);
+                    }
+                }
+            }
+        }
+        WaitForClock(t0 + readEnd + writeOffset);
+#pragma unroll
+        for (uint32_t j = 0; j < kItems; ++j) {
+            const uint32_t item = base + j * gridDim.x + blockIdx.x;
+            if (j < readParts && item < items) {
+                const uint32_t token = item / parts;
+                const uint32_t begin = (item - token * parts) * perPart;
+                const uint32_t end = begin + perPart < unitsPerRow ? begin + perPart : unitsPerRow;
+#pragma unroll
+                for (uint32_t b = 0; b < kBatch; ++b) {
+                    const uint32_t u = begin + b * 64 + threadIdx.x;
+                    if (u < end) {
+                        __builtin_nontemporal_store(o[j][b], out + static_cast<uint64_t>(token) * unitsPerRow + u);
+                    }
+                }
+            }
+        }
+    }
+}
+
+// Pace of the windowed combine, MB/s of HBM traffic in the read parts and in the write parts; 0 = never windowed.
+std::atomic<uint32_t> g_combineReadMBps{6600000};
+std::atomic<uint32_t> g_combineWriteMBps{6000000};
+
 }  // namespace
 }  // namespace mf
 
@@ -552,9 +689,26 @@ extern "C" int mfk_moe_combine(const void *rows, const void *rowOf, const void *
         // positions per lane in flight (16 loads), the fastest shape measured on 7168-element rows
         // (178 us; one four-wave workgroup per token 188 us; plain instead of nontemporal loads 194 us).
         if (upr >= 256) {
-            const uint32_t parts = (upr + 127) / 128;
-            hipLaunchKernelGGL((MoeCombineKernel<8, 64, true, 2>), dim3(tokens * parts), dim3(64), 0, s, in, ro, w, topK, upr,
-                               parts, o);
+            const uint32_t parts = (upr + kCombineSliceUnits - 1) / kCombineSliceUnits;
+            const uint32_t perPart = (upr + parts - 1) / parts;
+            const uint64_t items = static_cast<uint64_t>(tokens) * parts;
+            const uint32_t waves = static_cast<uint32_t>(mfrt_cu_count() > 0 ? mfrt_cu_count() : 256) * kCombineWavesPerCu;
+            // From six items per wave on, waves that stay and keep reads and writes apart in time; below that the
+            // first read part and the last write part, in which the chip only reads or only writes for want of
+            // work, cost what the separation gains (16 800 items on 4096 waves: 51.4 against 50.5 us; 19 200: the
+            // same; 25 200: 74.4 against 76.7 us).
+            const uint32_t readTicks = WindowPeriodTicks(static_cast<uint64_t>(waves) * 8 * perPart * 16,
+                                                         g_combineReadMBps.load(std::memory_order_relaxed));
+            const uint32_t writeTicks = WindowPeriodTicks(static_cast<uint64_t>(waves) * kCombineItems * perPart * 16,
+                                                          g_combineWriteMBps.load(std::memory_order_relaxed));
+            if (items >= static_cast<uint64_t>(waves) * kCombineMinItemsPerWave && items < 0x40000000ull && readTicks != 0 &&
+                writeTicks != 0) {
+                hipLaunchKernelGGL((MoeCombineWindowKernel<kCombineItems>), dim3(waves), dim3(64), 0, s, in, ro, w, upr, parts,
+                                   static_cast<uint32_t>(items), o, readTicks, writeTicks, NextWindowSeq());
+            } else {
+                hipLaunchKernelGGL((MoeCombineKernel<8, 64, true, 2>), dim3(tokens * parts), dim3(64), 0, s, in, ro, w, topK,
+                                   upr, parts, o);
+            }
         } else {
             hipLaunchKernelGGL((MoeCombineKernel<8, 256, true>), dim3(tokens), dim3(256), 0, s, in, ro, w, topK, upr, 1u, o);
         }
@@ -562,4 +716,10 @@ extern "C" int mfk_moe_combine(const void *rows, const void *rowOf, const void *
         hipLaunchKernelGGL((MoeCombineKernel<0, 256, true>), dim3(tokens), dim3(256), 0, s, in, ro, w, topK, upr, 1u, o);
     }
     return static_cast<int>(hipGetLastError());
+}
+
+extern "C" void mfk_moe_combine_windows(uint32_t readMBps, uint32_t writeMBps)
+{
+    mf::g_combineReadMBps.store(readMBps, std::memory_order_relaxed);
+    mf::g_combineWriteMBps.store(writeMBps, std::memory_order_relaxed);
 }

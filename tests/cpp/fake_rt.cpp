@@ -346,4 +346,5 @@ uint64_t mfk_moe_workspace_bytes(uint32_t, uint32_t, uint32_t) { return 0; }
 int mfk_moe_dispatch(const void *, const void *, uint32_t, uint32_t, uint32_t, uint32_t, void *, void *, void *, void *, void *,
                      void *, void *) { return -1; }
 int mfk_moe_combine(const void *, const void *, const void *, uint32_t, uint32_t, uint32_t, void *, void *) { return -1; }
+void mfk_moe_combine_windows(uint32_t, uint32_t) {}
 }

@@ -179,6 +179,46 @@ def test_out_of_range_expert_ids_are_flagged_not_followed(gpu, oracle):
         _free(bufs)
 
 
+@pytest.mark.parametrize("T,H", [
+    (3600, 7168),   # 25 200 slices: one full period for 4096 waves and a last period of two read parts and a short third
+    (3300, 8000),   # rows of 1000 units in eight slices of 125: ragged slices, a last period of three read parts
+])
+def test_combine_in_read_and_write_windows(gpu, oracle, T, H):
+    """Enough tokens of wide rows for the combine whose waves stay and alternate between reading and writing:
+    same bits as the oracle at the default pace, at a slow and at an absurdly fast one, with slots without a
+    row, and the same bits with the form switched off."""
+    K = 8
+    rng = np.random.default_rng(T)
+    rows = (rng.integers(0x3800, 0x4000, (T * K, H), dtype=np.uint16) | (rng.integers(0, 2, (T * K, H), dtype=np.uint16) << 15))
+    row_of = rng.permutation(T * K).astype(np.int32)
+    row_of[rng.integers(0, T * K, 50)] = -1
+    victim = int(np.where(row_of == 0)[0][0]) if np.any(row_of == 0) else None
+    if victim is not None:
+        row_of[victim] = 1                      # nobody reads row 0, which holds a NaN and an infinity
+    rows[0, 0::2] = 0x7FC0
+    rows[0, 1::2] = 0x7F80
+    w = rng.random((T, K), dtype=np.float32)
+    exp_y = np.zeros((T, H), dtype=np.uint16)
+    oracle.orc_moe_combine(np_ptr(rows), np_ptr(row_of), np_ptr(w), T, H, K, np_ptr(exp_y))
+    rdev, rodev, wdev = _dev(gpu, rows), _dev(gpu, row_of), _dev(gpu, w)
+    y = gpu_util.DeviceBuffer(gpu, T * H * 2)
+    try:
+        for rates in ((6600000, 6000000), (1000000, 1000000), (16000000, 16000000), (0, 0)):
+            assert gpu.mf_moe_combine_windows(*rates) == 0, native.last_error()
+            y.fill(0xEE)
+            assert gpu.mf_moe_combine(rdev.ptr, rodev.ptr, wdev.ptr, T, H, K, y.ptr, None) == 0, native.last_error()
+            assert gpu.mfrt_device_sync() == 0
+            got = _fetch(y, np.uint16, (T, H))
+            assert np.array_equal(got, exp_y), rates
+            assert not np.any((got & 0x7F80) == 0x7F80)
+        assert gpu.mf_moe_combine_windows(500, 6500000) == native.BM_INVALID_PARAM
+        assert gpu.mf_moe_combine_windows(0, 6500000) == native.BM_INVALID_PARAM
+    finally:
+        assert gpu.mf_moe_combine_windows(6600000, 6000000) == 0
+        for b in (rdev, rodev, wdev, y):
+            b.free()
+
+
 def test_same_workspace_reused_by_calls_of_different_sizes(gpu, oracle):
     """Histograms and status of one call must not leak into the next call on the same workspace."""
     E, K, H = 64, 4, 64
