@@ -546,7 +546,7 @@ def extras_moe(lib):
         shipped.append(timer.run(combine, 30, warm=3)[0])
         assert lib.mf_moe_combine_windows(0, 0) == 0
         one_shot.append(timer.run(combine, 30, warm=3)[0])
-        assert lib.mf_moe_combine_windows(6600000, 6000000) == 0
+        assert lib.mf_moe_combine_windows(*native.MOE_COMBINE_WINDOWS_DEFAULT) == 0
     c_us = sorted(shipped)[1]
     d_bytes = T * H * 2 + T * K * H * 2 + T * K * 4
     c_bytes = T * K * H * 2 + T * K * 4 + T * K * 4 + T * H * 2

@@ -486,8 +486,9 @@ __global__ __launch_bounds__(kThreads) void MoeCombineKernel(const u32x4 *__rest
 // AgreedStart(); after that every wave goes by the constant-rate clock alone.  Measured on
 // 8192 tokens of 7168 elements: 164-168 us against 177-181 us for one workgroup per item, on
 // 16 384 tokens 323-330 against 359-365 us (read parts paced at 6.6-6.8 TB/s, write parts at
-// 6.0-6.5; at 7.0 the waves fall behind now and then, and on some boxes already at 6.8 when the
-// launch runs for seven periods).  From about six items per wave on it is the faster form.
+// 6.0-6.5; reads at 7.0 make the waves fall behind now and then, and so did 6.8 with writes at
+// 6.5 on one machine when the launch ran for seven periods; the default is 6.8 and 6.2).  From
+// about six items per wave on it is the faster form.
 // Arithmetic and the rule for slots without a row are MoeCombineKernel's.
 constexpr uint32_t kCombineItems = 4;                  // 32 result registers, 116 in all: sixteen waves per CU
 constexpr uint32_t kCombineWavesPerCu = 16;
@@ -603,8 +604,8 @@ __global__ __launch_bounds__(64) void MoeCombineWindowKernel(const u32x4 *__rest
 }
 
 // Pace of the windowed combine, MB/s of HBM traffic in the read parts and in the write parts; 0 = never windowed.
-std::atomic<uint32_t> g_combineReadMBps{6600000};
-std::atomic<uint32_t> g_combineWriteMBps{6000000};
+std::atomic<uint32_t> g_combineReadMBps{6800000};
+std::atomic<uint32_t> g_combineWriteMBps{6200000};
 
 }  // namespace
 }  // namespace mf

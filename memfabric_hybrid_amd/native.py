@@ -290,6 +290,10 @@ _plugin = None
 _yardstick = None
 
 
+# pace of the combine's read and write parts the library starts with (MB/s), for callers that switch it and back
+MOE_COMBINE_WINDOWS_DEFAULT = (6800000, 6200000)
+
+
 def _bind(handle, table):
     for name, (restype, argtypes) in table.items():
         fn = getattr(handle, name)  # AttributeError names the missing symbol

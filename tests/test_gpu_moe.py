@@ -179,15 +179,18 @@ def test_out_of_range_expert_ids_are_flagged_not_followed(gpu, oracle):
         _free(bufs)
 
 
-@pytest.mark.parametrize("T,H", [
-    (3600, 7168),   # 25 200 slices: one full period for 4096 waves and a last period of two read parts and a short third
-    (3300, 8000),   # rows of 1000 units in eight slices of 125: ragged slices, a last period of three read parts
+@pytest.mark.parametrize("T,H,K", [
+    (3600, 7168, 8),   # 25 200 slices: one full period for 4096 waves and a last period of two read parts and a short third
+    (3300, 8000, 8),   # rows of 1000 units in eight slices of 125: ragged slices, a last period of three read parts
+    (700, 1024, 8),    # narrow rows: one four-wave workgroup per token
+    (60, 7168, 8),     # wide rows, few tokens: one workgroup per slice
+    (300, 16384, 3),   # any other topK
 ])
-def test_combine_in_read_and_write_windows(gpu, oracle, T, H):
-    """Enough tokens of wide rows for the combine whose waves stay and alternate between reading and writing:
-    same bits as the oracle at the default pace, at a slow and at an absurdly fast one, with slots without a
-    row, and the same bits with the form switched off."""
-    K = 8
+def test_combine_of_rows_that_differ_within_a_token(gpu, oracle, T, H, K):
+    """After a dispatch the rows of a token are copies of one another, so a combine that mixed them up would still pass
+    the dispatch-then-combine tests; here every row is different.  The first two shapes have enough tokens of wide rows
+    for the combine whose waves stay and alternate between reading and writing: same bits as the oracle at the
+    default pace, at a slow and at an absurdly fast one, with slots without a row, and with the form switched off."""
     rng = np.random.default_rng(T)
     rows = (rng.integers(0x3800, 0x4000, (T * K, H), dtype=np.uint16) | (rng.integers(0, 2, (T * K, H), dtype=np.uint16) << 15))
     row_of = rng.permutation(T * K).astype(np.int32)
@@ -203,7 +206,7 @@ def test_combine_in_read_and_write_windows(gpu, oracle, T, H):
     rdev, rodev, wdev = _dev(gpu, rows), _dev(gpu, row_of), _dev(gpu, w)
     y = gpu_util.DeviceBuffer(gpu, T * H * 2)
     try:
-        for rates in ((6600000, 6000000), (1000000, 1000000), (16000000, 16000000), (0, 0)):
+        for rates in (native.MOE_COMBINE_WINDOWS_DEFAULT, (1000000, 1000000), (16000000, 16000000), (0, 0)):
             assert gpu.mf_moe_combine_windows(*rates) == 0, native.last_error()
             y.fill(0xEE)
             assert gpu.mf_moe_combine(rdev.ptr, rodev.ptr, wdev.ptr, T, H, K, y.ptr, None) == 0, native.last_error()
@@ -214,7 +217,7 @@ def test_combine_in_read_and_write_windows(gpu, oracle, T, H):
         assert gpu.mf_moe_combine_windows(500, 6500000) == native.BM_INVALID_PARAM
         assert gpu.mf_moe_combine_windows(0, 6500000) == native.BM_INVALID_PARAM
     finally:
-        assert gpu.mf_moe_combine_windows(6600000, 6000000) == 0
+        assert gpu.mf_moe_combine_windows(*native.MOE_COMBINE_WINDOWS_DEFAULT) == 0
         for b in (rdev, rodev, wdev, y):
             b.free()
 

@@ -302,3 +302,13 @@ def test_2d_row_and_column_of_every_unit_in_a_chunk(lib):
         assert lib.mf_copy2d_rowcol_mismatches(wu, rpc.value, magic.value, units) == 0, wu
     # the formula the one-row case must not use: the multiply-high alone, on a row of 65 537 units
     assert lib.mf_copy2d_rowcol_mismatches(65537, 2, (1 << 32) // 65537 + 1, 65537) != 0
+
+
+def test_python_side_knows_the_combine_pace_the_library_starts_with():
+    """bench.py and the GPU tests switch the windowed combine off and back on with native.MOE_COMBINE_WINDOWS_DEFAULT."""
+    import pathlib
+    import re
+    text = (pathlib.Path(native.__file__).parent / "csrc" / "kernels" / "moe.hip").read_text()
+    read = int(re.search(r"g_combineReadMBps\{(\d+)\}", text).group(1))
+    write = int(re.search(r"g_combineWriteMBps\{(\d+)\}", text).group(1))
+    assert (read, write) == native.MOE_COMBINE_WINDOWS_DEFAULT
