@@ -132,12 +132,14 @@ __global__ __launch_bounds__(kRankThreads) void MoeRankKernel(const int32_t *__r
                                                               uint32_t histStride, int32_t *__restrict__ counts, int32_t *__restrict__ offsets,
                                                               int32_t *__restrict__ rowOf, int32_t *__restrict__ srcOf,
                                                               const uint32_t *__restrict__ blockBad,
-                                                              uint32_t *__restrict__ status)
+                                                              uint32_t *__restrict__ status, uint32_t topK,
+                                                              int2 *__restrict__ runOrder)
 {
     extern __shared__ uint32_t lds[];
     uint32_t *hist = lds;                                 // [kRankSlices][experts]
     uint32_t *base = lds + kRankSlices * experts;         // [experts] first row of this block's entries per expert
-    uint32_t *scan = base + experts;                      // [kRankThreads] scratch of the block scan
+    uint32_t *scan = base + experts;                      // [kRankThreads] scratch of the block scans
+    uint32_t *cum = scan + kRankThreads;                  // [experts] entries of this block with a smaller expert id
     uint32_t myExpert[kRankRounds];
     uint32_t myRank[kRankRounds];
     uint32_t bad = 0;
@@ -213,13 +215,53 @@ __global__ __launch_bounds__(kRankThreads) void MoeRankKernel(const int32_t *__r
         }
     }
     __syncthreads();
-    // turn slice histograms into exclusive prefixes over the slices of this block
-    for (uint32_t x = threadIdx.x; x < experts; x += kRankThreads) {
-        uint32_t acc = base[x];
-        for (uint32_t s = 0; s < kRankSlices; ++s) {
-            const uint32_t v = hist[s * experts + x];
-            hist[s * experts + x] = acc;
-            acc += v;
+    // turn slice histograms into exclusive prefixes over the slices of this block; the same threads own the same
+    // experts as above, so the block's own entries per expert can be scanned over the experts next
+    uint32_t ownOf[kMaxExperts / kRankThreads];          // this block's entries per owned expert
+    uint32_t own = 0;
+#pragma unroll
+    for (uint32_t j = 0; j < kMaxExperts / kRankThreads; ++j) {
+        ownOf[j] = 0;
+        const uint32_t x = threadIdx.x * per + j;
+        if (j < per && x < experts) {
+            uint32_t acc = base[x];
+            for (uint32_t s = 0; s < kRankSlices; ++s) {
+                const uint32_t v = hist[s * experts + x];
+                hist[s * experts + x] = acc;
+                acc += v;
+            }
+            ownOf[j] = acc - base[x];
+            own += ownOf[j];
+        }
+    }
+    uint32_t valid = 0;
+    if (runOrder != nullptr) {
+        // cum[x] = entries of this block routed to an expert below x: where the block's rows of expert x start in
+        // the list of the block's rows in ascending order
+        uint32_t inclOwn = own;
+#pragma unroll
+        for (uint32_t step = 1; step < 64; step <<= 1) {
+            const uint32_t up = __shfl_up(inclOwn, step, 64);
+            inclOwn += (threadIdx.x & 63u) >= step ? up : 0u;
+        }
+        __syncthreads();                                  // the first scan's readers are done with scan[]
+        if ((threadIdx.x & 63u) == 63u) {
+            scan[threadIdx.x >> 6] = inclOwn;
+        }
+        __syncthreads();
+        uint32_t ownBase = 0;
+        for (uint32_t wv = 0; wv < kRankThreads / 64; ++wv) {
+            ownBase += wv < (threadIdx.x >> 6) ? scan[wv] : 0u;
+            valid += scan[wv];
+        }
+        uint32_t at = inclOwn + ownBase - own;
+#pragma unroll
+        for (uint32_t j = 0; j < kMaxExperts / kRankThreads; ++j) {
+            const uint32_t x = threadIdx.x * per + j;
+            if (j < per && x < experts) {
+                cum[x] = at;
+                at += ownOf[j];
+            }
         }
     }
     __syncthreads();
@@ -236,8 +278,19 @@ __global__ __launch_bounds__(kRankThreads) void MoeRankKernel(const int32_t *__r
                 if (srcOf != nullptr) {
                     srcOf[row] = static_cast<int32_t>(idx);
                 }
+                if (runOrder != nullptr) {
+                    const uint32_t at = cum[myExpert[r]] + (static_cast<uint32_t>(row) - base[myExpert[r]]);
+                    runOrder[static_cast<uint64_t>(blockIdx.x) * kRankBlock + at] =
+                        make_int2(row, static_cast<int32_t>(idx / topK));
+                }
             }
             rowOf[idx] = row;
+        }
+    }
+    if (runOrder != nullptr) {
+        // slots past the block's valid entries (ids out of range, the tail of the last block) name no row
+        for (uint32_t at = valid + threadIdx.x; at < kRankBlock; at += kRankThreads) {
+            runOrder[static_cast<uint64_t>(blockIdx.x) * kRankBlock + at] = make_int2(-1, 0);
         }
     }
 }
@@ -372,6 +425,60 @@ __global__ __launch_bounds__(64) void MoePermuteLoopKernel(const u32x4 *__restri
         spread(ib, b, rb);
         if (!hasA) {
             break;
+        }
+    }
+}
+
+// The permute of wide rows when a block of kRankBlock entries holds no more of x than an XCD's L2 keeps:
+// output-ordered, in tiles.  runOrder lists, block of entries by block, the block's output rows in ascending
+// order (runs of consecutive rows per expert) with the token each row is a copy of.  Workgroup i, a single
+// wave, belongs to stream i % 8 (the dispatcher deals consecutive workgroups to the eight XCDs in turn);
+// stream s takes the blocks s, s + 8, ... one after the other and walks a block's rows in list order, a row in
+// tiles of 128 units (2 KiB).  So an XCD writes runs of consecutive rows front to back, two stores per wave,
+// which is the only store pattern this part takes at more than 5.4 TB/s (6.1 in runs of 128 KiB, 6.6 in
+// eight sequential streams; waves that store 14 KiB each: 5.4 in any order), and the K reads of a token row
+// all come from the same XCD within the time it spends on the block: the first from HBM, the others from its
+// L2 (plain loads), which stores that are written through pass without evicting x (plain stores: 244 us).
+// 8192 x 7168, top-8, 256 experts: 163-166 us against 192 us for the token-ordered loop kernel; tiles of
+// 64 / 192 / 256 / 448 units 207 / 171 / 178 / 193 us, nontemporal stores that are not written through 166-172 us,
+// blocks of 2048 entries per stream step 165-171 us, streams that do not follow the XCDs 283 us.
+constexpr uint32_t kTileUnits = 128;
+constexpr uint32_t kTileStreams = 8;
+
+__global__ __launch_bounds__(64) void MoePermuteTileKernel(const u32x4 *__restrict__ x, const int2 *__restrict__ runOrder,
+                                                           uint32_t unitsPerRow, uint32_t tilesPerRow, uint32_t blocks,
+                                                           u32x4 *__restrict__ out)
+{
+    const uint32_t stream = blockIdx.x % kTileStreams;
+    const uint32_t q = blockIdx.x / kTileStreams;
+    const uint32_t tilesPerBlock = kRankBlock * tilesPerRow;
+    const uint32_t block = (q / tilesPerBlock) * kTileStreams + stream;
+    const uint32_t within = q % tilesPerBlock;
+    if (block >= blocks) {
+        return;
+    }
+    const int2 rowAndToken = runOrder[static_cast<uint64_t>(block) * kRankBlock + within / tilesPerRow];
+    if (rowAndToken.x < 0) {
+        return;
+    }
+    const uint32_t begin = (within % tilesPerRow) * kTileUnits;
+    const MF_GLOBAL u32x4 *src = reinterpret_cast<const MF_GLOBAL u32x4 *>(reinterpret_cast<uint64_t>(x)) +
+                                 static_cast<uint64_t>(rowAndToken.y) * unitsPerRow;
+    MF_GLOBAL u32x4 *dst = reinterpret_cast<MF_GLOBAL u32x4 *>(reinterpret_cast<uint64_t>(out)) +
+                           static_cast<uint64_t>(rowAndToken.x) * unitsPerRow;
+    u32x4 v[kTileUnits / 64];
+#pragma unroll
+    for (uint32_t j = 0; j < kTileUnits / 64; ++j) {
+        const uint32_t u = begin + j * 64 + threadIdx.x;
+        if (u < unitsPerRow) {
+            v[j] = src[u];
+        }
+    }
+#pragma unroll
+    for (uint32_t j = 0; j < kTileUnits / 64; ++j) {
+        const uint32_t u = begin + j * 64 + threadIdx.x;
+        if (u < unitsPerRow) {
+            RowStore<2>(dst + u, v[j]);
         }
     }
 }
@@ -615,7 +722,9 @@ extern "C" uint64_t mfk_moe_workspace_bytes(uint32_t tokens, uint32_t topK, uint
     const uint64_t total = static_cast<uint64_t>(tokens) * topK;
     const uint64_t blocks = (total + mf::kRankBlock - 1) / mf::kRankBlock;
     const uint64_t stride = (blocks + 3) / 4 * 4;
-    return 256 + stride * sizeof(uint32_t) + stride * experts * sizeof(uint32_t);
+    // status words, per-block flags, the [expert][block] histogram, the run-ordered row list (8 bytes per entry slot)
+    const uint64_t tables = 256 + stride * sizeof(uint32_t) + stride * experts * sizeof(uint32_t);
+    return (tables + 15) / 16 * 16 + blocks * mf::kRankBlock * sizeof(int2);
 }
 
 extern "C" int mfk_moe_dispatch(const void *x, const void *topk, uint32_t tokens, uint32_t hidden, uint32_t topK,
@@ -636,17 +745,26 @@ extern "C" int mfk_moe_dispatch(const void *x, const void *topk, uint32_t tokens
     uint32_t *blockBad = status + 64;
     uint32_t *blockHist = blockBad + histStride;
     const size_t histLds = static_cast<size_t>(kRankSlices) * experts * sizeof(uint32_t);
-    const size_t rankLds = histLds + (experts + kRankThreads) * sizeof(uint32_t);
+    const size_t rankLds = histLds + (2 * experts + kRankThreads) * sizeof(uint32_t);
+    const uint32_t upr = hidden / 8;
+    // The output-ordered tile permute needs the token rows of one block of entries (kRankBlock / topK tokens) to
+    // stay in an XCD's 4 MiB L2 while the block's rows are written, and enough blocks for the eight streams.
+    const uint64_t blockTokenBytes = static_cast<uint64_t>(kRankBlock / topK + 1) * hidden * 2;
+    const uint32_t tilesPerRow = (upr + kTileUnits - 1) / kTileUnits;
+    const uint64_t tileGrid = static_cast<uint64_t>((blocks + kTileStreams - 1) / kTileStreams * kTileStreams) * kRankBlock * tilesPerRow;
+    const bool tiles = x != nullptr && out != nullptr && upr >= 512 && blockTokenBytes <= (5ull << 19) &&
+                       blocks >= 2 * kTileStreams && tileGrid <= 0x7FFFFFFFull;
+    const uint64_t tableBytes = 256 + histStride * sizeof(uint32_t) + static_cast<uint64_t>(histStride) * experts * sizeof(uint32_t);
+    int2 *runOrder = tiles ? reinterpret_cast<int2 *>(static_cast<char *>(workspace) + (tableBytes + 15) / 16 * 16) : nullptr;
     hipLaunchKernelGGL(MoeHistKernel, dim3(blocks), dim3(kRankThreads), histLds, s, static_cast<const int32_t *>(topk),
                        total, experts, blockHist, histStride, blockBad);
     hipLaunchKernelGGL(MoeRankKernel, dim3(blocks), dim3(kRankThreads), rankLds, s, static_cast<const int32_t *>(topk),
                        total, experts, blockHist, histStride, static_cast<int32_t *>(counts), static_cast<int32_t *>(offsets),
-                       static_cast<int32_t *>(rowOf), static_cast<int32_t *>(srcOf), blockBad, status);
+                       static_cast<int32_t *>(rowOf), static_cast<int32_t *>(srcOf), blockBad, status, topK, runOrder);
     if (x != nullptr && out != nullptr && hidden != 0) {
         const u32x4 *xi = static_cast<const u32x4 *>(x);
         const int32_t *ro = static_cast<const int32_t *>(rowOf);
         u32x4 *oo = static_cast<u32x4 *>(out);
-        const uint32_t upr = hidden / 8;
         // Wide rows: single-wave workgroups that hold up to 14 pieces per lane (a whole 7168-element
         // row) and write them with plain stores.  Storing alone takes 177 us of the 200 us such a
         // kernel needs when every wave reads its row first; with sixteen waves per CU that each
@@ -658,7 +776,10 @@ extern "C" int mfk_moe_dispatch(const void *x, const void *topk, uint32_t tokens
         // row reading x[srcOf[row]], 271 us: its eight reads of every token row are not absorbed by
         // the caches.
         // Narrow rows: one four-wave workgroup per token.
-        if (upr >= 512) {
+        if (tiles) {
+            hipLaunchKernelGGL(MoePermuteTileKernel, dim3(static_cast<uint32_t>(tileGrid)), dim3(64), 0, s, xi, runOrder, upr,
+                               tilesPerRow, blocks, oo);
+        } else if (upr >= 512) {
             // 123 vector registers per lane: four waves per SIMD, sixteen per CU, all resident at once
             const uint32_t wideParts = (upr + 64 * 14 - 1) / (64 * 14);
             const uint32_t items = tokens * wideParts;

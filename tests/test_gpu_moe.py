@@ -118,6 +118,47 @@ def test_dispatch_and_combine_match_the_specification(gpu, oracle, T, H, K, E):
         _free(bufs)
 
 
+@pytest.mark.parametrize("T,H,E,routing", [
+    (2000, 4096, 64, "router"),     # 16 000 entries: fifteen full blocks and a last one of 640 entries
+    (2500, 7168, 300, "router"),    # twenty blocks, which the eight streams do not divide
+    (2200, 7168, 256, "five"),      # everything lands on five experts, duplicates inside a token included: long runs
+    (2200, 5120, 256, "bad ids"),   # some ids out of range: their slots name no row, the lists of their blocks are shorter
+])
+def test_output_ordered_permute(gpu, oracle, T, H, E, routing):
+    """Rows wide enough and blocks enough for the permute that walks the output in runs of consecutive rows per
+    expert, in tiles: every output row and every map against the oracle."""
+    K = 8
+    x, topk, _ = _inputs(oracle, 0xD1 + T, T, H, K, E)
+    rng = np.random.default_rng(T)
+    if routing == "five":
+        topk = rng.integers(0, 5, (T, K)).astype(np.int32)
+        topk[::7, 0] = E - 1
+    elif routing == "bad ids":
+        topk = topk.copy()
+        topk[rng.integers(0, T, 300), rng.integers(0, K, 300)] = E + 3
+        topk[5, :] = -1                                     # a token nobody takes
+    if routing == "bad ids":
+        # the oracle refuses ids out of range; it is asked about the same routing with those entries sent to one
+        # more expert behind the others, which leaves every row of the real experts where it is
+        bad = (topk < 0) | (topk >= E)
+        exp_out, exp_counts, exp_offsets, exp_row, exp_src = _oracle_dispatch(oracle, x, np.where(bad, E, topk).astype(np.int32), E + 1)
+        exp_counts, exp_offsets = exp_counts[:E], exp_offsets[:E]
+        exp_row = np.where(bad.reshape(-1), -1, exp_row)
+    else:
+        exp_out, exp_counts, exp_offsets, exp_row, exp_src = _oracle_dispatch(oracle, x, topk, E)
+    bufs = _gpu_dispatch(gpu, x, topk, E)
+    try:
+        valid = int(exp_counts.sum())
+        assert np.array_equal(_fetch(bufs["counts"], np.int32, (E,)), exp_counts)
+        assert np.array_equal(_fetch(bufs["offsets"], np.int32, (E,)), exp_offsets)
+        assert np.array_equal(_fetch(bufs["row_of"], np.int32, (T * K,)), exp_row)
+        assert np.array_equal(_fetch(bufs["src_of"], np.int32, (T * K,))[:valid], exp_src[:valid])
+        assert np.array_equal(_fetch(bufs["out"], np.uint16, (T * K, H))[:valid], exp_out[:valid])
+        assert _fetch(bufs["ws"], np.uint32, (1,))[0] == (1 if routing == "bad ids" else 0)
+    finally:
+        _free(bufs)
+
+
 def test_skewed_routing_with_empty_and_hot_experts(gpu, oracle):
     rng = np.random.default_rng(3)
     T, H, K, E = 3000, 128, 8, 256
