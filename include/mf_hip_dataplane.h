@@ -156,8 +156,9 @@ int64_t mf_xcopy_describe_plan(const uint64_t *src, const uint64_t *dst, const u
  *   [0, experts)), srcOf[tokens*topK] (inverse, may be NULL),
  *   out[tokens*topK][hidden] expert-contiguous (x and out may both be NULL to
  *   compute the permutation only).
- * workspace: mf_moe_workspace_bytes() bytes of device memory, no initialisation
- *   needed; after the stream has drained its first uint32 is 1 if any expert id
+ * workspace: mf_moe_workspace_bytes() bytes of device memory (status, the
+ *   [expert][block] histogram and 8 bytes per entry for the order in which the
+ *   rows are written), no initialisation needed; after the stream has drained its first uint32 is 1 if any expert id
  *   was out of range.  Enqueues on `stream` (NULL: thread stream), does not wait. */
 uint64_t mf_moe_workspace_bytes(uint32_t tokens, uint32_t topK, uint32_t experts);
 int32_t mf_moe_dispatch(const void *x, const int32_t *topk, uint32_t tokens, uint32_t hidden, uint32_t topK,
