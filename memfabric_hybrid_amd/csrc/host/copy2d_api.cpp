@@ -82,6 +82,7 @@ MF_EXPORT int32_t mf_xcopy_2d_batch(const mf_copy2d_desc *descs, uint32_t n, int
             plan.rowsPerChunk[i] = 1;
             plan.magic[i] = 0;
             plan.first[i] = 0xFFFFFFFFu;
+            plan.mate[i] = 0;
         }
         plan.nchunk = static_cast<uint32_t>(run);
         const uint32_t perCu = engine.Tuning().wgPerCu;   // 0: one workgroup per row group
@@ -122,6 +123,13 @@ MF_EXPORT int32_t mf_xcopy_2d_batch(const mf_copy2d_desc *descs, uint32_t n, int
         plan.rowsPerChunk[used] = rpc;
         plan.magic[used] = RectMagic(wu);
         plan.first[used] = static_cast<uint32_t>(run);
+        plan.mate[used] = 0;
+        if (used > 0 && plan.mate[used - 1] == 0 &&
+            RectsSideBySide(plan.dst[used - 1], d.dst, static_cast<uint64_t>(plan.widthUnits[used - 1]) * 16, d.width,
+                            plan.height[used - 1], d.height, static_cast<uint64_t>(plan.dpitchUnits[used - 1]) * 16, d.dpitch)) {
+            plan.mate[used - 1] = 1;
+            plan.mate[used] = 2;
+        }
         run += chunks;
         ++used;
     }

@@ -34,10 +34,21 @@ __global__ __launch_bounds__(kRectThreads) void Copy2dKernel(const RectPlan p)
     const uint32_t ht = p.height[lane];
     const uint32_t rpc = p.rowsPerChunk[lane];
     const uint32_t mg = p.magic[lane];
+    const uint32_t mt = p.mate[lane];
     const uint32_t nchunk = p.nchunk;
     uint32_t c = blockIdx.x;
     do {
-        const uint32_t r = __popcll(__ballot(first <= c)) - 1;
+        // Two rectangles side by side in the destination take the chunks of their common range in turn, so that
+        // workgroups launched together write both parts of the same destination rows.
+        uint32_t r = __popcll(__ballot(first <= c)) - 1;
+        uint32_t k = c - __builtin_amdgcn_readlane(first, r);
+        const uint32_t m = __builtin_amdgcn_readlane(mt, r);
+        if (m != 0) {
+            const uint32_t r0 = r - (m - 1);
+            const uint32_t both = c - __builtin_amdgcn_readlane(first, r0);
+            r = r0 + (both & 1u);
+            k = both >> 1;
+        }
         const uint64_t rs = ReadLane64(src, r);
         const uint64_t rd = ReadLane64(dst, r);
         const uint32_t rsp = __builtin_amdgcn_readlane(sp, r);
@@ -46,7 +57,6 @@ __global__ __launch_bounds__(kRectThreads) void Copy2dKernel(const RectPlan p)
         const uint32_t rht = __builtin_amdgcn_readlane(ht, r);
         const uint32_t rrpc = __builtin_amdgcn_readlane(rpc, r);
         const uint32_t rmg = __builtin_amdgcn_readlane(mg, r);
-        const uint32_t k = c - __builtin_amdgcn_readlane(first, r);
         const uint32_t row0 = k * rrpc;
         const uint32_t rows = rht - row0 < rrpc ? rht - row0 : rrpc;
         const uint32_t units = rows * rwu;

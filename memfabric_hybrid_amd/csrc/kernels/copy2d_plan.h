@@ -24,6 +24,8 @@ struct RectPlan {
     uint32_t rowsPerChunk[kRectInline];
     uint32_t magic[kRectInline];          // floor(2^32 / widthUnits) + 1, see RectRowCol; unused when rowsPerChunk == 1
     uint32_t first[kRectInline];          // exclusive prefix of chunk counts, 0xFFFFFFFF past the end
+    uint32_t mate[kRectInline];           // 0: alone; 1 / 2: first / second of two rectangles that lie side by side in the
+                                          // destination (RectsSideBySide) and whose chunks are dealt out in turn
     uint32_t nchunk;
 };
 
@@ -70,6 +72,31 @@ MF_RECT_HD inline bool RectFitsPlan(uint64_t src, uint64_t dst, uint64_t width, 
 {
     return ((src | dst | width | spitch | dpitch) & 15u) == 0 && width / 16 <= 0xFFFFFFFFull &&
            spitch / 16 <= 0xFFFFFFFFull && dpitch / 16 <= 0xFFFFFFFFull && height <= 0xFFFFFFFFull;
+}
+
+// Two rectangles of the same shape whose destination rows continue one another: b's rows start where a's end,
+// in the same destination pitch (the two old column blocks of a row-parallel weight, side by side in the new shard).
+MF_RECT_HD inline bool RectsSideBySide(uint64_t dstA, uint64_t dstB, uint64_t widthA, uint64_t widthB, uint64_t heightA,
+                                       uint64_t heightB, uint64_t dpitchA, uint64_t dpitchB)
+{
+    return widthA == widthB && heightA == heightB && dpitchA == dpitchB && dstB == dstA + widthA && dpitchA >= 2 * widthA;
+}
+
+// Rectangle r and chunk k inside it that chunk c of a plan stands for; what Copy2dKernel works out with a ballot over
+// `first` and lane reads, restated for host code.  Rectangles that are mates take the chunks of their common range in turn.
+inline void RectOfChunk(const RectPlan &plan, uint32_t c, uint32_t &r, uint32_t &k)
+{
+    r = 0;
+    while (r + 1 < kRectInline && plan.first[r + 1] <= c) {
+        ++r;
+    }
+    k = c - plan.first[r];
+    if (plan.mate[r] != 0) {
+        const uint32_t r0 = r - (plan.mate[r] - 1);
+        const uint32_t both = c - plan.first[r0];
+        r = r0 + (both & 1u);
+        k = both >> 1;
+    }
 }
 
 }  // namespace mf

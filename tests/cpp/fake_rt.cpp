@@ -326,15 +326,24 @@ int mfk_xcopy_table_static(const void *triples, uint32_t nseg, uint32_t units, i
     return err != 0 ? err : mfk_xcopy_table(triples, scratch, scratch + nseg + 1, nseg, 0, units, nullptr, route, grid, nullptr, 0, stream);
 }
 
+static uint32_t g_lastRectMates = 0;
+extern "C" uint32_t fake_rt_last_rect_mates() { return g_lastRectMates; }
+
+// Walks the chunks as the kernel's workgroups do, so a wrong chunk-to-rectangle rule leaves rows uncopied.
 int mfk_copy2d(const void *rectPlan, uint32_t, void *)
 {
     const mf::RectPlan &p = *static_cast<const mf::RectPlan *>(rectPlan);
     ++g_launches;
+    g_lastRectMates = 0;
     for (uint32_t r = 0; r < mf::kRectInline; ++r) {
-        if (p.first[r] == 0xFFFFFFFFu) {
-            break;
-        }
-        for (uint32_t row = 0; row < p.height[r]; ++row) {
+        g_lastRectMates += p.mate[r] != 0 ? 1u : 0u;
+    }
+    for (uint32_t c = 0; c < p.nchunk; ++c) {
+        uint32_t r = 0;
+        uint32_t k = 0;
+        mf::RectOfChunk(p, c, r, k);
+        const uint32_t row0 = k * p.rowsPerChunk[r];
+        for (uint32_t row = row0; row < row0 + p.rowsPerChunk[r] && row < p.height[r]; ++row) {
             std::memmove(reinterpret_cast<void *>(p.dst[r] + 16ull * p.dpitchUnits[r] * row),
                          reinterpret_cast<void *>(p.src[r] + 16ull * p.spitchUnits[r] * row), 16ull * p.widthUnits[r]);
         }

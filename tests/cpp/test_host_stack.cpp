@@ -21,6 +21,7 @@
 
 extern "C" uint64_t fake_rt_launches(void);
 extern "C" uint32_t fake_rt_last_hold(void);
+extern "C" uint32_t fake_rt_last_rect_mates(void);
 extern "C" uint32_t fake_rt_last_window(void);
 extern "C" void fake_rt_seal(void);
 extern "C" void fake_rt_fail_launches(int n);
@@ -279,6 +280,35 @@ static void TestCApi()
     }
     for (int r = 0; r < 50; ++r) {
         ok = ok && std::memcmp(dev + (1u << 20) + 3 + r * 300, host + 5 + r * 160, 100) == 0;
+    }
+    CHECK(ok);
+    // two rectangles side by side in the destination become mates and share their chunks in turn; a third of another
+    // height and one whose destination does not continue the row stay alone; every row still arrives
+    std::memset(dev, 0, pool);
+    const uint64_t h0 = reinterpret_cast<uint64_t>(host);
+    const uint64_t d0 = reinterpret_cast<uint64_t>(dev);
+    mf_copy2d_desc sideBySide[5] = {
+        {h0, d0, 896, 101, 896, 1792},
+        {h0 + 101 * 896, d0 + 896, 896, 101, 896, 1792},
+        {h0 + 202 * 896, d0 + (1u << 20), 896, 77, 896, 1792},
+        {h0 + 300 * 896, d0 + (1u << 20) + 896, 896, 76, 896, 1792},
+        {h0 + 400 * 896, d0 + (2u << 20), 4736, 9, 4736, 9472},
+    };
+    CHECK(mf_xcopy_2d_batch(sideBySide, 5, MF_ROUTE_FROM_HOST, nullptr) == BM_OK);
+    CHECK(fake_rt_last_rect_mates() == 2);
+    ok = true;
+    for (int r = 0; r < 101; ++r) {
+        ok = ok && std::memcmp(dev + r * 1792, host + r * 896, 896) == 0;
+        ok = ok && std::memcmp(dev + r * 1792 + 896, host + (101 + r) * 896, 896) == 0;
+    }
+    for (int r = 0; r < 77; ++r) {
+        ok = ok && std::memcmp(dev + (1u << 20) + r * 1792, host + (202 + r) * 896, 896) == 0;
+    }
+    for (int r = 0; r < 76; ++r) {
+        ok = ok && std::memcmp(dev + (1u << 20) + 896 + r * 1792, host + (300 + r) * 896, 896) == 0;
+    }
+    for (int r = 0; r < 9; ++r) {
+        ok = ok && std::memcmp(dev + (2u << 20) + r * 9472, host + 400 * 896 + r * 4736, 4736) == 0;
     }
     CHECK(ok);
     CHECK(smem_bm_leave(bm, 0) == SM_OK);
