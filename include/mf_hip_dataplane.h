@@ -176,6 +176,10 @@ int32_t mf_moe_combine(const void *rows, const int32_t *rowOf, const float *weig
  * 6 200 000, both 0 turns the form off (one workgroup per slice, as for smaller inputs).  Results do not depend on
  * it.  No counterpart in the reference.  Returns BM_INVALID_PARAM for other values. */
 int32_t mf_moe_combine_windows(uint32_t readMBps, uint32_t writeMBps);
+/* 1 if hybm_init found that the GPU deals consecutive workgroups to its eight XCDs in turn (an MI355X in its default
+ * partition does): the dispatch of wide rows then writes its output in runs of consecutive rows, one stream of runs
+ * per XCD; 0: it keeps to the token-ordered permute.  No counterpart in the reference. */
+int32_t mf_moe_xcd_streams(void);
 
 /* ---- runtime services (thin layer over HIP) ------------------------------ */
 int mfrt_init(int device);

@@ -46,6 +46,9 @@ MF_EXPORT int32_t hybm_init(uint16_t deviceId, uint64_t flags)
         return ret;
     }
     VaManager::Global().SetDeviceProbe(HipDeviceProbe);
+    if (mfk_moe_setup() != 0) {
+        MF_ERROR("the MoE dispatch could not probe the XCD order and keeps to its token-ordered permute");
+    }
     g_initCount = 1;
     return BM_OK;
 }

@@ -104,3 +104,8 @@ MF_EXPORT int32_t mf_moe_combine_windows(uint32_t readMBps, uint32_t writeMBps)
     mfk_moe_combine_windows(readMBps, writeMBps);
     return BM_OK;
 }
+
+MF_EXPORT int32_t mf_moe_xcd_streams(void)
+{
+    return mfk_moe_xcd_streams();
+}

@@ -713,6 +713,19 @@ __global__ __launch_bounds__(64) void MoeCombineWindowKernel(const u32x4 *__rest
     }
 }
 
+// Which XCD a wave runs on (XCC_ID, hardware register 20, bits 3:0), for mfk_moe_setup().
+__global__ void XcdProbeKernel(uint32_t *__restrict__ ids)
+{
+    if (threadIdx.x == 0) {
+        ids[blockIdx.x] = static_cast<uint32_t>(__builtin_amdgcn_s_getreg((3 << 11) | 20)) & 0xFu;
+    }
+}
+
+// 1 once mfk_moe_setup() has seen consecutive workgroups go to kTileStreams different XCDs in turn, which is what the
+// streams of MoePermuteTileKernel stand on; 0 (the loop kernel is used) before that and where the GPU deals them
+// otherwise (a partition of one XCD, for instance).
+std::atomic<int> g_xcdStreams{0};
+
 // Pace of the windowed combine, MB/s of HBM traffic in the read parts and in the write parts; 0 = never windowed.
 std::atomic<uint32_t> g_combineReadMBps{6800000};
 std::atomic<uint32_t> g_combineWriteMBps{6200000};
@@ -758,7 +771,8 @@ extern "C" int mfk_moe_dispatch(const void *x, const void *topk, uint32_t tokens
     const uint64_t blockTokenBytes = static_cast<uint64_t>(kRankBlock / topK + 1) * hidden * 2;
     const uint32_t tilesPerRow = (upr + kTileUnits - 1) / kTileUnits;
     const uint64_t tileGrid = static_cast<uint64_t>((blocks + kTileStreams - 1) / kTileStreams * kTileStreams) * kRankBlock * tilesPerRow;
-    const bool tiles = x != nullptr && out != nullptr && upr >= 512 && blockTokenBytes <= 2200000ull &&
+    const bool tiles = g_xcdStreams.load(std::memory_order_relaxed) != 0 && x != nullptr && out != nullptr && upr >= 512 &&
+                       blockTokenBytes <= 2200000ull &&
                        blocks >= 2 * kTileStreams && tileGrid <= 0x7FFFFFFFull;
     const uint64_t tableBytes = 256 + histStride * sizeof(uint32_t) + static_cast<uint64_t>(histStride) * experts * sizeof(uint32_t);
     int2 *runOrder = tiles ? reinterpret_cast<int2 *>(static_cast<char *>(workspace) + (tableBytes + 15) / 16 * 16) : nullptr;
@@ -850,4 +864,39 @@ extern "C" void mfk_moe_combine_windows(uint32_t readMBps, uint32_t writeMBps)
 {
     mf::g_combineReadMBps.store(readMBps, std::memory_order_relaxed);
     mf::g_combineWriteMBps.store(writeMBps, std::memory_order_relaxed);
+}
+
+// Once per process, after the GPU has been bound and outside any stream capture (it waits for a small kernel):
+// checks that workgroup i of a launch runs on XCD i mod 8.
+extern "C" int mfk_moe_setup(void)
+{
+    constexpr uint32_t kProbe = 256;
+    uint32_t *dev = nullptr;
+    hipError_t err = hipMalloc(reinterpret_cast<void **>(&dev), kProbe * sizeof(uint32_t));
+    if (err != hipSuccess) {
+        return static_cast<int>(err);
+    }
+    uint32_t ids[kProbe];
+    hipLaunchKernelGGL(mf::XcdProbeKernel, dim3(kProbe), dim3(64), 0, nullptr, dev);
+    err = hipMemcpy(ids, dev, sizeof(ids), hipMemcpyDeviceToHost);
+    (void)hipFree(dev);
+    if (err != hipSuccess) {
+        return static_cast<int>(err);
+    }
+    bool inTurn = true;
+    for (uint32_t i = 0; i < kProbe; ++i) {
+        inTurn = inTurn && ids[i] == ids[i % mf::kTileStreams];
+    }
+    for (uint32_t a = 0; a < mf::kTileStreams; ++a) {
+        for (uint32_t b = a + 1; b < mf::kTileStreams; ++b) {
+            inTurn = inTurn && ids[a] != ids[b];
+        }
+    }
+    mf::g_xcdStreams.store(inTurn ? 1 : 0, std::memory_order_relaxed);
+    return 0;
+}
+
+extern "C" int mfk_moe_xcd_streams(void)
+{
+    return mf::g_xcdStreams.load(std::memory_order_relaxed);
 }

@@ -104,6 +104,10 @@ int mfk_moe_dispatch(const void *x, const void *topk, uint32_t tokens, uint32_t 
                      void *out, void *counts, void *offsets, void *rowOf, void *srcOf, void *workspace, void *stream);
 int mfk_moe_combine(const void *rows, const void *rowOf, const void *weights, uint32_t tokens, uint32_t hidden,
                     uint32_t topK, void *y, void *stream);
+/* once after the GPU is bound: finds out whether consecutive workgroups go to the eight XCDs in turn (the tile permute
+ * of the dispatch needs it); mfk_moe_xcd_streams() is 1 if they do */
+int mfk_moe_setup(void);
+int mfk_moe_xcd_streams(void);
 /* pace of the combine that keeps reads and writes apart in time, MB/s for its read and write parts; 0 = never */
 void mfk_moe_combine_windows(uint32_t readMBps, uint32_t writeMBps);
 

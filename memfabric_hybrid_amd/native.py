@@ -201,6 +201,7 @@ _SIGNATURES = {
     "mf_moe_dispatch": (i32, [vp, vp, u32, u32, u32, u32, vp, vp, vp, vp, vp, vp, u64, vp]),
     "mf_moe_combine": (i32, [vp, vp, vp, u32, u32, u32, vp, vp]),
     "mf_moe_combine_windows": (i32, [u32, u32]),
+    "mf_moe_xcd_streams": (i32, []),
     "mfrt_init": (ctypes.c_int, [ctypes.c_int]),
     "mfrt_shutdown": (None, []),
     "mfrt_is_initialised": (ctypes.c_int, []),

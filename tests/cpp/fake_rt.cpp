@@ -356,4 +356,6 @@ int mfk_moe_dispatch(const void *, const void *, uint32_t, uint32_t, uint32_t, u
                      void *, void *) { return -1; }
 int mfk_moe_combine(const void *, const void *, const void *, uint32_t, uint32_t, uint32_t, void *, void *) { return -1; }
 void mfk_moe_combine_windows(uint32_t, uint32_t) {}
+int mfk_moe_setup(void) { return 0; }
+int mfk_moe_xcd_streams(void) { return 0; }
 }

@@ -128,6 +128,7 @@ def test_output_ordered_permute(gpu, oracle, T, H, E, routing):
     """Rows wide enough and blocks enough for the permute that walks the output in runs of consecutive rows per
     expert, in tiles: every output row and every map against the oracle."""
     K = 8
+    assert gpu.mf_moe_xcd_streams() == 1        # an MI355X in its default partition: the form under test is the one that runs
     x, topk, _ = _inputs(oracle, 0xD1 + T, T, H, K, E)
     rng = np.random.default_rng(T)
     if routing == "five":
