@@ -118,20 +118,24 @@ def test_dispatch_and_combine_match_the_specification(gpu, oracle, T, H, K, E):
         _free(bufs)
 
 
-@pytest.mark.parametrize("T,H,E,routing", [
-    (2000, 4096, 64, "router"),     # 16 000 entries: fifteen full blocks and a last one of 640 entries
-    (2500, 7168, 300, "router"),    # twenty blocks, which the eight streams do not divide
-    (2200, 7168, 256, "five"),      # everything lands on five experts, duplicates inside a token included: long runs
-    (2200, 5120, 256, "bad ids"),   # some ids out of range: their slots name no row, the lists of their blocks are shorter
+@pytest.mark.parametrize("T,H,K,E,routing", [
+    (2000, 4096, 8, 64, "router"),     # 16 000 entries: fifteen full blocks and a last one of 640 entries
+    (2500, 7168, 8, 300, "router"),    # twenty blocks, which the eight streams do not divide
+    (2200, 7168, 8, 256, "five"),      # everything lands on five experts, duplicates inside a token included: long runs
+    (2200, 5120, 8, 256, "bad ids"),   # some ids out of range: their slots name no row, the lists of their blocks are shorter
+    (1200, 4096, 16, 128, "router"),   # sixty-four tokens per block
+    (2800, 4096, 6, 64, "router"),     # blocks that begin and end inside a token
+    (3000, 8200, 8, 1, "one"),         # one expert: the output is the input, every row eight times; rows that end inside a tile
 ])
-def test_output_ordered_permute(gpu, oracle, T, H, E, routing):
+def test_output_ordered_permute(gpu, oracle, T, H, K, E, routing):
     """Rows wide enough and blocks enough for the permute that walks the output in runs of consecutive rows per
     expert, in tiles: every output row and every map against the oracle."""
-    K = 8
     assert gpu.mf_moe_xcd_streams() == 1        # an MI355X in its default partition: the form under test is the one that runs
-    x, topk, _ = _inputs(oracle, 0xD1 + T, T, H, K, E)
+    x, topk, _ = _inputs(oracle, 0xD1 + T, T, H, min(K, E), E)
     rng = np.random.default_rng(T)
-    if routing == "five":
+    if routing == "one":
+        topk = np.zeros((T, K), dtype=np.int32)
+    elif routing == "five":
         topk = rng.integers(0, 5, (T, K)).astype(np.int32)
         topk[::7, 0] = E - 1
     elif routing == "bad ids":
