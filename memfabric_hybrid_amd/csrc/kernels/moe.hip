@@ -40,6 +40,7 @@ constexpr uint32_t kRankSlices = kRankBlock / 64;      // 16 wave-sized slices, 
 constexpr uint32_t kMaxExperts = 512;
 constexpr uint32_t kRowThreads = 256;
 constexpr uint32_t kMaxTopK = 16;
+constexpr uint32_t kHistPad = 32;                      // rows of the [expert][block] table are padded to this many blocks
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 #define MF_GLOBAL __attribute__((address_space(1)))
@@ -116,7 +117,7 @@ __global__ __launch_bounds__(kRankThreads) void MoeHistKernel(const int32_t *__r
         for (uint32_t s = 0; s < kRankSlices; ++s) {
             sum += hist[s * experts + x];
         }
-        blockHist[static_cast<uint64_t>(x) * histStride + blockIdx.x] = sum;  // [expert][block], rows padded to 4
+        blockHist[static_cast<uint64_t>(x) * histStride + blockIdx.x] = sum;  // [expert][block], rows padded to kHistPad
         if (blockIdx.x == 0) {
             for (uint32_t pad = gridDim.x; pad < histStride; ++pad) {
                 blockHist[static_cast<uint64_t>(x) * histStride + pad] = 0;
@@ -176,12 +177,21 @@ __global__ __launch_bounds__(kRankThreads) void MoeRankKernel(const int32_t *__r
             const uint32_t *rowHist = blockHist + static_cast<uint64_t>(x) * histStride;
             uint32_t t = 0;
             uint32_t b = 0;
-            for (uint32_t blk = 0; blk < gridDim.x; blk += 4) {
-                const u32x4 v = *reinterpret_cast<const u32x4 *>(rowHist + blk);  // padded with zeros up to histStride
+            // kHistPad blocks per step, all their loads requested before the first is used: with one load per step the
+            // loop waited a full round trip per four blocks (8 of the kernel's 10 us at 64 blocks)
+            for (uint32_t blk = 0; blk < gridDim.x; blk += kHistPad) {
+                u32x4 v[kHistPad / 4];
 #pragma unroll
-                for (uint32_t i = 0; i < 4; ++i) {
-                    t += v[i];
-                    b += blk + i < blockIdx.x ? v[i] : 0u;
+                for (uint32_t q = 0; q < kHistPad / 4; ++q) {
+                    v[q] = *reinterpret_cast<const u32x4 *>(rowHist + blk + 4 * q);  // rows are padded with zeros up to histStride
+                }
+#pragma unroll
+                for (uint32_t q = 0; q < kHistPad / 4; ++q) {
+#pragma unroll
+                    for (uint32_t i = 0; i < 4; ++i) {
+                        t += v[q][i];
+                        b += blk + 4 * q + i < blockIdx.x ? v[q][i] : 0u;
+                    }
                 }
             }
             tot[j] = t;
@@ -737,7 +747,7 @@ extern "C" uint64_t mfk_moe_workspace_bytes(uint32_t tokens, uint32_t topK, uint
 {
     const uint64_t total = static_cast<uint64_t>(tokens) * topK;
     const uint64_t blocks = (total + mf::kRankBlock - 1) / mf::kRankBlock;
-    const uint64_t stride = (blocks + 3) / 4 * 4;
+    const uint64_t stride = (blocks + mf::kHistPad - 1) / mf::kHistPad * mf::kHistPad;
     // status words, per-block flags, the [expert][block] histogram, the run-ordered row list (8 bytes per entry slot)
     const uint64_t tables = 256 + stride * sizeof(uint32_t) + stride * experts * sizeof(uint32_t);
     return (tables + 15) / 16 * 16 + blocks * mf::kRankBlock * sizeof(int2);
@@ -757,7 +767,7 @@ extern "C" int mfk_moe_dispatch(const void *x, const void *topk, uint32_t tokens
     const uint32_t blocks = (total + kRankBlock - 1) / kRankBlock;
     hipStream_t s = static_cast<hipStream_t>(stream);
     uint32_t *status = static_cast<uint32_t *>(workspace);
-    const uint32_t histStride = (blocks + 3) / 4 * 4;     // rows of the [expert][block] table, 16-byte granular
+    const uint32_t histStride = (blocks + kHistPad - 1) / kHistPad * kHistPad;   // rows of the [expert][block] table
     uint32_t *blockBad = status + 64;
     uint32_t *blockHist = blockBad + histStride;
     const size_t histLds = static_cast<size_t>(kRankSlices) * experts * sizeof(uint32_t);
