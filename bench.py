@@ -303,7 +303,7 @@ def extras_block(lib, pool, dev, batches, tables, steps):
         held.append(timed_steps(lib, handle, batches, g2g, ku, 0, native.ASYNC_COPY_FLAG)[1] * 1e3 / ku)
     out["kv122_held_stores"] = {
         "us_per_batch_not_held": round(median(not_held), 2), "us_per_batch_held": round(median(held), 2),
-        "note": "mf_xcopy_hold_stores(0) against the default (every wave of a 960 to 5632 chunk launch keeps its data until the "
+        "note": "mf_xcopy_hold_stores(0) against the default (every wave of a 960 to 6144 chunk launch keeps its data until the "
                 "loads of the whole launch are out, so HBM sees a read burst and then a write burst); 5 alternations, medians"}
     conc = {}
     kc = max(MIN_BATCHES, steps)

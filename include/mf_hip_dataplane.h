@@ -117,7 +117,7 @@ uint32_t mf_copy2d_rowcol_mismatches(uint32_t widthUnits, uint32_t rowsPerChunk,
  * default: one workgroup per chunk, no cap); wgPerCuLink: workgroups per CU
  * on host-link routes (0 = the default, 1). */
 int32_t mf_xcopy_tune(uint32_t units, uint32_t wgPerCu, uint32_t wgPerCuLink);
-/* Stores held back.  A batch of 960 to 5632 chunks of 4 KiB between HBM addresses (4 to 23 MB in up
+/* Stores held back.  A batch of 960 to 6144 chunks of 4 KiB between HBM addresses (4 to 25 MB in up
  * to 128 segments) is copied 7 to 20 % faster when every wave waits with its stores until the loads of
  * the whole launch are out, so that HBM sees a burst of reads and then a burst of writes instead of both
  * mixed.  nanos: -1 = the library's rule for how long a wave waits after its start (the default),
