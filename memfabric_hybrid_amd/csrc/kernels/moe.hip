@@ -795,21 +795,20 @@ extern "C" int mfk_moe_dispatch(const void *x, const void *topk, uint32_t tokens
         const u32x4 *xi = static_cast<const u32x4 *>(x);
         const int32_t *ro = static_cast<const int32_t *>(rowOf);
         u32x4 *oo = static_cast<u32x4 *>(out);
-        // Wide rows: single-wave workgroups that hold up to 14 pieces per lane (a whole 7168-element
-        // row) and write them with plain stores.  Storing alone takes 177 us of the 200 us such a
-        // kernel needs when every wave reads its row first; with sixteen waves per CU that each
-        // take several tokens and fetch the next row while they store the current one
-        // the dispatch takes 207 us instead of 215.  Other shapes measured on these rows: two waves
-        // per row 221 us; four-wave workgroups with nontemporal stores 237 us; the row staged in LDS
-        // instead of registers 221 us (one wave) and 227 us (four waves); buffer-addressed
-        // stores at eight waves per SIMD 224 us; the destination-side form, one workgroup per output
-        // row reading x[srcOf[row]], 271 us: its eight reads of every token row are not absorbed by
-        // the caches.
-        // Narrow rows: one four-wave workgroup per token.
         if (tiles) {
             hipLaunchKernelGGL(MoePermuteTileKernel, dim3(static_cast<uint32_t>(tileGrid)), dim3(64), 0, s, xi, runOrder, upr,
                                tilesPerRow, blocks, oo);
         } else if (upr >= 512) {
+            // Wide rows: single-wave workgroups that hold up to 14 pieces per lane (a whole 7168-element
+            // row) and write them with plain stores.  Storing alone takes 177 us of the 200 us such a
+            // kernel needs when every wave reads its row first; with sixteen waves per CU that each
+            // take several tokens and fetch the next row while they store the current one
+            // the dispatch takes 207 us instead of 215.  Other shapes measured on these rows: two waves
+            // per row 221 us; four-wave workgroups with nontemporal stores 237 us; the row staged in LDS
+            // instead of registers 221 us (one wave) and 227 us (four waves); buffer-addressed
+            // stores at eight waves per SIMD 224 us; the destination-side form, one workgroup per output
+            // row reading x[srcOf[row]], 271 us: its eight reads of every token row are not absorbed by
+            // the caches.
             // 123 vector registers per lane: four waves per SIMD, sixteen per CU, all resident at once
             const uint32_t wideParts = (upr + 64 * 14 - 1) / (64 * 14);
             const uint32_t items = tokens * wideParts;
@@ -817,6 +816,7 @@ extern "C" int mfk_moe_dispatch(const void *x, const void *topk, uint32_t tokens
             hipLaunchKernelGGL((MoePermuteLoopKernel<14>), dim3(items < waves ? items : waves), dim3(64), 0, s, xi, ro, topK, upr,
                                wideParts, items, oo);
         } else {
+            // Narrow rows: one four-wave workgroup per token.
             hipLaunchKernelGGL((MoePermuteKernel<256, 4, 1>), dim3(tokens), dim3(256), 0, s, xi, ro, topK, upr, 1u, oo);
         }
     }
