@@ -27,8 +27,11 @@ __device__ __forceinline__ void WaitForClock(uint64_t t)
 // (Deriving the start from the clock alone, as the next multiple of the period, costs every launch half a
 // period on average: 10 us, 3 % of a 1 GiB copy.  Letting whichever wave comes first publish with a
 // compare-and-swap serialises 4096 same-address atomics across the XCDs: 1.2 ms.)  A wave that does not see
-// the value within a few microseconds goes by its own clock, so no wave waits on another for long.  One slot
-// per launch in flight; a slot is reused after kEpochSlots launches.
+// a fresh value within its polls (workgroup 0 has not started yet, or started more than kEpochFreshTicks ago:
+// other work holds part of the chip and the waves of this launch are not all resident together) gets 0, a
+// start so long ago that every slot of its schedule has passed: it runs unpaced, as fast as it can, instead
+// of holding a schedule cut for a chip it does not have.  One slot per launch in flight; a slot is reused
+// after kEpochSlots launches.
 constexpr uint32_t kEpochSlots = 64;
 constexpr uint32_t kEpochPolls = 64;
 constexpr uint32_t kEpochFreshTicks = 2000;                 // workgroup 0 starts at most 20 us before any other wave of its launch
@@ -56,7 +59,7 @@ __device__ __forceinline__ uint64_t AgreedStart(uint32_t seq)
         }
         __builtin_amdgcn_s_sleep(4);
     }
-    return mine;
+    return 0;
 }
 
 // Period (ticks of the constant-rate clock) in which `bytes` of HBM traffic, read + written, pass at windowMBps
