@@ -173,8 +173,8 @@ int32_t mf_moe_combine(const void *rows, const int32_t *rowOf, const float *weig
  * slices of 128 x 8 elements (about 3500 tokens of 7168 elements on 256 CUs), runs as waves that stay for the whole
  * launch and alternate, chip-wide and by the clock, between reading rows and writing results.  readMBps / writeMBps
  * (MB/s of HBM traffic, 1 000 000 ... 16 000 000) set the pace of the two parts; the defaults are 6 800 000 and
- * 6 200 000, both 0 turns the form off (one workgroup per slice, as for smaller inputs).  Results do not depend on
- * it.  No counterpart in the reference.  Returns BM_INVALID_PARAM for other values. */
+ * 6 200 000, both 0 turns the form off (one workgroup per slice, as for smaller inputs, and as long as a second
+ * thread holds a stream of the library).  Results do not depend on it.  No counterpart in the reference.  Returns BM_INVALID_PARAM for other values. */
 int32_t mf_moe_combine_windows(uint32_t readMBps, uint32_t writeMBps);
 /* 1 if hybm_init found that the GPU deals consecutive workgroups to its eight XCDs in turn (an MI355X in its default
  * partition does): the dispatch of wide rows then writes its output in runs of consecutive rows, one stream of runs

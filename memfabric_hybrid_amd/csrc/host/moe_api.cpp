@@ -86,7 +86,10 @@ MF_EXPORT int32_t mf_moe_combine(const void *rows, const int32_t *rowOf, const f
     if (ret != BM_OK) {
         return ret;
     }
-    int err = mfk_moe_combine(rows, rowOf, weights, tokens, hidden, topK, y, stream);
+    // A kernel that paces itself for the whole chip's rate is the wrong one while other threads submit work of their
+    // own (beside a stream of 1 GiB copies the paced combine took 555 us, the other form 400 us), as for the copies.
+    const int paced = XcopyEngine::Instance().SingleSubmitter() ? 1 : 0;
+    int err = mfk_moe_combine(rows, rowOf, weights, tokens, hidden, topK, y, stream, paced);
     if (err != 0) {
         MF_FAIL(BM_ERROR, "mf_moe_combine: launch failed: " << (err > 0 ? mfrt_error_string(err) : "bad shape"));
     }

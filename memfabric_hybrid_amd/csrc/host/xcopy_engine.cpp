@@ -774,6 +774,11 @@ bool XcopyEngine::WindowsApply(uint64_t bytes, int route) const
            g_leasesOut.load(std::memory_order_relaxed) <= 1;
 }
 
+bool XcopyEngine::SingleSubmitter() const
+{
+    return g_leasesOut.load(std::memory_order_relaxed) <= 1;
+}
+
 int XcopyEngine::Submit(const uint64_t *src, const uint64_t *dst, const uint64_t *len, uint32_t n, int route,
                         void *stream, void *mask, uint32_t maskValue, bool unordered)
 {

@@ -91,6 +91,8 @@ public:
 
     // Whether an ordered launch that moves `bytes` on `route` takes the form with read and write windows.
     bool WindowsApply(uint64_t bytes, int route) const;
+    // No second thread holds a stream of the library: kernels that pace themselves for the whole chip may be used.
+    bool SingleSubmitter() const;
 
     // The calling thread's own stream (created on first use).
     void *ThreadStream();

@@ -824,7 +824,7 @@ extern "C" int mfk_moe_dispatch(const void *x, const void *topk, uint32_t tokens
 }
 
 extern "C" int mfk_moe_combine(const void *rows, const void *rowOf, const void *weights, uint32_t tokens,
-                               uint32_t hidden, uint32_t topK, void *y, void *stream)
+                               uint32_t hidden, uint32_t topK, void *y, void *stream, int paced)
 {
     using namespace mf;
     if (tokens == 0 || topK == 0 || topK > kMaxTopK || hidden == 0 || (static_cast<uint64_t>(hidden) * 2) % 16 != 0) {
@@ -853,8 +853,8 @@ extern "C" int mfk_moe_combine(const void *rows, const void *rowOf, const void *
                                                          g_combineReadMBps.load(std::memory_order_relaxed));
             const uint32_t writeTicks = WindowPeriodTicks(static_cast<uint64_t>(waves) * kCombineItems * perPart * 16,
                                                           g_combineWriteMBps.load(std::memory_order_relaxed));
-            if (items >= static_cast<uint64_t>(waves) * kCombineMinItemsPerWave && items < 0x40000000ull && readTicks != 0 &&
-                writeTicks != 0) {
+            if (paced != 0 && items >= static_cast<uint64_t>(waves) * kCombineMinItemsPerWave && items < 0x40000000ull &&
+                readTicks != 0 && writeTicks != 0) {
                 hipLaunchKernelGGL((MoeCombineWindowKernel<kCombineItems>), dim3(waves), dim3(64), 0, s, in, ro, w, upr, parts,
                                    static_cast<uint32_t>(items), o, readTicks, writeTicks, NextWindowSeq());
             } else {

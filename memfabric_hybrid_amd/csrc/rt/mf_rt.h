@@ -102,8 +102,9 @@ int mfk_xcopy_table_static(const void *triples, uint32_t nseg, uint32_t units, i
 uint64_t mfk_moe_workspace_bytes(uint32_t tokens, uint32_t topK, uint32_t experts);
 int mfk_moe_dispatch(const void *x, const void *topk, uint32_t tokens, uint32_t hidden, uint32_t topK, uint32_t experts,
                      void *out, void *counts, void *offsets, void *rowOf, void *srcOf, void *workspace, void *stream);
+/* paced != 0: the form whose waves stay and alternate between reading and writing may be used (see mfk_moe_combine_windows) */
 int mfk_moe_combine(const void *rows, const void *rowOf, const void *weights, uint32_t tokens, uint32_t hidden,
-                    uint32_t topK, void *y, void *stream);
+                    uint32_t topK, void *y, void *stream, int paced);
 /* once after the GPU is bound: finds out whether consecutive workgroups go to the eight XCDs in turn (the tile permute
  * of the dispatch needs it); mfk_moe_xcd_streams() is 1 if they do */
 int mfk_moe_setup(void);

@@ -354,7 +354,13 @@ int mfk_copy2d(const void *rectPlan, uint32_t, void *)
 uint64_t mfk_moe_workspace_bytes(uint32_t, uint32_t, uint32_t) { return 0; }
 int mfk_moe_dispatch(const void *, const void *, uint32_t, uint32_t, uint32_t, uint32_t, void *, void *, void *, void *, void *,
                      void *, void *) { return -1; }
-int mfk_moe_combine(const void *, const void *, const void *, uint32_t, uint32_t, uint32_t, void *, void *) { return -1; }
+static int g_lastCombinePaced = -1;
+extern "C" int fake_rt_last_combine_paced() { return g_lastCombinePaced; }
+int mfk_moe_combine(const void *, const void *, const void *, uint32_t, uint32_t, uint32_t, void *, void *, int paced)
+{
+    g_lastCombinePaced = paced;
+    return 0;
+}
 void mfk_moe_combine_windows(uint32_t, uint32_t) {}
 int mfk_moe_setup(void) { return 0; }
 int mfk_moe_xcd_streams(void) { return 0; }

@@ -22,6 +22,7 @@
 extern "C" uint64_t fake_rt_launches(void);
 extern "C" uint32_t fake_rt_last_hold(void);
 extern "C" uint32_t fake_rt_last_rect_mates(void);
+extern "C" int fake_rt_last_combine_paced(void);
 extern "C" uint32_t fake_rt_last_window(void);
 extern "C" void fake_rt_seal(void);
 extern "C" void fake_rt_fail_launches(int n);
@@ -891,8 +892,16 @@ static void TestHeldStores()
         CHECK(fake_rt_last_hold() == 0);
         CHECK(engine.Submit(src.data(), dst.data(), len.data(), count, MF_ROUTE_HBM, stream, nullptr, 0) == BM_OK);
         CHECK(fake_rt_last_hold() == HoldNanosFor(1024, 1024, 256, false));   // small launches keep the wait
+        // the MoE combine leaves its paced form alone as long as the second thread has its stream
+        alignas(16) static uint8_t moeBuf[64];
+        CHECK(mf_moe_combine(moeBuf, reinterpret_cast<const int32_t *>(moeBuf), reinterpret_cast<const float *>(moeBuf), 1, 8, 1,
+                             moeBuf + 16, nullptr) == BM_OK);
+        CHECK(fake_rt_last_combine_paced() == 0);
         phase.store(2);
         other.join();
+        CHECK(mf_moe_combine(moeBuf, reinterpret_cast<const int32_t *>(moeBuf), reinterpret_cast<const float *>(moeBuf), 1, 8, 1,
+                             moeBuf + 16, nullptr) == BM_OK);
+        CHECK(fake_rt_last_combine_paced() == 1);
         CHECK(engine.Submit(s5, d5, l5, 2, MF_ROUTE_HBM, stream, nullptr, 0) == BM_OK);
         CHECK(fake_rt_last_hold() == HoldNanosFor(5120, 5120, 256, false));
         CHECK(engine.DrainThread() == BM_OK);
