@@ -137,13 +137,14 @@ __global__ __launch_bounds__(kRankThreads) void MoeRankKernel(const int32_t *__r
                                                               int32_t *__restrict__ rowOf, int32_t *__restrict__ srcOf,
                                                               const uint32_t *__restrict__ blockBad,
                                                               uint32_t *__restrict__ status, uint32_t topK,
-                                                              int2 *__restrict__ runOrder)
+                                                              int2 *__restrict__ runOrder, uint32_t stepSlices)
 {
     extern __shared__ uint32_t lds[];
     uint32_t *hist = lds;                                 // [kRankSlices][experts]
     uint32_t *base = lds + kRankSlices * experts;         // [experts] first row of this block's entries per expert
-    uint32_t *scan = base + experts;                      // [kRankThreads] scratch of the block scans
-    uint32_t *cum = scan + kRankThreads;                  // [experts] entries of this block with a smaller expert id
+    uint32_t *scan = base + experts;                      // [kRankThreads] scratch of the block scan
+    uint32_t *stepValid = scan + kRankThreads;            // [kRankSlices] entries with a row in each step of the block
+    uint32_t *cum = stepValid + kRankSlices;              // [steps][experts] entries of the step with a smaller expert id
     uint32_t myExpert[kRankRounds];
     uint32_t myRank[kRankRounds];
     uint32_t bad = 0;
@@ -228,58 +229,60 @@ __global__ __launch_bounds__(kRankThreads) void MoeRankKernel(const int32_t *__r
         }
     }
     __syncthreads();
-    // turn slice histograms into exclusive prefixes over the slices of this block; the same threads own the same
-    // experts as above, so the block's own entries per expert can be scanned over the experts next
-    uint32_t ownOf[kMaxExperts / kRankThreads];          // this block's entries per owned expert
-    uint32_t own = 0;
-#pragma unroll
-    for (uint32_t j = 0; j < kMaxExperts / kRankThreads; ++j) {
-        ownOf[j] = 0;
-        const uint32_t x = threadIdx.x * per + j;
-        if (j < per && x < experts) {
-            uint32_t acc = base[x];
-            for (uint32_t s = 0; s < kRankSlices; ++s) {
-                const uint32_t v = hist[s * experts + x];
-                hist[s * experts + x] = acc;
-                acc += v;
-            }
-            ownOf[j] = acc - base[x];
-            own += ownOf[j];
-        }
-    }
-    uint32_t valid = 0;
-    if (runOrder != nullptr) {
-        // cum[x] = entries of this block routed to an expert below x: where the block's rows of expert x start in
-        // the list of the block's rows in ascending order
-        uint32_t inclOwn = own;
-#pragma unroll
-        for (uint32_t step = 1; step < 64; step <<= 1) {
-            const uint32_t up = __shfl_up(inclOwn, step, 64);
-            inclOwn += (threadIdx.x & 63u) >= step ? up : 0u;
-        }
-        __syncthreads();                                  // the first scan's readers are done with scan[]
-        if ((threadIdx.x & 63u) == 63u) {
-            scan[threadIdx.x >> 6] = inclOwn;
-        }
-        __syncthreads();
-        uint32_t ownBase = 0;
-        for (uint32_t wv = 0; wv < kRankThreads / 64; ++wv) {
-            ownBase += wv < (threadIdx.x >> 6) ? scan[wv] : 0u;
-            valid += scan[wv];
-        }
-        uint32_t at = inclOwn + ownBase - own;
-#pragma unroll
-        for (uint32_t j = 0; j < kMaxExperts / kRankThreads; ++j) {
-            const uint32_t x = threadIdx.x * per + j;
-            if (j < per && x < experts) {
-                cum[x] = at;
-                at += ownOf[j];
+    // Turn slice histograms into exclusive prefixes over the slices of this block.  For the run-ordered list the
+    // block is cut into steps of stepSlices slices (the tile permute works through one step at a time); the
+    // entries per (step, expert) are what the prefix gains over a step.
+    const uint32_t steps = runOrder != nullptr ? kRankSlices / stepSlices : 0;
+    for (uint32_t x = threadIdx.x; x < experts; x += kRankThreads) {
+        uint32_t acc = base[x];
+        uint32_t stepStart = acc;
+        for (uint32_t s = 0; s < kRankSlices; ++s) {
+            const uint32_t v = hist[s * experts + x];
+            hist[s * experts + x] = acc;
+            acc += v;
+            if (steps != 0 && (s + 1) % stepSlices == 0) {
+                cum[(s / stepSlices) * experts + x] = acc - stepStart;
+                stepStart = acc;
             }
         }
     }
     __syncthreads();
     const uint32_t lane = threadIdx.x & 63u;
     const uint32_t wave = threadIdx.x >> 6;
+    if (steps != 0) {
+        // cum[j][x]: entries of step j routed to an expert below x, i.e. where the rows of expert x start in the list
+        // of the step's rows in ascending order.  One wave per step; a lane scans experts/64 neighbours itself.
+        const uint32_t perLane = (experts + 63) / 64;     // at most kMaxExperts / 64
+        for (uint32_t j = wave; j < steps; j += kRankThreads / 64) {
+            uint32_t mineOf[kMaxExperts / 64];
+            uint32_t sum = 0;
+#pragma unroll
+            for (uint32_t i = 0; i < kMaxExperts / 64; ++i) {
+                const uint32_t x = lane * perLane + i;
+                mineOf[i] = i < perLane && x < experts ? cum[j * experts + x] : 0u;
+                sum += mineOf[i];
+            }
+            uint32_t incl2 = sum;
+#pragma unroll
+            for (uint32_t step = 1; step < 64; step <<= 1) {
+                const uint32_t up = __shfl_up(incl2, step, 64);
+                incl2 += lane >= step ? up : 0u;
+            }
+            uint32_t at = incl2 - sum;
+#pragma unroll
+            for (uint32_t i = 0; i < kMaxExperts / 64; ++i) {
+                const uint32_t x = lane * perLane + i;
+                if (i < perLane && x < experts) {
+                    cum[j * experts + x] = at;
+                    at += mineOf[i];
+                }
+            }
+            if (lane == 63) {
+                stepValid[j] = incl2;
+            }
+        }
+        __syncthreads();
+    }
 #pragma unroll
     for (uint32_t r = 0; r < kRankRounds; ++r) {
         const uint32_t slice = wave + r * (kRankThreads / 64);
@@ -292,8 +295,10 @@ __global__ __launch_bounds__(kRankThreads) void MoeRankKernel(const int32_t *__r
                     srcOf[row] = static_cast<int32_t>(idx);
                 }
                 if (runOrder != nullptr) {
-                    const uint32_t at = cum[myExpert[r]] + (static_cast<uint32_t>(row) - base[myExpert[r]]);
-                    runOrder[static_cast<uint64_t>(blockIdx.x) * kRankBlock + at] =
+                    const uint32_t j = slice / stepSlices;
+                    const uint32_t firstOfStep = hist[j * stepSlices * experts + myExpert[r]];
+                    const uint32_t at = cum[j * experts + myExpert[r]] + (static_cast<uint32_t>(row) - firstOfStep);
+                    runOrder[static_cast<uint64_t>(blockIdx.x) * kRankBlock + j * stepSlices * 64 + at] =
                         make_int2(row, static_cast<int32_t>(idx / topK));
                 }
             }
@@ -301,9 +306,13 @@ __global__ __launch_bounds__(kRankThreads) void MoeRankKernel(const int32_t *__r
         }
     }
     if (runOrder != nullptr) {
-        // slots past the block's valid entries (ids out of range, the tail of the last block) name no row
-        for (uint32_t at = valid + threadIdx.x; at < kRankBlock; at += kRankThreads) {
-            runOrder[static_cast<uint64_t>(blockIdx.x) * kRankBlock + at] = make_int2(-1, 0);
+        // slots past a step's valid entries (ids out of range, the tail of the last block) name no row
+        const uint32_t stepEntries = stepSlices * 64;
+        for (uint32_t slot = threadIdx.x; slot < kRankBlock; slot += kRankThreads) {
+            const uint32_t j = slot / stepEntries;
+            if (slot - j * stepEntries >= stepValid[j]) {
+                runOrder[static_cast<uint64_t>(blockIdx.x) * kRankBlock + slot] = make_int2(-1, 0);
+            }
         }
     }
 }
@@ -443,10 +452,11 @@ __global__ __launch_bounds__(64) void MoePermuteLoopKernel(const u32x4 *__restri
 }
 
 // The permute of wide rows when a block of kRankBlock entries holds no more of x than an XCD's L2 keeps:
-// output-ordered, in tiles.  runOrder lists, block of entries by block, the block's output rows in ascending
+// output-ordered, in tiles.  runOrder lists, step by step (a step is a block of kRankBlock entries or a power-of-two
+// part of one, chosen so that the token rows of a step fit), the step's output rows in ascending
 // order (runs of consecutive rows per expert) with the token each row is a copy of.  Workgroup i, a single
 // wave, belongs to stream i % 8 (the dispatcher deals consecutive workgroups to the eight XCDs in turn);
-// stream s takes the blocks s, s + 8, ... one after the other and walks a block's rows in list order, a row in
+// stream s takes the steps s, s + 8, ... one after the other and walks a step's rows in list order, a row in
 // tiles of 128 units (2 KiB).  So an XCD writes runs of consecutive rows front to back, two stores per wave,
 // which is the only store pattern this part takes at more than 5.4 TB/s (6.1 in runs of 128 KiB, 6.6 in
 // eight sequential streams; waves that store 14 KiB each: 5.4 in any order), and the K reads of a token row
@@ -459,18 +469,18 @@ constexpr uint32_t kTileUnits = 128;
 constexpr uint32_t kTileStreams = 8;
 
 __global__ __launch_bounds__(64) void MoePermuteTileKernel(const u32x4 *__restrict__ x, const int2 *__restrict__ runOrder,
-                                                           uint32_t unitsPerRow, uint32_t tilesPerRow, uint32_t blocks,
-                                                           u32x4 *__restrict__ out)
+                                                           uint32_t unitsPerRow, uint32_t tilesPerRow, uint32_t steps,
+                                                           uint32_t stepEntries, u32x4 *__restrict__ out)
 {
     const uint32_t stream = blockIdx.x % kTileStreams;
     const uint32_t q = blockIdx.x / kTileStreams;
-    const uint32_t tilesPerBlock = kRankBlock * tilesPerRow;
-    const uint32_t block = (q / tilesPerBlock) * kTileStreams + stream;
-    const uint32_t within = q % tilesPerBlock;
-    if (block >= blocks) {
+    const uint32_t tilesPerStep = stepEntries * tilesPerRow;
+    const uint32_t step = (q / tilesPerStep) * kTileStreams + stream;
+    const uint32_t within = q % tilesPerStep;
+    if (step >= steps) {
         return;
     }
-    const int2 rowAndToken = runOrder[static_cast<uint64_t>(block) * kRankBlock + within / tilesPerRow];
+    const int2 rowAndToken = runOrder[static_cast<uint64_t>(step) * stepEntries + within / tilesPerRow];
     if (rowAndToken.x < 0) {
         return;
     }
@@ -771,33 +781,44 @@ extern "C" int mfk_moe_dispatch(const void *x, const void *topk, uint32_t tokens
     uint32_t *blockBad = status + 64;
     uint32_t *blockHist = blockBad + histStride;
     const size_t histLds = static_cast<size_t>(kRankSlices) * experts * sizeof(uint32_t);
-    const size_t rankLds = histLds + (2 * experts + kRankThreads) * sizeof(uint32_t);
     const uint32_t upr = hidden / 8;
-    // The output-ordered tile permute needs the token rows of one block of entries (kRankBlock / topK tokens) to
-    // stay in an XCD's 4 MiB L2 while the block's rows are written, and enough blocks for the eight streams.
+    // The output-ordered tile permute needs the token rows of one step (a block of kRankBlock entries, or a half, a
+    // quarter ... down to one slice of 64 entries: stepEntries / topK tokens) to stay in an XCD's 4 MiB L2 while the
+    // step's rows are written, and enough steps for the eight streams.
     // 8192 tokens, 256 experts, top-8, rows of 4096 / 7168 / 8192 elements (1.1 / 1.8 / 2.1 MB of x per block):
-    // 102 / 174 / 187 us against 125 / 208 / 249 us with the loop kernel; 10 000 elements (2.6 MB): 356 against 337 us.
-    // 512 / 64 / 8 experts at 7168 elements: 194 / 155 / 154 us (the fewer experts, the longer the runs).
-    const uint64_t blockTokenBytes = static_cast<uint64_t>(kRankBlock / topK + 1) * hidden * 2;
+    // 102 / 174 / 187 us against 125 / 208 / 249 us with the loop kernel; 12 288 / 16 384 elements in steps of half a
+    // block: 268 / 381 against 359 / 546 us.  512 / 64 / 8 experts at 7168 elements: 194 / 155 / 154 us (the fewer
+    // experts, the longer the runs).  16 384 tokens, top-2, 8 experts, 4096 / 6144 / 8192 elements: 67 / 94 / 126 against
+    // 70 / 123 / 170 us; top-4: 94 against 117 us (7168 elements, 64 experts), 72 against 82 us (5120, 128).
+    // Rows that are not whole cache lines (10 000 elements: 20 000 bytes) lose, 362 against 337 us, whatever the step:
+    // every tile then begins and ends inside a line; they keep the loop kernel.
+    uint32_t stepSlices = kRankSlices;
+    while (stepSlices > 1 && static_cast<uint64_t>(stepSlices * 64 / topK + 1) * hidden * 2 > 2200000ull) {
+        stepSlices /= 2;
+    }
+    const uint32_t stepEntries = stepSlices * 64;
+    const uint32_t stepsPerBlock = kRankSlices / stepSlices;
+    const uint64_t steps = static_cast<uint64_t>(blocks) * stepsPerBlock;
     const uint32_t tilesPerRow = (upr + kTileUnits - 1) / kTileUnits;
-    const uint64_t tileGrid = static_cast<uint64_t>((blocks + kTileStreams - 1) / kTileStreams * kTileStreams) * kRankBlock * tilesPerRow;
+    const uint64_t tileGrid = (steps + kTileStreams - 1) / kTileStreams * kTileStreams * stepEntries * tilesPerRow;
     const bool tiles = g_xcdStreams.load(std::memory_order_relaxed) != 0 && x != nullptr && out != nullptr && upr >= 512 &&
-                       blockTokenBytes <= 2200000ull &&
-                       blocks >= 2 * kTileStreams && tileGrid <= 0x7FFFFFFFull;
+                       hidden % 64 == 0 && static_cast<uint64_t>(stepEntries / topK + 1) * hidden * 2 <= 2200000ull &&
+                       stepsPerBlock * experts <= 4096 && steps >= 2 * kTileStreams && tileGrid <= 0x7FFFFFFFull;
+    const size_t rankLds = histLds + (experts + kRankThreads + kRankSlices + (tiles ? stepsPerBlock * experts : 0)) * sizeof(uint32_t);
     const uint64_t tableBytes = 256 + histStride * sizeof(uint32_t) + static_cast<uint64_t>(histStride) * experts * sizeof(uint32_t);
     int2 *runOrder = tiles ? reinterpret_cast<int2 *>(static_cast<char *>(workspace) + (tableBytes + 15) / 16 * 16) : nullptr;
     hipLaunchKernelGGL(MoeHistKernel, dim3(blocks), dim3(kRankThreads), histLds, s, static_cast<const int32_t *>(topk),
                        total, experts, blockHist, histStride, blockBad);
     hipLaunchKernelGGL(MoeRankKernel, dim3(blocks), dim3(kRankThreads), rankLds, s, static_cast<const int32_t *>(topk),
                        total, experts, blockHist, histStride, static_cast<int32_t *>(counts), static_cast<int32_t *>(offsets),
-                       static_cast<int32_t *>(rowOf), static_cast<int32_t *>(srcOf), blockBad, status, topK, runOrder);
+                       static_cast<int32_t *>(rowOf), static_cast<int32_t *>(srcOf), blockBad, status, topK, runOrder, stepSlices);
     if (x != nullptr && out != nullptr && hidden != 0) {
         const u32x4 *xi = static_cast<const u32x4 *>(x);
         const int32_t *ro = static_cast<const int32_t *>(rowOf);
         u32x4 *oo = static_cast<u32x4 *>(out);
         if (tiles) {
             hipLaunchKernelGGL(MoePermuteTileKernel, dim3(static_cast<uint32_t>(tileGrid)), dim3(64), 0, s, xi, runOrder, upr,
-                               tilesPerRow, blocks, oo);
+                               tilesPerRow, static_cast<uint32_t>(steps), stepEntries, oo);
         } else if (upr >= 512) {
             // Wide rows: single-wave workgroups that hold up to 14 pieces per lane (a whole 7168-element
             // row) and write them with plain stores.  Storing alone takes 177 us of the 200 us such a

@@ -125,7 +125,11 @@ def test_dispatch_and_combine_match_the_specification(gpu, oracle, T, H, K, E):
     (2200, 5120, 8, 256, "bad ids"),   # some ids out of range: their slots name no row, the lists of their blocks are shorter
     (1200, 4096, 16, 128, "router"),   # sixty-four tokens per block
     (2800, 4096, 6, 64, "router"),     # blocks that begin and end inside a token
-    (3000, 8200, 8, 1, "one"),         # one expert: the output is the input, every row eight times; rows that end inside a tile
+    (3000, 8256, 8, 1, "one"),         # one expert: the output is the input, every row eight times; rows that end inside a tile
+    (2100, 16384, 8, 256, "router"),   # rows so wide that a step is half a block of entries
+    (6000, 4096, 2, 8, "router"),      # top-2: 512 tokens per block, steps of half a block
+    (2500, 12288, 8, 512, "bad ids"),  # 512 experts, half-block steps, slots without a row
+    (700, 16384, 3, 37, "router"),     # steps of two slices (128 entries) that begin and end inside tokens
 ])
 def test_output_ordered_permute(gpu, oracle, T, H, K, E, routing):
     """Rows wide enough and blocks enough for the permute that walks the output in runs of consecutive rows per
