@@ -790,6 +790,8 @@ extern "C" int mfk_moe_dispatch(const void *x, const void *topk, uint32_t tokens
     // block: 268 / 381 against 359 / 546 us.  512 / 64 / 8 experts at 7168 elements: 194 / 155 / 154 us (the fewer
     // experts, the longer the runs).  16 384 tokens, top-2, 8 experts, 4096 / 6144 / 8192 elements: 67 / 94 / 126 against
     // 70 / 123 / 170 us; top-4: 94 against 117 us (7168 elements, 64 experts), 72 against 82 us (5120, 128).
+    // Narrower rows (8192 tokens, top-8, 256 experts, 1024 / 2048 / 3072 elements): 44 / 62 / 91 against 49 / 75 / 108 us
+    // with one four-wave workgroup per token; 16 384 tokens of 2048 elements over 64 experts 102 against 136 us.
     // Rows that are not whole cache lines (10 000 elements: 20 000 bytes) lose, 362 against 337 us, whatever the step:
     // every tile then begins and ends inside a line; they keep the loop kernel.
     uint32_t stepSlices = kRankSlices;
@@ -801,7 +803,7 @@ extern "C" int mfk_moe_dispatch(const void *x, const void *topk, uint32_t tokens
     const uint64_t steps = static_cast<uint64_t>(blocks) * stepsPerBlock;
     const uint32_t tilesPerRow = (upr + kTileUnits - 1) / kTileUnits;
     const uint64_t tileGrid = (steps + kTileStreams - 1) / kTileStreams * kTileStreams * stepEntries * tilesPerRow;
-    const bool tiles = g_xcdStreams.load(std::memory_order_relaxed) != 0 && x != nullptr && out != nullptr && upr >= 512 &&
+    const bool tiles = g_xcdStreams.load(std::memory_order_relaxed) != 0 && x != nullptr && out != nullptr && upr >= kTileUnits &&
                        hidden % 64 == 0 && static_cast<uint64_t>(stepEntries / topK + 1) * hidden * 2 <= 2200000ull &&
                        stepsPerBlock * experts <= 4096 && steps >= 2 * kTileStreams && tileGrid <= 0x7FFFFFFFull;
     const size_t rankLds = histLds + (experts + kRankThreads + kRankSlices + (tiles ? stepsPerBlock * experts : 0)) * sizeof(uint32_t);

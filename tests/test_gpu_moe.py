@@ -130,6 +130,8 @@ def test_dispatch_and_combine_match_the_specification(gpu, oracle, T, H, K, E):
     (6000, 4096, 2, 8, "router"),      # top-2: 512 tokens per block, steps of half a block
     (2500, 12288, 8, 512, "bad ids"),  # 512 experts, half-block steps, slots without a row
     (700, 16384, 3, 37, "router"),     # steps of two slices (128 entries) that begin and end inside tokens
+    (2100, 1024, 8, 32, "router"),     # rows of one tile
+    (4000, 1600, 5, 100, "bad ids"),   # rows of one tile and a part of one
 ])
 def test_output_ordered_permute(gpu, oracle, T, H, K, E, routing):
     """Rows wide enough and blocks enough for the permute that walks the output in runs of consecutive rows per
