@@ -9,12 +9,15 @@
 //
 // Three launches for dispatch, one for combine:
 //   MoeHistKernel    per-block expert histograms (wave ballots + LDS)
-//   MoeRankKernel    cross-block scan, stable rank of every entry -> rowOf/srcOf, counts, offsets
-//   MoePermuteKernel one workgroup per token: the row is read once into registers and
-//                    stored to its K destination rows (HBM bound: H*2*(1+K) bytes per token)
-//   MoePermuteLoopKernel  the same for wide rows, by waves that walk the tokens
-//   MoePermuteTileKernel  wide rows whose share of x per block of entries fits an XCD's L2:
-//                    the output walked in runs of consecutive rows, in 2 KiB tiles
+//   MoeRankKernel    cross-block scan, stable rank of every entry -> rowOf/srcOf, counts, offsets,
+//                    and for the tile permute the rows of every step of entries in ascending order
+//   the permute, one of
+//   MoePermuteTileKernel  rows of whole cache lines, enough work: the output walked in runs of
+//                    consecutive rows, in 2 KiB tiles, one stream of steps per XCD, token rows
+//                    re-read from that XCD's L2 (HBM bound: H*2*(1+K) bytes per token)
+//   MoePermuteLoopKernel  other wide rows: waves that walk the tokens, a row read once into
+//                    registers and stored to its K destination rows
+//   MoePermuteKernel other narrow rows: one workgroup per token
 //   MoeCombineKernel one workgroup per token: K rows gathered, fp32 FMA chain in slot
 //                    order, one rounding to bf16 (HBM bound: H*2*(K+1) bytes per token)
 //   MoeCombineWindowKernel  the same arithmetic for wide rows and many tokens, by waves that
