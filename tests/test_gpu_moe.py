@@ -237,6 +237,9 @@ def test_out_of_range_expert_ids_are_flagged_not_followed(gpu, oracle):
     (700, 1024, 8),    # narrow rows: one four-wave workgroup per token
     (60, 7168, 8),     # wide rows, few tokens: one workgroup per slice
     (300, 16384, 3),   # any other topK
+    (500, 4096, 2),    # the slice kernel compiled for top-2
+    (400, 7168, 4),    # ... top-4
+    (300, 5120, 6),    # ... top-6
 ])
 def test_combine_of_rows_that_differ_within_a_token(gpu, oracle, T, H, K):
     """After a dispatch the rows of a token are copies of one another, so a combine that mixed them up would still pass
