@@ -686,6 +686,16 @@ def main():
     payload = batches[0].payload
     g2g = int(bm.BmCopyType.G2G)
 
+    # The submitting thread runs where a launch costs it least (mf_pin_thread_near_gpu: 3.1 against 4.3 us per call
+    # between the two halves of the CPUs on the hosts of this pool, which decides whether the host or the GPU sets
+    # the pace of this loop); extras.kv122_any_cpu has the same loop with the scheduler free to put it anywhere.
+    all_cpus = sorted(os.sched_getaffinity(0))
+    cpu_ids, cpu_us = (ctypes.c_uint32 * 1024)(), (ctypes.c_float * 1024)()
+    measured = lib.mf_host_launch_costs(cpu_ids, cpu_us, 1024)
+    launch_us_by_cpu = {int(cpu_ids[i]): round(float(cpu_us[i]), 2) for i in range(max(measured, 0))}
+    kept = lib.mf_pin_thread_near_gpu()
+    near_cpus = sorted(os.sched_getaffinity(0))
+
     wall, ms, rep_us = steady_state_headline(lib, pool.handle, batches, g2g, args.steps, args.warmup)
     per_launch_us = ms * 1e3 / args.steps
     value = payload * args.steps / wall / GB
@@ -710,11 +720,14 @@ def main():
                         "4 KiB-aligned random offsets in a 4 GiB HBM pool, D2D, 64 rotating tables",
             "api": "smem_bm_copy_batch(SMEMB_COPY_G2G, ASYNC_COPY_FLAG) on one stream + one wait; the K calls are "
                    "issued by a C loop (mf_bm_copy_batch_replay), extras.kv122_python_caller has one ctypes call per batch",
-            "timing": f"untimed ramp of {RAMP_BATCHES} batches + --warmup, then {REPETITIONS} repetitions of --steps batches, "
+            "timing": f"submitting thread pinned near the GPU; untimed ramp of {RAMP_BATCHES} batches + --warmup, then {REPETITIONS} repetitions of --steps batches, "
                       "each between two synchronisations; ms_per_step / value: median repetition by the host clock "
                       "(includes one stream wait per repetition), roofline: median repetition by HIP events",
             "payload_bytes": payload,
             "cu_count": lib.mfrt_cu_count(),
+            "submitting_thread": {"empty_launch_us_by_cpu": launch_us_by_cpu, "runs_on_cpus": near_cpus if kept > 0 else all_cpus,
+                                  "note": "mf_pin_thread_near_gpu: the CPUs from which a launch with a full argument block is "
+                                          "cheapest, measured at start; the threads of the concurrency extras inherit the set"},
         },
         "roofline": {
             "bound": "hbm",
@@ -741,12 +754,24 @@ def main():
 
     extras = {}
     if not args.no_extras:
+        def any_cpu():
+            os.sched_setaffinity(0, all_cpus)
+            try:
+                w, m, _ = steady_state_headline(lib, pool.handle, batches, g2g, max(args.steps, 2000), 0)
+                n = max(args.steps, 2000)
+                return {"us_per_batch_wall": round(w * 1e6 / n, 2), "us_per_batch_events": round(m * 1e3 / n, 2),
+                        "note": "the headline loop without the pinning: the scheduler may run the submitting thread on any of "
+                                "the process's CPUs"}
+            finally:
+                os.sched_setaffinity(0, near_cpus)
+        any_cpu_result = guarded(any_cpu)
         block = guarded(extras_block, lib, pool, dev, batches, tables, args.steps)
         if isinstance(block, tuple):
             extras, copy_ceiling = block
             result["roofline"]["frac_of_measured_copy_ceiling"] = frac(achieved, copy_ceiling)
         else:
             extras = {"kv122_and_link": block}
+        extras["kv122_any_cpu"] = any_cpu_result
         extras["kv122_transfer_write"] = guarded(extras_transfer, lib, dev, batches, args.steps)
         extras["kv122_plugin"] = guarded(extras_plugin, lib, dev, tables, args.steps)
     pool.destroy()  # give the pools back before the larger workloads allocate
@@ -758,6 +783,7 @@ def main():
         extras["paged_kv_40GiB"] = guarded(extras_paged, lib)
         result["extras"] = extras
 
+    os.sched_setaffinity(0, all_cpus)   # the CPU baselines use every core
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(tables)
         if not args.no_extras:

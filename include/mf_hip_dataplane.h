@@ -181,6 +181,19 @@ int32_t mf_moe_combine_windows(uint32_t readMBps, uint32_t writeMBps);
  * per XCD; 0: it keeps to the token-ordered permute.  No counterpart in the reference. */
 int32_t mf_moe_xcd_streams(void);
 
+/* Host side of a launch.  What one launch costs the submitting thread depends on the CPU it runs on (3.1 against
+ * 4.3 us per smem_bm_copy_batch call on the hosts this was built on, half of the CPUs each, with nothing in the
+ * operating system's topology to tell them apart), and a thread the scheduler moves between the two kinds changes
+ * pace mid-run.  mf_host_launch_costs measures it: it pins the calling thread to each CPU of its affinity set in
+ * turn, times 256 launches of an empty kernel with a full argument block from there, restores the set, and
+ * returns how many (cpu, microseconds per launch) pairs it wrote (at most `capacity`).  mf_pin_thread_near_gpu
+ * leaves the set alone where the dearest CPU is within 25 % of the cheapest (hosts with one kind of CPU measure
+ * 2.5 to 3.0 us) and otherwise narrows the calling thread's affinity set to the CPUs within 15 % of the cheapest;
+ * it returns the size of the resulting set, and threads created afterwards inherit it.  Both take some 20 ms and wait for the thread's stream.  No
+ * counterpart in the reference (a deployment would use numactl where the topology is visible). */
+int32_t mf_host_launch_costs(uint32_t *cpus, float *micros, uint32_t capacity);
+int32_t mf_pin_thread_near_gpu(void);
+
 /* ---- runtime services (thin layer over HIP) ------------------------------ */
 int mfrt_init(int device);
 void mfrt_shutdown(void);

@@ -197,6 +197,8 @@ _SIGNATURES = {
     "mf_xcopy_choose_units": (u32, [u64, u32, i32]),
     "mf_xcopy_launch_count": (u64, []),
     "mf_xcopy_describe_plan": (i64, [u64p, u64p, u64p, u32, u32, u64p, u64, ctypes.POINTER(i32)]),
+    "mf_host_launch_costs": (i32, [vp, vp, u32]),
+    "mf_pin_thread_near_gpu": (i32, []),
     "mf_moe_workspace_bytes": (u64, [u32, u32, u32]),
     "mf_moe_dispatch": (i32, [vp, vp, u32, u32, u32, u32, vp, vp, vp, vp, vp, vp, u64, vp]),
     "mf_moe_combine": (i32, [vp, vp, vp, u32, u32, u32, vp, vp]),

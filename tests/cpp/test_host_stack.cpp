@@ -12,6 +12,8 @@
 #include <thread>
 #include <vector>
 
+#include <sched.h>
+
 #include "../../include/mf_hip_dataplane.h"
 #include "../../include/mf_xcopy_api.h"
 #include "../../memfabric_hybrid_amd/csrc/host/compose_data_op.h"
@@ -323,6 +325,36 @@ static void TestCApi()
 // (test/ut/testcase/smem/smem_trans_test.cpp:145-168 create, :170-219 register, :1016-1098 batch
 // write); the data cases follow its two-object write / read tests (:272-373, :655-779) with both
 // objects in this process.
+// Launch cost per CPU and the pinning built on it: every CPU of the thread's set is measured, the set is put back,
+// and the pinned set is a part of it.
+static void TestHostLaunchCosts()
+{
+    CHECK(hybm_init(0, 0) == BM_OK);
+    cpu_set_t before;
+    CHECK(sched_getaffinity(0, sizeof(before), &before) == 0);
+    uint32_t cpus[1024];
+    float micros[1024];
+    const int32_t n = mf_host_launch_costs(cpus, micros, 1024);
+    CHECK(n == CPU_COUNT(&before));
+    cpu_set_t after;
+    CHECK(sched_getaffinity(0, sizeof(after), &after) == 0);
+    CHECK(CPU_EQUAL(&before, &after));
+    for (int32_t i = 0; i < n; ++i) {
+        CHECK(CPU_ISSET(static_cast<int>(cpus[i]), &before) && micros[i] >= 0.0f);
+    }
+    CHECK(mf_host_launch_costs(cpus, micros, 1) == 1);          // no more than there is room for
+    CHECK(mf_host_launch_costs(nullptr, micros, 4) == BM_INVALID_PARAM);
+    const int32_t kept = mf_pin_thread_near_gpu();
+    CHECK(kept >= 1 && kept <= n);
+    CHECK(sched_getaffinity(0, sizeof(after), &after) == 0);
+    CHECK(CPU_COUNT(&after) == kept);
+    for (int cpu = 0; cpu < CPU_SETSIZE; ++cpu) {
+        CHECK(!CPU_ISSET(cpu, &after) || CPU_ISSET(cpu, &before));
+    }
+    CHECK(sched_setaffinity(0, sizeof(before), &before) == 0);
+    hybm_uninit();
+}
+
 static void TestTrans()
 {
     const char *store = "tcp://127.0.0.1:5432";
@@ -1033,6 +1065,7 @@ int main()
     TestPlugin();
     TestHeldStores();
     TestWindows();
+    TestHostLaunchCosts();
     if (g_failed != 0) {
         std::printf("%d check(s) failed\n", g_failed);
         return 1;

@@ -377,3 +377,33 @@ def test_plugin_abi(pool, lib, oracle):
         params.free()
         table_dev.free()
         lib.mfrt_stream_destroy(stream)
+
+
+def test_launch_cost_per_cpu_and_pinning_near_the_gpu(lib, pool):
+    """Every CPU of the thread's set is measured and the set is put back; the pinned set is a part of it and copies
+    still work from there."""
+    import os
+    before = os.sched_getaffinity(0)
+    cpus, micros = (ctypes.c_uint32 * 1024)(), (ctypes.c_float * 1024)()
+    n = lib.mf_host_launch_costs(cpus, micros, 1024)
+    assert n == len(before), native.last_error()
+    assert os.sched_getaffinity(0) == before
+    assert {int(cpus[i]) for i in range(n)} == set(before)
+    assert all(0.5 < float(micros[i]) < 100.0 for i in range(n)), [float(micros[i]) for i in range(n)]
+    try:
+        kept = lib.mf_pin_thread_near_gpu()
+        assert 1 <= kept <= n
+        near = os.sched_getaffinity(0)
+        assert len(near) == kept and near <= before
+        src = gpu_util.DeviceBuffer(lib, 1 << 20)
+        dst = gpu_util.DeviceBuffer(lib, 1 << 20)
+        data = np.random.default_rng(5).integers(0, 256, 1 << 20, dtype=np.uint8)
+        src.upload(data)
+        s, d, l = native.u64_array([src.ptr]), native.u64_array([dst.ptr]), native.u64_array([1 << 20])
+        assert lib.mf_xcopy_batch(s, d, l, 1, native.ROUTE_HBM, None) == 0
+        assert lib.mfrt_device_sync() == 0
+        assert np.array_equal(dst.download(0, 1 << 20), data)
+        src.free()
+        dst.free()
+    finally:
+        os.sched_setaffinity(0, before)
