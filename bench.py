@@ -105,8 +105,8 @@ def timed_steps(lib, handle, batches, copy_type, steps, warmup, flags, caller="c
         assert ret == 0, native.last_error()
     assert lib.mfrt_stream_sync(stream) == 0
     assert lib.mfrt_device_sync() == 0
-    t0 = time.perf_counter()
     lib.mfrt_event_record(start, stream)
+    t0 = time.perf_counter()
     if caller == "c":
         if lib.mf_bm_copy_batch_replay(handle, table, nb, steps, copy_type, flags) != 0:
             raise RuntimeError(native.last_error())
