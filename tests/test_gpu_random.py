@@ -143,3 +143,57 @@ def test_random_moe_shapes_against_the_oracle(gpu, oracle, seed):
         finally:
             for b in bufs:
                 b.free()
+
+
+@pytest.mark.parametrize("seed", [31, 32])
+def test_random_rectangles_side_by_side_and_alone(gpu, seed):
+    """Twenty batches per seed of 1 to 200 rectangles: groups of two or three column blocks laid side by side in the
+    destination (the first two of a group of one shape share their chunks in turn inside the kernel; a third, or one
+    of another height, does not), blocks alone, widths from one unit to rows wider than a chunk, some unaligned
+    (those go row by row).  Every destination byte is compared, the space between rectangles included."""
+    rng = np.random.default_rng(seed)
+    src_bytes, dst_bytes = 32 << 20, 96 << 20
+    data = rng.integers(0, 256, src_bytes, dtype=np.uint8)
+    sbuf = gpu_util.DeviceBuffer(gpu, src_bytes)
+    dbuf = gpu_util.DeviceBuffer(gpu, dst_bytes)
+    sbuf.upload(data)
+    try:
+        for it in range(20):
+            rects, model = [], []
+            cursor = int(rng.integers(0, 64)) * 16
+            groups = int(rng.integers(1, 80))
+            for _ in range(groups):
+                blocks = int(rng.choice([1, 1, 2, 2, 2, 3]))
+                width = int(rng.choice([16, 48, 896, 1000, 2368, 4736, 20000, 40000]))
+                if rng.integers(0, 8) == 0:
+                    width += int(rng.integers(1, 16))           # unaligned: row by row
+                height = int(rng.integers(1, 120))
+                dpitch = blocks * width + int(rng.integers(0, 3)) * 16
+                used = 0
+                for b in range(blocks):
+                    h = height if b < 2 or rng.integers(0, 2) == 0 else max(1, height - int(rng.integers(1, 5)))
+                    spitch = width + int(rng.integers(0, 4)) * 16
+                    soff = int(rng.integers(0, src_bytes - spitch * h - 64)) // 16 * 16
+                    if width % 16 != 0:
+                        soff += int(rng.integers(0, 16))
+                    rects.append((sbuf.ptr + soff, dbuf.ptr + cursor + b * width, width, h, spitch, dpitch))
+                    model.append((soff, cursor + b * width, width, h, spitch, dpitch))
+                    used = max(used, dpitch * h)
+                cursor += (used + 255) // 256 * 256
+                if cursor > dst_bytes - (8 << 20):
+                    break
+            descs = (native.Copy2dDesc * len(rects))()
+            for i, r in enumerate(rects):
+                descs[i] = native.Copy2dDesc(*[int(v) for v in r])
+            dbuf.fill(0x3D)
+            assert gpu.mf_xcopy_2d_batch(descs, len(rects), native.ROUTE_HBM, None) == 0, native.last_error()
+            assert gpu.mfrt_device_sync() == 0
+            expect = np.full(cursor, 0x3D, dtype=np.uint8)
+            for soff, doff, width, h, spitch, dpitch in model:
+                rows_src = np.lib.stride_tricks.as_strided(data[soff:], shape=(h, width), strides=(spitch, 1))
+                rows_dst = np.lib.stride_tricks.as_strided(expect[doff:], shape=(h, width), strides=(dpitch, 1))
+                rows_dst[:] = rows_src
+            assert np.array_equal(dbuf.download(0, cursor), expect), (seed, it, len(rects))
+    finally:
+        sbuf.free()
+        dbuf.free()
