@@ -153,9 +153,12 @@ __global__ __launch_bounds__(kRankThreads) void MoeRankKernel(const int32_t *__r
     uint32_t bad = 0;
     SliceHistograms(topk, total, experts, blockIdx.x * kRankBlock, hist, myExpert, myRank, &bad);
 
+    // blockHist == nullptr: the launch is a single block and no histogram kernel ran before it; the block's own slice
+    // histograms and its own flag are all there is (a dispatch of up to 1024 entries: 128 tokens at top-8).
+    const bool alone = blockHist == nullptr;
     if (blockIdx.x == 0) {
-        uint32_t any = 0;
-        for (uint32_t blk = threadIdx.x; blk < gridDim.x; blk += kRankThreads) {
+        uint32_t any = alone ? bad : 0;
+        for (uint32_t blk = threadIdx.x; !alone && blk < gridDim.x; blk += kRankThreads) {
             any |= blockBad[blk];
         }
         any = __syncthreads_or(static_cast<int>(any)) != 0 ? 1u : 0u;
@@ -181,9 +184,12 @@ __global__ __launch_bounds__(kRankThreads) void MoeRankKernel(const int32_t *__r
             const uint32_t *rowHist = blockHist + static_cast<uint64_t>(x) * histStride;
             uint32_t t = 0;
             uint32_t b = 0;
-            // kHistPad blocks per step, all their loads requested before the first is used: with one load per step the
-            // loop waited a full round trip per four blocks (8 of the kernel's 10 us at 64 blocks)
-            for (uint32_t blk = 0; blk < gridDim.x; blk += kHistPad) {
+            for (uint32_t sl = 0; alone && sl < kRankSlices; ++sl) {
+                t += hist[sl * experts + x];
+            }
+            // kHistPad blocks per step, all their loads requested before the first is used (with one load per step the
+            // loop waited a round trip per four blocks)
+            for (uint32_t blk = 0; !alone && blk < gridDim.x; blk += kHistPad) {
                 u32x4 v[kHistPad / 4];
 #pragma unroll
                 for (uint32_t q = 0; q < kHistPad / 4; ++q) {
@@ -801,6 +807,11 @@ extern "C" int mfk_moe_dispatch(const void *x, const void *topk, uint32_t tokens
     while (stepSlices > 1 && static_cast<uint64_t>(stepSlices * 64 / topK + 1) * hidden * 2 > 2200000ull) {
         stepSlices /= 2;
     }
+    // a small call is cut finer, so that every XCD gets steps to work on (256 / 512 tokens of 7168 elements at top-8:
+    // 24 / 28 us per dispatch, 34 / 35 us with the loop kernel, whose single wave per token writes its 112 KiB alone)
+    while (stepSlices > 1 && static_cast<uint64_t>(blocks) * (kRankSlices / stepSlices) < 2 * kTileStreams) {
+        stepSlices /= 2;
+    }
     const uint32_t stepEntries = stepSlices * 64;
     const uint32_t stepsPerBlock = kRankSlices / stepSlices;
     const uint64_t steps = static_cast<uint64_t>(blocks) * stepsPerBlock;
@@ -808,12 +819,18 @@ extern "C" int mfk_moe_dispatch(const void *x, const void *topk, uint32_t tokens
     const uint64_t tileGrid = (steps + kTileStreams - 1) / kTileStreams * kTileStreams * stepEntries * tilesPerRow;
     const bool tiles = g_xcdStreams.load(std::memory_order_relaxed) != 0 && x != nullptr && out != nullptr && upr >= kTileUnits &&
                        hidden % 64 == 0 && static_cast<uint64_t>(stepEntries / topK + 1) * hidden * 2 <= 2200000ull &&
-                       stepsPerBlock * experts <= 4096 && steps >= 2 * kTileStreams && tileGrid <= 0x7FFFFFFFull;
+                       stepsPerBlock * experts <= 4096 && tileGrid <= 0x7FFFFFFFull;
     const size_t rankLds = histLds + (experts + kRankThreads + kRankSlices + (tiles ? stepsPerBlock * experts : 0)) * sizeof(uint32_t);
     const uint64_t tableBytes = 256 + histStride * sizeof(uint32_t) + static_cast<uint64_t>(histStride) * experts * sizeof(uint32_t);
     int2 *runOrder = tiles ? reinterpret_cast<int2 *>(static_cast<char *>(workspace) + (tableBytes + 15) / 16 * 16) : nullptr;
-    hipLaunchKernelGGL(MoeHistKernel, dim3(blocks), dim3(kRankThreads), histLds, s, static_cast<const int32_t *>(topk),
-                       total, experts, blockHist, histStride, blockBad);
+    if (blocks == 1) {
+        blockHist = nullptr;   // one block ranks from its own histograms: no launch in front of it (16 / 64 / 128 tokens of
+                               // 7168 elements at top-8: 12 / 12.5 / 14 us per dispatch; 22 / 23 / 24 us before, with the
+                               // histogram launch and the token-ordered permute)
+    } else {
+        hipLaunchKernelGGL(MoeHistKernel, dim3(blocks), dim3(kRankThreads), histLds, s, static_cast<const int32_t *>(topk),
+                           total, experts, blockHist, histStride, blockBad);
+    }
     hipLaunchKernelGGL(MoeRankKernel, dim3(blocks), dim3(kRankThreads), rankLds, s, static_cast<const int32_t *>(topk),
                        total, experts, blockHist, histStride, static_cast<int32_t *>(counts), static_cast<int32_t *>(offsets),
                        static_cast<int32_t *>(rowOf), static_cast<int32_t *>(srcOf), blockBad, status, topK, runOrder, stepSlices);

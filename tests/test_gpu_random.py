@@ -127,6 +127,7 @@ def test_random_moe_shapes_against_the_oracle(gpu, oracle, seed):
             assert gpu.mfrt_device_sync() == 0
             assert np.array_equal(drow.download(0, T * K * 4).view(np.int32), exp_row), case
             assert np.array_equal(dcounts.download(0, E * 4).view(np.int32), counts[:E]), case
+            assert dws.download(0, 4).view(np.uint32)[0] == (1 if invalid.any() else 0), case
             got = dout.download(0, T * K * H * 2).view(np.uint16).reshape(T * K, H)
             assert np.array_equal(got[:valid], out[:valid]), case
             assert np.all(got[valid:] == 0x7777), case
