@@ -177,7 +177,7 @@ int32_t mf_moe_combine(const void *rows, const int32_t *rowOf, const float *weig
  * thread holds a stream of the library).  Results do not depend on it.  No counterpart in the reference.  Returns BM_INVALID_PARAM for other values. */
 int32_t mf_moe_combine_windows(uint32_t readMBps, uint32_t writeMBps);
 /* 1 if hybm_init found that the GPU deals consecutive workgroups to its eight XCDs in turn (an MI355X in its default
- * partition does): the dispatch of wide rows then writes its output in runs of consecutive rows, one stream of runs
+ * partition does): the dispatch of rows of whole cache lines then writes its output in runs of consecutive rows, one stream of runs
  * per XCD; 0: it keeps to the token-ordered permute.  No counterpart in the reference. */
 int32_t mf_moe_xcd_streams(void);
 
