@@ -96,7 +96,9 @@ struct InlinePlan {
 // wait gains nothing), and it is the same for every wave: shortening it for waves that start later did
 // not help.  The best wait grows with the number of waves the dispatcher has to start.  100 to 200 ns
 // short of it the gain is lost (2196 chunks: 1700 ns 4.87 us, 1600 ns 5.09 us), each 100 ns beyond it
-// costs 0.1 us, so the rule aims a little long.  From about 7000 chunks on the gain is below 5 % and the
+// costs 0.1 us, so the rule aims a little long: in steps of 50 ns, on four machines, 2196 chunks took 4.57 us at
+// 1750 ns, 4.44 at 1800, 4.30 at 1850 to 1950, 4.35 at 2000 and 4.42 at 2050, and the rule gives 1957 ns; from 1220
+// to 5124 chunks the rule is within 50 ns of the best step or level with it.  From about 7000 chunks on the gain is below 5 % and the
 // best wait no longer follows the line: not every wave of such a launch is resident at once, and a wait
 // only delays the ones behind (11956 chunks: 19.3 us without, 20.2 us with).  Below about
 // 1000 chunks the period is the cost of a dependent launch and no wait changes it.
@@ -127,9 +129,9 @@ inline uint32_t HoldNanosFor(uint32_t nchunk, uint32_t grid, uint32_t units, boo
         return 0;
     }
     if (nchunk <= kHoldKneeChunks) {
-        return 700 + nchunk * 6 / 10;
+        return 640 + nchunk * 6 / 10;
     }
-    return 700 + kHoldKneeChunks * 6 / 10 + (nchunk - kHoldKneeChunks) * 33 / 100;
+    return 640 + kHoldKneeChunks * 6 / 10 + (nchunk - kHoldKneeChunks) * 33 / 100;
 }
 
 // The start of a windowed launch's first period travels between its waves as the low kEpochClockBits bits of a

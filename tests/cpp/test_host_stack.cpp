@@ -847,10 +847,10 @@ static void TestPlugin()
 // Which launches are told to hold their stores back, and for how long.
 static void TestHeldStores()
 {
-    CHECK(HoldNanosFor(959, 959, 256, false) == 0 && HoldNanosFor(960, 960, 256, false) == 700 + 576);
-    CHECK(HoldNanosFor(2196, 2196, 256, false) == 700 + 1317);
-    CHECK(HoldNanosFor(3904, 3904, 256, false) == 3042 && HoldNanosFor(3905, 3905, 256, false) == 3042);
-    CHECK(HoldNanosFor(6144, 6144, 256, false) == 3042 + 739 && HoldNanosFor(6145, 6145, 256, false) == 0);
+    CHECK(HoldNanosFor(959, 959, 256, false) == 0 && HoldNanosFor(960, 960, 256, false) == 640 + 576);
+    CHECK(HoldNanosFor(2196, 2196, 256, false) == 640 + 1317);
+    CHECK(HoldNanosFor(3904, 3904, 256, false) == 2982 && HoldNanosFor(3905, 3905, 256, false) == 2982);
+    CHECK(HoldNanosFor(6144, 6144, 256, false) == 2982 + 739 && HoldNanosFor(6145, 6145, 256, false) == 0);
     CHECK(HoldNanosFor(2196, 2195, 256, false) == 0);    // a workgroup with two chunks
     CHECK(HoldNanosFor(2196, 2196, 512, false) == 0);    // chunks of 8 KiB
     CHECK(HoldNanosFor(1399, 1399, 256, true) == 0 && HoldNanosFor(1400, 1400, 256, true) == 100 + 798);
