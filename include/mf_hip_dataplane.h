@@ -169,7 +169,7 @@ int32_t mf_moe_dispatch(const void *x, const int32_t *topk, uint32_t tokens, uin
  * round-to-nearest-even; entries with rowOf < 0 contribute nothing. */
 int32_t mf_moe_combine(const void *rows, const int32_t *rowOf, const float *weights, uint32_t tokens, uint32_t hidden,
                        uint32_t topK, void *y, void *stream);
-/* A combine of topK == 8 with rows of 2048 elements and more, on enough tokens to give every wave of the chip six
+/* A combine of topK == 8 or 6 with rows of 2048 elements and more, on enough tokens to give every wave of the chip six
  * slices of 128 x 8 elements (about 3500 tokens of 7168 elements on 256 CUs), runs as waves that stay for the whole
  * launch and alternate, chip-wide and by the clock, between reading rows and writing results.  readMBps / writeMBps
  * (MB/s of HBM traffic, 1 000 000 ... 16 000 000) set the pace of the two parts; the defaults are 6 800 000 and

@@ -621,8 +621,8 @@ __global__ __launch_bounds__(kThreads) void MoeCombineKernel(const u32x4 *__rest
 // part j a wave requests the 16 pieces of its j-th item of the period (eight rows, two column
 // positions per lane) at its own offset of the part, reduces them when they have arrived and
 // keeps the result, 8 registers per item; in the write part it stores the kItems results at
-// its own offset of that part.  The start of the first period is agreed through
-// AgreedStart(); after that every wave goes by the constant-rate clock alone.  Measured on
+// its own offset of that part (top-6: six rows, twelve pieces).  The start of the first period is agreed through
+// AgreedStart(); after that every wave goes by the constant-rate clock alone.  Measured at top-8 on
 // 8192 tokens of 7168 elements: 164-168 us against 177-181 us for one workgroup per item, on
 // 16 384 tokens 323-330 against 359-365 us (read parts paced at 6.6-6.8 TB/s, write parts at
 // 6.0-6.5; reads at 7.0 make the waves fall behind now and then, and so did 6.8 with writes at
@@ -634,14 +634,13 @@ constexpr uint32_t kCombineWavesPerCu = 16;
 constexpr uint32_t kCombineSliceUnits = 128;           // two column positions per lane
 constexpr uint32_t kCombineMinItemsPerWave = 6;
 
-template <uint32_t kItems>
+template <uint32_t kItems, uint32_t kSlots>
 __global__ __launch_bounds__(64) void MoeCombineWindowKernel(const u32x4 *__restrict__ rowsIn,
                                                              const int32_t *__restrict__ rowOf,
                                                              const float *__restrict__ weights, uint32_t unitsPerRow,
                                                              uint32_t parts, uint32_t items, u32x4 *__restrict__ y,
                                                              uint32_t readTicks, uint32_t writeTicks, uint32_t seq)
 {
-    constexpr uint32_t kSlots = 8;
     constexpr uint32_t kBatch = kCombineSliceUnits / 64;
     const uint64_t start = AgreedStart(seq);
     const uint32_t period = kItems * readTicks + writeTicks;
@@ -879,47 +878,54 @@ extern "C" int mfk_moe_combine(const void *rows, const void *rowOf, const void *
     const float *w = static_cast<const float *>(weights);
     u32x4 *o = static_cast<u32x4 *>(y);
     const uint32_t upr = hidden / 8;
-    if (topK == 8) {
-        // Wide rows: single-wave workgroups, each on a 128-unit slice of the row with two column
-        // positions per lane in flight (16 loads), the fastest shape measured on 7168-element rows
-        // (178 us; one four-wave workgroup per token 188 us; plain instead of nontemporal loads 194 us).
-        if (upr >= 256) {
-            const uint32_t parts = (upr + kCombineSliceUnits - 1) / kCombineSliceUnits;
-            const uint32_t perPart = (upr + parts - 1) / parts;
-            const uint64_t items = static_cast<uint64_t>(tokens) * parts;
-            const uint32_t waves = static_cast<uint32_t>(mfrt_cu_count() > 0 ? mfrt_cu_count() : 256) * kCombineWavesPerCu;
-            // From six items per wave on, waves that stay and keep reads and writes apart in time; below that the
-            // first read part and the last write part, in which the chip only reads or only writes for want of
-            // work, cost what the separation gains (16 800 items on 4096 waves: 51.4 against 50.5 us; 19 200: the
-            // same; 25 200: 74.4 against 76.7 us).
-            const uint32_t readTicks = WindowPeriodTicks(static_cast<uint64_t>(waves) * 8 * perPart * 16,
-                                                         g_combineReadMBps.load(std::memory_order_relaxed));
-            const uint32_t writeTicks = WindowPeriodTicks(static_cast<uint64_t>(waves) * kCombineItems * perPart * 16,
-                                                          g_combineWriteMBps.load(std::memory_order_relaxed));
-            if (paced != 0 && items >= static_cast<uint64_t>(waves) * kCombineMinItemsPerWave && items < 0x40000000ull &&
-                readTicks != 0 && writeTicks != 0) {
-                hipLaunchKernelGGL((MoeCombineWindowKernel<kCombineItems>), dim3(waves), dim3(64), 0, s, in, ro, w, upr, parts,
-                                   static_cast<uint32_t>(items), o, readTicks, writeTicks, NextWindowSeq());
-            } else {
-                hipLaunchKernelGGL((MoeCombineKernel<8, 64, true, 2>), dim3(tokens * parts), dim3(64), 0, s, in, ro, w, topK,
-                                   upr, parts, o);
-            }
-        } else {
-            hipLaunchKernelGGL((MoeCombineKernel<8, 256, true>), dim3(tokens), dim3(256), 0, s, in, ro, w, topK, upr, 1u, o);
-        }
-    } else if (upr >= 256 && (topK == 2 || topK == 4 || topK == 6)) {
-        // The slice kernel compiled for the common smaller fan-ins, so that all of a lane's loads are in flight
-        // together: top-2 16 384 x 4096 65 against 74 us, top-4 8192 x 7168 96 against 106 us, top-6 139 against 152 us
-        // (against the kernel below, which walks a run-time number of slots).
+    if (upr >= 256 && (topK == 2 || topK == 4 || topK == 6 || topK == 8)) {
+        // Wide rows: single-wave workgroups, each on a 128-unit slice of the row with two column positions per
+        // lane in flight (2 x topK loads), the fastest shape measured on 7168-element rows at top-8 (178 us; one
+        // four-wave workgroup per token 188 us; plain instead of nontemporal loads 194 us).  Compiled for the common
+        // fan-ins, so that all of a lane's loads are in flight together: top-2 16 384 x 4096 65 against 74 us,
+        // top-4 8192 x 7168 96 against 106 us, top-6 139 against 152 us (against the kernel that walks a run-time
+        // number of slots).
         const uint32_t parts = (upr + kCombineSliceUnits - 1) / kCombineSliceUnits;
-        const dim3 grid(tokens * parts);
+        const uint32_t perPart = (upr + parts - 1) / parts;
+        const uint64_t items = static_cast<uint64_t>(tokens) * parts;
+        const uint32_t waves = static_cast<uint32_t>(mfrt_cu_count() > 0 ? mfrt_cu_count() : 256) * kCombineWavesPerCu;
+        // From six items per wave on, waves that stay and keep reads and writes apart in time; below that the
+        // first read part and the last write part, in which the chip only reads or only writes for want of
+        // work, cost what the separation gains (top-8, 16 800 items on 4096 waves: 51.4 against 50.5 us; 19 200: the
+        // same; 25 200: 74.4 against 76.7 us).
+        const uint32_t readTicks = WindowPeriodTicks(static_cast<uint64_t>(waves) * topK * perPart * 16,
+                                                     g_combineReadMBps.load(std::memory_order_relaxed));
+        const uint32_t writeTicks = WindowPeriodTicks(static_cast<uint64_t>(waves) * kCombineItems * perPart * 16,
+                                                      g_combineWriteMBps.load(std::memory_order_relaxed));
+        // Top-6 gains as top-8 does (8192 x 7168: 131-133 against 138-140 us); top-4 gains nothing (98 against 97 us)
+        // and top-2 loses (16 384 x 4096: 79 against 66 us): their read parts are too short for the switch to pay.
+        const bool windows = paced != 0 && topK >= 6 && items >= static_cast<uint64_t>(waves) * kCombineMinItemsPerWave &&
+                             items < 0x40000000ull && readTicks != 0 && writeTicks != 0;
+        const dim3 grid(windows ? waves : tokens * parts);
+#define MF_COMBINE_SLICES(K)                                                                                           \
+    hipLaunchKernelGGL((MoeCombineKernel<K, 64, true, 2>), grid, dim3(64), 0, s, in, ro, w, topK, upr, parts, o)
+#define MF_COMBINE_WINDOWS(K)                                                                                          \
+    hipLaunchKernelGGL((MoeCombineWindowKernel<kCombineItems, K>), grid, dim3(64), 0, s, in, ro, w, upr, parts,        \
+                       static_cast<uint32_t>(items), o, readTicks, writeTicks, NextWindowSeq())
         if (topK == 2) {
-            hipLaunchKernelGGL((MoeCombineKernel<2, 64, true, 2>), grid, dim3(64), 0, s, in, ro, w, topK, upr, parts, o);
+            MF_COMBINE_SLICES(2);
         } else if (topK == 4) {
-            hipLaunchKernelGGL((MoeCombineKernel<4, 64, true, 2>), grid, dim3(64), 0, s, in, ro, w, topK, upr, parts, o);
+            MF_COMBINE_SLICES(4);
+        } else if (topK == 6) {
+            if (windows) {
+                MF_COMBINE_WINDOWS(6);
+            } else {
+                MF_COMBINE_SLICES(6);
+            }
+        } else if (windows) {
+            MF_COMBINE_WINDOWS(8);
         } else {
-            hipLaunchKernelGGL((MoeCombineKernel<6, 64, true, 2>), grid, dim3(64), 0, s, in, ro, w, topK, upr, parts, o);
+            MF_COMBINE_SLICES(8);
         }
+#undef MF_COMBINE_SLICES
+#undef MF_COMBINE_WINDOWS
+    } else if (topK == 8) {
+        hipLaunchKernelGGL((MoeCombineKernel<8, 256, true>), dim3(tokens), dim3(256), 0, s, in, ro, w, topK, upr, 1u, o);
     } else {
         hipLaunchKernelGGL((MoeCombineKernel<0, 256, true>), dim3(tokens), dim3(256), 0, s, in, ro, w, topK, upr, 1u, o);
     }

@@ -240,10 +240,12 @@ def test_out_of_range_expert_ids_are_flagged_not_followed(gpu, oracle):
     (500, 4096, 2),    # the slice kernel compiled for top-2
     (400, 7168, 4),    # ... top-4
     (300, 5120, 6),    # ... top-6
+    (5100, 5120, 6),   # top-6, 25 500 slices: waves that stay, as in the first shape
+    (3600, 7168, 4),   # top-4 with as many slices: still one workgroup per slice
 ])
 def test_combine_of_rows_that_differ_within_a_token(gpu, oracle, T, H, K):
     """After a dispatch the rows of a token are copies of one another, so a combine that mixed them up would still pass
-    the dispatch-then-combine tests; here every row is different.  The first two shapes have enough tokens of wide rows
+    the dispatch-then-combine tests; here every row is different.  The first two shapes and the top-6 shape of 5100 tokens have enough tokens of wide rows
     for the combine whose waves stay and alternate between reading and writing: same bits as the oracle at the
     default pace, at a slow and at an absurdly fast one, with slots without a row, and with the form switched off."""
     rng = np.random.default_rng(T)
