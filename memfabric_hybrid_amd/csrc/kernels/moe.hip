@@ -43,6 +43,7 @@ constexpr uint32_t kRankSlices = kRankBlock / 64;      // 16 wave-sized slices, 
 constexpr uint32_t kMaxExperts = 512;
 constexpr uint32_t kRowThreads = 256;
 constexpr uint32_t kMaxTopK = 16;
+constexpr uint32_t kCountingBlocks = 8;                 // launches of up to this many rank blocks need no histogram kernel
 constexpr uint32_t kHistPad = 32;                      // rows of the [expert][block] table are padded to this many blocks
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
@@ -151,14 +152,50 @@ __global__ __launch_bounds__(kRankThreads) void MoeRankKernel(const int32_t *__r
     uint32_t myExpert[kRankRounds];
     uint32_t myRank[kRankRounds];
     uint32_t bad = 0;
+    // blockHist == nullptr: no histogram kernel ran before this launch.  A single block has all it needs in its own
+    // slice histograms and its own flag (a dispatch of up to 1024 entries: 128 tokens at top-8).  The blocks of a
+    // launch of a few count the entries of the other blocks themselves, each for itself: per expert, the entries of
+    // all other blocks and those of the blocks before it (plain counts, so LDS atomics give the same result every time).
+    const bool tabled = blockHist != nullptr;
+    const bool counting = !tabled && gridDim.x > 1;
+    const uint32_t steps = runOrder != nullptr ? kRankSlices / stepSlices : 0;
+    uint32_t *others = cum + steps * experts;             // [2][experts], counting only
+    for (uint32_t i = threadIdx.x; counting && i < 2 * experts; i += kRankThreads) {
+        others[i] = 0;
+    }
     SliceHistograms(topk, total, experts, blockIdx.x * kRankBlock, hist, myExpert, myRank, &bad);
-
-    // blockHist == nullptr: the launch is a single block and no histogram kernel ran before it; the block's own slice
-    // histograms and its own flag are all there is (a dispatch of up to 1024 entries: 128 tokens at top-8).
-    const bool alone = blockHist == nullptr;
+    if (counting) {
+        const uint32_t blockBase = blockIdx.x * kRankBlock;
+        for (uint32_t start = 0; start < total; start += kRankBlock) {
+            if (start == blockBase) {
+                continue;
+            }
+            int32_t id[kRankRounds];
+#pragma unroll
+            for (uint32_t q = 0; q < kRankRounds; ++q) {
+                const uint32_t idx = start + q * kRankThreads + threadIdx.x;
+                id[q] = idx < total ? topk[idx] : 0;
+            }
+#pragma unroll
+            for (uint32_t q = 0; q < kRankRounds; ++q) {
+                const uint32_t idx = start + q * kRankThreads + threadIdx.x;
+                if (idx < total) {
+                    if (id[q] >= 0 && static_cast<uint32_t>(id[q]) < experts) {
+                        atomicAdd(&others[id[q]], 1u);
+                        if (start < blockBase) {
+                            atomicAdd(&others[experts + id[q]], 1u);
+                        }
+                    } else {
+                        bad = 1;
+                    }
+                }
+            }
+        }
+        __syncthreads();
+    }
     if (blockIdx.x == 0) {
-        uint32_t any = alone ? bad : 0;
-        for (uint32_t blk = threadIdx.x; !alone && blk < gridDim.x; blk += kRankThreads) {
+        uint32_t any = tabled ? 0 : bad;
+        for (uint32_t blk = threadIdx.x; tabled && blk < gridDim.x; blk += kRankThreads) {
             any |= blockBad[blk];
         }
         any = __syncthreads_or(static_cast<int>(any)) != 0 ? 1u : 0u;
@@ -184,12 +221,16 @@ __global__ __launch_bounds__(kRankThreads) void MoeRankKernel(const int32_t *__r
             const uint32_t *rowHist = blockHist + static_cast<uint64_t>(x) * histStride;
             uint32_t t = 0;
             uint32_t b = 0;
-            for (uint32_t sl = 0; alone && sl < kRankSlices; ++sl) {
+            for (uint32_t sl = 0; !tabled && sl < kRankSlices; ++sl) {
                 t += hist[sl * experts + x];
+            }
+            if (counting) {
+                t += others[x];
+                b = others[experts + x];
             }
             // kHistPad blocks per step, all their loads requested before the first is used (with one load per step the
             // loop waited a round trip per four blocks)
-            for (uint32_t blk = 0; !alone && blk < gridDim.x; blk += kHistPad) {
+            for (uint32_t blk = 0; tabled && blk < gridDim.x; blk += kHistPad) {
                 u32x4 v[kHistPad / 4];
 #pragma unroll
                 for (uint32_t q = 0; q < kHistPad / 4; ++q) {
@@ -241,7 +282,6 @@ __global__ __launch_bounds__(kRankThreads) void MoeRankKernel(const int32_t *__r
     // Turn slice histograms into exclusive prefixes over the slices of this block.  For the run-ordered list the
     // block is cut into steps of stepSlices slices (the tile permute works through one step at a time); the
     // entries per (step, expert) are what the prefix gains over a step.
-    const uint32_t steps = runOrder != nullptr ? kRankSlices / stepSlices : 0;
     for (uint32_t x = threadIdx.x; x < experts; x += kRankThreads) {
         uint32_t acc = base[x];
         uint32_t stepStart = acc;
@@ -819,13 +859,21 @@ extern "C" int mfk_moe_dispatch(const void *x, const void *topk, uint32_t tokens
     const bool tiles = g_xcdStreams.load(std::memory_order_relaxed) != 0 && x != nullptr && out != nullptr && upr >= kTileUnits &&
                        hidden % 64 == 0 && static_cast<uint64_t>(stepEntries / topK + 1) * hidden * 2 <= 2200000ull &&
                        stepsPerBlock * experts <= 4096 && tileGrid <= 0x7FFFFFFFull;
-    const size_t rankLds = histLds + (experts + kRankThreads + kRankSlices + (tiles ? stepsPerBlock * experts : 0)) * sizeof(uint32_t);
+    // Up to kCountingBlocks blocks rank without a histogram launch in front of them: every block counts the entries
+    // of the others itself.  129 / 256 / 512 / 1024 tokens of 7168 elements at top-8, 256 experts: 13.3 / 15.5 / 20.1 /
+    // 29.5 us per dispatch against 22.0 / 24.1 / 27.7 / 35.1 with the launch; 640 tokens over 512 experts 26 against 38.
+    // At sixteen blocks the two are level (50.5 us), at thirty-two the counting costs 10 us; over 8 or 16 experts,
+    // where the counts of a wave land on few LDS words, eight blocks are level (23.9 against 23.4 us) and sixteen
+    // lose 4 us.
+    const bool counting = blocks > 1 && blocks <= kCountingBlocks;
+    const size_t rankLds = histLds + (experts + kRankThreads + kRankSlices + (tiles ? stepsPerBlock * experts : 0) +
+                                      (counting ? 2 * experts : 0)) * sizeof(uint32_t);
     const uint64_t tableBytes = 256 + histStride * sizeof(uint32_t) + static_cast<uint64_t>(histStride) * experts * sizeof(uint32_t);
     int2 *runOrder = tiles ? reinterpret_cast<int2 *>(static_cast<char *>(workspace) + (tableBytes + 15) / 16 * 16) : nullptr;
-    if (blocks == 1) {
+    if (blocks == 1 || counting) {
         blockHist = nullptr;   // one block ranks from its own histograms: no launch in front of it (16 / 64 / 128 tokens of
                                // 7168 elements at top-8: 12 / 12.5 / 14 us per dispatch; 22 / 23 / 24 us before, with the
-                               // histogram launch and the token-ordered permute)
+                               // histogram launch and the token-ordered permute); a few blocks count for themselves
     } else {
         hipLaunchKernelGGL(MoeHistKernel, dim3(blocks), dim3(kRankThreads), histLds, s, static_cast<const int32_t *>(topk),
                            total, experts, blockHist, histStride, blockBad);

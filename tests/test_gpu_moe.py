@@ -186,6 +186,44 @@ def test_skewed_routing_with_empty_and_hot_experts(gpu, oracle):
         _free(bufs)
 
 
+@pytest.mark.parametrize("T,K,E", [(300, 8, 256), (600, 8, 64), (1024, 8, 512), (2048, 2, 8), (1100, 5, 17), (1025, 8, 256)])
+def test_few_blocks_that_count_one_anothers_entries(gpu, oracle, T, K, E):
+    """Two to eight blocks of 1024 entries rank without a histogram launch: each block counts the entries of the
+    others.  Everything against the oracle, then with one id out of range in the last block only (block 0 has to
+    find it for the status word), then clean again."""
+    H = 1024
+    x, topk, _ = _inputs(oracle, 0xF0 + T, T, H, K, E)
+    exp_out, exp_counts, exp_offsets, exp_row, exp_src = _oracle_dispatch(oracle, x, topk, E)
+    bufs = _gpu_dispatch(gpu, x, topk, E)
+    try:
+        assert _fetch(bufs["ws"], np.uint32, (1,))[0] == 0
+        assert np.array_equal(_fetch(bufs["counts"], np.int32, (E,)), exp_counts)
+        assert np.array_equal(_fetch(bufs["offsets"], np.int32, (E,)), exp_offsets)
+        assert np.array_equal(_fetch(bufs["row_of"], np.int32, (T * K,)), exp_row)
+        assert np.array_equal(_fetch(bufs["src_of"], np.int32, (T * K,)), exp_src)
+        assert np.array_equal(_fetch(bufs["out"], np.uint16, (T * K, H)), exp_out)
+    finally:
+        _free(bufs)
+    late = topk.copy()
+    late[T - 1, K - 1] = E + 7
+    sent = np.where(late >= E, E, late).astype(np.int32)
+    exp_out, exp_counts, _, exp_row, _ = _oracle_dispatch(oracle, x, sent, E + 1)
+    exp_row = np.where((late >= E).reshape(-1), -1, exp_row)
+    bufs = _gpu_dispatch(gpu, x, late, E)
+    try:
+        assert _fetch(bufs["ws"], np.uint32, (1,))[0] == 1
+        assert np.array_equal(_fetch(bufs["counts"], np.int32, (E,)), exp_counts[:E])
+        assert np.array_equal(_fetch(bufs["row_of"], np.int32, (T * K,)), exp_row)
+        assert np.array_equal(_fetch(bufs["out"], np.uint16, (T * K - 1, H)), exp_out[:T * K - 1])
+    finally:
+        _free(bufs)
+    bufs = _gpu_dispatch(gpu, x, topk, E)
+    try:
+        assert _fetch(bufs["ws"], np.uint32, (1,))[0] == 0
+    finally:
+        _free(bufs)
+
+
 def test_out_of_range_expert_ids_are_flagged_not_followed(gpu, oracle):
     T, H, K, E = 500, 64, 4, 32
     x, topk, _ = _inputs(oracle, 9, T, H, K, E)
