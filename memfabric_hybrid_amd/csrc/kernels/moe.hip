@@ -7,8 +7,9 @@
 //             (a stable counting sort of the flat (t,k) order by expert id)
 //   combine   y[t][h] = bf16_rne(fma(w[t][K-1], v[K-1], ... fma(w[t][0], v[0], 0)))
 //
-// Three launches for dispatch, one for combine:
-//   MoeHistKernel    per-block expert histograms (wave ballots + LDS)
+// Three launches for dispatch (two when the entries fill at most eight rank blocks), one for combine:
+//   MoeHistKernel    per-block expert histograms (wave ballots + LDS); not launched for a few blocks,
+//                    which count one another's entries inside the rank kernel
 //   MoeRankKernel    cross-block scan, stable rank of every entry -> rowOf/srcOf, counts, offsets,
 //                    and for the tile permute the rows of every step of entries in ascending order
 //   the permute, one of
@@ -24,7 +25,8 @@
 //                    stay for the whole launch and, chip-wide and by the clock, read for
 //                    most of a period and write at its end
 // Ranks come from ballots and prefix sums, never from atomics on a shared
-// cursor, so the permutation is the same on every run and equals the CPU sort.
+// cursor (the only atomics add up plain counts), so the permutation is the same on
+// every run and equals the CPU sort.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
