@@ -115,9 +115,12 @@ def timed_steps(lib, handle, batches, copy_type, steps, warmup, flags, caller="c
             if call(handle, refs[i % nb], copy_type, flags) != 0:
                 raise RuntimeError(native.last_error())
     lib.mfrt_event_record(stop, stream)
+    # the wait a caller of the API uses; it returns when everything queued on the thread's stream is done
+    ret = lib.smem_bm_wait(handle)
+    wall = time.perf_counter() - t0
+    assert ret == 0, native.last_error()
     assert lib.mfrt_stream_sync(stream) == 0
     assert lib.mfrt_device_sync() == 0
-    wall = time.perf_counter() - t0
     ms = lib.mfrt_event_elapsed_ms(start, stop)
     lib.mfrt_event_destroy(start)
     lib.mfrt_event_destroy(stop)
@@ -721,8 +724,10 @@ def main():
             "api": "smem_bm_copy_batch(SMEMB_COPY_G2G, ASYNC_COPY_FLAG) on one stream + one wait; the K calls are "
                    "issued by a C loop (mf_bm_copy_batch_replay), extras.kv122_python_caller has one ctypes call per batch",
             "timing": f"submitting thread pinned near the GPU; untimed ramp of {RAMP_BATCHES} batches + --warmup, then {REPETITIONS} repetitions of --steps batches, "
-                      "each between two synchronisations; ms_per_step / value: median repetition by the host clock "
-                      "(includes one stream wait per repetition), roofline: median repetition by HIP events",
+                      "each between two synchronisations; ms_per_step / value: median repetition by the host clock, "
+                      "from the first call to the return of smem_bm_wait (behind a queue of up to 256 MiB it polls a word that a "
+                      "one-lane launch stores behind the last batch, behind more it is hipStreamSynchronize; hipStreamSynchronize "
+                      "and hipDeviceSynchronize follow before the next repetition), roofline: median repetition by HIP events",
             "payload_bytes": payload,
             "cu_count": lib.mfrt_cu_count(),
             "submitting_thread": {"empty_launch_us_by_cpu": launch_us_by_cpu, "runs_on_cpus": near_cpus if kept > 0 else all_cpus,

@@ -57,6 +57,7 @@ MF_EXPORT int32_t mf_xcopy_2d_batch(const mf_copy2d_desc *descs, uint32_t n, int
     if (stream == nullptr) {
         stream = engine.ThreadStream();
     }
+    engine.NoteQueued(stream, ~0ull);   // a wait behind these kernels sleeps on the stream
     for (uint32_t i = 0; i < n; ++i) {
         if (descs[i].width > descs[i].spitch && descs[i].height > 1) {
             MF_FAIL(BM_INVALID_PARAM, "rectangle " << i << ": width exceeds the source pitch");

@@ -27,6 +27,7 @@ int Prepare(void *&stream)
             MF_FAIL(BM_ERROR, "cannot create the thread's stream");
         }
     }
+    engine.NoteQueued(stream, ~0ull);   // a wait behind these kernels sleeps on the stream
     return BM_OK;
 }
 

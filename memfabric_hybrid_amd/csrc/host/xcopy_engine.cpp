@@ -51,6 +51,7 @@ struct ThreadLease {
     bool adopted = false;           // taken over from a thread that ended: its queued kernels ran on streams unknown here
     uint64_t *doneWord = nullptr;   // pinned; a one-lane launch stores doneSeq there behind a blocking copy
     uint32_t doneSeq = 0;
+    uint64_t pendingBytes = 0;      // bytes of the copies queued on `stream` since the thread last waited for it
     void *bounce = nullptr;
     uint64_t bounceBytes = 0;
     void *bounceEvents[XcopyEngine::kBounceEvents] = {};
@@ -198,6 +199,15 @@ struct ThreadCtx {
 };
 
 thread_local ThreadCtx t_ctx;
+
+// Copies queued on the calling thread's own stream are added up, so that its next wait knows whether polling pays.
+void NotePending(void *stream, uint64_t bytes)
+{
+    if (t_ctx.HasLiveLease() && stream == t_ctx.lease->stream) {
+        uint64_t &pending = t_ctx.lease->pendingBytes;
+        pending = pending + bytes < pending ? ~0ull : pending + bytes;
+    }
+}
 
 uint64_t RoundUp(uint64_t v, uint64_t to)
 {
@@ -693,11 +703,8 @@ int XcopyEngine::DrainThread()
     if (!t_ctx.HasLiveLease() || t_ctx.lease->stream == nullptr) {
         return BM_OK;
     }
-    int err = mfrt_stream_sync(t_ctx.lease->stream);
-    if (err != 0) {
-        MF_FAIL(BM_ERROR, "stream wait failed: " << mfrt_error_string(err));
-    }
-    return BM_OK;
+    // a short queue is awaited like a blocking call: by polling (20 KV batches and a wait: 3 us sooner than the stream wait)
+    return WaitStream(t_ctx.lease->stream, t_ctx.lease->pendingBytes);
 }
 
 // A blocking call is a launch and a wait.  hipStreamSynchronize first has to put a marker with a
@@ -712,6 +719,11 @@ int XcopyEngine::DrainThread()
 // issued, in order, before the word's.
 int XcopyEngine::WaitStream(void *stream, uint64_t bytes)
 {
+    if (t_ctx.HasLiveLease() && stream == t_ctx.lease->stream) {
+        const uint64_t queued = t_ctx.lease->pendingBytes;
+        bytes = queued > bytes ? queued : bytes;     // what else the thread has queued there is waited for as well
+        t_ctx.lease->pendingBytes = 0;
+    }
     if (bytes != 0 && bytes <= kSpinBytes) {
         ThreadLease &lease = t_ctx.Lease();
         if (lease.doneWord == nullptr) {
@@ -742,6 +754,11 @@ int XcopyEngine::WaitStream(void *stream, uint64_t bytes)
         MF_FAIL(BM_ERROR, "copy failed on the GPU: " << mfrt_error_string(err));
     }
     return BM_OK;
+}
+
+void XcopyEngine::NoteQueued(void *stream, uint64_t bytes)
+{
+    NotePending(stream, bytes);
 }
 
 uint64_t XcopyEngine::LaunchCount() const
@@ -801,11 +818,13 @@ int XcopyEngine::Submit(const uint64_t *src, const uint64_t *dst, const uint64_t
     uint32_t units = 0;
     bool oversized = false;      // a run the 32-bit length of the inline table cannot hold is possible
     bool windowed = false;
+    uint64_t queuedBytes = 0;
     if (n <= 4 * kInlineSegs) {  // small enough that a failed attempt costs next to nothing
         uint64_t total = 0;
         for (uint32_t i = 0; i < n; ++i) {
             total += len[i];
         }
+        queuedBytes = total;
         oversized = total > 0xFFFFFFFFull;
         units = ChooseUnits(total, cu, route, tuning_);
         // Large HBM copies of one submitter: 16 KiB chunks for the kernel that alternates between read and write windows.
@@ -827,6 +846,7 @@ int XcopyEngine::Submit(const uint64_t *src, const uint64_t *dst, const uint64_t
             MF_FAIL(BM_ERROR, "xcopy launch failed: " << mfrt_error_string(err));
         }
         g_launches.fetch_add(1, std::memory_order_relaxed);
+        NotePending(stream, queuedBytes);
         return BM_OK;
     }
     if (inlined) {
@@ -838,6 +858,7 @@ int XcopyEngine::Submit(const uint64_t *src, const uint64_t *dst, const uint64_t
             MF_FAIL(BM_ERROR, "xcopy launch failed: " << mfrt_error_string(err));
         }
         g_launches.fetch_add(1, std::memory_order_relaxed);
+        NotePending(stream, queuedBytes);
         return BM_OK;
     }
 
@@ -850,6 +871,7 @@ int XcopyEngine::Submit(const uint64_t *src, const uint64_t *dst, const uint64_t
             total += len[i];
             longest = len[i] > longest ? len[i] : longest;
         }
+        queuedBytes = total;
         // A table of long segments between HBM addresses is cut into launches of kInlineSegs segments, each of which
         // then takes the form with read and write windows: the few extra launches cost microseconds, the windows
         // gain 8 % (896 segments, 8.5 GB: 2.55 ms in seven launches against 2.78 ms in one).  The table kernel
@@ -945,6 +967,7 @@ int XcopyEngine::Submit(const uint64_t *src, const uint64_t *dst, const uint64_t
         (void)MarkQueued(lease, slot, stream, true);
         MF_FAIL(BM_ERROR, "xcopy table launch failed: " << mfrt_error_string(err));
     }
+    NotePending(stream, queuedBytes);
     return MarkQueued(lease, slot, stream, false);
 }
 
@@ -997,6 +1020,7 @@ int XcopyEngine::SubmitDeviceTable(const void *triples, uint32_t n, int route, v
         MF_FAIL(BM_ERROR, "xcopy table launch failed: " << mfrt_error_string(err));
     }
     g_launches.fetch_add(2, std::memory_order_relaxed);
+    NotePending(stream, ~0ull);   // sizes unknown here: the next wait sleeps on the stream
     return MarkQueued(lease, slot, stream, false);
 }
 
@@ -1024,6 +1048,7 @@ int XcopyEngine::SubmitDeviceTableStatic(const void *triples, uint32_t n, int ro
         MF_FAIL(BM_ERROR, "static-scratch table launch failed (" << err << ")");
     }
     g_launches.fetch_add(2, std::memory_order_relaxed);
+    NotePending(stream, ~0ull);
     return BM_OK;
 }
 #endif

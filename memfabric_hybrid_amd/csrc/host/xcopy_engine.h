@@ -111,6 +111,9 @@ public:
     static constexpr uint64_t kSpinBytes = 256ull << 20;
     static constexpr uint32_t kSpinMicros = 200;
     int WaitStream(void *stream, uint64_t bytes);
+    // Work that another part of the library has queued on `stream`: if it is the calling thread's own stream, the next
+    // DrainThread() takes `bytes` into account when it chooses between polling and sleeping (~0: sleep).
+    void NoteQueued(void *stream, uint64_t bytes);
 
     // Enqueue one batch.  Addresses must be device-accessible.  stream may be
     // NULL (thread stream).  mask/maskValue: plugin completion word or NULL.

@@ -200,7 +200,8 @@ uint64_t fake_rt_in_flight(void)
     return g_inFlight.size();
 }
 
-int mfrt_stream_sync(void *) { Guard("mfrt_stream_sync"); Retire(~0ull); return 0; }
+extern "C" void fake_rt_count_stream_sync(void);
+int mfrt_stream_sync(void *) { Guard("mfrt_stream_sync"); Retire(~0ull); fake_rt_count_stream_sync(); return 0; }
 int mfrt_device_sync(void) { Guard("mfrt_device_sync"); Retire(~0ull); return 0; }
 void *mfrt_event_create(void) { return calloc(1, 8); }
 int mfrt_event_destroy(void *e) { Guard("mfrt_event_destroy"); free(e); return 0; }
@@ -309,9 +310,15 @@ int mfk_xcopy_plan(const void *triples, uint32_t nseg, uint32_t units, void *fir
     return 0;
 }
 
+static uint64_t g_signals = 0;
+static uint64_t g_streamSyncs = 0;
+extern "C" uint64_t fake_rt_signals() { return g_signals; }
+extern "C" uint64_t fake_rt_stream_syncs() { return g_streamSyncs; }
+extern "C" void fake_rt_count_stream_sync(void) { ++g_streamSyncs; }
 int mfk_xcopy_signal(void *word, uint32_t value, void *)
 {
     // not counted: fake_rt_launches() counts the launches that move data
+    ++g_signals;
     __atomic_store_n(static_cast<uint64_t *>(word), static_cast<uint64_t>(value), __ATOMIC_RELEASE);
     return 0;
 }

@@ -25,6 +25,8 @@ extern "C" uint64_t fake_rt_launches(void);
 extern "C" uint32_t fake_rt_last_hold(void);
 extern "C" uint32_t fake_rt_last_rect_mates(void);
 extern "C" int fake_rt_last_combine_paced(void);
+extern "C" uint64_t fake_rt_signals(void);
+extern "C" uint64_t fake_rt_stream_syncs(void);
 extern "C" uint32_t fake_rt_last_window(void);
 extern "C" void fake_rt_seal(void);
 extern "C" void fake_rt_fail_launches(int n);
@@ -352,6 +354,63 @@ static void TestHostLaunchCosts()
         CHECK(!CPU_ISSET(cpu, &after) || CPU_ISSET(cpu, &before));
     }
     CHECK(sched_setaffinity(0, sizeof(before), &before) == 0);
+    hybm_uninit();
+}
+
+// A wait behind a short queue of copies polls a word that a one-lane launch stores; behind a long queue, behind
+// kernels of the other entry points and behind tables of unknown size it sleeps on the stream.
+static void TestWaitOfShortQueues()
+{
+    CHECK(hybm_init(0, 0) == BM_OK);
+    XcopyEngine &engine = XcopyEngine::Instance();
+    void *stream = engine.ThreadStream();
+    CHECK(stream != nullptr);
+    std::vector<uint8_t> from(1 << 20, 7), to(1 << 20, 0);
+    uint64_t s = reinterpret_cast<uint64_t>(from.data()), d = reinterpret_cast<uint64_t>(to.data()), l = from.size();
+    for (int i = 0; i < 3; ++i) {
+        CHECK(engine.Submit(&s, &d, &l, 1, MF_ROUTE_HBM, stream, nullptr, 0) == BM_OK);
+    }
+    uint64_t signals = fake_rt_signals(), syncs = fake_rt_stream_syncs();
+    CHECK(engine.DrainThread() == BM_OK);
+    CHECK(fake_rt_signals() == signals + 1 && fake_rt_stream_syncs() == syncs);       // polled
+    CHECK(to == from);
+    signals = fake_rt_signals();
+    syncs = fake_rt_stream_syncs();
+    CHECK(engine.DrainThread() == BM_OK);                                               // nothing queued: the stream wait
+    CHECK(fake_rt_signals() == signals && fake_rt_stream_syncs() == syncs + 1);
+    // more than the polling limit in the queue
+    uint64_t big = XcopyEngine::kSpinBytes / 2 + 4096;
+    std::vector<uint8_t> wide(big, 1), wide2(big, 0);
+    uint64_t ws = reinterpret_cast<uint64_t>(wide.data()), wd = reinterpret_cast<uint64_t>(wide2.data());
+    CHECK(engine.Submit(&ws, &wd, &big, 1, MF_ROUTE_HBM, stream, nullptr, 0) == BM_OK);
+    CHECK(engine.Submit(&ws, &wd, &big, 1, MF_ROUTE_HBM, stream, nullptr, 0) == BM_OK);
+    signals = fake_rt_signals();
+    syncs = fake_rt_stream_syncs();
+    CHECK(engine.DrainThread() == BM_OK);
+    CHECK(fake_rt_signals() == signals && fake_rt_stream_syncs() == syncs + 1);
+    // a copy on another stream is not this thread's queue
+    int other = 0;
+    CHECK(engine.Submit(&s, &d, &l, 1, MF_ROUTE_HBM, &other, nullptr, 0) == BM_OK);
+    signals = fake_rt_signals();
+    syncs = fake_rt_stream_syncs();
+    CHECK(engine.DrainThread() == BM_OK);
+    CHECK(fake_rt_signals() == signals && fake_rt_stream_syncs() == syncs + 1);
+    // kernels of the other entry points behind a short copy
+    CHECK(engine.Submit(&s, &d, &l, 1, MF_ROUTE_HBM, stream, nullptr, 0) == BM_OK);
+    alignas(16) static uint8_t moeBuf[64];
+    CHECK(mf_moe_combine(moeBuf, reinterpret_cast<const int32_t *>(moeBuf), reinterpret_cast<const float *>(moeBuf), 1, 8, 1,
+                         moeBuf + 16, nullptr) == BM_OK);
+    signals = fake_rt_signals();
+    syncs = fake_rt_stream_syncs();
+    CHECK(engine.DrainThread() == BM_OK);
+    CHECK(fake_rt_signals() == signals && fake_rt_stream_syncs() == syncs + 1);
+    // a blocking call drains the queue, so the wait after it has nothing to poll for
+    CHECK(engine.Submit(&s, &d, &l, 1, MF_ROUTE_HBM, stream, nullptr, 0) == BM_OK);
+    CHECK(engine.WaitStream(stream, l) == BM_OK);
+    signals = fake_rt_signals();
+    syncs = fake_rt_stream_syncs();
+    CHECK(engine.DrainThread() == BM_OK);
+    CHECK(fake_rt_signals() == signals && fake_rt_stream_syncs() == syncs + 1);
     hybm_uninit();
 }
 
@@ -1066,6 +1125,7 @@ int main()
     TestHeldStores();
     TestWindows();
     TestHostLaunchCosts();
+    TestWaitOfShortQueues();
     if (g_failed != 0) {
         std::printf("%d check(s) failed\n", g_failed);
         return 1;
