@@ -319,6 +319,45 @@ def extras_block(lib, pool, dev, batches, tables, steps):
                     "on its own stream, wall clock from the release of the warmed-up threads to the last wait; median of 5")
     out["kv122_d2d_concurrent_streams"] = conc
 
+    # ---- several requests' KV blocks in one call (the serving case: smem_trans_entry.cpp:363-376 of the reference batches what its
+    # caller hands it), and 32 x 1 MiB, the largest block of the reference's own grid that one launch holds in registers
+    multi = {}
+    eighth = POOL_BYTES // 8
+    for requests in (2, 4, 8):
+        group = []
+        for b in range(16):
+            parts = [workloads.kv_batch(0xC1 + 1000 * requests + 8 * b + r, eighth) for r in range(requests)]
+            src = np.concatenate([p[0] + np.uint64(r * eighth) for r, p in enumerate(parts)])
+            dst = np.concatenate([p[1] + np.uint64(r * eighth) for r, p in enumerate(parts)])
+            group.append(Batch(dev + src, dev + dst, np.concatenate([p[2] for p in parts])))
+        entry = {}
+        for name, hold in (("us_per_call", -1), ("us_per_call_stores_not_held", 0)):
+            assert lib.mf_xcopy_hold_stores(hold) == 0
+            reps = sorted(timed_steps(lib, handle, group, g2g, 400, 50, native.ASYNC_COPY_FLAG)[1] * 1e3 / 400 for _ in range(5))
+            entry[name] = round(reps[2], 2)
+        assert lib.mf_xcopy_hold_stores(-1) == 0
+        us = entry["us_per_call"]
+        entry.update({"segments": group[0].n, "payload_bytes": group[0].payload, "us_per_request": round(us / requests, 2),
+                      "hbm_GBps": round(2 * group[0].payload / us / 1e3, 1),
+                      "frac_of_hbm_peak": frac(2 * group[0].payload / us / 1e3, HBM_PEAK_GBPS)})
+        multi[f"kv_{group[0].n}_segments"] = entry
+    blocks = [Batch(dev + np.uint64(b * (64 << 20)) + np.arange(32, dtype=np.uint64) * np.uint64(1 << 20),
+                    dev + np.uint64(POOL_BYTES // 2 + b * (64 << 20)) + np.arange(32, dtype=np.uint64)[::-1] * np.uint64(1 << 20),
+                    np.full(32, 1 << 20, dtype=np.uint64)) for b in range(16)]
+    entry = {}
+    for name, hold in (("us_per_call", -1), ("us_per_call_stores_not_held", 0)):
+        assert lib.mf_xcopy_hold_stores(hold) == 0
+        reps = sorted(timed_steps(lib, handle, blocks, g2g, 400, 50, native.ASYNC_COPY_FLAG)[1] * 1e3 / 400 for _ in range(5))
+        entry[name] = round(reps[2], 2)
+    assert lib.mf_xcopy_hold_stores(-1) == 0
+    entry.update({"payload_bytes": blocks[0].payload, "hbm_GBps": round(2 * blocks[0].payload / entry["us_per_call"] / 1e3, 1),
+                  "frac_of_hbm_peak": frac(2 * blocks[0].payload / entry["us_per_call"] / 1e3, HBM_PEAK_GBPS)})
+    multi["32_x_1MiB"] = entry
+    multi["note"] = ("asynchronous smem_bm_copy_batch calls back to back on one stream, 16 tables in turn, HIP events, median of 5 runs; more than "
+                     "128 segments take the table form (descriptors read from the pinned staging slot), up to 24 MiB in 4 KiB chunks and up "
+                     "to 64 MiB in 16 KiB chunks with the stores held back until the loads of the launch are out")
+    out["batches_of_several_requests"] = multi
+
     # ---- the grid the reference publishes for its transfer benchmark (example/trans/perf/README.md:61-70 there:
     # 32 equal blocks per batch, blocking calls, GB/s = block * 32 / time per call), here HBM to HBM on one GPU
     grid = []
@@ -489,7 +528,41 @@ def extras_paged(lib):
         res[name] = {"us": round(us, 1), "hbm_GBps": round(hbm, 1), "frac_of_hbm_peak": frac(hbm, HBM_PEAK_GBPS)}
     res["shape"] = "4096 x 32 KiB pages, 40 GiB pool, one K-or-V plane of one layer per call (134 217 728 B)"
     lib.mfrt_device_sync()
+
+    def device_table(src, dst, lens):
+        t = np.stack([np.asarray(src, dtype=np.uint64), np.asarray(dst, dtype=np.uint64), np.asarray(lens, dtype=np.uint64)], axis=1)
+        t = np.ascontiguousarray(t).reshape(-1)
+        p = lib.mfrt_alloc_device(t.nbytes)
+        assert p and lib.mfrt_memcpy(p, t.ctypes.data, t.nbytes) == 0
+        return p
+
+    # the same gather with its {src, dst, len} table resident in device memory (the plugin ABI's other legal form): planned on the GPU
+    ids = workloads.page_ids(0xC3, pool_bytes // page, count)
+    tab = device_table(pool + ids * page, buf + np.arange(count, dtype=np.uint64) * page, np.full(count, page))
+    us, _ = timer.run(lambda: lib.mf_xcopy_device_table(tab, count, native.ROUTE_HBM, None), 40, warm=10)
+    table_path = {"device_table_4096_pages": {"us": round(us, 1), "hbm_GBps": round(2 * count * page / us / 1e3, 1),
+                                               "frac_of_hbm_peak": frac(2 * count * page / us / 1e3, HBM_PEAK_GBPS),
+                                               "us_descriptors_from_host_arrays": res["gather"]["us"]}}
+    lib.mfrt_device_sync()
+    lib.mfrt_free_device(tab)
     lib.mfrt_free_device(buf)
+    # 16 384 ragged segments of 2 to 262 KB at odd addresses: no pattern, the group map finds a chunk's segment
+    rng = np.random.default_rng(7)
+    n_ragged, slot = 16384, 512 << 10
+    lens = rng.integers(2000, 262144, size=n_ragged).astype(np.uint64)
+    src = pool + rng.permutation(2 * n_ragged)[:n_ragged].astype(np.uint64) * np.uint64(slot) + rng.integers(0, 64, n_ragged).astype(np.uint64)
+    dst = pool + np.uint64(20 << 30) + np.arange(n_ragged, dtype=np.uint64) * np.uint64(slot) + rng.integers(0, 64, n_ragged).astype(np.uint64)
+    s_r, d_r, l_r = native.u64_array(src.tolist()), native.u64_array(dst.tolist()), native.u64_array(lens.tolist())
+    moved = int(lens.sum())
+    us, _ = timer.run(lambda: lib.mf_xcopy_batch(s_r, d_r, l_r, n_ragged, native.ROUTE_HBM, None), 20, warm=10)
+    tab = device_table(src, dst, lens)
+    us_dev, _ = timer.run(lambda: lib.mf_xcopy_device_table(tab, n_ragged, native.ROUTE_HBM, None), 20, warm=10)
+    table_path["ragged_16384"] = {"payload_bytes": moved, "us": round(us, 1), "hbm_GBps": round(2 * moved / us / 1e3, 1),
+                                  "frac_of_hbm_peak": frac(2 * moved / us / 1e3, HBM_PEAK_GBPS),
+                                  "us_table_in_device_memory": round(us_dev, 1),
+                                  "frac_of_hbm_peak_table_in_device_memory": frac(2 * moved / us_dev / 1e3, HBM_PEAK_GBPS)}
+    lib.mfrt_device_sync()
+    lib.mfrt_free_device(tab)
     # The whole set of a 32-layer model (K and V planes: 64 x 4096 pages) as ONE call of 262 144 descriptors.
     planes = 64
     big = lib.mfrt_alloc_device(planes * count * page)
@@ -507,8 +580,19 @@ def extras_paged(lib):
         hbm = 2 * total * page / us / 1e3
         res["gather_full_set_one_call"] = {"descriptors": total, "us": round(us, 1), "hbm_GBps": round(hbm, 1),
                                            "frac_of_hbm_peak": frac(hbm, HBM_PEAK_GBPS)}
+        tab = device_table(pool + ids * page, big + np.arange(total, dtype=np.uint64) * page, np.full(total, page))
+        us_dev, _ = timer.run(lambda: lib.mf_xcopy_device_table(tab, total, native.ROUTE_HBM, None), 8, warm=4)
+        table_path["device_table_262144_pages"] = {"us": round(us_dev, 1), "hbm_GBps": round(2 * total * page / us_dev / 1e3, 1),
+                                                   "frac_of_hbm_peak": frac(2 * total * page / us_dev / 1e3, HBM_PEAK_GBPS),
+                                                   "us_descriptors_from_host_arrays": round(us, 1)}
         lib.mfrt_device_sync()
+        lib.mfrt_free_device(tab)
         lib.mfrt_free_device(big)
+    table_path["note"] = ("device_table_*: mf_xcopy_device_table, the table planned on the GPU (chunk prefix, group map, and the repeating chunk "
+                          "counts of equal pages found there) in one launch up to 8192 segments, two beyond, in front of the copy launch; "
+                          "ragged_16384: mf_xcopy_batch from host arrays (descriptors, prefix and group map uploaded by a launch of its own) "
+                          "and the same table resident in device memory")
+    res["table_path"] = table_path
     lib.mfrt_free_device(pool)
     return res
 
@@ -653,7 +737,8 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--calibrate", action="store_true", help="only run the plain copy kernel (counter calibration)")
     ap.add_argument("--phases", action="store_true",
-                    help="only run the stand-alone program that takes the KV batch apart (lib/mf_batch_phases) and print its JSON")
+                    help="only run the stand-alone program that takes KV batches apart (bench_phases/mf_batch_phases) and print its JSON")
+    ap.add_argument("phase_args", nargs="*", help="with --phases: requests per batch to take apart (1 2 4 8), default 1 and 4")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build is a single-GPU data plane (no collectives, no sharding); run with --gpus 1")
@@ -661,8 +746,10 @@ def main():
     if args.phases:
         # a child process of its own, started before this one touches the GPU
         import subprocess
-        exe = os.path.join(ROOT, "memfabric_hybrid_amd", "lib", "mf_batch_phases")
-        done = subprocess.run([exe], stdout=subprocess.PIPE, text=True, timeout=300)
+        exe = os.path.join(ROOT, "bench_phases", "mf_batch_phases")
+        if not os.path.exists(exe):   # not part of the product build: compiled on demand
+            subprocess.run(["make", "-C", os.path.join(ROOT, "bench_phases")], check=True, stdout=subprocess.DEVNULL)
+        done = subprocess.run([exe] + args.phase_args, stdout=subprocess.PIPE, text=True, timeout=600)
         sys.stdout.write(done.stdout)
         sys.exit(done.returncode)
 

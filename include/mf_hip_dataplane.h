@@ -1,11 +1,14 @@
 /*
  * Native entry points of libmf_hip_dataplane.so beyond the drop-in surface of
- * mf_xcopy_api.h: the raw batch enqueue the benchmark times, runtime services
- * a host program needs to own GPU memory and streams without touching HIP
- * itself, and read-only views of the host logic (planner, address registry,
- * direction algebra) for tests.  Plain C types only; a stream or event is an
- * opaque void*.  Functions returning int32_t give 0 or a negative BM_* code
- * unless stated; the mfrt_* services return 0 or a positive HIP error number.
+ * mf_xcopy_api.h: raw batch enqueues (host arrays, a table in device memory,
+ * strided rectangles), the local MoE dispatch / combine, and the runtime
+ * services a host program needs to own GPU memory and streams without
+ * touching HIP itself.  This is the stable native ABI.  Test views, replay
+ * loops for benchmarks and tuning switches are exported too but declared in
+ * mf_hip_dataplane_internal.h, without a stability promise.
+ * Plain C types only; a stream or event is an opaque void*.  Functions
+ * returning int32_t give 0 or a negative BM_* code unless stated; the mfrt_*
+ * services return 0 or a positive HIP error number.
  *
  * None of these has a counterpart in the reference's public headers; where
  * one stands in for reference-internal code the comment says which.
@@ -46,30 +49,6 @@ extern "C" {
 int32_t mf_xcopy_batch(const uint64_t *src, const uint64_t *dst, const uint64_t *len, uint32_t n, int32_t route,
                        void *stream);
 
-/* `steps` calls of smem_bm_copy_batch(handle, batches[i % count], t, flags), i = 0 .. steps-1,
- * issued from C: what the loop of a C or C++ caller does (the reference's benchmark,
- * example/bm/BmBenchmark/band_width_calculator.cpp:530-590, is such a loop), for callers
- * written in an interpreted language whose per-call overhead would otherwise set the pace.
- * Stops at the first call that fails and returns its code. */
-int32_t mf_bm_copy_batch_replay(smem_bm_t handle, smem_batch_copy_params *const *batches, uint32_t count,
-                                uint32_t steps, smem_bm_copy_type t, uint32_t flags);
-
-/* The same for the transfer front-end: `steps` calls of smem_trans_batch_write_submit(handle, sources, remoteUniqueId,
- * destinations, dataSizes, batchSize, stream, 0) with the arrays of batches[i % count] (sources = local addresses,
- * destinations = addresses in the peer's registered memory). */
-int32_t mf_trans_batch_write_replay(smem_trans_t handle, smem_batch_copy_params *const *batches, uint32_t count, uint32_t steps,
-                                    const char *remoteUniqueId, void *stream);
-
-/* The same `steps` calls shared out over `threads` host threads (call i goes to thread
- * i % threads), each thread on its own stream as the reference gives every calling thread its
- * own (src/hybm/csrc/ts_engine/hybm_stream_manager.cpp:73-90), all asynchronous with one
- * smem_bm_wait per thread at the end.  *seconds receives the wall-clock time from the moment
- * all threads (already warmed up) are released until the last one has returned from its wait.
- * The threads share `batches`: the library rewrites the address arrays in place with the same
- * values, which is harmless.  Returns the first failing call's code. */
-int32_t mf_bm_copy_batch_replay_threads(smem_bm_t handle, smem_batch_copy_params *const *batches, uint32_t count,
-                                        uint32_t steps, smem_bm_copy_type t, uint32_t threads, double *seconds);
-
 /* An enqueue of mf_xcopy_batch for a {src,dst,len} triple table that already lives in device memory. */
 int32_t mf_xcopy_device_table(const void *triples, uint32_t n, int32_t route, void *stream);
 
@@ -105,45 +84,6 @@ typedef struct {
 } mf_copy2d_desc;
 int32_t mf_xcopy_2d_batch(const mf_copy2d_desc *descs, uint32_t n, int32_t route, void *stream);
 
-/* Host-only views of the 2-D kernel's index arithmetic, for tests.  mf_copy2d_describe: rows one
- * workgroup takes and the division constant for rows of `width` bytes.  mf_copy2d_rowcol_mismatches:
- * how many of the units 0 .. unitsInChunk-1 of a chunk the kernel's (row, column) formula places
- * differently from u / widthUnits, u % widthUnits (0 for every plan the library builds). */
-void mf_copy2d_describe(uint64_t width, uint32_t *rowsPerChunk, uint32_t *magic);
-uint32_t mf_copy2d_rowcol_mismatches(uint32_t widthUnits, uint32_t rowsPerChunk, uint32_t magic, uint32_t unitsInChunk);
-
-/* Launch-shape knobs.  units: 16-byte units per workgroup chunk (0 = choose
- * per batch); wgPerCu: grid cap in workgroups per CU on HBM routes (0 = the
- * default: one workgroup per chunk, no cap); wgPerCuLink: workgroups per CU
- * on host-link routes (0 = the default, 1). */
-int32_t mf_xcopy_tune(uint32_t units, uint32_t wgPerCu, uint32_t wgPerCuLink);
-/* Stores held back.  A batch of 960 to 6144 chunks of 4 KiB between HBM addresses (4 to 25 MB in up
- * to 128 segments) is copied 7 to 20 % faster when every wave waits with its stores until the loads of
- * the whole launch are out, so that HBM sees a burst of reads and then a burst of writes instead of both
- * mixed.  nanos: -1 = the library's rule for how long a wave waits after its start (the default),
- * 0 = never wait, otherwise that many ns for every launch the rule would pick.  Other launches, and
- * batches submitted with MF_COPY_UNORDERED_FLAG, never wait. */
-int32_t mf_xcopy_hold_stores(int32_t nanos);
-/* Read and write windows.  A batch of up to 128 segments and 512 MiB or more between HBM addresses is copied
- * by 4096 waves that alternate, all together and by the GPU's constant-rate clock, between a read half and a
- * write half of a period, so that HBM sees long bursts of one direction: 6.65-6.75 TB/s instead of 6.1-6.35 on
- * aligned copies of 512 MiB to 2 GiB, 6.05-6.3 instead of 5.75-5.85 when sources sit at odd addresses.  The
- * period is cut for a rate of HBM traffic (read + written) in MB/s, 6 800 000 by default; at 7 000 000 the waves
- * of a 2 GiB copy now and then no longer keep up, the windows dissolve and the copy runs at about the rate it
- * has without them; at 7 200 000 and above most launches do.  0 switches the form off.  While several threads
- * submit on streams of their own it is not used. */
-int32_t mf_xcopy_windows(uint32_t megabytesPerSecond);
-uint32_t mf_xcopy_choose_units(uint64_t totalBytes, uint32_t cuCount, int32_t route);
-uint64_t mf_xcopy_launch_count(void);
-
-/* Host-only view of the work decomposition: writes, for every chunk of the
- * normalised batch, up to three byte ranges {srcAddr, dstAddr, bytes, chunk}
- * (head, 16-byte body, tail) into out[4*i..].  Returns the number of ranges,
- * or -(needed) when capacity (in ranges) is too small.  inlineForm receives 1
- * when the batch fits the kernel-argument form. */
-int64_t mf_xcopy_describe_plan(const uint64_t *src, const uint64_t *dst, const uint64_t *len, uint32_t n,
-                               uint32_t units, uint64_t *out, uint64_t capacity, int32_t *inlineForm);
-
 /* ---- local MoE dispatch / combine over pooled memory ------------------------
  * No reference implementation exists; the specification is the stable counting
  * sort / fixed-order fp32 FMA chain stated in oracle/mf_oracle.c.  All buffers
@@ -169,19 +109,11 @@ int32_t mf_moe_dispatch(const void *x, const int32_t *topk, uint32_t tokens, uin
  * round-to-nearest-even; entries with rowOf < 0 contribute nothing. */
 int32_t mf_moe_combine(const void *rows, const int32_t *rowOf, const float *weights, uint32_t tokens, uint32_t hidden,
                        uint32_t topK, void *y, void *stream);
-/* A combine of topK == 8 or 6 with rows of 2048 elements and more, on enough tokens to give every wave of the chip six
- * slices of 128 x 8 elements (about 3500 tokens of 7168 elements on 256 CUs), runs as waves that stay for the whole
- * launch and alternate, chip-wide and by the clock, between reading rows and writing results.  readMBps / writeMBps
- * (MB/s of HBM traffic, 1 000 000 ... 16 000 000) set the pace of the two parts; the defaults are 6 800 000 and
- * 6 200 000, both 0 turns the form off (one workgroup per slice, as for smaller inputs, and as long as a second
- * thread holds a stream of the library).  Results do not depend on it.  No counterpart in the reference.  Returns BM_INVALID_PARAM for other values. */
-int32_t mf_moe_combine_windows(uint32_t readMBps, uint32_t writeMBps);
-/* 1 if hybm_init found that the GPU deals consecutive workgroups to its eight XCDs in turn (an MI355X in its default
- * partition does): the dispatch of rows of whole cache lines then writes its output in runs of consecutive rows, one stream of runs
- * per XCD; 0: it keeps to the token-ordered permute.  No counterpart in the reference. */
-int32_t mf_moe_xcd_streams(void);
-
-/* Host side of a launch.  What one launch costs the submitting thread depends on the CPU it runs on (3.1 against
+/* ---- optional: where the submitting thread runs ------------------------------
+ * The only two functions of this header that touch anything outside the library: they CHANGE THE CALLING
+ * THREAD'S CPU AFFINITY (mf_host_launch_costs restores it, mf_pin_thread_near_gpu keeps the narrowed set, and
+ * threads created afterwards inherit it).  Nothing in the library calls them on its own.
+ * What one launch costs the submitting thread depends on the CPU it runs on (3.1 against
  * 4.3 us per smem_bm_copy_batch call on the hosts this was built on, half of the CPUs each, with nothing in the
  * operating system's topology to tell them apart), and a thread the scheduler moves between the two kinds changes
  * pace mid-run.  mf_host_launch_costs measures it: it pins the calling thread to each CPU of its affinity set in
@@ -221,43 +153,6 @@ float mfrt_event_elapsed_ms(void *start, void *stop);
 int mfrt_memcpy(void *dst, const void *src, uint64_t bytes);
 int mfrt_memset(void *dst, int value, uint64_t bytes);
 int mfrt_memcpy_async(void *dst, const void *src, uint64_t bytes, void *stream);
-
-/* ---- address registry view (HybmVaManager counterpart,
- *      src/hybm/csrc/mm/hybm_va_manager.h:175-264) -------------------------- */
-void mf_va_clear(void);
-int32_t mf_va_add(uint64_t gva, uint64_t size, int32_t memType, uint64_t lva, uint32_t localRank);
-int32_t mf_va_add_external(uint64_t gva, uint64_t size, int32_t memType, uint64_t lva, uint32_t localRank,
-                           uint32_t importedRank);
-void mf_va_remove(uint64_t va);
-uint64_t mf_va_gva_of_lva(uint64_t lva);
-uint64_t mf_va_lva_of_gva(uint64_t gva);
-int32_t mf_va_is_gva(uint64_t va);
-int32_t mf_va_is_known(uint64_t va);
-int32_t mf_va_mem_type(uint64_t va);
-int64_t mf_va_rank(uint64_t gva);                    /* -1 when not found */
-int32_t mf_va_infer_direction(uint64_t srcVa, uint64_t dstVa);
-uint64_t mf_va_reserve(uint32_t localRank, uint64_t size, int32_t memType);
-void mf_va_unreserve(uint64_t start);
-uint64_t mf_va_range_count(void);
-uint64_t mf_va_reserved_count(void);
-
-/* ---- direction algebra and window arithmetic views ------------------------ */
-int32_t mf_dir_compose(int32_t srcPool, int32_t srcDevice, int32_t dstPool, int32_t dstDevice);
-int32_t mf_dir_translate_smem(int32_t copyType, int32_t srcPoolType, int32_t dstPoolType);
-int32_t mf_dir_checks(int32_t direction);            /* bit 0: source checked, bit 1: destination checked */
-int32_t mf_gva_contains(uint64_t base, uint64_t stride, uint64_t rankCount, uint64_t addr, uint64_t size);
-uint32_t mf_gva_rank(uint64_t base, uint64_t stride, uint64_t rankCount, uint64_t rankSpace, uint64_t addr);
-uint64_t mf_gva_mask48(uint64_t addr);
-
-/* ---- transfer front-end arithmetic views ----------------------------------
- * mf_trans_combine: union of n (start, size) pairs (pairs[2*n]) into sorted, disjoint runs
- * written to out[2*k..] (room for n pairs); returns k.  mf_trans_translate: look one peer range
- * up in n runs {start, size, mapped} (slices[3*n]); the mapped address or 0 when the range is not
- * inside one run.  mf_trans_parse_name: 1 when the name is a valid "ip:port" / "[ipv6]:port" and,
- * then, its 20-byte binary form in key. */
-uint32_t mf_trans_combine(const uint64_t *pairs, uint32_t n, uint64_t *out);
-uint64_t mf_trans_translate(const uint64_t *slices, uint32_t n, uint64_t remote, uint64_t size);
-int32_t mf_trans_parse_name(const char *name, uint8_t *key);
 
 #ifdef __cplusplus
 }

@@ -4,7 +4,7 @@
 // one segment per row and takes the ordinary batch path.
 #include <vector>
 
-#include "../../../include/mf_hip_dataplane.h"
+#include "../../../include/mf_hip_dataplane_internal.h"
 #include "../../../include/mf_xcopy_types.h"
 #include "../kernels/copy2d_plan.h"
 #include "../rt/mf_rt.h"

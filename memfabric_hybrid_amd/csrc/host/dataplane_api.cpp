@@ -1,4 +1,4 @@
-// Native C entry points declared in include/mf_hip_dataplane.h.
+// Native C entry points declared in include/mf_hip_dataplane.h and include/mf_hip_dataplane_internal.h.
 #include <atomic>
 #include <chrono>
 #include <cstring>
@@ -7,7 +7,7 @@
 
 #include <sched.h>
 
-#include "../../../include/mf_hip_dataplane.h"
+#include "../../../include/mf_hip_dataplane_internal.h"
 #include "../../../include/mf_xcopy_types.h"
 #include "copy_direction.h"
 #include "../rt/mf_rt.h"
@@ -153,6 +153,22 @@ MF_EXPORT int32_t mf_xcopy_tune(uint32_t units, uint32_t wgPerCu, uint32_t wgPer
     t.unitsOverride = units;
     t.wgPerCu = wgPerCu;                               // 0: no cap, one workgroup per chunk
     t.wgPerCuLink = wgPerCuLink == 0 ? 1 : wgPerCuLink;
+    return BM_OK;
+}
+
+MF_EXPORT int32_t mf_xcopy_tune_table(uint32_t stageUnordered, uint32_t deviceTableWgPerCu)
+{
+    XcopyTuning &t = XcopyEngine::Instance().Tuning();
+    t.stageUnordered = stageUnordered != 0;
+    t.deviceTableWgPerCu = deviceTableWgPerCu;
+    return BM_OK;
+}
+
+MF_EXPORT int32_t mf_xcopy_tune_hold(uint32_t deepHold, int32_t pinnedExtraNanos)
+{
+    XcopyTuning &t = XcopyEngine::Instance().Tuning();
+    t.deepHold = deepHold != 0;
+    t.holdPinnedExtraNanos = pinnedExtraNanos;
     return BM_OK;
 }
 

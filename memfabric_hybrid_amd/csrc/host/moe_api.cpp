@@ -1,6 +1,6 @@
 // Native C entry points of the local MoE dispatch / combine (declared in
 // include/mf_hip_dataplane.h).
-#include "../../../include/mf_hip_dataplane.h"
+#include "../../../include/mf_hip_dataplane_internal.h"
 #include "../../../include/mf_xcopy_types.h"
 #include "../rt/mf_rt.h"
 #include "mf_log.h"

@@ -1,5 +1,6 @@
 #include "xcopy_engine.h"
 
+#include <algorithm>
 #include <atomic>
 #include <chrono>
 #include <cstring>
@@ -356,6 +357,21 @@ uint32_t GridFor(uint64_t nchunk, uint32_t cuCount, int route, const XcopyTuning
     }
     uint64_t grid = nchunk < cap ? nchunk : cap;
     return grid == 0 ? 1u : static_cast<uint32_t>(grid);
+}
+
+// Grid of a table launch whose chunk count only the GPU knows: workgroups walk the chunks with the grid as their
+// stride, surplus workgroups leave at once.  Eight workgroups per segment (pages of 32 KiB have eight chunks)
+// between 32 and 4096 per CU: measured on 262 144 pages of 32 KiB, 256 / 512 / 1024 / 2048 / 4096 per CU take
+// 3.27 / 3.21 / 3.15 / 3.09 / 3.06 ms (one workgroup per chunk, which needs the count: 3.05 ms), while on 4096 pages
+// 512 per CU cost 14 us in workgroups that find nothing to do (69 against 55 us).
+uint32_t DeviceTableGrid(uint32_t nseg, uint32_t cuCount, int route, const XcopyTuning &tuning)
+{
+    const uint64_t cus = cuCount == 0 ? 256 : cuCount;
+    uint64_t want = tuning.deviceTableWgPerCu != 0 ? cus * tuning.deviceTableWgPerCu : 8ull * nseg;
+    if (tuning.deviceTableWgPerCu == 0) {
+        want = want < 32 * cus ? 32 * cus : (want > 4096 * cus ? 4096 * cus : want);
+    }
+    return GridFor(want, cuCount, route, tuning);
 }
 
 }  // namespace
@@ -776,11 +792,39 @@ uint32_t XcopyEngine::HoldFor(const InlinePlan &plan, uint32_t grid, int route, 
     // With launches of another thread's stream on the chip at the same time not every wave of a large launch is
     // resident at once, and the wait costs instead of gaining (two submitting threads, 24 MiB copies: 8.2 us per
     // copy without, 9.0 us with; 21 MB batches 7.9 / 8.2 us; 16 MB and below: the same or better with the wait).
-    if (plan.nchunk > kHoldSharedMaxChunks && g_leasesOut.load(std::memory_order_relaxed) > 1) {
+    if ((plan.nchunk > kHoldSharedMaxChunks || plan.units == kDeepUnits) && g_leasesOut.load(std::memory_order_relaxed) > 1) {
         return 0;
     }
-    const uint32_t rule = HoldNanosFor(plan.nchunk, grid, plan.units, plan.first[1] == kNoChunk);
+    const uint32_t rule = HoldNanosFor(plan.nchunk, grid, plan.units, plan.first[1] == kNoChunk && plan.units != kDeepUnits);
     return rule != 0 && tuning_.holdNanos > 0 ? static_cast<uint32_t>(tuning_.holdNanos) : rule;
+}
+
+// Hold of a table launch under a pattern: its waves fetch their descriptors across the host link and issue their
+// loads that much later than those of a launch whose descriptors are kernel arguments.
+uint32_t XcopyEngine::HoldForTable(uint32_t nchunk, uint32_t grid, uint32_t units, int route, bool unordered) const
+{
+    if (route != MFRT_ROUTE_HBM || unordered || tuning_.holdNanos == 0) {
+        return 0;
+    }
+    if ((nchunk > kHoldSharedMaxChunks || units == kDeepUnits) && g_leasesOut.load(std::memory_order_relaxed) > 1) {
+        return 0;
+    }
+    const uint32_t rule = HoldNanosFor(nchunk, grid, units, false);
+    if (rule == 0) {
+        return 0;
+    }
+    if (tuning_.holdNanos > 0) {
+        return static_cast<uint32_t>(tuning_.holdNanos);
+    }
+    const int64_t with = static_cast<int64_t>(rule) + tuning_.holdPinnedExtraNanos;
+    return with > 0 ? static_cast<uint32_t>(with) : 0;
+}
+
+bool XcopyEngine::DeepHoldApplies(uint64_t bytes, uint32_t n, int route, bool unordered) const
+{
+    return route == MFRT_ROUTE_HBM && !unordered && tuning_.holdNanos != 0 && tuning_.unitsOverride == 0 && tuning_.deepHold &&
+           bytes > kDeepMinBytes && bytes <= kDeepMaxBytes && n != 0 && bytes / n >= kDeepMinSegmentBytes &&
+           g_leasesOut.load(std::memory_order_relaxed) <= 1;
 }
 
 bool XcopyEngine::WindowsApply(uint64_t bytes, int route) const
@@ -798,6 +842,15 @@ bool XcopyEngine::SingleSubmitter() const
 
 int XcopyEngine::Submit(const uint64_t *src, const uint64_t *dst, const uint64_t *len, uint32_t n, int route,
                         void *stream, void *mask, uint32_t maskValue, bool unordered)
+{
+    return SubmitOne(src, dst, len, n, route, stream, mask, maskValue, unordered, true);
+}
+
+// maySlice: a table of long segments may be cut into launches of kInlineSegs segments; a slice is submitted
+// with false, so that one that cannot take the kernel-argument form (a segment of 4 GiB and more is cut into
+// pieces, which can carry it past kInlineSegs rows) goes to the table form instead of being sliced again.
+int XcopyEngine::SubmitOne(const uint64_t *src, const uint64_t *dst, const uint64_t *len, uint32_t n, int route,
+                           void *stream, void *mask, uint32_t maskValue, bool unordered, bool maySlice)
 {
     if (!Started()) {
         MF_FAIL(BM_NOT_INITIALIZED, "xcopy engine not started");
@@ -832,7 +885,11 @@ int XcopyEngine::Submit(const uint64_t *src, const uint64_t *dst, const uint64_t
         if (windowed) {
             units = mfk_xcopy_window_units();
         }
-        inlined = BuildInlineDirect(src, dst, len, n, units, plan);
+        const bool deep = !windowed && DeepHoldApplies(total, n, route, unordered);
+        inlined = BuildInlineDirect(src, dst, len, n, deep ? kDeepUnits : units, plan);
+        if (inlined && deep && HoldNanosFor(plan.nchunk, plan.nchunk, kDeepUnits, false) == 0) {
+            inlined = BuildInlineDirect(src, dst, len, n, units, plan);   // ragged enough to exceed the waves that hold: the usual chunks
+        }
     }
     if (!inlined && oversized) {
         // a run of 4 GiB and more may have made the one-pass attempt give up: the general inline path cuts it into pieces
@@ -864,6 +921,7 @@ int XcopyEngine::Submit(const uint64_t *src, const uint64_t *dst, const uint64_t
 
     // Table form: {triples, prefix} are built in a pinned slot; the general form moves them to HBM
     // with a copy launch and searches them there.  The slot is sized for n segments; merging can only make the table shorter.
+    bool deepTable = false;
     {
         uint64_t total = 0;
         uint64_t longest = 0;
@@ -878,12 +936,14 @@ int XcopyEngine::Submit(const uint64_t *src, const uint64_t *dst, const uint64_t
         // itself was measured under windows and is left without them: its chunk search lowers the rate it
         // sustains (6.56 TB/s at a target of 6.6, erratic at 6.8), and 262 144 pages of 32 KiB at random
         // places lose (5.1 against 5.4 TB/s).
-        if (route == MFRT_ROUTE_HBM && !unordered && tuning_.windowMBps != 0 && tuning_.unitsOverride == 0 &&
-            total / n >= kWindowSliceMinSegmentBytes && g_leasesOut.load(std::memory_order_relaxed) <= 1) {
+        if (maySlice && n > kInlineSegs && route == MFRT_ROUTE_HBM && !unordered && tuning_.windowMBps != 0 &&
+            tuning_.unitsOverride == 0 && total / n >= kWindowSliceMinSegmentBytes &&
+            g_leasesOut.load(std::memory_order_relaxed) <= 1) {
             for (uint32_t at = 0; at < n; at += kInlineSegs) {
                 const uint32_t m = n - at < kInlineSegs ? n - at : kInlineSegs;
                 const bool last = at + m == n;
-                const int ret = Submit(src + at, dst + at, len + at, m, route, stream, last ? mask : nullptr, maskValue, false);
+                const int ret = SubmitOne(src + at, dst + at, len + at, m, route, stream, last ? mask : nullptr, maskValue, false,
+                                          false);
                 if (ret != BM_OK) {
                     return ret;
                 }
@@ -891,10 +951,11 @@ int XcopyEngine::Submit(const uint64_t *src, const uint64_t *dst, const uint64_t
             return BM_OK;
         }
         units = ChooseUnits(total, cu, route, tuning_);
+        deepTable = DeepHoldApplies(total, n, route, unordered);
         // Many short segments: a chunk size that holds the longest of them gives every segment exactly
         // one chunk, which is the equal-count form below (no prefix, no search, no upload): 16 384
         // segments of 2-14 KB take 62 us instead of 74 us.
-        if (tuning_.unitsOverride == 0 && longest != 0) {
+        if (tuning_.unitsOverride == 0 && longest != 0 && !deepTable) {
             for (uint32_t u = units; u <= 4 * kXcopyThreads; u *= 2) {
                 if (longest <= static_cast<uint64_t>(u) * kUnitBytes - kUnitBytes) {
                     units = u;
@@ -903,11 +964,17 @@ int XcopyEngine::Submit(const uint64_t *src, const uint64_t *dst, const uint64_t
             }
         }
     }
+    // Slot layout: triples | prefix | group map.  The map's size follows from the chunk count, which is bounded
+    // here by one chunk per segment plus one per full chunk of payload.
     const uint64_t tripleBytes = 24ull * n;
-    const uint64_t tableBytes = RoundUp(tripleBytes + 4ull * (n + 1), kUnitBytes);
+    const uint64_t prefixBytes = RoundUp(4ull * (n + 1), 8);
+    const uint64_t chunkBound = static_cast<uint64_t>(n) + queuedBytes / (static_cast<uint64_t>(units) * kUnitBytes);
+    const uint32_t groupCapacity = static_cast<uint32_t>(
+        std::min<uint64_t>(GroupCapacityFor(n), (chunkBound >> kGroupShiftMin) + 2));
+    const uint64_t slotBytes = RoundUp(tripleBytes + prefixBytes + 4ull * groupCapacity, kUnitBytes);
     StagingSlot *slot = nullptr;
     ThreadLease &lease = ctx.Lease();
-    int ret = AcquireSlot(lease, tableBytes, stream, slot);
+    int ret = AcquireSlot(lease, slotBytes, stream, slot);
     if (ret != BM_OK) {
         return ret;
     }
@@ -915,7 +982,18 @@ int XcopyEngine::Submit(const uint64_t *src, const uint64_t *dst, const uint64_t
     uint32_t *first = reinterpret_cast<uint32_t *>(static_cast<uint8_t *>(slot->host) + tripleBytes);
     uint32_t count = 0;
     ChunkPattern pattern;
-    const uint64_t nchunk = BuildTableDirect(src, dst, len, n, units, triples, first, count, &pattern);
+    uint64_t nchunk = 0;
+    if (deepTable) {
+        nchunk = BuildTableDirect(src, dst, len, n, kDeepUnits, triples, first, count, &pattern);
+        if (HoldNanosFor(static_cast<uint32_t>(nchunk < kNoChunk ? nchunk : 0), static_cast<uint32_t>(nchunk), kDeepUnits, false) != 0) {
+            units = kDeepUnits;
+        } else {
+            deepTable = false;   // ragged enough to exceed the waves that hold: the usual chunks
+        }
+    }
+    if (!deepTable) {
+        nchunk = BuildTableDirect(src, dst, len, n, units, triples, first, count, &pattern);
+    }
     if (nchunk >= kNoChunk) {
         MF_FAIL(BM_INVALID_PARAM, "batch too large for one launch: " << nchunk << " chunks");
     }
@@ -928,38 +1006,55 @@ int XcopyEngine::Submit(const uint64_t *src, const uint64_t *dst, const uint64_t
     }
 
     const uint32_t grid = GridFor(nchunk, cu, route, tuning_);
+    TablePlan table{};
+    table.nseg = count;
+    table.nchunk = static_cast<uint32_t>(nchunk);
+    table.units = units;
     int err = 0;
+    // Chunk counts that repeat (pages of one size, K and V blocks in turn): a workgroup finds its descriptor by
+    // a division and a few comparisons, so the only thing it needs from the table is that one descriptor, which it
+    // can read straight out of the pinned slot.  No upload launch, nothing serial in front of the copy (a 4096-page
+    // gather on an idle stream: 50 us instead of 55); the 64 bytes per workgroup that cross the host link stay
+    // below 2 % of the payload rate.  (Uploading the table by a launch of its own that carries no barrier, so that
+    // it runs beside the caller's earlier copies, was measured for these batches too: the extra launch costs the
+    // stream 2 us whether it overlaps or not, more than the fetch from HBM saves: 36 MB of K and V blocks 20.5
+    // against 18.4 us per call.)
     if (pattern.period != 0) {
-        // Chunk counts that repeat (pages of one size, K and V blocks in turn): a workgroup finds its
-        // descriptor by a division and a few comparisons, so the only
-        // thing it needs from the table is that one descriptor, and it reads it straight out of
-        // the pinned slot.  No upload launch, nothing serial in front of the copy: a 4096-page gather
-        // takes 50 us instead of 55, the 64 bytes per workgroup that cross the host link stay below
-        // 2 % of the payload rate.  (With the chunk prefix in host memory as well the search of the
-        // general form pays a link round trip per level: 16 384 ragged segments 135 us against 74.)
-        err = mfk_xcopy_table(slot->host, nullptr, nullptr, count, static_cast<uint32_t>(nchunk), units, &pattern, route,
-                              grid, mask, maskValue, stream);
+        const uint32_t hold = HoldForTable(static_cast<uint32_t>(nchunk), grid, units, route, unordered);
+        table.triples = triples;
+        table.pattern = pattern;
+        err = mfk_xcopy_table(&table, route, grid, mask, maskValue, stream, hold);
         g_launches.fetch_add(1, std::memory_order_relaxed);
     } else {
-        ret = EnsureDevice(*slot, tableBytes);
+        // Ragged segments: prefix and group map go to HBM with the triples (with them in host memory every
+        // step of the lookup is a link round trip: 16 384 ragged segments 135 us against 74).  The upload is
+        // launched without a barrier: the slot's device half is free (AcquireSlot has waited for its last
+        // reader), so it may run while the caller's earlier copies still do; the table launch behind it waits
+        // for both.
+        uint32_t *group = reinterpret_cast<uint32_t *>(static_cast<uint8_t *>(slot->host) + tripleBytes + prefixBytes);
+        table.groupShift = BuildGroupMap(first, count, group, groupCapacity);
+        const uint64_t usedBytes =
+            RoundUp(tripleBytes + prefixBytes + 4ull * (GroupCount(nchunk, table.groupShift) + 1), kUnitBytes);
+        ret = EnsureDevice(*slot, slotBytes);
         if (ret != BM_OK) {
             return ret;
         }
         const uint64_t hostAddr = reinterpret_cast<uint64_t>(slot->host);
         const uint64_t devAddr = reinterpret_cast<uint64_t>(slot->dev);
         InlinePlan stagePlan;
-        if (!BuildInlineDirect(&hostAddr, &devAddr, &tableBytes, 1, kXcopyThreads, stagePlan)) {
-            MF_FAIL(BM_INVALID_PARAM, "descriptor table of " << tableBytes << " bytes is too large");
+        if (!BuildInlineDirect(&hostAddr, &devAddr, &usedBytes, 1, kXcopyThreads, stagePlan)) {
+            MF_FAIL(BM_INVALID_PARAM, "descriptor table of " << usedBytes << " bytes is too large");
         }
-        // (Uploading on a stream of its own, with the copy stream waiting for an event, was measured: the
-        // two extra queue operations cost what the overlap gains, 56 us per 4096-page gather either way.)
-        err = mfk_xcopy_inline(&stagePlan, MFRT_ROUTE_FROM_HOST, stagePlan.nchunk, nullptr, 0, stream, 0, 0);
+        err = mfk_xcopy_inline(&stagePlan, MFRT_ROUTE_FROM_HOST, stagePlan.nchunk, nullptr, 0, stream,
+                               tuning_.stageUnordered ? 1 : 0, 0);
         if (err != 0) {
             MF_FAIL(BM_ERROR, "descriptor staging launch failed: " << mfrt_error_string(err));
         }
         const uint8_t *devBase = static_cast<const uint8_t *>(slot->dev);
-        err = mfk_xcopy_table(devBase, devBase + tripleBytes, nullptr, count, static_cast<uint32_t>(nchunk), units, nullptr, route,
-                              grid, mask, maskValue, stream);
+        table.triples = reinterpret_cast<const uint64_t *>(devBase);
+        table.first = reinterpret_cast<const uint32_t *>(devBase + tripleBytes);
+        table.group = reinterpret_cast<const uint32_t *>(devBase + tripleBytes + prefixBytes);
+        err = mfk_xcopy_table(&table, route, grid, mask, maskValue, stream, 0);
         g_launches.fetch_add(2, std::memory_order_relaxed);
     }
     if (err != 0) {
@@ -993,28 +1088,28 @@ int XcopyEngine::SubmitDeviceTable(const void *triples, uint32_t n, int route, v
         int err = mfk_xcopy_inline(&empty, route, 1, mask, maskValue, stream, 0, 0);
         return err == 0 ? BM_OK : BM_ERROR;
     }
-    // The prefix is computed on the GPU; its slot is only ever touched by kernels of this stream.
+    // Prefix, group map and pattern are computed on the GPU; their slot is only ever touched by kernels of this stream.
     ThreadCtx &ctx = t_ctx;
     StagingSlot *slot = nullptr;
-    const uint64_t prefixBytes = RoundUp(4ull * (n + 2), kUnitBytes);
+    const uint32_t groupCapacity = GroupCapacityFor(n);
+    const uint64_t scratchBytes = RoundUp(4ull * mfk_xcopy_plan_scratch_words(n, groupCapacity), kUnitBytes);
     ThreadLease &lease = ctx.Lease();
     int ret = AcquireSlot(lease, 0, stream, slot);
     if (ret == BM_OK) {
-        ret = EnsureDevice(*slot, prefixBytes);
+        ret = EnsureDevice(*slot, scratchBytes);
     }
     if (ret != BM_OK) {
         return ret;
     }
-    const uint32_t units = ChooseUnits(0, mfrt_cu_count(), route, tuning_);   // sizes are only known on the GPU
-    uint32_t *first = static_cast<uint32_t *>(slot->dev);
-    uint32_t *nchunkDev = first + n + 1;
-    int err = mfk_xcopy_plan(triples, n, units, first, nchunkDev, stream);
+    const uint32_t cu = mfrt_cu_count();
+    const uint32_t units = ChooseUnits(0, cu, route, tuning_);   // sizes are only known on the GPU
+    TablePlan table;
+    int err = mfk_xcopy_plan(triples, n, units, slot->dev, groupCapacity, &table, stream);
     if (err != 0) {
         MF_FAIL(BM_ERROR, "xcopy plan launch failed: " << mfrt_error_string(err));
     }
-    const uint32_t cu = mfrt_cu_count();
-    const uint32_t grid = GridFor(static_cast<uint64_t>(cu == 0 ? 256 : cu) * 256, cu, route, tuning_);   // chunk count is only known on the GPU; surplus workgroups leave at once
-    err = mfk_xcopy_table(triples, first, nchunkDev, n, 0, units, nullptr, route, grid, mask, maskValue, stream);
+    const uint32_t grid = DeviceTableGrid(n, cu, route, tuning_);
+    err = mfk_xcopy_table(&table, route, grid, mask, maskValue, stream, 0);
     if (err != 0) {
         (void)MarkQueued(lease, slot, stream, true);   // the plan launch writes the slot
         MF_FAIL(BM_ERROR, "xcopy table launch failed: " << mfrt_error_string(err));
@@ -1042,7 +1137,7 @@ int XcopyEngine::SubmitDeviceTableStatic(const void *triples, uint32_t n, int ro
     }
     const uint32_t cu = mfrt_cu_count();
     const uint32_t units = ChooseUnits(0, cu, route, tuning_);   // sizes are only known on the GPU
-    const uint32_t grid = GridFor(static_cast<uint64_t>(cu == 0 ? 256 : cu) * 256, cu, route, tuning_);   // surplus workgroups leave at once
+    const uint32_t grid = DeviceTableGrid(n, cu, route, tuning_);
     const int err = mfk_xcopy_table_static(triples, n, units, route, grid, stream);
     if (err != 0) {
         MF_FAIL(BM_ERROR, "static-scratch table launch failed (" << err << ")");

@@ -47,6 +47,10 @@ struct XcopyTuning {
     uint32_t wgPerCuLink = 1;    // routes bound by the host link: workgroups per CU
     uint32_t minUnits = kXcopyThreads;   // 4 KiB: the chunk of HBM routes
     int32_t holdNanos = -1;      // stores held back in inline launches: -1 = HoldNanosFor's rule, 0 = never, else that long
+    bool deepHold = true;        // batches of 24 to 64 MiB hold the stores of 16 KiB per wave
+    int32_t holdPinnedExtraNanos = 1600;   // added to the rule for table launches, whose descriptors come from pinned host memory: a link round trip before the loads
+    bool stageUnordered = true;  // the upload of a ragged table's descriptors is launched without a barrier
+    uint32_t deviceTableWgPerCu = 0;   // grid of a device-resident table in workgroups per CU, 0 = eight per segment between 32 and 4096 per CU
     uint32_t windowMBps = 6800000;   // HBM copies of kWindowMinBytes and more alternate between read and write windows cut for this rate; 0 = never
 };
 
@@ -137,6 +141,11 @@ private:
     XcopyEngine() = default;
 
     uint32_t HoldFor(const InlinePlan &plan, uint32_t grid, int route, bool unordered) const;
+    uint32_t HoldForTable(uint32_t nchunk, uint32_t grid, uint32_t units, int route, bool unordered) const;
+    // Whether a batch of `bytes` in n segments is planned in chunks of kDeepUnits units, to hold the stores of 16 KiB per wave.
+    bool DeepHoldApplies(uint64_t bytes, uint32_t n, int route, bool unordered) const;
+    int SubmitOne(const uint64_t *src, const uint64_t *dst, const uint64_t *len, uint32_t n, int route, void *stream,
+                  void *mask, uint32_t maskValue, bool unordered, bool maySlice);
 
     XcopyTuning tuning_;
     std::atomic<bool> started_{false};   // read by every calling thread, flipped by Start / Stop

@@ -168,11 +168,18 @@ __device__ __forceinline__ uint64_t ReadLane64(uint64_t v, uint32_t lane)
 //
 // kHold: every wave keeps its loaded data until `holdTicks` of the constant-rate clock after its own
 // start, which separates the read burst of the launch from its write burst (HoldNanosFor has the
-// measurements); such a launch has one chunk per workgroup.
-template <bool kNtLoad, int kStore, bool kHold = false>
+// rule); such a launch has one chunk per workgroup: of 4 KiB (kHoldShallow, four loads per lane) or, for
+// batches whose 4 KiB chunks would outnumber the waves the chip holds at once, of 16 KiB (kHoldDeep).
+enum HoldMode : int { kHoldNone = 0, kHoldShallow = 1, kHoldDeep = 2 };
+
+template <bool kNtLoad, int kStore, int kHold>
+__device__ __forceinline__ void CopyChunkHeld(uint64_t src, uint64_t dst, uint64_t len, uint64_t k, uint32_t units, uint64_t t0,
+                                              uint32_t ticks);
+
+template <bool kNtLoad, int kStore, int kHold = kHoldNone>
 __global__ __launch_bounds__(kXcopyThreads) void XcopyInlineKernel(const InlinePlan p, uint32_t holdTicks)
 {
-    const uint64_t t0 = kHold ? wall_clock64() : 0;
+    const uint64_t t0 = kHold != kHoldNone ? wall_clock64() : 0;
     const uint32_t lane = threadIdx.x & 63u;
     const uint32_t f0 = p.first[lane];
     const uint32_t f1 = p.first[lane + 64];
@@ -207,33 +214,21 @@ __global__ __launch_bounds__(kXcopyThreads) void XcopyInlineKernel(const InlineP
             len = __builtin_amdgcn_readlane(l1, row);
             first = __builtin_amdgcn_readlane(f1, row);
         }
-        CopyChunk<kNtLoad, kStore, kHold>(src, dst, len, c - first, units, t0, holdTicks);
+        CopyChunkHeld<kNtLoad, kStore, kHold>(src, dst, len, c - first, units, t0, holdTicks);
         c += gridDim.x;
     } while (c < nchunk);
 }
 
 // Read and write windows.  A copy that runs for hundreds of microseconds streams faster when the whole chip
 // alternates between reading and writing than when every wave stores as soon as its loads have landed:
-// HBM then sees long bursts of one direction instead of a mix.  The waves need no communication for
-// that, only the constant-rate clock every wave can read: a period is cut into a read half and a write
-// half, wave i of a launch of G waves issues the 16 loads per lane of its next 16 KiB chunk at
-// offset i * (period / 2) / G into the read half, waits for them, and issues the stores at the same
-// offset into the write half.  The period is the time the launch's 2 * G * 16 KiB per round need at a
-// target rate; up to a target the part sustains, the copy simply runs at the pace the clock sets.
-// Measured with a stand-alone kernel of this shape on 1 and 2 GiB (4096 waves: 64 MiB read and 64 MiB
-// written per 18 to 20 us period): target 6.6 / 6.8 / 7.0 / 7.2 / 7.4 TB/s -> 6.39 / 6.59 / 6.7 / 6.97 / 7.15 TB/s
-// achieved, against 6.1-6.2 TB/s for one wave per 4 KiB chunk that stores at once; at 7.6 TB/s the waves no
-// longer keep up, the windows dissolve and the copy falls back to 5.8-6.1 TB/s.  This kernel, which also
-// looks its chunk up in the plan, through smem_bm_copy_batch on a pool, target 6.8 against no windows:
-// 512 MiB 6.65 / 6.34 TB/s, 1 GiB 6.73 / 6.23, 2 GiB 6.6-6.7 / 6.12, 100 segments of about 10 MB at odd addresses
-// 6.28 / 5.84, 3 x 700 MB at odd addresses 6.05 / 5.73; at 6.6 it measures 6.47 / 6.54 / 6.57 / 6.09 / 6.1-6.2, at
-// 7.0 the 2 GiB copy dissolves now and then (6.2-6.3), at 7.2 and above most launches do.  256 MiB gains nothing
-// (the first and the last half period, in which the chip only reads or only writes, cost what the windows
-// gain), 128 MiB loses.  Memory that has never been written copies erratically under windows (6.0 to 6.8 TB/s
-// from one launch to the next); initialised memory does not.  2048 waves dissolve one step earlier than 4096;
-// 4, 8 or 32 loads per lane and windows that are not spread over their half were slower or less stable.  A wave
-// that is late proceeds at once: letting it skip to its slot in a later period made a dissolved launch slower
-// (4.4 instead of 5.7 TB/s).
+// HBM then sees long bursts of one direction instead of a mix (6.7 against 6.2 TB/s on 1 to 2 GiB).  The
+// waves need no communication for that beyond the start, only the constant-rate clock every wave can read:
+// a period is cut into a read half and a write half, wave i of a launch of G waves issues the 16 loads per
+// lane of its next 16 KiB chunk at offset i * (period / 2) / G into the read half, waits for them, and
+// issues the stores at the same offset into the write half.  The period is the time the launch's
+// 2 * G * 16 KiB per round need at a target rate; up to a rate the part sustains, the copy runs at the pace
+// the clock sets, beyond it the windows dissolve and the copy runs as it does without them.  A wave that
+// is late proceeds at once (skipping to a later period made a dissolved launch slower).
 constexpr uint32_t kWindowDepth = 16;                       // 128-bit loads per lane and round
 constexpr uint32_t kWindowUnits = 64 * kWindowDepth;        // 16 KiB chunks, one wave each
 constexpr uint32_t kWindowWaves = 4096;                     // 16 per CU
@@ -265,6 +260,59 @@ __device__ __forceinline__ void CopyChunkWindowed(uint64_t src, uint64_t dst, ui
 #pragma unroll
     for (uint32_t j = 0; j < kWindowDepth; ++j) {
         StoreUnit<kStore>(d + j * 64 * kUnitBytes, v[j]);
+    }
+}
+
+// One chunk under a hold mode.  kHoldDeep: a chunk of up to kWindowUnits units is read by a single wave with up to
+// 16 loads per lane in flight and stored when the wave's hold is over; units past the end of the segment's
+// body are skipped lane by lane, head and tail bytes travel as in CopyChunk.
+template <bool kNtLoad, int kStore, int kHold>
+__device__ __forceinline__ void CopyChunkHeld(uint64_t src, uint64_t dst, uint64_t len, uint64_t k, uint32_t units, uint64_t t0,
+                                              uint32_t ticks)
+{
+    if (kHold != kHoldDeep) {
+        CopyChunk<kNtLoad, kStore, kHold == kHoldShallow>(src, dst, len, k, units, t0, ticks);
+        return;
+    }
+    const SegGeom g = SegmentGeometry(dst, len);
+    const uint64_t u0 = k * kWindowUnits;
+    const uint64_t left = g.body > u0 ? g.body - u0 : 0;
+    const uint32_t n = left < kWindowUnits ? static_cast<uint32_t>(left) : kWindowUnits;
+    const uint32_t tid = threadIdx.x;                       // 64 lanes
+    const uint64_t s = src + g.head + u0 * kUnitBytes + tid * kUnitBytes;
+    const uint64_t d = dst + g.head + u0 * kUnitBytes + tid * kUnitBytes;
+    u32x4 v[kWindowDepth];
+    if (n == kWindowUnits) {    // the common case without a test per load: the sixteen loads leave back to back
+#pragma unroll
+        for (uint32_t j = 0; j < kWindowDepth; ++j) {
+            v[j] = LoadUnit<kNtLoad>(s + j * 64 * kUnitBytes);
+        }
+        HoldStores(t0, ticks);
+#pragma unroll
+        for (uint32_t j = 0; j < kWindowDepth; ++j) {
+            StoreUnit<kStore>(d + j * 64 * kUnitBytes, v[j]);
+        }
+    } else {
+#pragma unroll
+        for (uint32_t j = 0; j < kWindowDepth; ++j) {
+            if (j * 64 + tid < n) {
+                v[j] = LoadUnit<kNtLoad>(s + j * 64 * kUnitBytes);
+            }
+        }
+        HoldStores(t0, ticks);
+#pragma unroll
+        for (uint32_t j = 0; j < kWindowDepth; ++j) {
+            if (j * 64 + tid < n) {
+                StoreUnit<kStore>(d + j * 64 * kUnitBytes, v[j]);
+            }
+        }
+    }
+    if (k == 0 && tid < g.head) {
+        CopyByte(src + tid, dst + tid);
+    }
+    if (u0 + kWindowUnits >= g.body && tid < g.tail) {
+        const uint64_t off = g.head + g.body * kUnitBytes + tid;
+        CopyByte(src + off, dst + off);
     }
 }
 
@@ -309,20 +357,19 @@ __global__ __launch_bounds__(64) void XcopyWindowKernel(const InlinePlan p, uint
     }
 }
 
-// A single segment needs no table: its three words travel as plain kernel arguments (28 bytes
-// instead of the 3080-byte plan), which is cheaper for the host to hand over and spares every
-// wave the table fetch.  Measured against the table form on one box: an 8 MiB copy 13.7 us instead
-// of 15.4 us per blocking call, back-to-back 32 MiB copies 10.8 us instead of 11.5 us each; from
-// about 200 MiB on the table form is 1 % faster (512 MiB: 166.4 us against 168.8 us), hence the limit.
+// A single segment needs no table: its three words travel as plain kernel arguments (28 bytes instead of
+// the 3080-byte plan), which is cheaper for the host to hand over and spares every wave the table fetch
+// (an 8 MiB copy: 13.7 instead of 15.4 us per blocking call).  From about 200 MiB on the table form is
+// 1 % faster, hence the limit.
 constexpr uint32_t kSingleMaxChunks = 49152;
-template <bool kNtLoad, int kStore, bool kHold = false>
+template <bool kNtLoad, int kStore, int kHold = kHoldNone>
 __global__ __launch_bounds__(kXcopyThreads) void XcopySingleKernel(uint64_t src, uint64_t dst, uint32_t len, uint32_t nchunk,
                                                                    uint32_t units, uint32_t holdTicks)
 {
-    const uint64_t t0 = kHold ? wall_clock64() : 0;
+    const uint64_t t0 = kHold != kHoldNone ? wall_clock64() : 0;
     uint32_t c = blockIdx.x;
     do {
-        CopyChunk<kNtLoad, kStore, kHold>(src, dst, len, c, units, t0, holdTicks);
+        CopyChunkHeld<kNtLoad, kStore, kHold>(src, dst, len, c, units, t0, holdTicks);
         c += gridDim.x;
     } while (c < nchunk);
 }
@@ -340,80 +387,417 @@ __global__ void XcopySignalKernel(uint64_t *mask, uint32_t maskValue)
     }
 }
 
-template <bool kNtLoad, int kStore>
-__global__ __launch_bounds__(kXcopyThreads) void XcopyTableKernel(const uint64_t *__restrict__ triples,
-                                                                  const uint32_t *__restrict__ first,
-                                                                  const uint32_t *__restrict__ nchunkDev, uint32_t nseg,
-                                                                  uint32_t nchunkHost, uint32_t units, const ChunkPattern pattern)
+// The table form: any number of segments, {src, dst, len} triples in memory.  A wave finds the owner of its
+// chunk either by a division (chunk counts that repeat: pages of one size, K and V blocks in turn) or
+// through the group map: two map entries bound the owner to a short range of segments, whose prefix
+// entries AND triples the lanes then fetch side by side, one segment per lane, so that the descriptor is
+// in registers two dependent loads after the wave started, whatever the size of the table.  (The form
+// this replaces searched the whole prefix 64 ways per round: three rounds for 262 144 segments, then the
+// prefix entry, then the triple.)  A wave that walks several chunks fetches what the next lookup starts
+// from before it copies the current chunk.
+struct ChunkRef {
+    uint64_t src;
+    uint64_t dst;
+    uint64_t len;
+    uint32_t k;
+};
+
+// Owner of chunk c, known to lie in segments [lo, hiEx): first[lo] <= c < first[hiEx].
+__device__ __forceinline__ ChunkRef OwnerOf(const uint64_t *__restrict__ triples, const uint32_t *__restrict__ first, uint32_t lo,
+                                            uint32_t hiEx, uint32_t c, uint32_t lane)
 {
-    const uint32_t nchunk = nchunkDev != nullptr ? *nchunkDev : nchunkHost;
+    // more than 64 candidates (a run of empty segments, or a map with coarse groups): narrow 64 ways per round
+    while (hiEx - lo > 64) {
+        const uint32_t span = hiEx - lo;
+        const uint32_t step = (span + 63u) >> 6;
+        const uint32_t probe = lo + (lane + 1) * step;
+        const bool inside = probe < hiEx;
+        const uint32_t v = inside ? first[probe] : 0xFFFFFFFFu;
+        const uint32_t hits = __popcll(__ballot(inside && v <= c));
+        lo += hits * step;
+        const uint32_t cap = lo + step;
+        hiEx = cap < hiEx ? cap : hiEx;
+    }
+    const uint32_t probe = lo + lane;
+    const bool inside = probe < hiEx;
+    uint32_t f = 0xFFFFFFFFu;
+    uint64_t ts = 0;
+    uint64_t td = 0;
+    uint64_t tl = 0;
+    if (inside) {
+        f = first[probe];
+        const uint64_t *t = triples + 3ull * probe;
+        ts = t[0];
+        td = t[1];
+        tl = t[2];
+    }
+    const uint32_t row = __popcll(__ballot(inside && f <= c)) - 1;   // first[lo] <= c: at least one hit
+    ChunkRef r;
+    r.src = ReadLane64(ts, row);
+    r.dst = ReadLane64(td, row);
+    r.len = ReadLane64(tl, row);
+    r.k = c - __builtin_amdgcn_readlane(f, row);
+    return r;
+}
+
+// A value every lane holds alike, moved to a scalar register: what a wave loads from a uniform address after its
+// first store lands in vector registers, and addresses and lengths computed from it would be computed per lane.
+__device__ __forceinline__ uint32_t Uniform(uint32_t v)
+{
+    return __builtin_amdgcn_readfirstlane(v);
+}
+
+__device__ __forceinline__ uint64_t Uniform(uint64_t v)
+{
+    return (static_cast<uint64_t>(Uniform(static_cast<uint32_t>(v >> 32))) << 32) | Uniform(static_cast<uint32_t>(v));
+}
+
+// kHeader: chunk count, group shift and pattern come from the header the device-side planner left in
+// device memory (the host knows none of them) instead of the kernel arguments.
+// kHold: as for the inline kernel, for launches of one chunk per workgroup (the host knows the chunk count).
+template <bool kNtLoad, int kStore, bool kHeader, int kHold = kHoldNone>
+__global__ __launch_bounds__(kXcopyThreads) void XcopyTableKernel(const TablePlan plan, uint32_t holdTicks)
+{
+    const uint64_t t0 = kHold != kHoldNone ? wall_clock64() : 0;
+    uint32_t nchunk = plan.nchunk;
+    uint32_t shift = plan.groupShift;
+    ChunkPattern pattern = plan.pattern;
+    if (kHeader) {
+        const TableHeader *__restrict__ header = plan.header;
+        nchunk = Uniform(header->nchunk);
+        shift = Uniform(header->groupShift);
+        pattern.period = Uniform(header->pattern.period);
+        pattern.chunksPerPeriod = Uniform(header->pattern.chunksPerPeriod);
+#pragma unroll
+        for (uint32_t i = 0; i <= kMaxPeriod; ++i) {
+            pattern.start[i] = Uniform(header->pattern.start[i]);
+        }
+    }
+    uint32_t c = blockIdx.x;
+    if (c >= nchunk) {
+        return;
+    }
+    const uint32_t units = plan.units;
+    if (pattern.period != 0) {
+        uint32_t seg;
+        uint32_t k;
+        PatternOwner(pattern, c, seg, k);
+        const uint64_t *t = plan.triples + 3ull * seg;
+        uint64_t src = t[0];
+        uint64_t dst = t[1];
+        uint64_t len = t[2];
+        for (;;) {
+            const uint32_t next = c + gridDim.x;
+            const bool more = next < nchunk;
+            uint64_t nsrc = 0;
+            uint64_t ndst = 0;
+            uint64_t nlen = 0;
+            uint32_t nk = 0;
+            if (more) {   // requested now, needed after the copy
+                PatternOwner(pattern, next, seg, nk);
+                t = plan.triples + 3ull * seg;
+                nsrc = t[0];
+                ndst = t[1];
+                nlen = t[2];
+            }
+            CopyChunkHeld<kNtLoad, kStore, kHold>(src, dst, len, k, units, t0, holdTicks);
+            if (!more) {
+                return;
+            }
+            src = Uniform(nsrc);
+            dst = Uniform(ndst);
+            len = Uniform(nlen);
+            k = nk;
+            c = next;
+        }
+    }
     const uint32_t lane = threadIdx.x & 63u;
-    for (uint32_t c = blockIdx.x; c < nchunk; c += gridDim.x) {
-        if (pattern.period != 0) {
-            // Chunk counts that repeat (pages of one size, K and V blocks in turn): the owner follows
-            // from a division and a few comparisons on kernel arguments, and the only memory round
-            // trip before the copy is the fetch of its descriptor.
-            uint32_t seg;
-            uint32_t k;
-            PatternOwner(pattern, c, seg, k);
-            const uint64_t *t = triples + 3ull * seg;
-            CopyChunk<kNtLoad, kStore>(t[0], t[1], t[2], k, units);
-            continue;
+    // even lanes fetch the map entry of the chunk's group, odd lanes the one behind it
+    uint32_t bounds = plan.group[(c >> shift) + (lane & 1u)];
+    for (;;) {
+        const uint32_t lo = __builtin_amdgcn_readlane(bounds, 0);
+        const uint32_t hiEx = __builtin_amdgcn_readlane(bounds, 1) + 1;
+        const ChunkRef r = OwnerOf(plan.triples, plan.first, lo, hiEx, c, lane);
+        const uint32_t next = c + gridDim.x;
+        const bool more = next < nchunk;
+        if (more) {
+            bounds = plan.group[(next >> shift) + (lane & 1u)];
         }
-        // 64-ary search for the last prefix entry <= c: every level is one load per lane and a
-        // ballot, so 4096 segments resolve in two memory round trips (a binary search by one
-        // lane would chain twelve).  Invariant: first[lo] <= c < first[hi].
-        uint32_t lo = 0;
-        uint32_t hi = nseg;
-        while (hi - lo > 1) {
-            const uint32_t span = hi - lo;
-            const uint32_t step = (span + 63u) >> 6;            // entries per lane at this level
-            const uint32_t probe = lo + (lane + 1) * step;      // lanes probe lo+step, lo+2*step, ...
-            const bool inside = probe < hi;
-            const uint32_t v = inside ? first[probe] : 0xFFFFFFFFu;
-            const uint32_t hits = __popcll(__ballot(inside && v <= c));
-            lo += hits * step;
-            const uint32_t cap = lo + step;
-            hi = cap < hi ? cap : hi;
+        CopyChunkHeld<kNtLoad, kStore, kHold>(r.src, r.dst, r.len, r.k, units, t0, holdTicks);
+        if (!more) {
+            return;
         }
-        const uint64_t *t = triples + 3ull * lo;
-        CopyChunk<kNtLoad, kStore>(t[0], t[1], t[2], c - first[lo], units);
+        c = next;
     }
 }
 
-// Device-side planner for a table the host cannot read: one workgroup turns
-// the triples into the chunk prefix the table kernel searches.
-constexpr uint32_t kPlanThreads = 1024;
-
-__global__ __launch_bounds__(kPlanThreads) void XcopyPlanKernel(const uint64_t *__restrict__ triples, uint32_t nseg,
-                                                                uint32_t units, uint32_t *__restrict__ first,
-                                                                uint32_t *__restrict__ nchunk)
+// Device-side planner for a table the host cannot read: chunk prefix, group map and, where the chunk
+// counts repeat with a short period, the pattern that lets the table kernel do without both.
+__device__ __forceinline__ uint32_t ChunksOf(const uint64_t *__restrict__ triples, uint32_t i, uint32_t units)
 {
-    __shared__ uint32_t partial[kPlanThreads];
+    return static_cast<uint32_t>(SegmentChunks(triples[3ull * i + 1], triples[3ull * i + 2], units));
+}
+
+__device__ __forceinline__ uint32_t WaveInclusiveSum(uint32_t v, uint32_t lane)
+{
+#pragma unroll
+    for (uint32_t d = 1; d < 64; d <<= 1) {
+        const uint32_t o = __shfl_up(v, d, 64);
+        v += lane >= d ? o : 0u;
+    }
+    return v;
+}
+
+__device__ __forceinline__ uint32_t WaveSum(uint32_t v)
+{
+#pragma unroll
+    for (uint32_t d = 32; d != 0; d >>= 1) {
+        v += __shfl_xor(v, d, 64);
+    }
+    return v;
+}
+
+__device__ __forceinline__ uint32_t WaveAnd(uint32_t v)
+{
+#pragma unroll
+    for (uint32_t d = 32; d != 0; d >>= 1) {
+        v &= __shfl_xor(v, d, 64);
+    }
+    return v;
+}
+
+constexpr uint32_t kPlanWaves = kPlanThreads / 64;
+constexpr uint32_t kAllPeriods = ((1u << kMaxPeriod) - 1) << 1;     // bit p: the counts repeat with period p
+
+// First of two launches for tables beyond kPlanSingleBlockSegs segments: every workgroup sums the chunk
+// counts of its kPlanThreads segments and notes which periods they contradict.
+__global__ __launch_bounds__(kPlanThreads) void XcopyPlanSumsKernel(const uint64_t *__restrict__ triples, uint32_t nseg, uint32_t units,
+                                                                    uint32_t *__restrict__ scratch, uint32_t groupCapacity)
+{
+    __shared__ uint32_t counts[kMaxPeriod + kPlanThreads];
+    __shared__ uint32_t waveSum[kPlanWaves];
+    __shared__ uint32_t waveAlive[kPlanWaves];
+    const ScratchLayout at = ScratchLayoutFor(nseg, groupCapacity);
     const uint32_t tid = threadIdx.x;
-    const uint32_t per = (nseg + kPlanThreads - 1) / kPlanThreads;
-    const uint32_t lo = tid * per;
-    const uint32_t hi = lo + per < nseg ? lo + per : nseg;
-    uint32_t sum = 0;
-    for (uint32_t i = lo; i < hi; ++i) {
-        sum += static_cast<uint32_t>(SegmentChunks(triples[3ull * i + 1], triples[3ull * i + 2], units));
+    const uint32_t seg0 = blockIdx.x * kPlanThreads;
+    const uint32_t i = seg0 + tid;
+    const uint32_t mine = i < nseg ? ChunksOf(triples, i, units) : 0u;
+    counts[kMaxPeriod + tid] = mine;
+    if (tid < kMaxPeriod) {
+        counts[tid] = seg0 + tid >= kMaxPeriod ? ChunksOf(triples, seg0 + tid - kMaxPeriod, units) : 0u;
     }
-    partial[tid] = sum;
     __syncthreads();
-    for (uint32_t step = 1; step < kPlanThreads; step <<= 1) {
-        const uint32_t add = tid >= step ? partial[tid - step] : 0;
-        __syncthreads();
-        partial[tid] += add;
-        __syncthreads();
+    uint32_t alive = kAllPeriods;
+    if (i < nseg) {
+#pragma unroll
+        for (uint32_t p = 1; p <= kMaxPeriod; ++p) {
+            if (i >= p && counts[kMaxPeriod + tid - p] != mine) {
+                alive &= ~(1u << p);
+            }
+        }
     }
-    uint32_t run = partial[tid] - sum;  // exclusive prefix of this lane's slice
-    for (uint32_t i = lo; i < hi; ++i) {
-        first[i] = run;
-        run += static_cast<uint32_t>(SegmentChunks(triples[3ull * i + 1], triples[3ull * i + 2], units));
+    const uint32_t sum = WaveSum(mine);
+    const uint32_t all = WaveAnd(alive);
+    if ((tid & 63u) == 0) {
+        waveSum[tid >> 6] = sum;
+        waveAlive[tid >> 6] = all;
     }
-    if (tid == kPlanThreads - 1) {
-        first[nseg] = partial[tid];
-        *nchunk = partial[tid];
+    __syncthreads();
+    if (tid == 0) {
+        uint32_t s = 0;
+        uint32_t a = kAllPeriods;
+        for (uint32_t w = 0; w < kPlanWaves; ++w) {
+            s += waveSum[w];
+            a &= waveAlive[w];
+        }
+        scratch[at.blockSum + blockIdx.x] = s;
+        scratch[at.blockAlive + blockIdx.x] = a;
+    }
+}
+
+// The planner proper.  Thread t takes kEach consecutive segments.  One workgroup and one launch for up to
+// kPlanSingleBlockSegs segments (kEach = 1, 2, 4 or 8); beyond, one workgroup per kPlanThreads segments
+// (kEach = 1) behind XcopyPlanSumsKernel, which has left the sums and the periods of all workgroups.
+template <uint32_t kEach>
+__global__ __launch_bounds__(kPlanThreads) void XcopyPlanKernel(const uint64_t *__restrict__ triples, uint32_t nseg, uint32_t units,
+                                                                uint32_t *__restrict__ scratch, uint32_t groupCapacity)
+{
+    __shared__ uint32_t counts[kMaxPeriod + kEach * kPlanThreads];
+    __shared__ uint32_t waveTotal[kPlanWaves];      // inclusive sums of the waves, then their exclusive prefix
+    __shared__ uint32_t reduced[2 * kPlanWaves + 4];
+    const ScratchLayout at = ScratchLayoutFor(nseg, groupCapacity);
+    const uint32_t tid = threadIdx.x;
+    const uint32_t lane = tid & 63u;
+    const uint32_t wave = tid >> 6;
+    const bool alone = gridDim.x == 1;
+    const uint32_t i0 = (blockIdx.x * kPlanThreads + tid) * kEach;
+
+    uint32_t mine[kEach];
+    uint32_t sum = 0;
+#pragma unroll
+    for (uint32_t q = 0; q < kEach; ++q) {
+        mine[q] = i0 + q < nseg ? ChunksOf(triples, i0 + q, units) : 0u;
+        sum += mine[q];
+        if (alone) {
+            counts[kMaxPeriod + tid * kEach + q] = mine[q];
+        }
+    }
+    if (alone && tid < kMaxPeriod) {
+        counts[tid] = 0;
+    }
+    const uint32_t incl = WaveInclusiveSum(sum, lane);
+    if (lane == 63) {
+        waveTotal[wave] = incl;
+    }
+    __syncthreads();
+
+    uint32_t aliveMine = kAllPeriods;
+    if (alone) {
+        // the eight counts in front of this thread's segments, then its own, checked against every period
+        uint32_t window[kMaxPeriod + kEach];
+#pragma unroll
+        for (uint32_t w = 0; w < kMaxPeriod; ++w) {
+            window[w] = counts[tid * kEach + w];
+        }
+#pragma unroll
+        for (uint32_t q = 0; q < kEach; ++q) {
+            window[kMaxPeriod + q] = mine[q];
+        }
+#pragma unroll
+        for (uint32_t q = 0; q < kEach; ++q) {
+#pragma unroll
+            for (uint32_t p = 1; p <= kMaxPeriod; ++p) {
+                if (i0 + q < nseg && i0 + q >= p && window[kMaxPeriod + q - p] != mine[q]) {
+                    aliveMine &= ~(1u << p);
+                }
+            }
+        }
+    }
+    const uint32_t aliveWave = WaveAnd(aliveMine);
+    // wave 0: exclusive prefix over the wave totals and their sum
+    if (wave == 0) {
+        const uint32_t own = lane < kPlanWaves ? waveTotal[lane] : 0u;
+        const uint32_t scan = WaveInclusiveSum(own, lane);
+        if (lane < kPlanWaves) {
+            waveTotal[lane] = scan - own;
+        }
+        if (lane == 63) {
+            reduced[2 * kPlanWaves] = scan;          // chunks of this workgroup's segments
+        }
+    }
+    if (lane == 0) {
+        reduced[wave] = aliveWave;
+    }
+    __syncthreads();
+
+    // chunks in front of this workgroup, chunks of the whole table, periods still alive
+    uint32_t base = 0;
+    uint32_t total = reduced[2 * kPlanWaves];
+    uint32_t alive = kAllPeriods;
+    if (alone) {
+        for (uint32_t w = 0; w < kPlanWaves; ++w) {
+            alive &= reduced[w];
+        }
+    } else {
+        uint32_t front = 0;
+        uint32_t whole = 0;
+        uint32_t bits = kAllPeriods;
+        for (uint32_t b = tid; b < gridDim.x; b += kPlanThreads) {
+            const uint32_t blockSum = scratch[at.blockSum + b];
+            whole += blockSum;
+            front += b < blockIdx.x ? blockSum : 0u;
+            bits &= scratch[at.blockAlive + b];
+        }
+        front = WaveSum(front);
+        whole = WaveSum(whole);
+        bits = WaveAnd(bits);
+        __syncthreads();                               // every thread has read reduced[] above
+        if (lane == 0) {
+            reduced[wave] = front;
+            reduced[kPlanWaves + wave] = whole;
+            counts[wave] = bits;
+        }
+        __syncthreads();
+        total = 0;
+        for (uint32_t w = 0; w < kPlanWaves; ++w) {
+            base += reduced[w];
+            total += reduced[kPlanWaves + w];
+            alive &= counts[w];
+        }
+    }
+
+    const uint32_t shift = GroupShiftFor(total, at.groupCapacity);
+    const uint32_t ngroups = GroupCount(total, shift);
+    uint32_t *first = scratch + at.first;
+    uint32_t *group = scratch + at.group;
+    uint32_t f = base + waveTotal[wave] + incl - sum;
+#pragma unroll
+    for (uint32_t q = 0; q < kEach; ++q) {
+        const uint32_t i = i0 + q;
+        const bool live = i < nseg;
+        if (live) {
+            first[i] = f;
+            if (i == nseg - 1) {
+                first[nseg] = f + mine[q];
+            }
+        }
+        // map entries of the groups whose first chunk this segment owns; the segment that owns the last chunk also closes the map
+        uint32_t gLo = 1;
+        uint32_t gHi = 0;
+        if (live && mine[q] != 0) {
+            gLo = static_cast<uint32_t>((static_cast<uint64_t>(f) + (1ull << shift) - 1) >> shift);
+            gHi = (f + mine[q] - 1) >> shift;
+            if (f + mine[q] == total) {
+                group[ngroups] = i;
+            }
+        }
+        const bool some = gLo <= gHi;
+        const bool many = some && gHi - gLo >= 4;
+        if (some && !many) {
+            for (uint32_t g = gLo; g <= gHi; ++g) {
+                group[g] = i;
+            }
+        }
+        // a segment of many groups is written by its whole wave
+        uint64_t todo = __ballot(many);
+        while (todo != 0) {
+            const uint32_t from = static_cast<uint32_t>(__builtin_ctzll(todo));
+            todo &= todo - 1;
+            const uint32_t lo = __builtin_amdgcn_readlane(gLo, from);
+            const uint32_t hi = __builtin_amdgcn_readlane(gHi, from);
+            const uint32_t owner = __builtin_amdgcn_readlane(i, from);
+            for (uint64_t g = static_cast<uint64_t>(lo) + lane; g <= hi; g += 64) {
+                group[g] = owner;
+            }
+        }
+        f += mine[q];
+    }
+
+    if (blockIdx.x == 0 && tid == 0) {
+        TableHeader *header = reinterpret_cast<TableHeader *>(scratch);
+        header->nchunk = total;
+        header->groupShift = shift;
+        header->reserved[0] = 0;
+        header->reserved[1] = 0;
+        ChunkPattern pattern{};
+        if (alive != 0 && total != 0) {
+            // the shortest period never exceeds the segment count: period nseg is never contradicted
+            const uint32_t period = static_cast<uint32_t>(__builtin_ctz(alive));
+            uint32_t run = 0;
+            for (uint32_t q = 0; q < period; ++q) {
+                pattern.start[q] = run;
+                run += ChunksOf(triples, q, units);
+            }
+            pattern.start[period] = run;
+            if (run != 0) {
+                pattern.period = period;
+                pattern.chunksPerPeriod = run;
+            } else {
+                pattern = ChunkPattern{};
+            }
+        }
+        header->pattern = pattern;
+        header->pad = 0;
     }
 }
 
@@ -493,20 +877,27 @@ uint32_t HoldTicks(uint32_t nanos)
 }
 
 // anyOrder: the launch carries no barrier, so the command processor may start it while launches queued
-// before it on the same stream still run (hipExtAnyOrderLaunch).  Measured on the 9 MB batch, one stream:
-// 5.3 us per launch against 5.9 us with the barrier.
-// holdNanos: the caller's HoldNanosFor(); the launch qualifies only if it still has one chunk per workgroup.
+// before it on the same stream still run (hipExtAnyOrderLaunch; a 9 MB batch on one stream: 5.3 against 5.9 us).
+// holdNanos: the caller's HoldNanosFor(); the launch qualifies only if it has one chunk per workgroup, of
+// 4 KiB (stores of four loads per lane held) or of kWindowUnits units (of sixteen).
 template <bool kNtLoad, int kStore>
 int LaunchInline(const InlinePlan &plan, uint32_t grid, uint32_t lanes, hipStream_t stream, bool anyOrder, uint32_t holdNanos)
 {
     const uint32_t flags = anyOrder ? hipExtAnyOrderLaunch : 0u;
+    const bool deep = plan.units == kWindowUnits && grid == plan.nchunk && holdNanos != 0 && !anyOrder;
+    if (deep) {
+        lanes = 64;
+    }
     const uint32_t ticks = grid == plan.nchunk && lanes == 64 ? HoldTicks(holdNanos) : 0;
     if (plan.first[1] == kNoChunk && plan.nchunk <= kSingleMaxChunks) {
         if (anyOrder) {
             hipExtLaunchKernelGGL((XcopySingleKernel<kNtLoad, kStore>), dim3(grid), dim3(lanes), 0, stream, nullptr, nullptr, flags,
                                   plan.src[0], plan.dst[0], plan.len[0], plan.nchunk, plan.units, 0u);
+        } else if (ticks != 0 && deep) {
+            hipLaunchKernelGGL((XcopySingleKernel<kNtLoad, kStore, kHoldDeep>), dim3(grid), dim3(lanes), 0, stream, plan.src[0],
+                               plan.dst[0], plan.len[0], plan.nchunk, plan.units, ticks);
         } else if (ticks != 0) {
-            hipLaunchKernelGGL((XcopySingleKernel<kNtLoad, kStore, true>), dim3(grid), dim3(lanes), 0, stream, plan.src[0],
+            hipLaunchKernelGGL((XcopySingleKernel<kNtLoad, kStore, kHoldShallow>), dim3(grid), dim3(lanes), 0, stream, plan.src[0],
                                plan.dst[0], plan.len[0], plan.nchunk, plan.units, ticks);
         } else {
             hipLaunchKernelGGL((XcopySingleKernel<kNtLoad, kStore>), dim3(grid), dim3(lanes), 0, stream, plan.src[0], plan.dst[0],
@@ -518,22 +909,17 @@ int LaunchInline(const InlinePlan &plan, uint32_t grid, uint32_t lanes, hipStrea
     // launch configuration around the same call, 0.15 us of host time per launch with this 3 KiB argument block.
     uint32_t holdTicks = ticks;
     void *args[] = {const_cast<InlinePlan *>(&plan), &holdTicks};
-    if (ticks != 0) {
-        if (anyOrder) {
-            hipExtLaunchKernelGGL((XcopyInlineKernel<kNtLoad, kStore, true>), dim3(grid), dim3(lanes), 0, stream, nullptr, nullptr,
-                                  flags, plan, ticks);
-        } else {
-            return static_cast<int>(hipLaunchKernel(reinterpret_cast<const void *>(&XcopyInlineKernel<kNtLoad, kStore, true>), dim3(grid),
-                                                    dim3(lanes), args, 0, stream));
-        }
-    } else if (anyOrder) {
+    const void *kernel = reinterpret_cast<const void *>(&XcopyInlineKernel<kNtLoad, kStore, kHoldNone>);
+    if (ticks != 0 && !anyOrder) {
+        kernel = deep ? reinterpret_cast<const void *>(&XcopyInlineKernel<kNtLoad, kStore, kHoldDeep>)
+                      : reinterpret_cast<const void *>(&XcopyInlineKernel<kNtLoad, kStore, kHoldShallow>);
+    }
+    if (anyOrder) {
         hipExtLaunchKernelGGL((XcopyInlineKernel<kNtLoad, kStore>), dim3(grid), dim3(lanes), 0, stream, nullptr, nullptr, flags, plan,
                               0u);
-    } else {
-        return static_cast<int>(hipLaunchKernel(reinterpret_cast<const void *>(&XcopyInlineKernel<kNtLoad, kStore, false>), dim3(grid),
-                                                dim3(lanes), args, 0, stream));
+        return static_cast<int>(hipGetLastError());
     }
-    return static_cast<int>(hipGetLastError());
+    return static_cast<int>(hipLaunchKernel(kernel, dim3(grid), dim3(lanes), args, 0, stream));
 }
 
 // windowMBps: the rate (MB/s of HBM traffic, read + written) the period of a windowed launch is cut for.
@@ -549,10 +935,51 @@ int LaunchWindowed(const InlinePlan &plan, uint32_t grid, uint32_t windowMBps, h
 }
 
 template <bool kNtLoad, int kStore>
-int LaunchTable(const TablePlan &plan, const uint32_t *nchunkDev, uint32_t grid, uint32_t lanes, hipStream_t stream)
+int LaunchTable(const TablePlan &plan, uint32_t grid, uint32_t lanes, hipStream_t stream, uint32_t holdNanos)
 {
-    hipLaunchKernelGGL((XcopyTableKernel<kNtLoad, kStore>), dim3(grid), dim3(lanes), 0, stream, plan.triples,
-                       plan.first, nchunkDev, plan.nseg, plan.nchunk, plan.units, plan.pattern);
+    if (plan.header != nullptr) {
+        hipLaunchKernelGGL((XcopyTableKernel<kNtLoad, kStore, true>), dim3(grid), dim3(lanes), 0, stream, plan, 0u);
+        return static_cast<int>(hipGetLastError());
+    }
+    const bool deep = plan.units == kWindowUnits && holdNanos != 0;
+    if (deep) {
+        lanes = 64;
+    }
+    const uint32_t ticks = grid == plan.nchunk && lanes == 64 ? HoldTicks(holdNanos) : 0;
+    if (ticks != 0 && deep) {
+        hipLaunchKernelGGL((XcopyTableKernel<kNtLoad, kStore, false, kHoldDeep>), dim3(grid), dim3(lanes), 0, stream, plan, ticks);
+    } else if (ticks != 0) {
+        hipLaunchKernelGGL((XcopyTableKernel<kNtLoad, kStore, false, kHoldShallow>), dim3(grid), dim3(lanes), 0, stream, plan, ticks);
+    } else {
+        hipLaunchKernelGGL((XcopyTableKernel<kNtLoad, kStore, false>), dim3(grid), dim3(lanes), 0, stream, plan, 0u);
+    }
+    return static_cast<int>(hipGetLastError());
+}
+
+// The planner's one or two launches for a table of nseg segments in device memory.
+int LaunchPlanner(const uint64_t *triples, uint32_t nseg, uint32_t units, uint32_t *scratch, uint32_t groupCapacity,
+                  hipStream_t stream)
+{
+    const uint32_t blocks = PlanBlocks(nseg);
+    if (blocks > 1) {
+        hipLaunchKernelGGL(XcopyPlanSumsKernel, dim3(blocks), dim3(kPlanThreads), 0, stream, triples, nseg, units, scratch,
+                           groupCapacity);
+        const hipError_t err = hipGetLastError();
+        if (err != hipSuccess) {
+            return static_cast<int>(err);
+        }
+    }
+    const uint32_t tiles = blocks > 1 ? 1u : (nseg + kPlanThreads - 1) / kPlanThreads;   // segments per thread
+    if (tiles <= 1) {
+        hipLaunchKernelGGL(XcopyPlanKernel<1>, dim3(blocks), dim3(kPlanThreads), 0, stream, triples, nseg, units, scratch, groupCapacity);
+    } else if (tiles <= 2) {
+        hipLaunchKernelGGL(XcopyPlanKernel<2>, dim3(1), dim3(kPlanThreads), 0, stream, triples, nseg, units, scratch, groupCapacity);
+    } else if (tiles <= 4) {
+        hipLaunchKernelGGL(XcopyPlanKernel<4>, dim3(1), dim3(kPlanThreads), 0, stream, triples, nseg, units, scratch, groupCapacity);
+    } else {
+        hipLaunchKernelGGL(XcopyPlanKernel<kPlanTiles>, dim3(1), dim3(kPlanThreads), 0, stream, triples, nseg, units, scratch,
+                           groupCapacity);
+    }
     return static_cast<int>(hipGetLastError());
 }
 
@@ -618,38 +1045,69 @@ extern "C" int mfk_xcopy_signal(void *word, uint32_t value, void *stream)
     return mf::Signal(word, value, static_cast<hipStream_t>(stream));
 }
 
-extern "C" int mfk_xcopy_table(const void *triples, const void *first, const void *nchunkDev, uint32_t nseg,
-                               uint32_t nchunk, uint32_t units, const void *pattern, int route, uint32_t grid, void *mask,
-                               uint32_t maskValue, void *stream)
+extern "C" int mfk_xcopy_table(const void *tablePlan, int route, uint32_t grid, void *mask, uint32_t maskValue, void *stream,
+                               uint32_t holdNanos)
 {
-    mf::ChunkPattern pat{};
-    if (pattern != nullptr) {
-        pat = *static_cast<const mf::ChunkPattern *>(pattern);
-    }
-    if (nseg == 0 || grid == 0 || (pat.period == 0 && first == nullptr)) {
+    const mf::TablePlan &plan = *static_cast<const mf::TablePlan *>(tablePlan);
+    const mf::ChunkPattern &pat = plan.pattern;
+    if (plan.nseg == 0 || grid == 0 || plan.triples == nullptr) {
         return -1;
     }
-    if (pat.period != 0 && (pat.period > mf::kMaxPeriod || pat.chunksPerPeriod == 0 || nchunkDev != nullptr ||
-                            pat.start[0] != 0 || pat.start[pat.period] != pat.chunksPerPeriod ||
-                            mf::PatternChunks(pat, nseg) != nchunk)) {
+    if (plan.header == nullptr) {
+        if (pat.period == 0 && (plan.first == nullptr || plan.group == nullptr || plan.groupShift < mf::kGroupShiftMin ||
+                                plan.groupShift > 31)) {
+            return -1;
+        }
+        if (pat.period != 0 && (pat.period > mf::kMaxPeriod || pat.chunksPerPeriod == 0 || pat.start[0] != 0 ||
+                                pat.start[pat.period] != pat.chunksPerPeriod || mf::PatternChunks(pat, plan.nseg) != plan.nchunk)) {
+            return -1;
+        }
+    } else if (plan.first == nullptr || plan.group == nullptr) {
         return -1;
     }
-    mf::TablePlan plan{static_cast<const uint64_t *>(triples), static_cast<const uint32_t *>(first), nseg, nchunk, units, pat};
-    const uint32_t *nd = static_cast<const uint32_t *>(nchunkDev);
     hipStream_t s = static_cast<hipStream_t>(stream);
     const int err = mf::WithPolicy(mf::PolicyOf(route), [&](auto ntLoad, auto store) {
-        return mf::LaunchTable<decltype(ntLoad)::value, decltype(store)::value>(plan, nd, grid, mf::LanesFor(units, route), s);
+        return mf::LaunchTable<decltype(ntLoad)::value, decltype(store)::value>(plan, grid, mf::LanesFor(plan.units, route), s,
+                                                                                route == MFRT_ROUTE_HBM ? holdNanos : 0u);
     });
     return err != 0 ? err : mf::Signal(mask, maskValue, s);
 }
 
+extern "C" uint64_t mfk_xcopy_plan_scratch_words(uint32_t nseg, uint32_t groupCapacity)
+{
+    return mf::ScratchLayoutFor(nseg, groupCapacity).words;
+}
+
+// scratch: mfk_xcopy_plan_scratch_words(nseg, groupCapacity) words of device memory.  *tablePlan receives the plan for
+// mfk_xcopy_table that reads what the planner leaves there.
+extern "C" int mfk_xcopy_plan(const void *triples, uint32_t nseg, uint32_t units, void *scratch, uint32_t groupCapacity,
+                              void *tablePlan, void *stream)
+{
+    if (nseg == 0 || scratch == nullptr || groupCapacity < 2 || tablePlan == nullptr) {
+        return -1;
+    }
+    uint32_t *words = static_cast<uint32_t *>(scratch);
+    const mf::ScratchLayout at = mf::ScratchLayoutFor(nseg, groupCapacity);
+    mf::TablePlan &plan = *static_cast<mf::TablePlan *>(tablePlan);
+    plan = mf::TablePlan{};
+    plan.triples = static_cast<const uint64_t *>(triples);
+    plan.first = words + at.first;
+    plan.group = words + at.group;
+    plan.header = reinterpret_cast<const mf::TableHeader *>(words);
+    plan.nseg = nseg;
+    plan.units = units;
+    return mf::LaunchPlanner(plan.triples, nseg, units, words, groupCapacity, static_cast<hipStream_t>(stream));
+}
+
 #ifndef MF_RT_HIDDEN   // the plugin library has no entry point that needs it
-// Scratch of the entry point that allocates nothing (mfk_xcopy_table_static): the chunk prefix
-// first[0 .. nseg] and, behind it, the chunk count, both written by XcopyPlanKernel and read by
-// XcopyTableKernel of the same call.  One copy per GPU, held until the process ends.  In host code
-// the array's name is only a handle for hipGetSymbolAddress: kernels and copies get the address that
-// call returned for the current device, never the name.
-static __device__ __align__(256) uint32_t scratch[MFK_STATIC_TABLE_SEGMENTS + 64];
+// Scratch of the entry point that allocates nothing (mfk_xcopy_table_static): header, chunk prefix,
+// the planner's partial sums and the group map, written by the planner and read by XcopyTableKernel of the
+// same call.  One copy per GPU, held until the process ends.  In host code the array's name is only a
+// handle for hipGetSymbolAddress: kernels get the address that call returned for the current device,
+// never the name.
+constexpr uint32_t kStaticGroupCapacity = MFK_STATIC_TABLE_SEGMENTS;
+constexpr uint64_t kStaticScratchWords = mf::ScratchLayoutFor(MFK_STATIC_TABLE_SEGMENTS, kStaticGroupCapacity).words;
+static __device__ __align__(256) uint32_t scratch[kStaticScratchWords];
 
 namespace {
 constexpr int kMaxDevices = 64;
@@ -685,31 +1143,12 @@ extern "C" int mfk_xcopy_table_static(const void *triples, uint32_t nseg, uint32
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices || g_scratchOf[dev] == nullptr) {
         return -2;   // mfk_xcopy_static_setup has not run on this device
     }
-    uint32_t *first = g_scratchOf[dev];
-    uint32_t *nchunkDev = first + nseg + 1;
-    hipStream_t s = static_cast<hipStream_t>(stream);
-    // the plan kernel writes every word the table kernel reads: nothing has to start at zero
-    hipLaunchKernelGGL(mf::XcopyPlanKernel, dim3(1), dim3(mf::kPlanThreads), 0, s, static_cast<const uint64_t *>(triples), nseg,
-                       units, first, nchunkDev);
-    hipError_t err = hipGetLastError();
-    if (err != hipSuccess) {
-        return static_cast<int>(err);
+    // the planner writes every word the table kernel reads: nothing has to start at zero
+    mf::TablePlan plan;
+    const int err = mfk_xcopy_plan(triples, nseg, units, g_scratchOf[dev], kStaticGroupCapacity, &plan, stream);
+    if (err != 0) {
+        return err;
     }
-    mf::TablePlan plan{static_cast<const uint64_t *>(triples), first, nseg, 0, units, mf::ChunkPattern{}};
-    return mf::WithPolicy(mf::PolicyOf(route), [&](auto ntLoad, auto store) {
-        return mf::LaunchTable<decltype(ntLoad)::value, decltype(store)::value>(plan, nchunkDev, grid, mf::LanesFor(units, route), s);
-    });
+    return mfk_xcopy_table(&plan, route, grid, nullptr, 0, stream, 0);
 }
 #endif  // MF_RT_HIDDEN
-
-extern "C" int mfk_xcopy_plan(const void *triples, uint32_t nseg, uint32_t units, void *first, void *nchunk,
-                              void *stream)
-{
-    if (nseg == 0) {
-        return -1;
-    }
-    hipLaunchKernelGGL(mf::XcopyPlanKernel, dim3(1), dim3(mf::kPlanThreads), 0, static_cast<hipStream_t>(stream),
-                       static_cast<const uint64_t *>(triples), nseg, units, static_cast<uint32_t *>(first),
-                       static_cast<uint32_t *>(nchunk));
-    return static_cast<int>(hipGetLastError());
-}

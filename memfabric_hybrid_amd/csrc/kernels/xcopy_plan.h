@@ -79,48 +79,37 @@ struct InlinePlan {
 
 // Stores held back: how long after its start a wave of the inline kernel waits before it stores.
 //
-// A launch of a few thousand single-chunk waves has every load in flight within the first two
-// microseconds and would issue its stores as the data trickle in, so HBM sees reads and writes mixed
-// for most of the kernel.  When every wave instead keeps its four loaded registers until the loads
-// of the whole launch are out, the reads run as one burst and the writes as another, and the kernel
-// is shorter.  Measured through smem_bm_copy_batch, batches back to back on one stream, K and V
-// blocks in turn (61 of each, V blocks of 16 KiB), period per batch without the wait / at the best wait:
-//    976 chunks 3.79 / 3.24 us (1300 ns)     2684 chunks 6.45 / 5.11 us (2200 ns)
-//   1220 chunks 4.11 / 3.47 us (1400 ns)     3172 chunks 6.86 / 5.78 us (2600 ns)
-//   1708 chunks 4.76 / 4.32 us (1500-1900)   3904 chunks 8.02 / 6.54 us (3000 ns)
-//   2196 chunks 5.29 / 4.56 us (1900 ns)     5124 chunks 9.72 / 8.79 us (3400 ns)
-// and for other mixes of about 2048 chunks: 64 x 128 KiB 5.05 / 4.64, 32 x 256 KiB 4.99 / 4.38,
-// 128 x 64 KiB 5.07 / 4.61, 8 x 1 MiB + 100 x 20 KiB 6.12 / 5.07 us; 128 ragged segments of about
-// 70000 bytes gain nothing and lose nothing (6.5 us either way).  The wait is counted from the start of
-// the wave, which absorbs the spread of the table fetch (counted from the issue of the loads the same
-// wait gains nothing), and it is the same for every wave: shortening it for waves that start later did
-// not help.  The best wait grows with the number of waves the dispatcher has to start.  100 to 200 ns
-// short of it the gain is lost (2196 chunks: 1700 ns 4.87 us, 1600 ns 5.09 us), each 100 ns beyond it
-// costs 0.1 us, so the rule aims a little long: in steps of 50 ns, on four machines, 2196 chunks took 4.57 us at
-// 1750 ns, 4.44 at 1800, 4.30 at 1850 to 1950, 4.35 at 2000 and 4.42 at 2050, and the rule gives 1957 ns; from 1220
-// to 5124 chunks the rule is within 50 ns of the best step or level with it.  From about 7000 chunks on the gain is below 5 % and the
-// best wait no longer follows the line: not every wave of such a launch is resident at once, and a wait
-// only delays the ones behind (11956 chunks: 19.3 us without, 20.2 us with).  Below about
-// 1000 chunks the period is the cost of a dependent launch and no wait changes it.
-// Launches that overlap on purpose (no barrier between them) lose with a wait: 4.53 us without, 4.81 with.
-//
-// A single segment (its three words are plain kernel arguments, no table to fetch) has its loads out
-// about 0.6 us earlier, and its best wait is shorter by as much; copies back to back on one stream,
-// without / at the best wait:
-//   1536 chunks (6 MiB) 3.64 / 3.39 us (1000 ns)     4096 chunks (16 MiB) 7.06 / 5.97 us (2300 ns)
-//   2048 chunks (8 MiB) 4.08 / 3.83 us (1300 ns)     5120 chunks (20 MiB) 8.74 / 7.07 us (2900 ns)
-//   3072 chunks (12 MiB) 5.71 / 4.90 us (1800 ns)    6144 chunks (24 MiB) 10.03 / 8.18 us (3400 ns)
-// 1024 chunks gain nothing (3.1 us either way); 7168 chunks gain 5 %, 8192 and more 3 % and less: past
-// 6144 single-wave workgroups (24 per CU) not every wave of the launch is resident at once.
+// A launch of a few thousand single-chunk waves has every load in flight within two microseconds and
+// would store as the data trickle in, so HBM sees reads and writes mixed.  When every wave keeps its four
+// loaded registers until the loads of the whole launch are out, the reads run as one burst and the
+// writes as another: a 2196-chunk batch takes 4.5 instead of 5.3 us.  The wait is counted from the start
+// of the wave, is the same for every wave, and grows with the number of waves the dispatcher has to start
+// (a line fitted to sweeps over 976 ... 7076 chunks; it aims 50 to 100 ns long, because falling 200 ns short
+// loses the gain while each 100 ns beyond costs 0.1 us).  It pays only while every wave of the launch is
+// resident at once (up to 24 single-wave workgroups per CU) and only for launches that do not overlap
+// others on purpose.  A single segment has no table to fetch and gets a line of its own.
 constexpr uint32_t kHoldMinChunks = 960;        // table in the kernel arguments
 constexpr uint32_t kHoldKneeChunks = 3904;
 constexpr uint32_t kHoldMinChunksSingle = 1400; // one segment
 constexpr uint32_t kHoldMaxChunks = 6144;
 constexpr uint32_t kHoldSharedMaxChunks = 4096; // the limit while several threads submit on streams of their own
+// Beyond kHoldMaxChunks chunks of 4 KiB the waves of a launch are no longer resident together.  Batches of up to
+// kDeepMaxChunks chunks of kDeepUnits units (16 KiB, sixteen loads per lane in flight: 64 MiB in 4096 waves, 16 per CU)
+// are, and hold their stores the same way.
+constexpr uint32_t kDeepUnits = 1024;
+constexpr uint32_t kDeepMaxChunks = 4096;
+constexpr uint64_t kDeepMinBytes = static_cast<uint64_t>(kHoldMaxChunks) * kXcopyThreads * kUnitBytes;   // 24 MiB
+constexpr uint64_t kDeepMaxBytes = static_cast<uint64_t>(kDeepMaxChunks) * kDeepUnits * kUnitBytes;      // 64 MiB
+constexpr uint64_t kDeepMinSegmentBytes = 32768;   // on average: short segments make chunks that are not whole
 inline uint32_t HoldNanosFor(uint32_t nchunk, uint32_t grid, uint32_t units, bool single)
 {
+    if (units == kDeepUnits && grid == nchunk && nchunk <= kDeepMaxChunks) {
+        // fitted to sweeps over 1664 ... 4096 waves (26 to 64 MiB in 32 segments, one segment, 100 ragged ones): the best wait is
+        // 600 ns and 2.15 ns per 16 KiB, a read rate of 7.6 TB/s; up to 10 % beyond costs 1 to 3 %, 10 % short loses half the gain
+        return nchunk < kHoldMinChunks / 4 ? 0 : 600 + nchunk * 215 / 100;
+    }
     if (units != kXcopyThreads || grid != nchunk || nchunk > kHoldMaxChunks) {
-        return 0;   // only launches of one 4 KiB chunk per single-wave workgroup were measured
+        return 0;   // only launches of one chunk per single-wave workgroup were measured
     }
     if (single) {
         return nchunk < kHoldMinChunksSingle ? 0 : 100 + nchunk * 57 / 100;
@@ -161,17 +150,22 @@ struct ChunkPattern {
     uint32_t start[kMaxPeriod + 1];     // exclusive prefix of the counts inside one period; start[period] == chunksPerPeriod
 };
 
-// Segment and chunk-in-segment of global chunk c under a pattern.
+// Segment and chunk-in-segment of global chunk c under a pattern.  Every start[] is read at a fixed index, so
+// that a kernel keeps the pattern in scalar registers (the member that owns r is the last one whose start
+// is <= r, and starts never decrease, so the hits form a prefix and the last hit's start is the owner's).
 MF_HD inline void PatternOwner(const ChunkPattern &p, uint32_t c, uint32_t &seg, uint32_t &k)
 {
     const uint32_t group = c / p.chunksPerPeriod;
     const uint32_t r = c - group * p.chunksPerPeriod;
     uint32_t j = 0;
+    uint32_t base = 0;
     for (uint32_t i = 1; i < kMaxPeriod; ++i) {
-        j += (i < p.period && p.start[i] <= r) ? 1u : 0u;
+        const bool hit = i < p.period && p.start[i] <= r;
+        j += hit ? 1u : 0u;
+        base = hit ? p.start[i] : base;
     }
     seg = group * p.period + j;
-    k = r - p.start[j];
+    k = r - base;
 }
 
 // Chunks of the first nseg segments under a pattern.
@@ -180,12 +174,115 @@ MF_HD inline uint64_t PatternChunks(const ChunkPattern &p, uint32_t nseg)
     return static_cast<uint64_t>(nseg / p.period) * p.chunksPerPeriod + p.start[nseg % p.period];
 }
 
-// A table-driven launch: triples and prefix live in device memory.
+// Group map of a table without a pattern.  The chunks are taken in groups of 2^shift; group[g] is the
+// segment that owns chunk g << shift, and one more entry names the segment that owns the last chunk.
+// The owner of chunk c then lies in [group[g], group[g + 1]] with g = c >> shift, a range the 64 lanes
+// of a wave probe in one round whenever it spans at most 64 segments: the lookup is two dependent loads
+// instead of a search over the whole prefix.  A group of 2^shift chunks touches at most 2^shift + 1
+// segments that are not empty, so groups of 32 chunks always resolve in that one round (groups of 64
+// would need a second one for a run of 65 single-chunk segments).  The shift grows until the map fits
+// the room there is for it.
+constexpr uint32_t kGroupShiftMin = 5;
+
+MF_HD constexpr inline uint32_t GroupCount(uint64_t nchunk, uint32_t shift)
+{
+    return static_cast<uint32_t>((nchunk + (1ull << shift) - 1) >> shift);
+}
+
+// Smallest shift from kGroupShiftMin on whose map (GroupCount + 1 entries) fits `capacity` entries.
+MF_HD constexpr inline uint32_t GroupShiftFor(uint64_t nchunk, uint32_t capacity)
+{
+    uint32_t shift = kGroupShiftMin;
+    while (shift < 32 && static_cast<uint64_t>(GroupCount(nchunk, shift)) + 1 > capacity) {
+        ++shift;
+    }
+    return shift;
+}
+
+// Room the engine gives the map of a table of nseg segments: the finest groups for every table whose chunks
+// number up to 32 times that (2 M chunks, 8 GiB in 4 KiB chunks, at the least), coarser ones beyond.
+MF_HD constexpr inline uint32_t GroupCapacityFor(uint32_t nseg)
+{
+    return (nseg > 65536u ? nseg : 65536u) + 1u;
+}
+
+// Host-side build of the map from a finished prefix (first[0 .. nseg], first[nseg] == nchunk != 0); returns the shift.
+// group: room for `capacity` entries.
+inline uint32_t BuildGroupMap(const uint32_t *first, uint32_t nseg, uint32_t *group, uint32_t capacity)
+{
+    const uint32_t nchunk = first[nseg];
+    const uint32_t shift = GroupShiftFor(nchunk, capacity);
+    const uint32_t ngroups = GroupCount(nchunk, shift);
+    uint32_t last = 0;
+    for (uint32_t i = 0; i < nseg; ++i) {
+        const uint32_t f = first[i];
+        const uint32_t cnt = first[i + 1] - f;
+        if (cnt == 0) {
+            continue;
+        }
+        last = i;
+        const uint32_t gLo = static_cast<uint32_t>((static_cast<uint64_t>(f) + (1ull << shift) - 1) >> shift);
+        const uint32_t gHi = (f + cnt - 1) >> shift;
+        for (uint64_t g = gLo; g <= gHi; ++g) {
+            group[g] = i;
+        }
+    }
+    group[ngroups] = last;
+    return shift;
+}
+
+// What the device-side planner leaves for the table kernel of the same call (64 bytes).
+struct TableHeader {
+    uint32_t nchunk;
+    uint32_t groupShift;
+    uint32_t reserved[2];
+    ChunkPattern pattern;               // period != 0: owner by division, prefix and group map are not read
+    uint32_t pad;
+};
+static_assert(sizeof(TableHeader) == 64, "the planner's scratch layout counts on a 64-byte header");
+
+// Segments one workgroup of the device-side planner takes, and its lanes.
+constexpr uint32_t kPlanThreads = 1024;
+constexpr uint32_t kPlanTiles = 8;                          // a workgroup walks up to this many tiles of kPlanThreads segments
+constexpr uint32_t kPlanSingleBlockSegs = kPlanThreads * kPlanTiles;   // up to here one workgroup plans the whole table in one launch
+
+// Words of device scratch the planner and the table kernel of a device-resident table share:
+// header | first[nseg + 1] | blockSum[blocks] | blockAlive[blocks] | group[groupCapacity].
+MF_HD constexpr inline uint32_t PlanBlocks(uint32_t nseg)
+{
+    return nseg <= kPlanSingleBlockSegs ? 1u : (nseg + kPlanThreads - 1) / kPlanThreads;
+}
+struct ScratchLayout {
+    uint32_t first;                     // word offsets
+    uint32_t blockSum;
+    uint32_t blockAlive;
+    uint32_t group;
+    uint32_t groupCapacity;             // entries
+    uint64_t words;
+};
+MF_HD constexpr inline ScratchLayout ScratchLayoutFor(uint32_t nseg, uint32_t groupCapacity)
+{
+    ScratchLayout l{};
+    const uint32_t blocks = PlanBlocks(nseg);
+    l.first = sizeof(TableHeader) / 4;
+    l.blockSum = l.first + nseg + 1;
+    l.blockAlive = l.blockSum + blocks;
+    l.group = (l.blockAlive + blocks + 3u) & ~3u;
+    l.groupCapacity = groupCapacity;
+    l.words = static_cast<uint64_t>(l.group) + groupCapacity;
+    return l;
+}
+
+// A table-driven launch: triples, prefix and group map live in device memory (under a pattern the
+// triples may sit in pinned host memory and the other two are not read).
 struct TablePlan {
     const uint64_t *triples;            // {src,dst,len} * nseg
-    const uint32_t *first;              // nseg + 1 entries, first[nseg] == nchunk; not read under a pattern
+    const uint32_t *first;              // nseg + 1 entries, first[nseg] == nchunk
+    const uint32_t *group;              // GroupCount(nchunk, groupShift) + 1 entries
+    const TableHeader *header;          // not NULL: nchunk, groupShift and pattern are read from there
     uint32_t nseg;
     uint32_t nchunk;
+    uint32_t groupShift;
     uint32_t units;
     ChunkPattern pattern;
 };

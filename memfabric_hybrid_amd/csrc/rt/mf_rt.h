@@ -72,7 +72,8 @@ int mfrt_memcpy_async(void *dst, const void *src, uint64_t bytes, void *stream);
 /* anyOrder != 0: the launch does not wait for launches queued before it on `stream` (it carries no barrier);
  * launches queued after it without that option still wait for it. */
 /* holdNanos != 0: every wave keeps its loaded data until that long after its own start (see HoldNanosFor in
- * kernels/xcopy_plan.h); honoured only by a launch of one 4 KiB chunk per workgroup. */
+ * kernels/xcopy_plan.h); honoured only by a launch of one chunk per workgroup, the chunk being 4 KiB or
+ * mfk_xcopy_window_units() units (16 KiB, copied by single waves with sixteen loads per lane in flight). */
 int mfk_xcopy_inline(const void *inlinePlan, int route, uint32_t grid, void *mask, uint32_t maskValue, void *stream,
                      int anyOrder, uint32_t holdNanos);
 /* HBM to HBM copies of hundreds of MiB: the plan's chunks are mfk_xcopy_window_units() units (16 KiB), copied by up to
@@ -81,16 +82,23 @@ int mfk_xcopy_inline(const void *inlinePlan, int route, uint32_t grid, void *mas
 uint32_t mfk_xcopy_window_units(void);
 uint32_t mfk_xcopy_window_waves(void);
 int mfk_xcopy_windowed(const void *inlinePlan, uint32_t windowMBps, void *mask, uint32_t maskValue, void *stream);
-/* pattern: NULL, or a mf::ChunkPattern (kernels/xcopy_plan.h) that the chunk counts of the segments follow;
- * then `first` is not read (may be NULL) and `triples` may live in pinned host memory. */
-int mfk_xcopy_table(const void *triples, const void *first, const void *nchunkDev, uint32_t nseg, uint32_t nchunk,
-                    uint32_t units, const void *pattern, int route, uint32_t grid, void *mask, uint32_t maskValue,
-                    void *stream);
+/* tablePlan: a mf::TablePlan (kernels/xcopy_plan.h).  Under a pattern its triples may live in pinned host
+ * memory and neither prefix nor group map is read; with a header (left by mfk_xcopy_plan on the same stream)
+ * chunk count, group shift and pattern are read from device memory and `grid` workgroups walk the chunks.
+ * holdNanos: as for mfk_xcopy_inline, for a launch of one chunk per workgroup between HBM addresses. */
+int mfk_xcopy_table(const void *tablePlan, int route, uint32_t grid, void *mask, uint32_t maskValue, void *stream,
+                    uint32_t holdNanos);
 /* One lane stores `value` (as a 64-bit word, released at system scope) into `word` once everything queued on
  * `stream` before it has finished. */
 int mfk_xcopy_signal(void *word, uint32_t value, void *stream);
-int mfk_xcopy_plan(const void *triples, uint32_t nseg, uint32_t units, void *first, void *nchunk, void *stream);
-/* The table form with its chunk prefix in a statically allocated device array instead of memory the
+/* Device-side planner for a triple table in device memory: one launch (two beyond 8192 segments) that leaves
+ * header, chunk prefix and group map in `scratch` (mfk_xcopy_plan_scratch_words(nseg, groupCapacity) 32-bit words of
+ * device memory; groupCapacity: entries of room for the group map, the more the finer) and fills *tablePlan
+ * (a mf::TablePlan) for the mfk_xcopy_table call behind it on the same stream. */
+uint64_t mfk_xcopy_plan_scratch_words(uint32_t nseg, uint32_t groupCapacity);
+int mfk_xcopy_plan(const void *triples, uint32_t nseg, uint32_t units, void *scratch, uint32_t groupCapacity, void *tablePlan,
+                   void *stream);
+/* The table form with the planner's scratch in a statically allocated device array instead of memory the
  * engine allocates: no allocation anywhere, at most MFK_STATIC_TABLE_SEGMENTS segments, one call at a
  * time per GPU.  mfk_xcopy_static_setup looks the array's address up for the current device (once per
  * device, at start-up); mfk_xcopy_table_static returns -2 when that has not happened. */

@@ -183,7 +183,7 @@ _SIGNATURES = {
     "smem_set_extern_logger": (i32, [vp]),
     "smem_set_log_level": (i32, [ctypes.c_int]),
     "smem_get_last_err_msg": (ctypes.c_char_p, []),
-    # mf_hip_dataplane.h
+    # mf_hip_dataplane.h and mf_hip_dataplane_internal.h
     "mf_xcopy_batch": (i32, [u64p, u64p, u64p, u32, i32, vp]),
     "mf_xcopy_device_table": (i32, [vp, u32, i32, vp]),
     "mf_xcopy_device_table_static": (i32, [vp, u32, i32, vp]),
@@ -192,6 +192,8 @@ _SIGNATURES = {
     "mf_copy2d_rowcol_mismatches": (u32, [u32, u32, u32, u32]),
     "mf_xcopy_thread_stream": (vp, []),
     "mf_xcopy_tune": (i32, [u32, u32, u32]),
+    "mf_xcopy_tune_table": (i32, [u32, u32]),
+    "mf_xcopy_tune_hold": (i32, [u32, i32]),
     "mf_xcopy_hold_stores": (i32, [i32]),
     "mf_xcopy_windows": (i32, [u32]),
     "mf_xcopy_choose_units": (u32, [u64, u32, i32]),

@@ -26,6 +26,10 @@ uint64_t g_launches = 0;
 uint32_t g_lastHold = 0;
 uint32_t g_lastWindow = 0;   // rate of the latest windowed launch, cleared by fake_rt_last_window()     // holdNanos of the latest inline launch
 uint64_t g_chunksRun = 0;
+bool g_skipCopies = false;       // launches count and check their plans but move nothing (tables of segments no test can back with memory)
+uint32_t g_lastTableShift = 0;   // group shift of the latest table launch that used a group map, 0 under a pattern
+uint64_t g_groupMapErrors = 0;
+uint32_t g_lastTableHold = 0;    // holdNanos of the latest table launch
 
 void *Track(uint64_t bytes, int kind)
 {
@@ -128,6 +132,10 @@ uint32_t fake_rt_last_window(void) { const uint32_t w = g_lastWindow; g_lastWind
 static int g_failLaunches = 0;
 void fake_rt_fail_launches(int n) { g_failLaunches = n; }
 uint64_t fake_rt_chunks(void) { return g_chunksRun; }
+void fake_rt_skip_copies(int on) { g_skipCopies = on != 0; }
+uint32_t fake_rt_last_table_shift(void) { return g_lastTableShift; }
+uint64_t fake_rt_group_map_errors(void) { return g_groupMapErrors; }
+uint32_t fake_rt_last_table_hold(void) { return g_lastTableHold; }
 
 int mfrt_init(int device)
 {
@@ -228,7 +236,10 @@ int mfk_xcopy_inline(const void *inlinePlan, int, uint32_t, void *mask, uint32_t
     }
     ++g_launches;
     static const bool skip = std::getenv("FAKE_RT_SKIP_COPY") != nullptr;   // host-path timing: the launch is free
-    if (skip) {
+    if (skip || g_skipCopies) {
+        if (mask != nullptr && g_skipCopies) {
+            *static_cast<uint64_t *>(mask) = maskValue;
+        }
         return 0;
     }
     for (uint32_t c = 0; c < p.nchunk; ++c) {
@@ -257,37 +268,62 @@ int mfk_xcopy_windowed(const void *inlinePlan, uint32_t windowMBps, void *mask, 
     return mfk_xcopy_inline(inlinePlan, 0, p.nchunk, mask, maskValue, stream, 0, 0);
 }
 
-int mfk_xcopy_table(const void *triples, const void *first, const void *nchunkDev, uint32_t nseg, uint32_t nchunk,
-                    uint32_t units, const void *pattern, int, uint32_t, void *mask, uint32_t maskValue, void *)
+// As the kernel: chunk count, group shift and pattern out of the header when there is one; the owner of a
+// chunk by division under a pattern, else from the two group-map entries around it and the prefix between
+// them.  A map whose entries do not bracket the owner fails the launch.
+int mfk_xcopy_table(const void *tablePlan, int, uint32_t grid, void *mask, uint32_t maskValue, void *, uint32_t holdNanos)
 {
-    const uint64_t *t = static_cast<const uint64_t *>(triples);
-    const uint32_t *f = static_cast<const uint32_t *>(first);
-    const uint32_t total = nchunkDev != nullptr ? *static_cast<const uint32_t *>(nchunkDev) : nchunk;
+    g_lastTableHold = holdNanos;
+    const mf::TablePlan &plan = *static_cast<const mf::TablePlan *>(tablePlan);
+    const uint64_t *t = plan.triples;
+    const uint32_t *f = plan.first;
+    uint32_t total = plan.nchunk;
+    uint32_t shift = plan.groupShift;
+    mf::ChunkPattern pat = plan.pattern;
+    if (plan.nseg == 0 || grid == 0 || t == nullptr) {
+        return -1;
+    }
+    if (plan.header != nullptr) {
+        total = plan.header->nchunk;
+        shift = plan.header->groupShift;
+        pat = plan.header->pattern;
+    } else if (pat.period != 0 && (pat.period > mf::kMaxPeriod || mf::PatternChunks(pat, plan.nseg) != total)) {
+        return -1;
+    }
+    if (pat.period == 0 && (f == nullptr || plan.group == nullptr || shift < mf::kGroupShiftMin || shift > 31)) {
+        return -1;
+    }
     if (g_failLaunches > 0) {
         --g_failLaunches;
         return 719;
     }
     ++g_launches;
-    uint32_t s = 0;
-    TrackTable(triples, 24ull * nseg);
-    mf::ChunkPattern pat{};
-    if (pattern != nullptr) {
-        pat = *static_cast<const mf::ChunkPattern *>(pattern);
-        if (pat.period == 0 || pat.period > mf::kMaxPeriod || mf::PatternChunks(pat, nseg) != total) {
-            return -1;
+    g_lastTableShift = pat.period != 0 ? 0 : shift;
+    TrackTable(t, 24ull * plan.nseg);
+    if (g_skipCopies) {
+        if (mask != nullptr) {
+            *static_cast<uint64_t *>(mask) = maskValue;
         }
+        return 0;
     }
-    for (uint32_t c = 0; pat.period != 0 && c < total; ++c) {   // as the kernel: owner by division, no prefix
+    for (uint32_t c = 0; pat.period != 0 && c < total; ++c) {
         uint32_t seg = 0;
         uint32_t k = 0;
         mf::PatternOwner(pat, c, seg, k);
-        RunChunk(t[3 * seg], t[3 * seg + 1], t[3 * seg + 2], k, units);
+        RunChunk(t[3 * seg], t[3 * seg + 1], t[3 * seg + 2], k, plan.units);
     }
     for (uint32_t c = 0; pat.period == 0 && c < total; ++c) {
-        while (s + 1 <= nseg && f[s + 1] <= c) {
+        const uint32_t lo = plan.group[c >> shift];
+        const uint32_t hiEx = plan.group[(c >> shift) + 1] + 1;
+        if (lo >= hiEx || hiEx > plan.nseg || f[lo] > c || f[hiEx] <= c) {
+            ++g_groupMapErrors;
+            return 720;
+        }
+        uint32_t s = lo;
+        while (s + 1 < hiEx && f[s + 1] <= c) {
             ++s;
         }
-        RunChunk(t[3 * s], t[3 * s + 1], t[3 * s + 2], c - f[s], units);
+        RunChunk(t[3 * s], t[3 * s + 1], t[3 * s + 2], c - f[s], plan.units);
     }
     if (mask != nullptr) {
         *static_cast<uint64_t *>(mask) = maskValue;
@@ -295,17 +331,66 @@ int mfk_xcopy_table(const void *triples, const void *first, const void *nchunkDe
     return 0;
 }
 
-int mfk_xcopy_plan(const void *triples, uint32_t nseg, uint32_t units, void *first, void *nchunk, void *)
+uint64_t mfk_xcopy_plan_scratch_words(uint32_t nseg, uint32_t groupCapacity)
 {
+    return mf::ScratchLayoutFor(nseg, groupCapacity).words;
+}
+
+// The device-side planner restated: same scratch layout, same header, prefix, group map and pattern rule.
+int mfk_xcopy_plan(const void *triples, uint32_t nseg, uint32_t units, void *scratch, uint32_t groupCapacity, void *tablePlan,
+                   void *)
+{
+    if (nseg == 0 || scratch == nullptr || groupCapacity < 2 || tablePlan == nullptr) {
+        return -1;
+    }
     const uint64_t *t = static_cast<const uint64_t *>(triples);
-    uint32_t *f = static_cast<uint32_t *>(first);
+    uint32_t *words = static_cast<uint32_t *>(scratch);
+    const mf::ScratchLayout at = mf::ScratchLayoutFor(nseg, groupCapacity);
+    uint32_t *f = words + at.first;
     uint32_t run = 0;
+    uint32_t alive = 0x1FEu;
+    std::vector<uint32_t> counts(nseg);
     for (uint32_t i = 0; i < nseg; ++i) {
         f[i] = run;
-        run += static_cast<uint32_t>(mf::SegmentChunks(t[3 * i + 1], t[3 * i + 2], units));
+        counts[i] = static_cast<uint32_t>(mf::SegmentChunks(t[3 * i + 1], t[3 * i + 2], units));
+        for (uint32_t p = 1; p <= mf::kMaxPeriod; ++p) {
+            if (i >= p && counts[i - p] != counts[i]) {
+                alive &= ~(1u << p);
+            }
+        }
+        run += counts[i];
     }
     f[nseg] = run;
-    *static_cast<uint32_t *>(nchunk) = run;
+    mf::TableHeader *header = reinterpret_cast<mf::TableHeader *>(words);
+    *header = mf::TableHeader{};
+    header->nchunk = run;
+    header->groupShift = mf::GroupShiftFor(run, groupCapacity);
+    if (run != 0) {
+        header->groupShift = mf::BuildGroupMap(f, nseg, words + at.group, groupCapacity);
+    }
+    if (alive != 0 && run != 0) {
+        const uint32_t period = static_cast<uint32_t>(__builtin_ctz(alive));
+        uint32_t sum = 0;
+        for (uint32_t q = 0; q < period; ++q) {
+            header->pattern.start[q] = sum;
+            sum += counts[q];
+        }
+        header->pattern.start[period] = sum;
+        if (sum != 0) {
+            header->pattern.period = period;
+            header->pattern.chunksPerPeriod = sum;
+        } else {
+            header->pattern = mf::ChunkPattern{};
+        }
+    }
+    mf::TablePlan &plan = *static_cast<mf::TablePlan *>(tablePlan);
+    plan = mf::TablePlan{};
+    plan.triples = t;
+    plan.first = f;
+    plan.group = words + at.group;
+    plan.header = header;
+    plan.nseg = nseg;
+    plan.units = units;
     ++g_launches;
     return 0;
 }
@@ -325,12 +410,13 @@ int mfk_xcopy_signal(void *word, uint32_t value, void *)
 int mfk_xcopy_static_setup(void) { return 0; }
 int mfk_xcopy_table_static(const void *triples, uint32_t nseg, uint32_t units, int route, uint32_t grid, void *stream)
 {
-    static uint32_t scratch[MFK_STATIC_TABLE_SEGMENTS + 64];
+    static std::vector<uint32_t> scratch(mf::ScratchLayoutFor(MFK_STATIC_TABLE_SEGMENTS, MFK_STATIC_TABLE_SEGMENTS).words);
     if (nseg == 0 || nseg > MFK_STATIC_TABLE_SEGMENTS) {
         return -1;
     }
-    int err = mfk_xcopy_plan(triples, nseg, units, scratch, scratch + nseg + 1, stream);
-    return err != 0 ? err : mfk_xcopy_table(triples, scratch, scratch + nseg + 1, nseg, 0, units, nullptr, route, grid, nullptr, 0, stream);
+    mf::TablePlan plan;
+    int err = mfk_xcopy_plan(triples, nseg, units, scratch.data(), MFK_STATIC_TABLE_SEGMENTS, &plan, stream);
+    return err != 0 ? err : mfk_xcopy_table(&plan, route, grid, nullptr, 0, stream, 0);
 }
 
 static uint32_t g_lastRectMates = 0;

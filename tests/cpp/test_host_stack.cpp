@@ -14,7 +14,7 @@
 
 #include <sched.h>
 
-#include "../../include/mf_hip_dataplane.h"
+#include "../../include/mf_hip_dataplane_internal.h"
 #include "../../include/mf_xcopy_api.h"
 #include "../../memfabric_hybrid_amd/csrc/host/compose_data_op.h"
 #include "../../memfabric_hybrid_amd/csrc/host/mf_log.h"
@@ -32,6 +32,9 @@ extern "C" void fake_rt_seal(void);
 extern "C" void fake_rt_fail_launches(int n);
 #include "../../include/mf_hip_copy_extend.h"
 extern "C" uint64_t fake_rt_violations(void);
+extern "C" void fake_rt_skip_copies(int on);
+extern "C" uint32_t fake_rt_last_table_shift(void);
+extern "C" uint64_t fake_rt_group_map_errors(void);
 extern "C" uint64_t fake_rt_in_flight(void);
 
 using namespace mf;
@@ -713,6 +716,29 @@ static void TestPlanners()
         }
         same = same && f1[segs.Size()] == f2[count];
         CHECK(same);
+        if (c1 != 0) {
+            // the group map brackets the owner of every chunk, at the finest shift its room allows
+            const uint32_t room[] = {GroupCapacityFor(count), static_cast<uint32_t>(c1 / 64 + 2), 17, 2};
+            for (uint32_t capacity : room) {
+                std::vector<uint32_t> group(capacity, 0xFFFFFFFFu);
+                const uint32_t shift = BuildGroupMap(f1.data(), segs.Size(), group.data(), capacity);
+                bool ok = shift >= kGroupShiftMin && GroupCount(c1, shift) + 1 <= capacity &&
+                          (shift == kGroupShiftMin || GroupCount(c1, shift - 1) + 1 > capacity);
+                uint32_t seg = 0;
+                for (uint32_t c = 0; ok && c < c1; ++c) {
+                    while (f1[seg + 1] <= c) {
+                        ++seg;
+                    }
+                    const uint32_t lo = group[c >> shift];
+                    const uint32_t hi = group[(c >> shift) + 1];
+                    ok = lo <= seg && seg <= hi && hi < segs.Size();
+                    if (shift == kGroupShiftMin) {
+                        ok = ok && hi - lo < 64;     // no empty segments after normalisation: one probe round
+                    }
+                }
+                CHECK(ok);
+            }
+        }
         InlinePlan a, b;
         NormalizeSegments(src.data(), dst.data(), len.data(), n, 1ull << 30, segs);
         const bool fitsA = BuildInlinePlan(segs, units, a);
@@ -722,6 +748,110 @@ static void TestPlanners()
             CHECK(std::memcmp(&a, &b, sizeof(a)) == 0);
         }
     }
+}
+
+// Tables the engine cannot back with memory in a test: the launches are planned and checked, nothing is moved.
+static void TestLongSegments()
+{
+    CHECK(hybm_init(0, 0) == BM_OK);
+    XcopyEngine &engine = XcopyEngine::Instance();
+    void *stream = mf_xcopy_thread_stream();
+    fake_rt_skip_copies(1);
+    const uint64_t gib = 1ull << 30;
+    const uint64_t base = 0x7f0000000000ull;
+    const uint64_t errorsBefore = fake_rt_group_map_errors();
+    {
+        // 128 segments that do not merge, one of them 4 GiB: cut into 1 GiB pieces it no longer fits the kernel-argument
+        // form, and its average length makes it a candidate for slicing.  It goes to the table form, once.
+        for (uint32_t n : {126u, 128u, 100u}) {
+            std::vector<uint64_t> src(n), dst(n), len(n, 4096);
+            for (uint32_t i = 0; i < n; ++i) {
+                src[i] = base + i * 16 * gib;
+                dst[i] = base + (2048 + i) * 16 * gib + 7;
+            }
+            len[n / 2] = 4 * gib;
+            const uint64_t before = mf_xcopy_launch_count();
+            CHECK(engine.Submit(src.data(), dst.data(), len.data(), n, MF_ROUTE_HBM, stream, nullptr, 0) == BM_OK);
+            CHECK(mf_xcopy_launch_count() - before <= 2);
+        }
+    }
+    {
+        // one segment beyond what 128 pieces of 1 GiB hold
+        uint64_t src = base;
+        uint64_t dst = base + 4096 * gib + 3;
+        uint64_t len = 129 * gib + 5;
+        const uint64_t before = mf_xcopy_launch_count();
+        CHECK(engine.Submit(&src, &dst, &len, 1, MF_ROUTE_HBM, stream, nullptr, 0) == BM_OK);
+        CHECK(mf_xcopy_launch_count() - before == 1);          // a pattern of period 1: no upload
+    }
+    {
+        // 600 long segments are cut into slices of 128; the slice that holds a 5 GiB segment takes the table form, the others the windowed one
+        const uint32_t n = 600;
+        std::vector<uint64_t> src(n), dst(n), len(n, 8u << 20);
+        for (uint32_t i = 0; i < n; ++i) {
+            src[i] = base + i * 16 * gib;
+            dst[i] = base + (2048 + i) * 16 * gib + 9;
+        }
+        len[300] = 5 * gib;
+        uint64_t word = 0;
+        const uint64_t before = mf_xcopy_launch_count();
+        (void)fake_rt_last_window();
+        CHECK(engine.Submit(src.data(), dst.data(), len.data(), n, MF_ROUTE_HBM, stream, &word, 32) == BM_OK);
+        CHECK(mf_xcopy_launch_count() - before == 6);          // 128 + 128 + (upload + table) + 128 + 88
+        CHECK(word == 32);
+        CHECK(fake_rt_last_window() != 0);
+    }
+    {
+        // a ragged table whose chunks outnumber the room of its map: coarser groups, the owner still bracketed
+        const uint32_t n = 500;     // beyond what is cut into launches of 128 segments
+        std::vector<uint64_t> src(n), dst(n), len(n);
+        for (uint32_t i = 0; i < n; ++i) {
+            src[i] = base + i * 64 * gib;
+            dst[i] = base + (2048 + i) * 64 * gib + (i % 16);
+            len[i] = (i % 7 == 0 ? 3 * gib : 70000) + i;
+        }
+        CHECK(mf_xcopy_windows(0) == BM_OK);                   // no slicing: one table
+        CHECK(engine.Submit(src.data(), dst.data(), len.data(), n, MF_ROUTE_HBM, stream, nullptr, 0) == BM_OK);
+        CHECK(fake_rt_last_table_shift() > kGroupShiftMin);
+        CHECK(mf_xcopy_windows(6800000) == BM_OK);
+    }
+    CHECK(fake_rt_group_map_errors() == errorsBefore);
+    CHECK(engine.DrainThread() == BM_OK);
+    fake_rt_skip_copies(0);
+    {
+        // the planner of a device-resident table, restated by the stand-in runtime: empty segments in runs longer than a
+        // probe round, a pattern with an empty member, a table of nothing but empty segments
+        std::mt19937_64 rng(0x6A09);
+        for (int trial = 0; trial < 60; ++trial) {
+            const uint32_t n = 1 + rng() % 700;
+            std::vector<uint8_t> from(1 << 20), to(1 << 20, 0), expect(1 << 20, 0);
+            for (auto &b : from) {
+                b = static_cast<uint8_t>(rng());
+            }
+            std::vector<uint64_t> triples(3 * n);
+            uint64_t at = 0;
+            for (uint32_t i = 0; i < n; ++i) {
+                uint64_t l = trial % 4 == 0 ? (i % 3 == 1 ? 0 : 1024) : (rng() % 5 == 0 ? rng() % 3000 : 0);
+                if (trial % 7 == 6) {
+                    l = 0;
+                }
+                if (at + l + 64 > from.size()) {
+                    l = 0;
+                }
+                triples[3 * i] = reinterpret_cast<uint64_t>(from.data()) + at + (rng() % 16);
+                triples[3 * i + 1] = reinterpret_cast<uint64_t>(to.data()) + at;
+                triples[3 * i + 2] = l;
+                std::memcpy(expect.data() + at, reinterpret_cast<void *>(triples[3 * i]), l);
+                at += l + (rng() % 48);
+            }
+            const uint64_t errors = fake_rt_group_map_errors();
+            CHECK(mf_xcopy_device_table(triples.data(), n, MF_ROUTE_HBM, stream) == BM_OK);
+            CHECK(fake_rt_group_map_errors() == errors);
+            CHECK(engine.DrainThread() == BM_OK);
+            CHECK(to == expect);
+        }
+    }
+    hybm_uninit();
 }
 
 // Copies shared with the helper thread move exactly the bytes memcpy would, also when two
@@ -1124,6 +1254,7 @@ int main()
     TestPlugin();
     TestHeldStores();
     TestWindows();
+    TestLongSegments();
     TestHostLaunchCosts();
     TestWaitOfShortQueues();
     if (g_failed != 0) {

@@ -115,6 +115,46 @@ def test_sizes_taking_turns_above_the_inline_limit(gpu, oracle, sizes, count):
     _check_d2d(gpu, oracle, 2 * half, src_off, dst_off, lens, count)
 
 
+def _held_case(rng, count, sizes, ragged):
+    """count segments whose lengths take turns over `sizes` (+ a ragged few bytes), sources and destinations at
+    random slots of the two halves of a pool; returns (pool bytes, src, dst, lens)."""
+    lens = np.array([sizes[i % len(sizes)] for i in range(count)], dtype=np.uint64)
+    if ragged:
+        lens = lens - rng.integers(0, 3000, count).astype(np.uint64)
+    slot = (int(lens.max()) + 64 + 4095) // 4096 * 4096
+    half = slot * count
+    odd = rng.integers(0, 16, count) if ragged else np.zeros(count, dtype=np.int64)
+    src = rng.permutation(count) * slot + odd
+    dst = half + rng.permutation(count) * slot + rng.integers(0, 16, count) * (1 if ragged else 0)
+    return 2 * half, src, dst, lens
+
+
+@pytest.mark.parametrize("count,sizes,ragged", [
+    (244, (131072, 16384), False),      # 4392 chunks of 4 KiB out of a table: stores of four loads held
+    (300, (65536, 20480), True),        # the same with a group map instead of a pattern
+    (32, (1 << 20,), False),            # 32 MiB in the kernel arguments: 16 KiB per wave, stores of sixteen loads held
+    (100, (400000,), True),             # the same with heads, tails and last chunks that are not whole
+    (488, (131072, 16384), False),      # 36 MB out of a table under a pattern, 16 KiB per wave
+    (400, (150000, 40000, 98304), True),  # 38 MB, ragged: group map, 16 KiB per wave
+    (1, (48 << 20,), False),            # one segment of 48 MiB
+    (1, ((40 << 20) + 12345,), True),
+    (976, (131072, 16384), False),      # 72 MB: beyond what the waves hold at once, the usual form
+])
+def test_batches_whose_stores_are_held_back(gpu, oracle, count, sizes, ragged):
+    """Batches of 4 to 64 MiB between device addresses wait with their stores until the loads of the launch are out
+    (4 KiB per wave up to 24 MiB, 16 KiB per wave beyond), whether their descriptors travel in the kernel
+    arguments or in a table.  With the wait at its rule, forced absurdly long (so that every wave does
+    wait) and off, the bytes are the oracle's."""
+    rng = np.random.default_rng(count * 7 + len(sizes))
+    pool, src, dst, lens = _held_case(rng, count, sizes, ragged)
+    for hold in (-1, 9000, 0):
+        assert gpu.mf_xcopy_hold_stores(hold) == 0
+        try:
+            _check_d2d(gpu, oracle, pool, src, dst, lens, count + hold + 1)
+        finally:
+            assert gpu.mf_xcopy_hold_stores(-1) == 0
+
+
 @pytest.mark.parametrize("count", [16384, 70000])
 def test_batches_at_and_beyond_the_reference_slot_size(gpu, oracle, count):
     """16 384 segments fill one parameter slot of the reference (hybm_data_op_sdma.cpp:25-31 there);
@@ -204,11 +244,52 @@ def test_pinned_host_routes(gpu, oracle):
         back.free()
 
 
-def test_device_resident_table(gpu, oracle):
-    pool = 48 * MIB
-    count = 3000
-    src, dst, lens = workloads.ragged_batch(77, pool, count, max_len=9000)
-    init = _random_bytes(oracle, pool, 77)
+def _device_table_case(kind, count, rng, pool):
+    """(src, dst, lens) offsets of one table for the device-side planner."""
+    half = pool // 2
+    if kind == "ragged":
+        return workloads.ragged_batch(count * 3 + 1, pool, count, max_len=min(9000, half // count - 64))
+    slot = half // count // 64 * 64
+    src = rng.permutation(count).astype(np.uint64) * np.uint64(slot)
+    dst = np.uint64(half) + rng.permutation(count).astype(np.uint64) * np.uint64(slot)
+    if kind == "pages":                       # one size: period 1
+        lens = np.full(count, min(slot - 64, 20000), dtype=np.uint64)
+    elif kind == "turns":                     # three sizes in turn, one of them empty: period 3 with an empty member
+        sizes = (min(slot - 64, 9000), 0, min(slot - 64, 4096))
+        lens = np.array([sizes[i % 3] for i in range(count)], dtype=np.uint64)
+        src += rng.integers(0, 16, count).astype(np.uint64)
+    elif kind == "gaps":                      # runs of empty segments longer than one probe round between live ones
+        lens = np.zeros(count, dtype=np.uint64)
+        live = rng.choice(count, size=max(2, count // 150), replace=False)
+        lens[live] = rng.integers(1, slot - 64, len(live)).astype(np.uint64)
+        dst += rng.integers(0, 16, count).astype(np.uint64)
+    elif kind == "empty":
+        lens = np.zeros(count, dtype=np.uint64)
+    else:                                     # "long": one segment of many groups among short ones
+        lens = rng.integers(0, min(slot - 64, 3000), count).astype(np.uint64)
+        big = count // 2
+        room = (count - big) * slot - 64
+        lens[big] = min(room, 24 * MIB)
+        lens[big + 1:] = 0
+        src[big], dst[big] = big * slot, half + big * slot
+        src[:big] = np.arange(big, dtype=np.uint64) * np.uint64(slot)
+        dst[:big] = np.uint64(half) + np.arange(big, dtype=np.uint64) * np.uint64(slot)
+    return src, dst, lens
+
+
+@pytest.mark.parametrize("kind,count", [
+    ("ragged", 3000), ("ragged", 1), ("ragged", 1000), ("ragged", 2048), ("ragged", 5000), ("ragged", 8192),
+    ("ragged", 8193), ("ragged", 40000), ("pages", 700), ("pages", 9000), ("turns", 1500), ("turns", 20001),
+    ("gaps", 6000), ("gaps", 30000), ("empty", 3000), ("long", 400), ("long", 12000),
+])
+def test_device_resident_table(gpu, oracle, kind, count):
+    """A {src, dst, len} table the host cannot read is planned on the GPU: by one workgroup up to 8192 segments (1, 2, 4 or
+    8 tiles of 1024), by one workgroup per 1024 segments beyond; chunk counts that repeat are found there and take the
+    launch without a prefix, the rest the group map, whose groups empty segments and long segments stretch."""
+    pool = 96 * MIB
+    rng = np.random.default_rng(count + len(kind))
+    src, dst, lens = _device_table_case(kind, count, rng, pool)
+    init = _random_bytes(oracle, pool, count)
     buf = gpu_util.DeviceBuffer(gpu, pool)
     table = gpu_util.DeviceBuffer(gpu, count * 24)
     try:
