@@ -297,6 +297,21 @@ def extras_block(lib, pool, dev, batches, tables, steps):
         "frac_of_hbm_peak": frac(2 * payload / reps_u[2] / 1e3, HBM_PEAK_GBPS),
         "note": "the headline loop with MF_COPY_UNORDERED_FLAG: the caller declares its batches independent and they are "
                 "launched without a barrier, so start-up and drain of consecutive batches overlap; one thread, one stream"}
+    # the same with the batches handed to submit threads of the library's (mf_xcopy_unordered_streams): one calling thread,
+    # several streams
+    fan = {}
+    for streams in (4, 6):
+        assert lib.mf_xcopy_unordered_streams(streams) == 0
+        walls = []
+        for _ in range(5):
+            w, _ = timed_steps(lib, handle, batches, g2g, ku, 0, unordered)
+            walls.append(w * 1e6 / ku)
+        fan[f"submit_threads_{streams}"] = {"us_per_batch": round(median(walls), 2), "hbm_GBps": round(2 * payload / median(walls) / 1e3, 1),
+                                     "frac_of_hbm_peak": frac(2 * payload / median(walls) / 1e3, HBM_PEAK_GBPS)}
+    assert lib.mf_xcopy_unordered_streams(0) == 0
+    fan["note"] = (f"{ku} batches with MF_COPY_UNORDERED_FLAG from ONE calling thread, planned by it and launched by submit threads of the "
+                   "library's, a stream each; wall clock from the first call to the return of smem_bm_wait (which joins their streams), median of 5")
+    out["kv122_unordered_fanout"] = fan
     # the headline loop with the held stores switched off and on in turn, in this process
     held, not_held = [], []
     for _ in range(5):

@@ -35,6 +35,22 @@ extern "C" {
  * flag cannot help (more than 128 segments, pageable memory, blocking calls) ignore it. */
 #define MF_COPY_UNORDERED_FLAG (1UL << 16)
 
+/* Who launches unordered copies.  0 or 1 (the default): the calling thread, on its own stream, without a barrier.
+ * 2 to 8: batches of up to 128 segments and 64 MiB between device addresses, submitted with MF_COPY_UNORDERED_FLAG and
+ * no stream of the caller's, are planned by the caller and handed in turn to that many submit threads of the
+ * library's, each with a stream of its own, which the GPU serves from different hardware queues: one calling
+ * thread then gets the overlap several submitting threads get (the reference gives every thread one stream,
+ * src/hybm/csrc/ts_engine/hybm_stream_manager.cpp:73-90): 9 MB batches take 4.4 / 4.1 / 3.9 / 4.0 us each with
+ * 4 / 5 / 6 / 8 submit threads against 4.5 us without, and 1.2 us of the calling thread's time instead of 3.5.  One
+ * thread that launches on several streams itself does not: the launches then cost it more than on one stream.
+ * The next copy WITHOUT the flag, smem_bm_wait / hybm_wait and every other call that uses the thread's stream first
+ * make that stream wait for them.  What changes for the caller: a synchronisation of mf_xcopy_thread_stream() that it
+ * issues itself covers the unordered copies only if it fetched the stream after the last of them (the fetch is
+ * such a call); a launch that fails is reported by that next call instead of the one that submitted it; the submit
+ * threads poll for some tens of microseconds after their last batch before they sleep, and live until hybm_uninit.
+ * Returns BM_INVALID_PARAM beyond 8. */
+int32_t mf_xcopy_unordered_streams(uint32_t count);
+
 /* ---- which memory a copy touches (selects the kernel's cache policy) ---- */
 #define MF_ROUTE_HBM 0
 #define MF_ROUTE_TO_HOST 1
@@ -53,14 +69,19 @@ int32_t mf_xcopy_batch(const uint64_t *src, const uint64_t *dst, const uint64_t 
 int32_t mf_xcopy_device_table(const void *triples, uint32_t n, int32_t route, void *stream);
 
 /* No counterpart in the reference.  mf_xcopy_device_table for callers that cannot allocate: code
- * under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  The chunk prefix
- * the kernels need lives in a statically allocated device array (132 KiB per GPU, held until the
- * process ends) instead of memory the library allocates on demand, and the call creates no stream,
- * event or staging either: `stream` is used as given (NULL is the null stream).
+ * under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  What the planner
+ * leaves for the copy launch (header, chunk prefix, group map) lives in a statically allocated device
+ * array (257 KiB per GPU, held until the process ends) instead of memory the library allocates on
+ * demand, and the call creates no stream, event or staging either: `stream` is used as given (NULL is
+ * the null stream).
  * Limits: n <= MF_XCOPY_STATIC_TABLE_MAX segments (BM_INVALID_PARAM beyond); every call on one GPU
- * uses the same array, so two calls whose kernels may run at the same time (different streams,
- * different threads) race: keep them on one stream or order them yourself.  hybm_init must have
- * run (it looks the array's address up).  Same results as mf_xcopy_device_table. */
+ * uses the same array.  Calls on one stream are ordered by the stream; a call on another stream than
+ * the call before is made to wait for that one (by an event created at hybm_init).  Outside that
+ * protection: calls under stream capture (replays of two graphs that hold such a call, or a replay
+ * and a plain call, must not run at the same time) and a graph replayed on several streams at once.
+ * Before a call is captured, one plain call must have run in the process (a kernel's first launch makes
+ * the runtime load its code, which is not capturable).  hybm_init must have run (it looks the array's
+ * address up).  Same results as mf_xcopy_device_table. */
 #define MF_XCOPY_STATIC_TABLE_MAX 32768u
 int32_t mf_xcopy_device_table_static(const void *triples, uint32_t n, int32_t route, void *stream);
 
@@ -148,6 +169,7 @@ void *mfrt_event_create(void);
 int mfrt_event_destroy(void *event);
 int mfrt_event_record(void *event, void *stream);
 int mfrt_event_sync(void *event);
+int mfrt_stream_wait_event(void *stream, void *event);
 int mfrt_event_done(void *event);
 float mfrt_event_elapsed_ms(void *start, void *stop);
 int mfrt_memcpy(void *dst, const void *src, uint64_t bytes);

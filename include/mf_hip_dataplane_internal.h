@@ -82,8 +82,10 @@ int32_t mf_xcopy_tune_table(uint32_t stageUnordered, uint32_t deviceTableWgPerCu
  * average 32 KiB and more be copied in 16 KiB chunks, one single wave each with sixteen loads per lane in flight,
  * stores held like those of the smaller batches; 0 keeps them on 4 KiB chunks that store at once.
  * pinnedExtraNanos: added to the wait of launches of more than 128 segments, whose descriptors come out of pinned
- * host memory rather than out of the kernel arguments (default 1600: a wave's loads start a link round trip later). */
-int32_t mf_xcopy_tune_hold(uint32_t deepHold, int32_t pinnedExtraNanos);
+ * host memory rather than out of the kernel arguments (default 1600: a wave's loads start a link round trip later).
+ * holdOnSideStreams: 1 lets batches launched by the submit threads (mf_xcopy_unordered_streams) hold their stores too;
+ * 0 (default): they overlap one another on purpose and store at once. */
+int32_t mf_xcopy_tune_hold(uint32_t deepHold, int32_t pinnedExtraNanos, uint32_t holdOnSideStreams);
 
 /* A combine of topK == 8 or 6 with rows of 2048 elements and more, on enough tokens to give every wave of the chip six
  * slices of 128 x 8 elements (about 3500 tokens of 7168 elements on 256 CUs), runs as waves that stay for the whole

@@ -156,6 +156,15 @@ MF_EXPORT int32_t mf_xcopy_tune(uint32_t units, uint32_t wgPerCu, uint32_t wgPer
     return BM_OK;
 }
 
+MF_EXPORT int32_t mf_xcopy_unordered_streams(uint32_t count)
+{
+    if (count > XcopyEngine::kFanStreams) {
+        MF_FAIL(BM_INVALID_PARAM, "unordered streams: 0 to " << XcopyEngine::kFanStreams << ", got " << count);
+    }
+    XcopyEngine::Instance().Tuning().unorderedStreams = count;
+    return BM_OK;
+}
+
 MF_EXPORT int32_t mf_xcopy_tune_table(uint32_t stageUnordered, uint32_t deviceTableWgPerCu)
 {
     XcopyTuning &t = XcopyEngine::Instance().Tuning();
@@ -164,11 +173,12 @@ MF_EXPORT int32_t mf_xcopy_tune_table(uint32_t stageUnordered, uint32_t deviceTa
     return BM_OK;
 }
 
-MF_EXPORT int32_t mf_xcopy_tune_hold(uint32_t deepHold, int32_t pinnedExtraNanos)
+MF_EXPORT int32_t mf_xcopy_tune_hold(uint32_t deepHold, int32_t pinnedExtraNanos, uint32_t holdOnSideStreams)
 {
     XcopyTuning &t = XcopyEngine::Instance().Tuning();
     t.deepHold = deepHold != 0;
     t.holdPinnedExtraNanos = pinnedExtraNanos;
+    t.holdOnSideStreams = holdOnSideStreams != 0;
     return BM_OK;
 }
 

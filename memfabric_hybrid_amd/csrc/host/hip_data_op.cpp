@@ -78,6 +78,7 @@ HipDataOp::Result HipDataOp::Wait(int32_t) noexcept
 void HipDataOp::CleanUp() noexcept
 {
     (void)XcopyEngine::Instance().DrainThread();
+    XcopyEngine::Instance().QuiesceSubmitters();   // batches of other threads that a submit thread has not launched yet
 }
 
 HipDataOp::Result HipDataOp::DataCopy(hybm_copy_params &params, hybm_data_copy_direction direction,
@@ -122,14 +123,18 @@ HipDataOp::Result HipDataOp::Run(void *const *src, void *const *dst, const uint6
     // Only caller-private host memory can be invisible to the GPU; pool memory is pinned by construction.
     const bool srcPageable = !se.pool && srcOnHost && AnyPageable(src, n);
     const bool dstPageable = !de.pool && dstOnHost && AnyPageable(dst, n);
-    void *stream = options.stream != nullptr ? options.stream : engine.ThreadStream();
-    if (stream == nullptr) {
-        MF_FAIL(BM_ERROR, "no stream available for the copy");
+    const bool unordered = async && (options.flags & MF_COPY_UNORDERED_FLAG) != 0;
+    void *stream = options.stream;
+    if (stream == nullptr && !(unordered && !srcPageable && !dstPageable)) {
+        // (an unordered copy without a stream of the caller's leaves the choice to the engine, which may deal it to a side stream)
+        stream = engine.ThreadStream();
+        if (stream == nullptr) {
+            MF_FAIL(BM_ERROR, "no stream available for the copy");
+        }
     }
 
     if (!srcPageable && !dstPageable) {
         static_assert(sizeof(void *) == sizeof(uint64_t), "64-bit addresses expected");
-        const bool unordered = async && (options.flags & MF_COPY_UNORDERED_FLAG) != 0;
         int ret = engine.Submit(reinterpret_cast<const uint64_t *>(src), reinterpret_cast<const uint64_t *>(dst), len, n,
                                 RouteOf(srcOnHost, dstOnHost), stream, nullptr, 0, unordered);
         if (ret != BM_OK) {

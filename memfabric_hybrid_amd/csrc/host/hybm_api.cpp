@@ -217,6 +217,7 @@ MF_EXPORT int32_t hybm_data_copy(hybm_entity_t e, hybm_copy_params *params, hybm
     if (entity == nullptr) {
         MF_FAIL(BM_INVALID_PARAM, "hybm_data_copy: unknown pool handle");
     }
+    MemEntity::SubmitScope inFlight(*entity);   // from the range check to the enqueue: a slice being freed waits for it
     bool ok = true;
     if (MustCheckDestination(direction)) {
         ok = entity->CheckAddressInEntity(params->dest, params->dataSize);
@@ -262,6 +263,7 @@ MF_EXPORT int32_t hybm_data_batch_copy(hybm_entity_t e, hybm_batch_copy_params *
     if (entity == nullptr) {
         MF_FAIL(BM_INVALID_PARAM, "hybm_data_batch_copy: unknown pool handle");
     }
+    MemEntity::SubmitScope inFlight(*entity);   // from the range check to the enqueue: a slice being freed waits for it
     const uint32_t n = params->batchSize;
     uint32_t bad = n;
     if (MustCheckDestination(direction)) {

@@ -2,6 +2,7 @@
 
 #include <cstdlib>
 #include <cstring>
+#include <thread>
 
 #include "../rt/mf_rt.h"
 #include "mf_log.h"
@@ -320,12 +321,16 @@ int MemEntity::FreeMapped(LocalSlice *slice)
     if (going == 0) {
         return BM_OK;
     }
-    // First the bound comes down, so that no new copy passes the range check for these bytes; then
-    // the copies already queued drain; only then the memory goes.  (A copy into a slice that is
-    // being freed is a caller error all the same: it may now fail its range check.)
-    deviceBacked_.store(deviceBacked_.load(std::memory_order_acquire) - going, std::memory_order_release);
+    // First the bound comes down, so that no new copy passes the range check for these bytes; then the copies that
+    // had passed it before are let through to their enqueue (and those handed to the engine's submit threads to
+    // their launch); then the GPU drains; only then the memory goes.  (A copy into a slice that is being freed
+    // is a caller error all the same: it may now fail its range check.)
+    deviceBacked_.store(deviceBacked_.load(std::memory_order_acquire) - going, std::memory_order_seq_cst);
+    while (submitsInFlight_.load(std::memory_order_seq_cst) != 0) {
+        std::this_thread::yield();
+    }
     if (dataOperator_ != nullptr) {
-        dataOperator_->CleanUp();
+        dataOperator_->CleanUp();   // also lets the engine's submit threads launch what they still hold
     }
     (void)mfrt_device_sync();
     while (!mappedSlices_.empty() && mappedSlices_.back()->released) {

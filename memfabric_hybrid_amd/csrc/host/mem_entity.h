@@ -61,6 +61,23 @@ public:
     }
 
     bool CheckAddressInEntity(const void *ptr, uint64_t length) const;
+    // Brackets range check and enqueue of one copy (see submitsInFlight_).
+    class SubmitScope {
+    public:
+        explicit SubmitScope(MemEntity &entity) : entity_(entity)
+        {
+            entity_.submitsInFlight_.fetch_add(1, std::memory_order_seq_cst);
+        }
+        ~SubmitScope()
+        {
+            entity_.submitsInFlight_.fetch_sub(1, std::memory_order_release);
+        }
+        SubmitScope(const SubmitScope &) = delete;
+        SubmitScope &operator=(const SubmitScope &) = delete;
+
+    private:
+        MemEntity &entity_;
+    };
     // The same test for every element of a batch in one pass; the index of the first element that
     // is null or leaves the entity, n when all are inside.
     uint32_t FirstOutside(void *const *ptrs, const uint64_t *lengths, uint32_t n) const;
@@ -91,6 +108,9 @@ private:
     // published with a release store after it exists, an unmap lowers the bound before it waits
     // for the GPU, so no new copy is admitted into memory that is about to go away.
     std::atomic<uint64_t> deviceBacked_{0};
+    // copies between their range check and the return of their enqueue: FreeMapped waits for the count to reach zero
+    // after it has lowered the bound, so that no copy that passed the old bound is enqueued after the GPU was drained
+    std::atomic<uint32_t> submitsInFlight_{0};
     std::atomic<uint64_t> hostBacked_{0};
     std::unique_ptr<LocalSlice> deviceSlice_;
     // Mapped-window mode (the default; MF_HIP_GVA_WINDOW=malloc turns it off): the device window is reserved address space of

@@ -3,9 +3,11 @@
 #include <algorithm>
 #include <atomic>
 #include <chrono>
+#include <condition_variable>
 #include <cstring>
 #include <memory>
 #include <mutex>
+#include <thread>
 
 #include "../../../include/mf_xcopy_types.h"
 #include "../rt/mf_rt.h"
@@ -56,6 +58,12 @@ struct ThreadLease {
     void *bounce = nullptr;
     uint64_t bounceBytes = 0;
     void *bounceEvents[XcopyEngine::kBounceEvents] = {};
+    // unordered batches handed to the submit threads: fanDirty bit w = submitter w holds batches of this thread that the
+    // thread's stream has not been made to wait for, the last of them under ticket fanTicket[w]
+    void *fanEvent[XcopyEngine::kFanStreams] = {};
+    uint64_t fanTicket[XcopyEngine::kFanStreams] = {};
+    uint32_t fanDirty = 0;
+    uint32_t fanCursor = 0;
 
     void Destroy()   // GPU calls: only from Stop(), on a thread that is alive and bound
     {
@@ -97,6 +105,13 @@ struct ThreadLease {
             (void)mfrt_free_host(doneWord);
             doneWord = nullptr;
         }
+        for (uint32_t i = 0; i < XcopyEngine::kFanStreams; ++i) {
+            if (fanEvent[i] != nullptr) {
+                (void)mfrt_event_destroy(fanEvent[i]);
+                fanEvent[i] = nullptr;
+            }
+        }
+        fanDirty = 0;
         for (void *&event : bounceEvents) {
             if (event != nullptr) {
                 (void)mfrt_event_destroy(event);
@@ -208,6 +223,216 @@ void NotePending(void *stream, uint64_t bytes)
         uint64_t &pending = t_ctx.lease->pendingBytes;
         pending = pending + bytes < pending ? ~0ull : pending + bytes;
     }
+}
+
+// Submit threads.  One thread that launches on several streams in turn gains nothing (the launches cost it more
+// than they cost on one stream: 4.6 to 5.1 us per 9 MB batch on two to four streams against 4.5 us), while several
+// threads with a stream each do overlap on the GPU (eight threads: 3.9 us).  So a caller that declares its batches
+// unordered can have them launched by up to kFanStreams threads of the library's, each with a stream of its own
+// (six of them: 3.87 us per batch with the caller's thread spending 1.2 us on each): the caller plans the batch and puts the
+// plan into a submitter's queue (a bounded queue of sequence-numbered cells, any number of producers, one consumer),
+// the submitter launches it.  A ticket per queue tells the caller how far the submitter has got.
+struct FanJob {
+    InlinePlan plan;
+    int route;
+    uint32_t grid;
+    uint32_t hold;
+};
+
+struct Submitter {
+    static constexpr uint32_t kCells = 64;
+    struct Cell {
+        std::atomic<uint64_t> seq;
+        FanJob job;
+    };
+    Cell cells[kCells];
+    std::atomic<uint64_t> head{0};          // tickets handed to producers
+    std::atomic<uint64_t> launched{0};      // jobs the thread has launched (in ticket order)
+    std::atomic<int> error{0};              // first launch error, sticky until a caller has seen it
+    std::atomic<bool> stop{false};
+    std::atomic<bool> asleep{false};
+    std::atomic<bool> ready{false};         // Run() has made its stream (or failed to)
+    std::mutex lock;
+    std::condition_variable wake;
+    void *stream = nullptr;
+    std::thread thread;
+
+    Submitter()
+    {
+        for (uint32_t i = 0; i < kCells; ++i) {
+            cells[i].seq.store(i, std::memory_order_relaxed);
+        }
+    }
+
+    // Producer: returns the job's ticket.  Waits while the queue is full.
+    uint64_t Push(const InlinePlan &plan, int route, uint32_t grid, uint32_t hold)
+    {
+        const uint64_t ticket = head.fetch_add(1, std::memory_order_relaxed);
+        Cell &cell = cells[ticket % kCells];
+        while (cell.seq.load(std::memory_order_acquire) != ticket) {
+            std::this_thread::yield();      // kCells jobs ahead: the submitter is behind, or asleep and about to be woken
+            Wake();
+        }
+        cell.job.plan = plan;
+        cell.job.route = route;
+        cell.job.grid = grid;
+        cell.job.hold = hold;
+        cell.seq.store(ticket + 1, std::memory_order_seq_cst);   // before the look at `asleep`: the submitter does both in the other order
+        Wake();
+        return ticket;
+    }
+
+    void Wake()
+    {
+        if (asleep.load(std::memory_order_seq_cst)) {
+            std::lock_guard<std::mutex> guard(lock);
+            wake.notify_one();
+        }
+    }
+
+    void Run()
+    {
+        if (mfrt_bind_thread() != 0) {
+            error.store(-1, std::memory_order_relaxed);
+        }
+        stream = mfrt_stream_create();      // by the thread that launches on it
+        ready.store(true, std::memory_order_release);
+        if (stream == nullptr) {
+            return;
+        }
+        uint64_t next = 0;
+        uint32_t idle = 0;
+        while (!stop.load(std::memory_order_acquire)) {
+            Cell &cell = cells[next % kCells];
+            if (cell.seq.load(std::memory_order_acquire) == next + 1) {
+                // a copy of its own first: the cell's lines come from the producer's core, and fetching them inside the launch
+                // call would keep whatever the runtime holds locked there for as long
+                const FanJob job = cell.job;
+                const int err = mfk_xcopy_inline(&job.plan, job.route, job.grid, nullptr, 0, stream, 0, job.hold);
+                if (err != 0) {
+                    int none = 0;
+                    (void)error.compare_exchange_strong(none, err, std::memory_order_relaxed);
+                }
+                cell.seq.store(next + kCells, std::memory_order_release);
+                ++next;
+                launched.store(next, std::memory_order_release);
+                idle = 0;
+                continue;
+            }
+            if (++idle < 20000) {           // some tens of microseconds of polling before the thread gives up its core
+                continue;
+            }
+            std::unique_lock<std::mutex> guard(lock);
+            asleep.store(true, std::memory_order_seq_cst);
+            if (cell.seq.load(std::memory_order_seq_cst) != next + 1 && !stop.load(std::memory_order_acquire)) {
+                wake.wait_for(guard, std::chrono::milliseconds(50));   // the bound is a net under the handshake, not part of it
+            }
+            asleep.store(false, std::memory_order_release);
+            idle = 0;
+        }
+    }
+};
+
+struct SubmitPool {
+    std::mutex lock;
+    Submitter *submitters[XcopyEngine::kFanStreams] = {};
+    std::atomic<uint32_t> alive{0};
+
+    // Submitter w, started on first use; NULL when its stream or thread cannot be had.
+    Submitter *Get(uint32_t w)
+    {
+        if (w < alive.load(std::memory_order_acquire)) {
+            return submitters[w];
+        }
+        std::lock_guard<std::mutex> guard(lock);
+        while (alive.load(std::memory_order_relaxed) <= w) {
+            const uint32_t at = alive.load(std::memory_order_relaxed);
+            Submitter *raw = new Submitter();
+            raw->thread = std::thread([raw] { raw->Run(); });
+            while (!raw->ready.load(std::memory_order_acquire)) {
+                std::this_thread::yield();
+            }
+            if (raw->stream == nullptr) {
+                raw->thread.join();
+                delete raw;
+                return nullptr;
+            }
+            submitters[at] = raw;
+            alive.store(at + 1, std::memory_order_release);
+        }
+        return submitters[w];
+    }
+
+    // Submitter w if it runs.
+    Submitter *Peek(uint32_t w)
+    {
+        return w < alive.load(std::memory_order_acquire) ? submitters[w] : nullptr;
+    }
+
+    // From Stop(): the threads end, their streams are drained and destroyed.
+    void Shutdown()
+    {
+        std::lock_guard<std::mutex> guard(lock);
+        const uint32_t count = alive.load(std::memory_order_relaxed);
+        for (uint32_t w = 0; w < count; ++w) {
+            Submitter *sub = submitters[w];
+            sub->stop.store(true, std::memory_order_release);
+            {
+                std::lock_guard<std::mutex> inner(sub->lock);
+                sub->wake.notify_one();
+            }
+            sub->thread.join();
+            (void)mfrt_stream_sync(sub->stream);
+            (void)mfrt_stream_destroy(sub->stream);
+            delete sub;
+            submitters[w] = nullptr;
+        }
+        alive.store(0, std::memory_order_release);
+    }
+};
+
+SubmitPool &Submitters()
+{
+    static SubmitPool *pool = new SubmitPool();   // never destroyed: see Leases()
+    return *pool;
+}
+
+// Makes `stream` (the lease's own) wait for the unordered batches the lease has handed to the submit threads: first until
+// each has been launched, then, by an event on the submitter's stream, until it has run.
+int JoinFan(ThreadLease &lease, void *stream)
+{
+    int failed = 0;
+    for (uint32_t w = 0; lease.fanDirty != 0 && w < XcopyEngine::kFanStreams; ++w) {
+        if ((lease.fanDirty & (1u << w)) == 0) {
+            continue;
+        }
+        lease.fanDirty &= ~(1u << w);
+        Submitter *sub = Submitters().Peek(w);
+        if (sub == nullptr) {
+            continue;   // stopped in the meantime: Stop() has drained it
+        }
+        while (sub->launched.load(std::memory_order_acquire) <= lease.fanTicket[w]) {
+            sub->Wake();
+            std::this_thread::yield();
+        }
+        const int err = sub->error.exchange(0, std::memory_order_relaxed);
+        failed = failed != 0 ? failed : err;
+        if (lease.fanEvent[w] == nullptr) {
+            lease.fanEvent[w] = mfrt_event_create();
+        }
+        const bool joined = lease.fanEvent[w] != nullptr && mfrt_event_record(lease.fanEvent[w], sub->stream) == 0 &&
+                            mfrt_stream_wait_event(stream, lease.fanEvent[w]) == 0;
+        if (!joined) {
+            const int syncErr = mfrt_stream_sync(sub->stream);
+            if (syncErr != 0) {
+                MF_FAIL(BM_ERROR, "unordered copies could not be awaited: " << mfrt_error_string(syncErr));
+            }
+        }
+    }
+    if (failed != 0) {
+        MF_FAIL(BM_ERROR, "an unordered copy failed to launch: " << mfrt_error_string(failed));
+    }
+    return BM_OK;
 }
 
 uint64_t RoundUp(uint64_t v, uint64_t to)
@@ -644,9 +869,11 @@ int XcopyEngine::Start(int device)
 #ifndef MF_RT_HIDDEN
     err = mfk_xcopy_static_setup();   // the device is current on this thread: mfrt_init has just selected it
     if (err != 0) {
-        MF_FAIL(BM_ERROR, "address of the static descriptor scratch not available: " << mfrt_error_string(err));
+        // only the entry point that allocates nothing needs it, and that one reports the missing set-up itself
+        MF_ERROR("address of the static descriptor scratch not available: " << mfrt_error_string(err));
     }
 #endif
+    windowsAvailable_ = mfk_xcopy_windows_available() != 0;
     started_.store(true, std::memory_order_release);
     return BM_OK;
 }
@@ -657,6 +884,7 @@ void XcopyEngine::Stop()
         return;
     }
     (void)mfrt_bind_thread();
+    Submitters().Shutdown();
     (void)mfrt_device_sync();
     Leases().DestroyAll();   // every thread's stream and staging memory, not only the caller's
     g_leaseEpoch.store(Leases().Epoch(), std::memory_order_release);
@@ -677,6 +905,9 @@ void *XcopyEngine::ThreadStream()
             return nullptr;
         }
         lease.stream = mfrt_stream_create();
+    }
+    if (lease.fanDirty != 0 && lease.stream != nullptr && JoinFan(lease, lease.stream) != BM_OK) {
+        return nullptr;
     }
     return lease.stream;
 }
@@ -739,6 +970,12 @@ int XcopyEngine::WaitStream(void *stream, uint64_t bytes)
         const uint64_t queued = t_ctx.lease->pendingBytes;
         bytes = queued > bytes ? queued : bytes;     // what else the thread has queued there is waited for as well
         t_ctx.lease->pendingBytes = 0;
+        if (t_ctx.lease->fanDirty != 0) {            // and the unordered batches on its side streams
+            const int ret = JoinFan(*t_ctx.lease, stream);
+            if (ret != BM_OK) {
+                return ret;
+            }
+        }
     }
     if (bytes != 0 && bytes <= kSpinBytes) {
         ThreadLease &lease = t_ctx.Lease();
@@ -775,6 +1012,21 @@ int XcopyEngine::WaitStream(void *stream, uint64_t bytes)
 void XcopyEngine::NoteQueued(void *stream, uint64_t bytes)
 {
     NotePending(stream, bytes);
+}
+
+void XcopyEngine::QuiesceSubmitters()
+{
+    for (uint32_t w = 0; w < kFanStreams; ++w) {
+        Submitter *sub = Submitters().Peek(w);
+        if (sub == nullptr) {
+            break;
+        }
+        const uint64_t handed = sub->head.load(std::memory_order_acquire);
+        while (sub->launched.load(std::memory_order_acquire) < handed) {
+            sub->Wake();
+            std::this_thread::yield();
+        }
+    }
 }
 
 uint64_t XcopyEngine::LaunchCount() const
@@ -832,7 +1084,7 @@ bool XcopyEngine::WindowsApply(uint64_t bytes, int route) const
     // Two such launches at a time would each cut their periods for the whole chip's rate, so a second thread with a
     // stream of its own switches the form off, as it does for the largest held launches.
     return route == MFRT_ROUTE_HBM && bytes >= kWindowMinBytes && tuning_.windowMBps != 0 && tuning_.unitsOverride == 0 &&
-           g_leasesOut.load(std::memory_order_relaxed) <= 1;
+           windowsAvailable_ && g_leasesOut.load(std::memory_order_relaxed) <= 1;
 }
 
 bool XcopyEngine::SingleSubmitter() const
@@ -858,15 +1110,45 @@ int XcopyEngine::SubmitOne(const uint64_t *src, const uint64_t *dst, const uint6
     if (mfrt_bind_thread() != 0) {
         MF_FAIL(BM_ERROR, "cannot make the GPU current on this thread");
     }
+    ThreadCtx &ctx = t_ctx;
+    const uint32_t cu = mfrt_cu_count();
+    InlinePlan plan;
     if (stream == nullptr) {
+        // An unordered batch that can travel in the kernel arguments is handed to one of the submit threads in turn, where
+        // the caller asked for them: launched there in order on the submitter's stream, beside whatever the others launch.
+        const uint32_t fanCount = tuning_.unorderedStreams < kFanStreams ? tuning_.unorderedStreams : kFanStreams;
+        if (unordered && fanCount >= 2 && n <= kInlineSegs && mask == nullptr && route == MFRT_ROUTE_HBM) {
+            uint64_t total = 0;
+            for (uint32_t i = 0; i < n; ++i) {
+                total += len[i];
+            }
+            const uint32_t fanUnits = ChooseUnits(total, cu, route, tuning_);
+            if (total <= kFanMaxBytes && BuildInlineDirect(src, dst, len, n, fanUnits, plan)) {
+                ThreadLease &lease = ctx.Lease();
+                if (lease.stream == nullptr && ThreadStream() == nullptr) {
+                    MF_FAIL(BM_ERROR, "cannot create the thread's stream");
+                }
+                const uint32_t w = lease.fanCursor % fanCount;
+                Submitter *sub = Submitters().Get(w);
+                if (sub != nullptr) {
+                    lease.fanCursor = w + 1;
+                    if (plan.nchunk != 0) {
+                        const uint32_t grid = GridFor(plan.nchunk, cu, route, tuning_);
+                        const uint32_t hold = tuning_.holdOnSideStreams ? HoldFor(plan, grid, route, false) : 0;
+                        lease.fanTicket[w] = sub->Push(plan, route, grid, hold);
+                        lease.fanDirty |= 1u << w;
+                        g_launches.fetch_add(1, std::memory_order_relaxed);
+                        NotePending(lease.stream, total);   // the thread's next wait covers the submitters' streams
+                    }
+                    return BM_OK;
+                }
+            }
+        }
         stream = ThreadStream();
         if (stream == nullptr) {
             MF_FAIL(BM_ERROR, "cannot create the thread's stream");
         }
     }
-    ThreadCtx &ctx = t_ctx;
-    const uint32_t cu = mfrt_cu_count();
-    InlinePlan plan;
     bool inlined = false;
     uint32_t units = 0;
     bool oversized = false;      // a run the 32-bit length of the inline table cannot hold is possible
@@ -936,7 +1218,7 @@ int XcopyEngine::SubmitOne(const uint64_t *src, const uint64_t *dst, const uint6
         // itself was measured under windows and is left without them: its chunk search lowers the rate it
         // sustains (6.56 TB/s at a target of 6.6, erratic at 6.8), and 262 144 pages of 32 KiB at random
         // places lose (5.1 against 5.4 TB/s).
-        if (maySlice && n > kInlineSegs && route == MFRT_ROUTE_HBM && !unordered && tuning_.windowMBps != 0 &&
+        if (maySlice && n > kInlineSegs && route == MFRT_ROUTE_HBM && !unordered && tuning_.windowMBps != 0 && windowsAvailable_ &&
             tuning_.unitsOverride == 0 && total / n >= kWindowSliceMinSegmentBytes &&
             g_leasesOut.load(std::memory_order_relaxed) <= 1) {
             for (uint32_t at = 0; at < n; at += kInlineSegs) {

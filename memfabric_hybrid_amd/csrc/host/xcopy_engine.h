@@ -47,6 +47,8 @@ struct XcopyTuning {
     uint32_t wgPerCuLink = 1;    // routes bound by the host link: workgroups per CU
     uint32_t minUnits = kXcopyThreads;   // 4 KiB: the chunk of HBM routes
     int32_t holdNanos = -1;      // stores held back in inline launches: -1 = HoldNanosFor's rule, 0 = never, else that long
+    uint32_t unorderedStreams = 0;   // unordered batches are launched by this many submit threads of the library's, a stream each (0, 1: by the caller on its own stream)
+    bool holdOnSideStreams = false;  // launches of the submit threads overlap on purpose: their stores are not held
     bool deepHold = true;        // batches of 24 to 64 MiB hold the stores of 16 KiB per wave
     int32_t holdPinnedExtraNanos = 1600;   // added to the rule for table launches, whose descriptors come from pinned host memory: a link round trip before the loads
     bool stageUnordered = true;  // the upload of a ragged table's descriptors is launched without a barrier
@@ -98,8 +100,11 @@ public:
     // No second thread holds a stream of the library: kernels that pace themselves for the whole chip may be used.
     bool SingleSubmitter() const;
 
-    // The calling thread's own stream (created on first use).
+    // The calling thread's own stream (created on first use).  Unordered batches that were handed to the submit
+    // threads are joined first: work queued on the returned stream afterwards waits for them.
     void *ThreadStream();
+    static constexpr uint32_t kFanStreams = 8;   // most submit threads for unordered batches (9 MB batches: 4 / 5 / 6 / 8 threads 4.40 / 4.07 / 3.87 / 4.00 us per batch)
+    static constexpr uint64_t kFanMaxBytes = 64ull << 20;   // larger batches gain nothing from a second queue
     // Pinned, device-mapped staging memory of the calling thread, at least `bytes` long; it lives
     // until Stop().  NULL when it cannot be allocated.
     void *ThreadBounce(uint64_t bytes);
@@ -135,6 +140,9 @@ public:
     // MFK_STATIC_TABLE_SEGMENTS segments, calls on one GPU must not overlap.
     int SubmitDeviceTableStatic(const void *triples, uint32_t n, int route, void *stream);
 
+    // Returns once every batch handed to the submit threads so far has been launched (a device wait then covers it).
+    void QuiesceSubmitters();
+
     uint64_t LaunchCount() const;
 
 private:
@@ -148,6 +156,7 @@ private:
                   void *mask, uint32_t maskValue, bool unordered, bool maySlice);
 
     XcopyTuning tuning_;
+    bool windowsAvailable_ = false;      // set by Start(): the device's constant-rate clock is known
     std::atomic<bool> started_{false};   // read by every calling thread, flipped by Start / Stop
 };
 

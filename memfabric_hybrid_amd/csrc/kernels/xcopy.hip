@@ -18,6 +18,7 @@
 #include <stdint.h>
 
 #include <atomic>
+#include <mutex>
 #include <type_traits>
 
 #include <cstdlib>
@@ -1021,6 +1022,12 @@ extern "C" uint32_t mfk_xcopy_window_units(void)
     return mf::kWindowUnits;
 }
 
+// 1 when the period of a windowed launch can be computed on the current device (its constant-rate clock is known).
+extern "C" int mfk_xcopy_windows_available(void)
+{
+    return mf::WindowPeriodTicks(2ull * mf::kWindowWaves * mf::kWindowUnits * mf::kUnitBytes, 6800000u) != 0 ? 1 : 0;
+}
+
 extern "C" uint32_t mfk_xcopy_window_waves(void)
 {
     return mf::kWindowWaves;
@@ -1112,6 +1119,13 @@ static __device__ __align__(256) uint32_t scratch[kStaticScratchWords];
 namespace {
 constexpr int kMaxDevices = 64;
 uint32_t *g_scratchOf[kMaxDevices] = {};   // device ordinal -> address of that device's copy of `scratch`
+// Calls on one GPU share the array.  The host side keeps them apart where it can without allocating: an event made at
+// set-up is recorded behind every call, and a call that comes on another stream than the one before first makes its
+// stream wait for that event.  Calls under stream capture are outside this (an event recorded there belongs to the graph).
+hipEvent_t g_staticDone[kMaxDevices] = {};
+hipStream_t g_staticLast[kMaxDevices] = {};
+bool g_staticUsed[kMaxDevices] = {};
+std::mutex g_staticLock;
 }  // namespace
 
 extern "C" int mfk_xcopy_static_setup(void)
@@ -1130,6 +1144,10 @@ extern "C" int mfk_xcopy_static_setup(void)
         return static_cast<int>(err);
     }
     g_scratchOf[dev] = static_cast<uint32_t *>(ptr);
+    if (g_staticDone[dev] == nullptr && hipEventCreateWithFlags(&g_staticDone[dev], hipEventDisableTiming) != hipSuccess) {
+        g_staticDone[dev] = nullptr;   // calls then go unguarded, as documented for callers that overlap them
+        (void)hipGetLastError();
+    }
     return 0;
 }
 
@@ -1143,12 +1161,24 @@ extern "C" int mfk_xcopy_table_static(const void *triples, uint32_t nseg, uint32
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices || g_scratchOf[dev] == nullptr) {
         return -2;   // mfk_xcopy_static_setup has not run on this device
     }
+    std::lock_guard<std::mutex> guard(g_staticLock);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+    const bool capturing = hipStreamIsCapturing(s, &capture) == hipSuccess && capture != hipStreamCaptureStatusNone;
+    const bool guarded = !capturing && g_staticDone[dev] != nullptr;
+    if (guarded && g_staticUsed[dev] && g_staticLast[dev] != s && hipStreamWaitEvent(s, g_staticDone[dev], 0) != hipSuccess) {
+        return static_cast<int>(hipGetLastError());
+    }
     // the planner writes every word the table kernel reads: nothing has to start at zero
     mf::TablePlan plan;
-    const int err = mfk_xcopy_plan(triples, nseg, units, g_scratchOf[dev], kStaticGroupCapacity, &plan, stream);
-    if (err != 0) {
-        return err;
+    int err = mfk_xcopy_plan(triples, nseg, units, g_scratchOf[dev], kStaticGroupCapacity, &plan, stream);
+    if (err == 0) {
+        err = mfk_xcopy_table(&plan, route, grid, nullptr, 0, stream, 0);
     }
-    return mfk_xcopy_table(&plan, route, grid, nullptr, 0, stream, 0);
+    if (guarded && hipEventRecord(g_staticDone[dev], s) == hipSuccess) {
+        g_staticLast[dev] = s;
+        g_staticUsed[dev] = true;
+    }
+    return err;
 }
 #endif  // MF_RT_HIDDEN

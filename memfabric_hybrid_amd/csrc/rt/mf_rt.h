@@ -61,6 +61,7 @@ void *mfrt_event_create(void);
 int mfrt_event_destroy(void *event);
 int mfrt_event_record(void *event, void *stream);
 int mfrt_event_sync(void *event);
+int mfrt_stream_wait_event(void *stream, void *event);   /* work queued on `stream` afterwards waits for the event */
 int mfrt_event_done(void *event);       /* 1 finished, 0 pending, <0 error */
 float mfrt_event_elapsed_ms(void *start, void *stop);
 
@@ -79,6 +80,7 @@ int mfk_xcopy_inline(const void *inlinePlan, int route, uint32_t grid, void *mas
 /* HBM to HBM copies of hundreds of MiB: the plan's chunks are mfk_xcopy_window_units() units (16 KiB), copied by up to
  * mfk_xcopy_window_waves() single-wave workgroups that alternate, chip-wide and by the clock, between a read half and a
  * write half of a period cut for `windowMBps` MB/s of HBM traffic (see XcopyWindowKernel). */
+int mfk_xcopy_windows_available(void);   /* 1 when the current device's constant-rate clock is known, which the period is cut by */
 uint32_t mfk_xcopy_window_units(void);
 uint32_t mfk_xcopy_window_waves(void);
 int mfk_xcopy_windowed(const void *inlinePlan, uint32_t windowMBps, void *mask, uint32_t maskValue, void *stream);

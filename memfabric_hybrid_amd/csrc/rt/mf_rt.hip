@@ -299,6 +299,11 @@ extern "C" int mfrt_event_record(void *event, void *stream)
     return Code(hipEventRecord(static_cast<hipEvent_t>(event), static_cast<hipStream_t>(stream)));
 }
 
+extern "C" int mfrt_stream_wait_event(void *stream, void *event)
+{
+    return Code(hipStreamWaitEvent(static_cast<hipStream_t>(stream), static_cast<hipEvent_t>(event), 0));
+}
+
 extern "C" int mfrt_event_sync(void *event)
 {
     return Code(hipEventSynchronize(static_cast<hipEvent_t>(event)));

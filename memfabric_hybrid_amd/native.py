@@ -192,8 +192,9 @@ _SIGNATURES = {
     "mf_copy2d_rowcol_mismatches": (u32, [u32, u32, u32, u32]),
     "mf_xcopy_thread_stream": (vp, []),
     "mf_xcopy_tune": (i32, [u32, u32, u32]),
+    "mf_xcopy_unordered_streams": (i32, [u32]),
     "mf_xcopy_tune_table": (i32, [u32, u32]),
-    "mf_xcopy_tune_hold": (i32, [u32, i32]),
+    "mf_xcopy_tune_hold": (i32, [u32, i32, u32]),
     "mf_xcopy_hold_stores": (i32, [i32]),
     "mf_xcopy_windows": (i32, [u32]),
     "mf_xcopy_choose_units": (u32, [u64, u32, i32]),
@@ -227,6 +228,7 @@ _SIGNATURES = {
     "mfrt_event_destroy": (ctypes.c_int, [vp]),
     "mfrt_event_record": (ctypes.c_int, [vp, vp]),
     "mfrt_event_sync": (ctypes.c_int, [vp]),
+    "mfrt_stream_wait_event": (ctypes.c_int, [vp, vp]),
     "mfrt_event_done": (ctypes.c_int, [vp]),
     "mfrt_event_elapsed_ms": (ctypes.c_float, [vp, vp]),
     "mfrt_memcpy": (ctypes.c_int, [vp, vp, u64]),

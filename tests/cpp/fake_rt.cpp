@@ -4,6 +4,7 @@
 // (test/ut/mock/acl_stub.cpp of the reference).  "Device" memory is host memory, a launch executes
 // its plan at once with the SAME chunk geometry the kernels use (csrc/kernels/xcopy_plan.h), streams
 // and events are tokens.  Never linked into the product libraries.
+#include <atomic>
 #include <cstdint>
 #include <cstdio>
 #include <cstdlib>
@@ -22,10 +23,10 @@ namespace {
 std::mutex g_lock;
 std::map<uint64_t, std::pair<uint64_t, int>> g_allocs;  // base -> (size, kind)
 int g_device = -1;
-uint64_t g_launches = 0;
-uint32_t g_lastHold = 0;
+std::atomic<uint64_t> g_launches{0};   // launches may come from the engine's submit threads
+std::atomic<uint32_t> g_lastHold{0};
 uint32_t g_lastWindow = 0;   // rate of the latest windowed launch, cleared by fake_rt_last_window()     // holdNanos of the latest inline launch
-uint64_t g_chunksRun = 0;
+std::atomic<uint64_t> g_chunksRun{0};
 bool g_skipCopies = false;       // launches count and check their plans but move nothing (tables of segments no test can back with memory)
 uint32_t g_lastTableShift = 0;   // group shift of the latest table launch that used a group map, 0 under a pattern
 uint64_t g_groupMapErrors = 0;
@@ -220,6 +221,9 @@ int mfrt_event_record(void *e, void *)
     return 0;
 }
 int mfrt_event_sync(void *e) { Retire(*static_cast<uint64_t *>(e)); return 0; }
+static uint64_t g_streamWaits = 0;
+extern "C" uint64_t fake_rt_stream_waits(void) { return g_streamWaits; }
+int mfrt_stream_wait_event(void *, void *) { ++g_streamWaits; return 0; }
 int mfrt_event_done(void *) { return 1; }
 float mfrt_event_elapsed_ms(void *, void *) { return 0.0f; }
 int mfrt_memcpy(void *dst, const void *src, uint64_t bytes) { std::memmove(dst, src, bytes); return 0; }
@@ -256,6 +260,7 @@ int mfk_xcopy_inline(const void *inlinePlan, int, uint32_t, void *mask, uint32_t
     return 0;
 }
 
+int mfk_xcopy_windows_available(void) { return 1; }
 uint32_t mfk_xcopy_window_units(void) { return 1024; }
 uint32_t mfk_xcopy_window_waves(void) { return 4096; }
 int mfk_xcopy_windowed(const void *inlinePlan, uint32_t windowMBps, void *mask, uint32_t maskValue, void *stream)

@@ -33,6 +33,7 @@ extern "C" void fake_rt_fail_launches(int n);
 #include "../../include/mf_hip_copy_extend.h"
 extern "C" uint64_t fake_rt_violations(void);
 extern "C" void fake_rt_skip_copies(int on);
+extern "C" uint64_t fake_rt_stream_waits(void);
 extern "C" uint32_t fake_rt_last_table_shift(void);
 extern "C" uint64_t fake_rt_group_map_errors(void);
 extern "C" uint64_t fake_rt_in_flight(void);
@@ -634,6 +635,43 @@ static void TestMappedWindow()
     CHECK(hybm_data_copy(e, &cp, HYBM_GLOBAL_DEVICE_TO_LOCAL_HOST, nullptr, 0) == BM_INVALID_PARAM);
     hybm_mem_slice_t s3 = hybm_alloc_local_memory(e, HYBM_MEM_TYPE_DEVICE, page, 0);
     CHECK(s3 != nullptr && hybm_get_slice_va(e, s3) == base);
+    {
+        // A thread keeps copying into a slice while it is freed: every copy either was enqueued before the memory went (the stand-in
+        // runtime executes it at once; a late one would touch a page without access rights and end the test) or fails its range check.
+        // With the copies unordered and handed to submit threads, which launch them later than the call returns.
+        for (uint32_t submitters : {0u, 2u}) {
+            CHECK(mf_xcopy_unordered_streams(submitters) == BM_OK);
+            hybm_mem_slice_t top = hybm_alloc_local_memory(e, HYBM_MEM_TYPE_DEVICE, 2 * page, 0);
+            CHECK(top != nullptr && hybm_get_slice_va(e, top) == base + page);
+            std::atomic<int> phase{0};
+            std::atomic<uint64_t> done{0};
+            std::atomic<uint64_t> refused{0};
+            std::atomic<uint64_t> other{0};
+            std::thread hammer([&] {
+                hybm_copy_params p{base, base + page + 4096, 65536};
+                while (phase.load() != 2) {
+                    const int ret = hybm_data_copy(e, &p, HYBM_GLOBAL_DEVICE_TO_GLOBAL_DEVICE, nullptr, ASYNC_COPY_FLAG | MF_COPY_UNORDERED_FLAG);
+                    (ret == BM_OK ? done : (ret == BM_INVALID_PARAM ? refused : other)).fetch_add(1);
+                    if (done.load() > 50) {
+                        { int zero = 0; phase.compare_exchange_strong(zero, 1); }
+                    }
+                }
+                (void)hybm_wait(e);
+            });
+            while (phase.load() == 0) {
+                std::this_thread::yield();
+            }
+            CHECK(hybm_free_local_memory(e, top, 1, 0) == BM_OK);
+            const uint64_t refusedAtFree = refused.load();
+            while (refused.load() < refusedAtFree + 50) {
+                std::this_thread::yield();
+            }
+            phase.store(2);
+            hammer.join();
+            CHECK(done.load() > 50 && other.load() == 0);
+        }
+        CHECK(mf_xcopy_unordered_streams(0) == BM_OK);
+    }
     hybm_destroy_entity(e, 0);
     hybm_uninit();
 }
@@ -748,6 +786,49 @@ static void TestPlanners()
             CHECK(std::memcmp(&a, &b, sizeof(a)) == 0);
         }
     }
+}
+
+// Unordered batches handed to submit threads: the thread's stream is made to wait for them exactly when something ordered follows.
+static void TestUnorderedFanOut()
+{
+    CHECK(hybm_init(0, 0) == BM_OK);
+    XcopyEngine &engine = XcopyEngine::Instance();
+    std::vector<uint8_t> from(1 << 20), to(1 << 20, 0);
+    Fill(from, 77);
+    auto batch = [&](uint32_t piece, bool unordered, void *stream) {
+        uint64_t s = reinterpret_cast<uint64_t>(from.data()) + piece * 4096;
+        uint64_t d = reinterpret_cast<uint64_t>(to.data()) + piece * 4096;
+        uint64_t l = 4096;
+        return engine.Submit(&s, &d, &l, 1, MF_ROUTE_HBM, stream, nullptr, 0, unordered);
+    };
+    CHECK(mf_xcopy_unordered_streams(9) == BM_INVALID_PARAM);
+    CHECK(mf_xcopy_unordered_streams(3) == BM_OK);
+    uint64_t waits = fake_rt_stream_waits();
+    for (uint32_t i = 0; i < 7; ++i) {
+        CHECK(batch(i, true, nullptr) == BM_OK);
+    }
+    CHECK(fake_rt_stream_waits() == waits);                     // nothing ordered yet: nothing joined
+    CHECK(batch(7, false, nullptr) == BM_OK);                   // an ordered copy: the three side streams are joined first
+    CHECK(fake_rt_stream_waits() == waits + 3);
+    CHECK(batch(8, false, nullptr) == BM_OK);
+    CHECK(fake_rt_stream_waits() == waits + 3);                 // nothing new to join
+    CHECK(batch(9, true, nullptr) == BM_OK);
+    CHECK(engine.DrainThread() == BM_OK);                       // the wait joins the one side stream that was used
+    CHECK(fake_rt_stream_waits() == waits + 4);
+    CHECK(batch(10, true, nullptr) == BM_OK);
+    CHECK(mf_xcopy_thread_stream() != nullptr);                 // fetching the thread's stream joins as well
+    CHECK(fake_rt_stream_waits() == waits + 5);
+    void *own = mfrt_stream_create();
+    CHECK(batch(11, true, own) == BM_OK);                       // a caller's stream is never fanned out
+    CHECK(engine.DrainThread() == BM_OK);
+    CHECK(fake_rt_stream_waits() == waits + 5);
+    CHECK(mf_xcopy_unordered_streams(0) == BM_OK);
+    CHECK(batch(12, true, nullptr) == BM_OK);
+    CHECK(engine.DrainThread() == BM_OK);
+    CHECK(fake_rt_stream_waits() == waits + 5);
+    CHECK(std::memcmp(from.data(), to.data(), 13 * 4096) == 0);
+    mfrt_stream_destroy(own);
+    hybm_uninit();
 }
 
 // Tables the engine cannot back with memory in a test: the launches are planned and checked, nothing is moved.
@@ -1255,6 +1336,7 @@ int main()
     TestHeldStores();
     TestWindows();
     TestLongSegments();
+    TestUnorderedFanOut();
     TestHostLaunchCosts();
     TestWaitOfShortQueues();
     if (g_failed != 0) {

@@ -194,11 +194,23 @@ def test_async_copy_completes_on_wait(pool, lib, oracle):
     assert np.array_equal(got, block)
 
 
-def test_unordered_batches_and_the_ordered_copy_behind_them(pool, lib, oracle):
-    """MF_COPY_UNORDERED_FLAG: batches the caller declares independent are launched without a barrier.
+@pytest.mark.parametrize("side_streams", [0, 2, 6])
+def test_unordered_batches_and_the_ordered_copy_behind_them(pool, lib, oracle, side_streams):
+    """MF_COPY_UNORDERED_FLAG: batches the caller declares independent are launched without a barrier on the
+    thread's stream, or (mf_xcopy_unordered_streams) handed in turn to submit threads of the library's.
     Sixty such batches of up to 100 ragged pieces, all with destinations of their own, then ONE ordinary
     asynchronous copy that reads what they wrote: it has to wait for all of them.  Compared with the
-    oracle applied in order; repeated so that an ordering slip has many chances to show."""
+    oracle applied in order; repeated so that an ordering slip has many chances to show.  The last round
+    ends in smem_bm_wait alone, which has to cover the submit threads' streams as well."""
+    assert lib.mf_xcopy_unordered_streams(side_streams) == 0
+    try:
+        _unordered_then_ordered(pool, lib, oracle)
+    finally:
+        assert lib.mf_xcopy_unordered_streams(0) == 0
+    assert lib.mf_xcopy_unordered_streams(9) == native.BM_INVALID_PARAM
+
+
+def _unordered_then_ordered(pool, lib, oracle):
     dev = pool.peer_rank_ptr(0, bm.BmMemType.DEVICE)
     half = 40 * MIB
     init = _rand(oracle, half, 0xD8)
@@ -226,6 +238,22 @@ def test_unordered_batches_and_the_ordered_copy_behind_them(pool, lib, oracle):
         assert pool.wait() == 0
         assert lib.mfrt_memcpy(np_ptr(got), dev + 2 * half, half) == 0
         assert np.array_equal(got, expect), rep
+    # unordered batches and nothing but the wait behind them
+    assert lib.mfrt_memset(dev + half, 0x77, half) == 0
+    expect = np.full(half, 0x77, dtype=np.uint8)
+    cursor = 0
+    for b in range(40):
+        count = int(rng.integers(1, 101))
+        lens = rng.integers(0, 20000, count)
+        src = rng.integers(0, half - 20000, count)
+        dst = cursor + np.cumsum(lens + 13) - lens - 13
+        cursor = int(dst[-1] + lens[-1] + 13)
+        assert pool.copy_data_batch((dev + src).tolist(), (dev + half + dst).tolist(), lens.tolist(), count, g2g, flags) == 0, \
+            native.last_error()
+        gpu_util.oracle_batch(oracle, init, expect, src, dst, lens)
+    assert pool.wait() == 0
+    assert lib.mfrt_memcpy(np_ptr(got), dev + half, half) == 0
+    assert np.array_equal(got, expect)
 
 
 def test_held_stores_copy_the_same_bytes(pool, lib, oracle):
