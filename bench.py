@@ -1,7 +1,8 @@
 #!/usr/bin/env python3
 """Benchmark of the MemFabric xcopy hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-extras] [--no-cpu] | --calibrate | --phases
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-extras] [--no-cpu] | --calibrate | --phases [requests ...]
+                    | --only paged|reshard|moe
 
 Headline (value / roofline): the 122-segment KV-block batch copy, device to device inside a
 4 GiB HBM pool, through smem_bm_copy_batch on one stream.  A step is one batch:
@@ -753,6 +754,8 @@ def main():
     ap.add_argument("--calibrate", action="store_true", help="only run the plain copy kernel (counter calibration)")
     ap.add_argument("--phases", action="store_true",
                     help="only run the stand-alone program that takes KV batches apart (bench_phases/mf_batch_phases) and print its JSON")
+    ap.add_argument("--only", choices=("paged", "reshard", "moe"),
+                    help="run one of the larger workloads alone and print its JSON (what the counter summaries under profiles/ are taken on)")
     ap.add_argument("phase_args", nargs="*", help="with --phases: requests per batch to take apart (1 2 4 8), default 1 and 4")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -780,6 +783,12 @@ def main():
                           "bytes_written_per_launch": 1 << 30}))
         lib.hybm_uninit()
         return
+    if args.only:
+        assert lib.hybm_init(0, 0) == 0, native.last_error()
+        fn = {"paged": extras_paged, "reshard": extras_reshard, "moe": extras_moe}[args.only]
+        print(json.dumps({args.only: fn(lib)}))
+        lib.hybm_uninit()
+        return
     assert bm.initialize("tcp://127.0.0.1:0", 1, 0) == 0, native.last_error()
     want_host = 0 if args.no_extras else POOL_BYTES
     pool = bm.create(0, want_host, POOL_BYTES)
@@ -800,6 +809,16 @@ def main():
     launch_us_by_cpu = {int(cpu_ids[i]): round(float(cpu_us[i]), 2) for i in range(max(measured, 0))}
     kept = lib.mf_pin_thread_near_gpu()
     near_cpus = sorted(os.sched_getaffinity(0))
+
+    cal_on, cal_delta, cal_rate = ctypes.c_int32(0), ctypes.c_int32(0), ctypes.c_uint32(0)
+    cal_us = (ctypes.c_float * 7)()
+    cal_ran = lib.mf_xcopy_calibration(ctypes.byref(cal_on), ctypes.byref(cal_delta), ctypes.byref(cal_rate), cal_us)
+    calibration = {"ran": bool(cal_ran), "held_stores": bool(cal_on.value), "hold_delta_ns": cal_delta.value,
+                   "window_MBps": cal_rate.value,
+                   "us_per_2196_chunk_batch_not_held_and_held_rule_minus_200_rule_plus_200": [round(v, 2) for v in cal_us[:4]],
+                   "us_per_512MiB_copy_plain_windows_default_windows_94_percent": [round(v, 1) for v in cal_us[4:]],
+                   "note": "measured by hybm_init on this GPU (about 15 ms): the wait of the held stores is the fitted rule plus the offset "
+                           "that was fastest here, the window rate the faster of two, either form off where it gains under 3 %"}
 
     wall, ms, rep_us = steady_state_headline(lib, pool.handle, batches, g2g, args.steps, args.warmup)
     per_launch_us = ms * 1e3 / args.steps
@@ -832,6 +851,7 @@ def main():
                       "and hipDeviceSynchronize follow before the next repetition), roofline: median repetition by HIP events",
             "payload_bytes": payload,
             "cu_count": lib.mfrt_cu_count(),
+            "calibration": calibration,
             "submitting_thread": {"empty_launch_us_by_cpu": launch_us_by_cpu, "runs_on_cpus": near_cpus if kept > 0 else all_cpus,
                                   "note": "mf_pin_thread_near_gpu: the CPUs from which a launch with a full argument block is "
                                           "cheapest, measured at start; the threads of the concurrency extras inherit the set"},

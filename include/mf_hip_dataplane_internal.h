@@ -72,6 +72,15 @@ uint64_t mf_xcopy_launch_count(void);
 int64_t mf_xcopy_describe_plan(const uint64_t *src, const uint64_t *dst, const uint64_t *len, uint32_t n,
                                uint32_t units, uint64_t *out, uint64_t capacity, int32_t *inlineForm);
 
+/* What hybm_init measured on its GPU and chose (about 15 ms, 1 GiB of HBM for that long; the environment variable
+ * MF_HIP_CALIBRATE=0 skips it and keeps the fitted defaults).  A batch of 2196 chunks is timed with its stores not held
+ * and held for the rule's wait and 200 ns either side: the best of the three becomes the process's offset to every wait
+ * (holdDeltaNanos), and holding is switched off where it does not beat the plain launch by 3 % (holdEnabled 0).  A copy
+ * of 512 MiB is timed without windows, at the default rate and at 94 % of it: windowMBps receives the rate in force
+ * (0: windows did not beat the plain kernel and are off).  micros (7 floats, may be NULL): the seven times in that order,
+ * us per batch / per copy.  Returns 1 if the calibration ran, 0 if not.  mf_xcopy_hold_stores / mf_xcopy_windows still
+ * override what it chose. */
+int32_t mf_xcopy_calibration(int32_t *holdEnabled, int32_t *holdDeltaNanos, uint32_t *windowMBps, float *micros);
 /* Table launches.  stageUnordered: 1 (default) launches the upload of a ragged table's descriptors without a
  * barrier, so that it runs while the caller's earlier copies still do; 0 orders it behind them.
  * deviceTableWgPerCu: workgroups per CU of the launch that copies a table in device memory, whose chunk

@@ -182,6 +182,29 @@ MF_EXPORT int32_t mf_xcopy_tune_hold(uint32_t deepHold, int32_t pinnedExtraNanos
     return BM_OK;
 }
 
+MF_EXPORT int32_t mf_xcopy_calibration(int32_t *holdEnabled, int32_t *holdDeltaNanos, uint32_t *windowMBps, float *micros)
+{
+    const XcopyCalibration &c = XcopyEngine::Instance().Calibration();
+    if (holdEnabled != nullptr) {
+        *holdEnabled = c.holdEnabled ? 1 : 0;
+    }
+    if (holdDeltaNanos != nullptr) {
+        *holdDeltaNanos = c.holdDeltaNanos;
+    }
+    if (windowMBps != nullptr) {
+        *windowMBps = XcopyEngine::Instance().Tuning().windowMBps;
+    }
+    if (micros != nullptr) {
+        for (int i = 0; i < 4; ++i) {
+            micros[i] = c.batchMicros[i];
+        }
+        for (int i = 0; i < 3; ++i) {
+            micros[4 + i] = c.copyMicros[i];
+        }
+    }
+    return c.ran ? 1 : 0;
+}
+
 MF_EXPORT int32_t mf_xcopy_hold_stores(int32_t nanos)
 {
     if (nanos < -1) {

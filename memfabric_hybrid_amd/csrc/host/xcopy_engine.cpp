@@ -4,6 +4,7 @@
 #include <atomic>
 #include <chrono>
 #include <condition_variable>
+#include <cstdlib>
 #include <cstring>
 #include <memory>
 #include <mutex>
@@ -854,6 +855,72 @@ uint64_t BuildTableDirect(const uint64_t *src, const uint64_t *dst, const uint64
     return run;
 }
 
+void ChooseCalibration(const float *batchMicros, const float *copyMicros, uint32_t defaultWindowMBps, XcopyCalibration &out)
+{
+    out = XcopyCalibration{};
+    out.windowMBps = defaultWindowMBps;
+    for (int i = 0; i < 4; ++i) {
+        out.batchMicros[i] = batchMicros[i];
+    }
+    for (int i = 0; i < 3; ++i) {
+        out.copyMicros[i] = copyMicros[i];
+    }
+    const bool batchMeasured = batchMicros[0] > 0 && batchMicros[1] > 0 && batchMicros[2] > 0 && batchMicros[3] > 0;
+    if (batchMeasured) {
+        // the rule's own wait unless a neighbour is clearly better (2 %: less is noise between rounds and between boxes)
+        int best = 2;
+        for (int v : {1, 3}) {
+            if (batchMicros[v] < batchMicros[best] * 0.98f) {
+                best = v;
+            }
+        }
+        out.holdDeltaNanos = (best - 2) * kCalibrateHoldStepNanos;
+        out.holdEnabled = batchMicros[best] <= batchMicros[0] * (1.0f - kCalibrateMinGain);
+        out.ran = true;
+    }
+    const bool copyMeasured = copyMicros[0] > 0 && copyMicros[1] > 0 && copyMicros[2] > 0;
+    if (copyMeasured) {
+        const bool slowerWins = copyMicros[2] < copyMicros[1] * 0.99f;
+        const float windowed = slowerWins ? copyMicros[2] : copyMicros[1];
+        const uint32_t rate = slowerWins ? static_cast<uint32_t>(static_cast<uint64_t>(defaultWindowMBps) * kCalibrateSlowerWindowPercent / 100)
+                                         : defaultWindowMBps;
+        out.windowMBps = windowed <= copyMicros[0] * (1.0f - kCalibrateMinWindowGain) ? rate : 0u;
+        out.ran = true;
+    }
+}
+
+int XcopyEngine::Calibrate()
+{
+    if (!Started()) {
+        return BM_NOT_INITIALIZED;
+    }
+    void *stream = ThreadStream();
+    if (stream == nullptr) {
+        return BM_ERROR;
+    }
+    const uint32_t rule = HoldNanosFor(2196, 2196, kXcopyThreads, false);
+    const uint32_t holds[3] = {rule - kCalibrateHoldStepNanos, rule, rule + kCalibrateHoldStepNanos};
+    const uint32_t defaultRate = XcopyTuning{}.windowMBps;
+    const uint32_t rates[2] = {defaultRate, static_cast<uint32_t>(static_cast<uint64_t>(defaultRate) * kCalibrateSlowerWindowPercent / 100)};
+    float us[7] = {};
+    const int err = mfk_xcopy_calibrate(stream, holds, rates, us);
+    if (err != 0) {
+        calibration_ = XcopyCalibration{};
+        MF_ERROR("calibration run failed (" << mfrt_error_string(err) << "): the fitted defaults stay");
+        return BM_ERROR;
+    }
+    ChooseCalibration(us, us + 4, defaultRate, calibration_);
+    if (calibration_.ran) {
+        tuning_.holdDeltaNanos = calibration_.holdDeltaNanos;
+        tuning_.holdCalibratedOff = !calibration_.holdEnabled;
+        if (windowsAvailable_) {
+            tuning_.windowMBps = calibration_.windowMBps;
+            windowRateCalibrated_ = true;
+        }
+    }
+    return BM_OK;
+}
+
 XcopyEngine &XcopyEngine::Instance()
 {
     static XcopyEngine engine;
@@ -874,6 +941,28 @@ int XcopyEngine::Start(int device)
     }
 #endif
     windowsAvailable_ = mfk_xcopy_windows_available() != 0;
+    tuning_.holdDeltaNanos = 0;
+    tuning_.holdCalibratedOff = false;
+    if (windowRateCalibrated_) {   // what an earlier start of this process chose does not outlive it
+        tuning_.windowMBps = XcopyTuning{}.windowMBps;
+        windowRateCalibrated_ = false;
+    }
+    calibration_ = XcopyCalibration{};
+    started_.store(true, std::memory_order_release);
+    {
+        // every copy kernel once, then the timing rules checked against this GPU
+        void *stream = ThreadStream();
+        if (stream == nullptr || mfk_xcopy_prelaunch(stream) != 0) {
+            MF_ERROR("the copy kernels could not be launched once at start");
+        }
+        const char *env = std::getenv("MF_HIP_CALIBRATE");
+        if (stream != nullptr && !(env != nullptr && env[0] == '0')) {
+            (void)Calibrate();
+        }
+        if (stream != nullptr) {
+            (void)mfrt_stream_sync(stream);
+        }
+    }
     started_.store(true, std::memory_order_release);
     return BM_OK;
 }
@@ -1048,7 +1137,14 @@ uint32_t XcopyEngine::HoldFor(const InlinePlan &plan, uint32_t grid, int route, 
         return 0;
     }
     const uint32_t rule = HoldNanosFor(plan.nchunk, grid, plan.units, plan.first[1] == kNoChunk && plan.units != kDeepUnits);
-    return rule != 0 && tuning_.holdNanos > 0 ? static_cast<uint32_t>(tuning_.holdNanos) : rule;
+    if (rule == 0 || tuning_.holdNanos > 0) {
+        return rule != 0 ? static_cast<uint32_t>(tuning_.holdNanos) : 0;
+    }
+    if (tuning_.holdCalibratedOff) {
+        return 0;
+    }
+    const int64_t with = static_cast<int64_t>(rule) + tuning_.holdDeltaNanos;
+    return with > 0 ? static_cast<uint32_t>(with) : 0;
 }
 
 // Hold of a table launch under a pattern: its waves fetch their descriptors across the host link and issue their
@@ -1068,7 +1164,10 @@ uint32_t XcopyEngine::HoldForTable(uint32_t nchunk, uint32_t grid, uint32_t unit
     if (tuning_.holdNanos > 0) {
         return static_cast<uint32_t>(tuning_.holdNanos);
     }
-    const int64_t with = static_cast<int64_t>(rule) + tuning_.holdPinnedExtraNanos;
+    if (tuning_.holdCalibratedOff) {
+        return 0;
+    }
+    const int64_t with = static_cast<int64_t>(rule) + tuning_.holdPinnedExtraNanos + tuning_.holdDeltaNanos;
     return with > 0 ? static_cast<uint32_t>(with) : 0;
 }
 

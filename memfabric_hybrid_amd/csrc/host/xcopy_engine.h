@@ -46,7 +46,9 @@ struct XcopyTuning {
     uint32_t wgPerCu = 0;        // HBM routes: grid cap in workgroups per CU, 0 = one workgroup per chunk
     uint32_t wgPerCuLink = 1;    // routes bound by the host link: workgroups per CU
     uint32_t minUnits = kXcopyThreads;   // 4 KiB: the chunk of HBM routes
-    int32_t holdNanos = -1;      // stores held back in inline launches: -1 = HoldNanosFor's rule, 0 = never, else that long
+    int32_t holdNanos = -1;      // stores held back in inline launches: -1 = HoldNanosFor's rule (+ holdDeltaNanos), 0 = never, else that long
+    int32_t holdDeltaNanos = 0;  // added to the rule's wait: what the calibration at start found best on this GPU
+    bool holdCalibratedOff = false;   // the calibration found no gain in holding stores on this GPU
     uint32_t unorderedStreams = 0;   // unordered batches are launched by this many submit threads of the library's, a stream each (0, 1: by the caller on its own stream)
     bool holdOnSideStreams = false;  // launches of the submit threads overlap on purpose: their stores are not held
     bool deepHold = true;        // batches of 24 to 64 MiB hold the stores of 16 KiB per wave
@@ -60,6 +62,22 @@ struct XcopyTuning {
 // (XcopyWindowKernel has the measurements; 512 MiB gains 2 %, 256 MiB nothing).
 constexpr uint64_t kWindowMinBytes = 512ull << 20;
 constexpr uint64_t kWindowSliceMinSegmentBytes = 4ull << 20;   // tables of segments this long on average are cut into windowed launches
+
+// What Start() measured on the GPU it runs on and chose from it (XcopyEngine::Calibrate).
+struct XcopyCalibration {
+    bool ran = false;               // false: skipped (MF_HIP_CALIBRATE=0), failed, or not run yet: the fitted defaults apply
+    bool holdEnabled = true;        // the held stores beat the launch that stores at once by kCalibrateMinGain
+    int32_t holdDeltaNanos = 0;     // added to every wait HoldNanosFor gives
+    uint32_t windowMBps = 0;        // rate the read and write windows are cut for; 0: the form lost against the plain kernel
+    float batchMicros[4] = {};      // 2196-chunk batch: not held, rule - step, rule, rule + step
+    float copyMicros[3] = {};       // 512 MiB copy: no windows, default rate, reduced rate
+};
+constexpr int32_t kCalibrateHoldStepNanos = 200;
+constexpr float kCalibrateMinGain = 0.03f;          // held stores that do not gain this much over the plain launch are switched off
+constexpr float kCalibrateMinWindowGain = 0.005f;   // windows stay unless they lose: on the 512 MiB that is measured they gain least (2 to 5 %, 8 % on 1 GiB)
+constexpr uint32_t kCalibrateSlowerWindowPercent = 94;   // the second window rate tried, in percent of the default
+// The choice, from the measured times alone (microseconds; a time of 0 means "not measured" and leaves the default).
+void ChooseCalibration(const float *batchMicros, const float *copyMicros, uint32_t defaultWindowMBps, XcopyCalibration &out);
 
 uint32_t ChooseUnits(uint64_t totalBytes, uint32_t cuCount, int route, const XcopyTuning &tuning);
 
@@ -94,6 +112,15 @@ public:
     {
         return tuning_;
     }
+    const XcopyCalibration &Calibration() const
+    {
+        return calibration_;
+    }
+    // Measures, on the calling thread's stream, the 2196-chunk batch with its stores not held and held for the rule's wait
+    // and kCalibrateHoldStepNanos either side of it, and a 512 MiB copy without windows and at two window rates; keeps
+    // the best wait (or none) and the best rate (or none) for the process.  About 15 ms and 1 GiB of HBM for its duration.
+    // Start() runs it unless the environment says MF_HIP_CALIBRATE=0.
+    int Calibrate();
 
     // Whether an ordered launch that moves `bytes` on `route` takes the form with read and write windows.
     bool WindowsApply(uint64_t bytes, int route) const;
@@ -156,6 +183,8 @@ private:
                   void *mask, uint32_t maskValue, bool unordered, bool maySlice);
 
     XcopyTuning tuning_;
+    XcopyCalibration calibration_;
+    bool windowRateCalibrated_ = false;  // tuning_.windowMBps holds what Calibrate() chose, not a caller's setting
     bool windowsAvailable_ = false;      // set by Start(): the device's constant-rate clock is known
     std::atomic<bool> started_{false};   // read by every calling thread, flipped by Start / Stop
 };

@@ -20,6 +20,7 @@
 #include <atomic>
 #include <mutex>
 #include <type_traits>
+#include <vector>
 
 #include <cstdlib>
 
@@ -1104,6 +1105,166 @@ extern "C" int mfk_xcopy_plan(const void *triples, uint32_t nseg, uint32_t units
     plan.nseg = nseg;
     plan.units = units;
     return mf::LaunchPlanner(plan.triples, nseg, units, words, groupCapacity, static_cast<hipStream_t>(stream));
+}
+
+// Every copy kernel once, on plans that hold nothing, so that a caller who captures a stream later finds the code of
+// this file loaded and every kernel known to the runtime (a kernel's first launch is not capturable).
+extern "C" int mfk_xcopy_prelaunch(void *stream)
+{
+    using namespace mf;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    InlinePlan empty{};
+    for (uint32_t i = 0; i < kInlineSegs; ++i) {
+        empty.first[i] = kNoChunk;
+    }
+    empty.units = kXcopyThreads;
+    TablePlan none{};
+    none.nseg = 1;
+    none.units = kXcopyThreads;
+    none.groupShift = kGroupShiftMin;
+    for (int route = MFRT_ROUTE_HBM; route <= MFRT_ROUTE_FROM_HOST; ++route) {
+        (void)WithPolicy(PolicyOf(route), [&](auto ntLoad, auto store) {
+            constexpr bool kNt = decltype(ntLoad)::value;
+            constexpr int kSt = decltype(store)::value;
+            hipLaunchKernelGGL((XcopyInlineKernel<kNt, kSt, kHoldNone>), dim3(1), dim3(64), 0, s, empty, 0u);
+            hipLaunchKernelGGL((XcopySingleKernel<kNt, kSt, kHoldNone>), dim3(1), dim3(64), 0, s, 0ull, 0ull, 0u, 0u, kXcopyThreads, 0u);
+            hipLaunchKernelGGL((XcopyTableKernel<kNt, kSt, false, kHoldNone>), dim3(1), dim3(64), 0, s, none, 0u);
+            if (route == MFRT_ROUTE_HBM) {
+                hipLaunchKernelGGL((XcopyInlineKernel<kNt, kSt, kHoldShallow>), dim3(1), dim3(64), 0, s, empty, 1u);
+                hipLaunchKernelGGL((XcopyInlineKernel<kNt, kSt, kHoldDeep>), dim3(1), dim3(64), 0, s, empty, 1u);
+                hipLaunchKernelGGL((XcopySingleKernel<kNt, kSt, kHoldShallow>), dim3(1), dim3(64), 0, s, 0ull, 0ull, 0u, 0u, kXcopyThreads, 1u);
+                hipLaunchKernelGGL((XcopySingleKernel<kNt, kSt, kHoldDeep>), dim3(1), dim3(64), 0, s, 0ull, 0ull, 0u, 0u, kWindowUnits, 1u);
+                hipLaunchKernelGGL((XcopyTableKernel<kNt, kSt, false, kHoldShallow>), dim3(1), dim3(64), 0, s, none, 1u);
+                hipLaunchKernelGGL((XcopyTableKernel<kNt, kSt, false, kHoldDeep>), dim3(1), dim3(64), 0, s, none, 1u);
+                hipLaunchKernelGGL((XcopyWindowKernel<kNt, kSt>), dim3(1), dim3(64), 0, s, empty, 64u, NextWindowSeq());
+            }
+            return 0;
+        });
+    }
+    return static_cast<int>(hipGetLastError());
+}
+
+// Calibration workloads, timed by events on `stream` (see XcopyEngine::Calibrate for what is chosen from them).
+// out[0 .. 3]: microseconds per batch of 122 segments (61 x 128 KiB and 16 KiB in turn, 2196 chunks, 32 tables in turn
+// inside 1 GiB of scratch) without a hold and held for holdNanos[0 .. 2]; out[4 .. 6]: microseconds per copy of 512 MiB by
+// the kernel without windows and in windows cut for windowMBps[0 .. 1].  The minimum of three rounds each.
+extern "C" int mfk_xcopy_calibrate(void *stream, const uint32_t *holdNanos, const uint32_t *windowMBps, float *out)
+{
+    using namespace mf;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const uint64_t half = 512ull << 20;
+    char *scratchMem = nullptr;
+    hipError_t err = hipMalloc(&scratchMem, 2 * half);
+    if (err != hipSuccess) {
+        return static_cast<int>(err);
+    }
+    hipEvent_t e0 = nullptr;
+    hipEvent_t e1 = nullptr;
+    auto release = [&](hipError_t code) {
+        (void)hipStreamSynchronize(s);
+        if (e0 != nullptr) {
+            (void)hipEventDestroy(e0);
+        }
+        if (e1 != nullptr) {
+            (void)hipEventDestroy(e1);
+        }
+        (void)hipFree(scratchMem);
+        return static_cast<int>(code);
+    };
+    if ((err = hipMemsetAsync(scratchMem, 0x5A, 2 * half, s)) != hipSuccess || (err = hipEventCreate(&e0)) != hipSuccess ||
+        (err = hipEventCreate(&e1)) != hipSuccess) {
+        return release(err);
+    }
+    // 32 tables of K and V blocks, every block in a 128 KiB slot of its own: sources in the lower half, destinations in
+    // the upper; together they touch 576 MB, more than the last-level cache holds, as a caller's batches do
+    constexpr uint32_t kTables = 32;
+    constexpr uint32_t kSlotsPerHalf = 4096;
+    std::vector<InlinePlan> plans(kTables);
+    const uint64_t base = reinterpret_cast<uint64_t>(scratchMem);
+    for (uint32_t t = 0; t < kTables; ++t) {
+        InlinePlan &plan = plans[t];
+        uint32_t run = 0;
+        for (uint32_t i = 0; i < kInlineSegs; ++i) {
+            if (i < 122) {
+                const uint32_t len = (i & 1u) != 0 ? 16384u : 131072u;
+                const uint32_t at = t * 122 + i;
+                plan.src[i] = base + static_cast<uint64_t>((at * 1103u + 17u) % kSlotsPerHalf) * (128u << 10);
+                plan.dst[i] = base + half + static_cast<uint64_t>((at * 757u + 5u) % kSlotsPerHalf) * (128u << 10);
+                plan.len[i] = len;
+                plan.first[i] = run;
+                run += len / 4096;
+            } else {
+                plan.src[i] = plan.dst[i] = 0;
+                plan.len[i] = 0;
+                plan.first[i] = kNoChunk;
+            }
+        }
+        plan.nchunk = run;
+        plan.units = kXcopyThreads;
+    }
+    InlinePlan big{};
+    for (uint32_t i = 0; i < kInlineSegs; ++i) {
+        big.first[i] = kNoChunk;
+    }
+    big.src[0] = base;
+    big.dst[0] = base + half;
+    big.len[0] = static_cast<uint32_t>(half);
+    big.first[0] = 0;
+    auto timed = [&](auto launch, int warm, int count, float &best) -> hipError_t {
+        for (int i = 0; i < warm; ++i) {
+            launch(i);
+        }
+        hipError_t code = hipEventRecord(e0, s);
+        for (int i = 0; i < count && code == hipSuccess; ++i) {
+            launch(i);
+        }
+        if (code == hipSuccess) {
+            code = hipEventRecord(e1, s);
+        }
+        if (code == hipSuccess) {
+            code = hipEventSynchronize(e1);
+        }
+        float ms = 0.0f;
+        if (code == hipSuccess) {
+            code = hipEventElapsedTime(&ms, e0, e1);
+        }
+        if (code == hipSuccess) {
+            const float us = ms * 1000.0f / static_cast<float>(count);
+            best = best == 0.0f || us < best ? us : best;
+        }
+        return code != hipSuccess ? code : hipGetLastError();
+    };
+    for (int i = 0; i < 7; ++i) {
+        out[i] = 0.0f;
+    }
+    for (int round = 0; round < 3; ++round) {
+        for (int v = 0; v < 4; ++v) {
+            const uint32_t nanos = v == 0 ? 0u : holdNanos[v - 1];
+            err = timed([&](int i) { (void)LaunchInline<true, kStoreStream>(plans[i % kTables], plans[0].nchunk, 64, s, false, nanos); }, 32, 128,
+                        out[v]);
+            if (err != hipSuccess) {
+                return release(err);
+            }
+        }
+    }
+    for (int round = 0; round < 3; ++round) {
+        for (int v = 0; v < 3; ++v) {
+            if (v == 0) {
+                big.units = kXcopyThreads;
+                big.nchunk = static_cast<uint32_t>(half / (kXcopyThreads * kUnitBytes));
+                err = timed([&](int) { (void)LaunchInline<true, kStoreStream>(big, big.nchunk, 64, s, false, 0); }, 1, 2, out[4]);
+            } else {
+                big.units = kWindowUnits;
+                big.nchunk = static_cast<uint32_t>(half / (kWindowUnits * kUnitBytes));
+                const uint32_t rate = windowMBps[v - 1];
+                err = timed([&](int) { (void)LaunchWindowed<true, kStoreStream>(big, kWindowWaves, rate, s); }, 1, 2, out[4 + v]);
+            }
+            if (err != hipSuccess) {
+                return release(err);
+            }
+        }
+    }
+    return release(hipSuccess);
 }
 
 #ifndef MF_RT_HIDDEN   // the plugin library has no entry point that needs it

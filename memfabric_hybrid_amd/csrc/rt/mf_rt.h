@@ -90,6 +90,12 @@ int mfk_xcopy_windowed(const void *inlinePlan, uint32_t windowMBps, void *mask, 
  * holdNanos: as for mfk_xcopy_inline, for a launch of one chunk per workgroup between HBM addresses. */
 int mfk_xcopy_table(const void *tablePlan, int route, uint32_t grid, void *mask, uint32_t maskValue, void *stream,
                     uint32_t holdNanos);
+/* Launches every copy kernel once on empty plans (a kernel's first launch is not capturable into a HIP graph). */
+int mfk_xcopy_prelaunch(void *stream);
+/* Times the calibration workloads on `stream` with HIP events, in 1 GiB of device memory it allocates and frees:
+ * out[0 .. 3] = us per 2196-chunk batch without a hold and held for holdNanos[0 .. 2]; out[4 .. 6] = us per 512 MiB
+ * copy without windows and in windows cut for windowMBps[0 .. 1].  0, or a HIP error number. */
+int mfk_xcopy_calibrate(void *stream, const uint32_t *holdNanos, const uint32_t *windowMBps, float *out);
 /* One lane stores `value` (as a 64-bit word, released at system scope) into `word` once everything queued on
  * `stream` before it has finished. */
 int mfk_xcopy_signal(void *word, uint32_t value, void *stream);

@@ -261,6 +261,18 @@ int mfk_xcopy_inline(const void *inlinePlan, int, uint32_t, void *mask, uint32_t
 }
 
 int mfk_xcopy_windows_available(void) { return 1; }
+int mfk_xcopy_prelaunch(void *) { return 0; }
+// The calibration "measures" what the test has put here (all zero: nothing measured, the defaults stay).
+static float g_calibration[7] = {};
+static uint32_t g_calibrationHolds[3] = {};
+extern "C" void fake_rt_set_calibration(const float *us) { std::memcpy(g_calibration, us, sizeof(g_calibration)); }
+extern "C" const uint32_t *fake_rt_calibration_holds(void) { return g_calibrationHolds; }
+int mfk_xcopy_calibrate(void *, const uint32_t *holdNanos, const uint32_t *, float *out)
+{
+    std::memcpy(g_calibrationHolds, holdNanos, sizeof(g_calibrationHolds));
+    std::memcpy(out, g_calibration, sizeof(g_calibration));
+    return 0;
+}
 uint32_t mfk_xcopy_window_units(void) { return 1024; }
 uint32_t mfk_xcopy_window_waves(void) { return 4096; }
 int mfk_xcopy_windowed(const void *inlinePlan, uint32_t windowMBps, void *mask, uint32_t maskValue, void *stream)

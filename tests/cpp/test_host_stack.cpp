@@ -34,6 +34,8 @@ extern "C" void fake_rt_fail_launches(int n);
 extern "C" uint64_t fake_rt_violations(void);
 extern "C" void fake_rt_skip_copies(int on);
 extern "C" uint64_t fake_rt_stream_waits(void);
+extern "C" void fake_rt_set_calibration(const float *us);
+extern "C" const uint32_t *fake_rt_calibration_holds(void);
 extern "C" uint32_t fake_rt_last_table_shift(void);
 extern "C" uint64_t fake_rt_group_map_errors(void);
 extern "C" uint64_t fake_rt_in_flight(void);
@@ -788,6 +790,82 @@ static void TestPlanners()
     }
 }
 
+// The choice hybm_init makes from what it measures on its GPU.
+static void TestCalibration()
+{
+    const uint32_t rate = XcopyTuning{}.windowMBps;
+    XcopyCalibration c;
+    {   // the usual picture: the rule's wait is best, held stores gain 14 %, windows 7 %
+        const float batch[4] = {5.30f, 4.62f, 4.55f, 4.60f};
+        const float copy[3] = {172.0f, 160.0f, 163.0f};
+        ChooseCalibration(batch, copy, rate, c);
+        CHECK(c.ran && c.holdEnabled && c.holdDeltaNanos == 0 && c.windowMBps == rate);
+    }
+    {   // a GPU whose loads land later: the longer wait wins clearly; windows only hold at the lower rate
+        const float batch[4] = {5.30f, 4.95f, 4.80f, 4.60f};
+        const float copy[3] = {172.0f, 171.0f, 161.0f};
+        ChooseCalibration(batch, copy, rate, c);
+        CHECK(c.holdEnabled && c.holdDeltaNanos == kCalibrateHoldStepNanos && c.windowMBps == static_cast<uint32_t>(static_cast<uint64_t>(rate) * 94 / 100));
+    }
+    {   // a neighbour that is better by less than 1 % does not move the wait
+        const float batch[4] = {5.30f, 4.53f, 4.55f, 4.60f};
+        const float copy[3] = {0.0f, 0.0f, 0.0f};
+        ChooseCalibration(batch, copy, rate, c);
+        CHECK(c.ran && c.holdDeltaNanos == 0 && c.windowMBps == rate);       // windows not measured: the default stays
+    }
+    {   // a busy or capped chip: holding gains 2 %, windows lose: both off
+        const float batch[4] = {5.30f, 5.25f, 5.20f, 5.28f};
+        const float copy[3] = {172.0f, 175.0f, 174.0f};
+        ChooseCalibration(batch, copy, rate, c);
+        CHECK(c.ran && !c.holdEnabled && c.windowMBps == 0);
+    }
+    {   // nothing measured
+        const float none[4] = {0, 0, 0, 0};
+        ChooseCalibration(none, none, rate, c);
+        CHECK(!c.ran && c.holdEnabled && c.holdDeltaNanos == 0 && c.windowMBps == rate);
+    }
+    // through hybm_init: the engine applies what it chose, and mf_xcopy_hold_stores(-1) means the calibrated rule
+    const float shorter[7] = {5.30f, 4.40f, 4.60f, 4.70f, 172.0f, 160.0f, 163.0f};
+    fake_rt_set_calibration(shorter);
+    CHECK(hybm_init(0, 0) == BM_OK);
+    const uint32_t rule = HoldNanosFor(2196, 2196, 256, false);
+    CHECK(fake_rt_calibration_holds()[0] == rule - 200 && fake_rt_calibration_holds()[1] == rule && fake_rt_calibration_holds()[2] == rule + 200);
+    int32_t enabled = -1;
+    int32_t delta = 0;
+    uint32_t mbps = 0;
+    float micros[7] = {};
+    CHECK(mf_xcopy_calibration(&enabled, &delta, &mbps, micros) == 1);
+    CHECK(enabled == 1 && delta == -200 && mbps == rate && micros[1] == 4.40f && micros[5] == 160.0f);
+    {
+        std::vector<uint8_t> from(12 << 20), to(12 << 20);
+        const uint64_t fromBase = (reinterpret_cast<uint64_t>(from.data()) + 4095) & ~4095ull;
+        const uint64_t toBase = (reinterpret_cast<uint64_t>(to.data()) + 4095) & ~4095ull;
+        std::vector<uint64_t> s(122), d(122), l(122);
+        uint64_t at = 0;
+        for (uint32_t i = 0; i < 122; ++i) {
+            l[i] = (i & 1) != 0 ? 16384 : 131072;
+            s[i] = fromBase + at + 4096;    // a page between neighbours on one side: no merging
+            d[i] = toBase + at;
+            at += l[i] + 4096 * (1 + i % 2);
+        }
+        CHECK(XcopyEngine::Instance().Submit(s.data(), d.data(), l.data(), 122, MF_ROUTE_HBM, nullptr, nullptr, 0) == BM_OK);
+        CHECK(fake_rt_last_hold() == HoldNanosFor(2196, 2196, 256, false) - 200);
+    }
+    hybm_uninit();
+    const float lost[7] = {5.30f, 5.29f, 5.31f, 5.30f, 172.0f, 175.0f, 176.0f};
+    fake_rt_set_calibration(lost);
+    CHECK(hybm_init(0, 0) == BM_OK);
+    CHECK(mf_xcopy_calibration(&enabled, &delta, &mbps, nullptr) == 1 && enabled == 0 && mbps == 0);
+    hybm_uninit();
+    setenv("MF_HIP_CALIBRATE", "0", 1);
+    CHECK(hybm_init(0, 0) == BM_OK);
+    CHECK(mf_xcopy_calibration(&enabled, &delta, &mbps, nullptr) == 0 && enabled == 1 && delta == 0 && mbps == rate);
+    hybm_uninit();
+    unsetenv("MF_HIP_CALIBRATE");
+    const float none[7] = {};
+    fake_rt_set_calibration(none);
+}
+
 // Unordered batches handed to submit threads: the thread's stream is made to wait for them exactly when something ordered follows.
 static void TestUnorderedFanOut()
 {
@@ -1336,6 +1414,7 @@ int main()
     TestHeldStores();
     TestWindows();
     TestLongSegments();
+    TestCalibration();
     TestUnorderedFanOut();
     TestHostLaunchCosts();
     TestWaitOfShortQueues();
