@@ -73,10 +73,17 @@ MF_EXPORT int32_t mf_xcopy_2d_batch(const mf_copy2d_desc *descs, uint32_t n, int
     RectPlan plan;
     uint32_t used = 0;
     uint64_t run = 0;
+    // the same launch in the chunks of the windowed form (RectWindowChunks), which a launch of kWindowMinBytes and
+    // more between device addresses takes where the segment path would
+    uint32_t firstWindowed[kRectInline];
+    uint64_t runWindowed = 0;
+    uint64_t bytes = 0;
+    bool allWindowable = true;
     auto flush = [&]() -> int {
         if (used == 0) {
             return 0;
         }
+        const bool windowed = allWindowable && runWindowed < 0xFFFFFFFFull && engine.WindowsApply(bytes, route);
         for (uint32_t i = used; i < kRectInline; ++i) {
             plan.src[i] = plan.dst[i] = 0;
             plan.spitchUnits[i] = plan.dpitchUnits[i] = plan.widthUnits[i] = plan.height[i] = 0;
@@ -85,12 +92,24 @@ MF_EXPORT int32_t mf_xcopy_2d_batch(const mf_copy2d_desc *descs, uint32_t n, int
             plan.first[i] = 0xFFFFFFFFu;
             plan.mate[i] = 0;
         }
-        plan.nchunk = static_cast<uint32_t>(run);
-        const uint32_t perCu = engine.Tuning().wgPerCu;   // 0: one workgroup per row group
-        const uint64_t cap = perCu == 0 ? run : static_cast<uint64_t>(cu) * perCu;
-        int err = mfk_copy2d(&plan, static_cast<uint32_t>(run < cap ? run : cap), stream);
+        int err;
+        if (windowed) {
+            for (uint32_t i = 0; i < used; ++i) {
+                plan.first[i] = firstWindowed[i];
+            }
+            plan.nchunk = static_cast<uint32_t>(runWindowed);
+            err = mfk_copy2d_windowed(&plan, engine.Tuning().windowMBps, stream);
+        } else {
+            plan.nchunk = static_cast<uint32_t>(run);
+            const uint32_t perCu = engine.Tuning().wgPerCu;   // 0: one workgroup per row group
+            const uint64_t cap = perCu == 0 ? run : static_cast<uint64_t>(cu) * perCu;
+            err = mfk_copy2d(&plan, static_cast<uint32_t>(run < cap ? run : cap), stream);
+        }
         used = 0;
         run = 0;
+        runWindowed = 0;
+        bytes = 0;
+        allWindowable = true;
         return err;
     };
     for (uint32_t i = 0; i < n; ++i) {
@@ -125,6 +144,11 @@ MF_EXPORT int32_t mf_xcopy_2d_batch(const mf_copy2d_desc *descs, uint32_t n, int
         plan.magic[used] = RectMagic(wu);
         plan.first[used] = static_cast<uint32_t>(run);
         plan.mate[used] = 0;
+        const uint64_t windowChunks = RectWindowChunks(wu, d.height);
+        firstWindowed[used] = static_cast<uint32_t>(runWindowed < 0xFFFFFFFFull ? runWindowed : 0xFFFFFFFFull);
+        allWindowable = allWindowable && windowChunks != 0;
+        runWindowed += windowChunks;
+        bytes += d.width * d.height;
         if (used > 0 && plan.mate[used - 1] == 0 &&
             RectsSideBySide(plan.dst[used - 1], d.dst, static_cast<uint64_t>(plan.widthUnits[used - 1]) * 16, d.width,
                             plan.height[used - 1], d.height, static_cast<uint64_t>(plan.dpitchUnits[used - 1]) * 16, d.dpitch)) {

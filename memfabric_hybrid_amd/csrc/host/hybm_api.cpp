@@ -46,6 +46,13 @@ MF_EXPORT int32_t hybm_init(uint16_t deviceId, uint64_t flags)
         return ret;
     }
     VaManager::Global().SetDeviceProbe(HipDeviceProbe);
+    {
+        // the rectangle kernels once, as the engine did with the copy kernels: a kernel's first launch is not capturable
+        void *stream = XcopyEngine::Instance().ThreadStream();
+        if (stream == nullptr || mfk_copy2d_prelaunch(stream) != 0 || mfrt_stream_sync(stream) != 0) {
+            MF_ERROR("the rectangle kernels could not be launched once at start");
+        }
+    }
     if (mfk_moe_setup() != 0) {
         MF_ERROR("the MoE dispatch could not probe the XCD order and keeps to its token-ordered permute");
     }

@@ -7,6 +7,7 @@
 
 #include "../rt/mf_rt.h"
 #include "copy2d_plan.h"
+#include "window_clock.h"
 
 namespace mf {
 namespace {
@@ -86,8 +87,133 @@ __global__ __launch_bounds__(kRectThreads) void Copy2dKernel(const RectPlan p)
     } while (c < nchunk);
 }
 
+// The same rectangles in read and write windows (the form XcopyWindowKernel gives long segments): single-wave
+// workgroups walk chunks of kRectWindowUnits units of a rectangle's payload taken row-major, whatever the width,
+// one chunk per period each; sixteen loads per lane at the wave's offset into the read half of the period, the
+// stores at the same offset into the write half.  plan.first counts these chunks (RectWindowChunks), a
+// rectangle holds fewer than 2^32 units, rowsPerChunk is not used.
+__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(4, 4))) void Copy2dWindowKernel(const RectPlan p, uint32_t period, uint32_t seq)
+{
+    // Only what the search needs stays in vector registers; the rectangle a chunk belongs to is read from the
+    // argument block by scalar loads once it is known (a period is microseconds long, their latency does not show).
+    const uint32_t lane = threadIdx.x & 63u;
+    const uint32_t first = p.first[lane];
+    const uint32_t mt = p.mate[lane];
+    const uint32_t nchunk = p.nchunk;
+    const uint32_t half = period / 2;
+    uint64_t slot = AgreedStart(seq) + static_cast<uint64_t>(blockIdx.x) * half / gridDim.x;
+    for (uint32_t c = blockIdx.x; c < nchunk; c += gridDim.x) {
+        uint32_t r = __popcll(__ballot(first <= c)) - 1;
+        uint32_t k = c - __builtin_amdgcn_readlane(first, r);
+        const uint32_t m = __builtin_amdgcn_readlane(mt, r);
+        if (m != 0) {
+            const uint32_t r0 = r - (m - 1);
+            const uint32_t both = c - __builtin_amdgcn_readlane(first, r0);
+            r = r0 + (both & 1u);
+            k = both >> 1;
+        }
+        r &= kRectInline - 1;
+        const uint64_t rs = p.src[r];
+        const uint64_t rd = p.dst[r];
+        const uint32_t rsp = p.spitchUnits[r];
+        const uint32_t rdp = p.dpitchUnits[r];
+        const uint32_t rwu = p.widthUnits[r];
+        const uint32_t rht = p.height[r];
+        const uint32_t rmg = p.magic[r];
+        const uint32_t base = k * kRectWindowUnits;
+        const uint32_t left = rht * rwu - base;
+        const uint32_t n = left < kRectWindowUnits ? left : kRectWindowUnits;
+        const uint32_t row0 = base / rwu;
+        const uint32_t col0 = base - row0 * rwu;
+        const MF_GLOBAL u32x4 *s = reinterpret_cast<const MF_GLOBAL u32x4 *>(rs) + static_cast<uint64_t>(row0) * rsp;
+        MF_GLOBAL u32x4 *d = reinterpret_cast<MF_GLOBAL u32x4 *>(rd) + static_cast<uint64_t>(row0) * rdp;
+        uint32_t row[kRectWindowDepth];   // the column follows from the row: kept in 16 registers, not 64 of offsets
+#pragma unroll
+        for (uint32_t j = 0; j < kRectWindowDepth; ++j) {
+            uint32_t col;
+            RectWindowRowCol(col0 + j * 64 + lane, rwu, rmg, row[j], col);
+        }
+        const uint32_t x0 = col0 + lane;
+        u32x4 v[kRectWindowDepth];
+        WaitForClock(slot);
+        // Addresses are worked out where they are used, from the sixteen row numbers: worked out ahead of the waits,
+        // as the compiler prefers, sixteen load and sixteen store addresses beside the data take the kernel past the
+        // 128 registers at which all kRectWindowWaves waves are resident together, which the schedule needs.
+#pragma unroll
+        for (uint32_t j = 0; j < kRectWindowDepth; ++j) {
+            asm volatile("" : "+v"(row[j]));
+        }
+        if (n == kRectWindowUnits) {
+#pragma unroll
+            for (uint32_t j = 0; j < kRectWindowDepth; ++j) {
+                v[j] = __builtin_nontemporal_load(s + (static_cast<uint64_t>(row[j]) * rsp + (x0 + j * 64 - row[j] * rwu)));
+            }
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            WaitForClock(slot + half);
+#pragma unroll
+            for (uint32_t j = 0; j < kRectWindowDepth; ++j) {
+                asm volatile("" : "+v"(row[j]));
+            }
+#pragma unroll
+            for (uint32_t j = 0; j < kRectWindowDepth; ++j) {
+                __builtin_nontemporal_store(v[j], d + (static_cast<uint64_t>(row[j]) * rdp + (x0 + j * 64 - row[j] * rwu)));
+            }
+        } else {
+#pragma unroll
+            for (uint32_t j = 0; j < kRectWindowDepth; ++j) {
+                if (j * 64 + lane < n) {
+                    v[j] = __builtin_nontemporal_load(s + (static_cast<uint64_t>(row[j]) * rsp + (x0 + j * 64 - row[j] * rwu)));
+                }
+            }
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            WaitForClock(slot + half);
+#pragma unroll
+            for (uint32_t j = 0; j < kRectWindowDepth; ++j) {
+                asm volatile("" : "+v"(row[j]));
+            }
+#pragma unroll
+            for (uint32_t j = 0; j < kRectWindowDepth; ++j) {
+                if (j * 64 + lane < n) {
+                    __builtin_nontemporal_store(v[j], d + (static_cast<uint64_t>(row[j]) * rdp + (x0 + j * 64 - row[j] * rwu)));
+                }
+            }
+        }
+        slot += period;
+    }
+}
+
 }  // namespace
 }  // namespace mf
+
+extern "C" int mfk_copy2d_windowed(const void *rectPlan, uint32_t windowMBps, void *stream)
+{
+    const mf::RectPlan &plan = *static_cast<const mf::RectPlan *>(rectPlan);
+    if (plan.nchunk == 0) {
+        return 0;
+    }
+    const uint32_t grid = plan.nchunk < mf::kRectWindowWaves ? plan.nchunk : mf::kRectWindowWaves;
+    const uint32_t ticks = mf::WindowPeriodTicks(2ull * grid * mf::kRectWindowUnits * 16u, windowMBps);
+    if (ticks == 0) {
+        return static_cast<int>(hipErrorInvalidValue);
+    }
+    hipLaunchKernelGGL(mf::Copy2dWindowKernel, dim3(grid), dim3(64), 0, static_cast<hipStream_t>(stream), plan, ticks,
+                       mf::NextWindowSeq());
+    return static_cast<int>(hipGetLastError());
+}
+
+// Both kernels once on a plan that holds nothing: a kernel's first launch is not capturable.
+extern "C" int mfk_copy2d_prelaunch(void *stream)
+{
+    mf::RectPlan empty{};
+    for (uint32_t i = 0; i < mf::kRectInline; ++i) {
+        empty.first[i] = 0xFFFFFFFFu;
+        empty.rowsPerChunk[i] = 1;
+    }
+    hipLaunchKernelGGL(mf::Copy2dKernel, dim3(1), dim3(mf::kRectThreads), 0, static_cast<hipStream_t>(stream), empty);
+    hipLaunchKernelGGL(mf::Copy2dWindowKernel, dim3(1), dim3(64), 0, static_cast<hipStream_t>(stream), empty, 64u,
+                       mf::NextWindowSeq());
+    return static_cast<int>(hipGetLastError());
+}
 
 extern "C" int mfk_copy2d(const void *rectPlan, uint32_t grid, void *stream)
 {

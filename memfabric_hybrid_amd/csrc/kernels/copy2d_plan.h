@@ -65,6 +65,35 @@ MF_RECT_HD inline void RectRowCol(uint32_t u, uint32_t widthUnits, uint32_t rows
     col = u - row * widthUnits;
 }
 
+// The windowed form cuts a rectangle's payload, taken row-major, into chunks of kRectWindowUnits units
+// regardless of row ends (16 loads per lane of a single wave).
+constexpr uint32_t kRectWindowDepth = 16;
+constexpr uint32_t kRectWindowUnits = 64 * kRectWindowDepth;
+constexpr uint32_t kRectWindowWaves = 4096;   // 16 per CU
+
+// Chunks of the windowed form, or 0 for a rectangle it cannot take (2^32 units and more).
+MF_RECT_HD inline uint64_t RectWindowChunks(uint64_t widthUnits, uint64_t height)
+{
+    const uint64_t units = widthUnits * height;
+    if (widthUnits == 0 || units / widthUnits != height || units > 0xFFFFFFFFull) {
+        return 0;
+    }
+    return (units + kRectWindowUnits - 1) / kRectWindowUnits;
+}
+
+// Row (relative to the row the chunk starts in) and column of the unit x units past the start of that row,
+// x < widthUnits + kRectWindowUnits: the quotient is 0 or 1 for rows of kRectWindowUnits units and more,
+// and below that x < 2 * kRectWindowUnits, where the multiply-high of RectRowCol is exact.
+MF_RECT_HD inline void RectWindowRowCol(uint32_t x, uint32_t widthUnits, uint32_t magic, uint32_t &row, uint32_t &col)
+{
+    if (widthUnits >= kRectWindowUnits) {
+        row = x >= widthUnits ? 1u : 0u;
+    } else {
+        row = widthUnits == 1 ? x : static_cast<uint32_t>((static_cast<uint64_t>(x) * magic) >> 32);
+    }
+    col = x - row * widthUnits;
+}
+
 // Whether a rectangle can take the 2-D kernel: everything a multiple of 16 and, in 16-byte units
 // (rows: in rows), within the 32-bit fields of the plan.
 MF_RECT_HD inline bool RectFitsPlan(uint64_t src, uint64_t dst, uint64_t width, uint64_t height, uint64_t spitch,

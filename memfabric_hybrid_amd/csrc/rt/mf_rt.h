@@ -130,6 +130,10 @@ void mfk_moe_combine_windows(uint32_t readMBps, uint32_t writeMBps);
 
 /* ---- 2-D copy launcher (kernels/copy2d.hip) ----------------------------------- */
 int mfk_copy2d(const void *rectPlan, uint32_t grid, void *stream);
+/* The same rectangles in read and write windows cut for windowMBps; plan.first counts chunks of RectWindowChunks(). */
+int mfk_copy2d_windowed(const void *rectPlan, uint32_t windowMBps, void *stream);
+/* Both rectangle kernels once on an empty plan. */
+int mfk_copy2d_prelaunch(void *stream);
 
 #ifndef MF_RT_HIDDEN
 #pragma GCC visibility pop

@@ -461,6 +461,38 @@ int mfk_copy2d(const void *rectPlan, uint32_t, void *)
     return 0;
 }
 
+// The windowed form: chunks of kRectWindowUnits units of the payload taken row-major, unit by unit as the kernel's lanes do.
+static uint32_t g_rectWindowed = 0;
+extern "C" uint32_t fake_rt_rect_windowed_launches() { return g_rectWindowed; }
+int mfk_copy2d_windowed(const void *rectPlan, uint32_t windowMBps, void *)
+{
+    const mf::RectPlan &p = *static_cast<const mf::RectPlan *>(rectPlan);
+    if (windowMBps == 0) {
+        return -1;
+    }
+    ++g_launches;
+    ++g_rectWindowed;
+    for (uint32_t c = 0; c < p.nchunk; ++c) {
+        uint32_t r = 0;
+        uint32_t k = 0;
+        mf::RectOfChunk(p, c, r, k);
+        const uint32_t wu = p.widthUnits[r];
+        const uint32_t base = k * mf::kRectWindowUnits;
+        const uint32_t total = p.height[r] * wu;
+        const uint32_t row0 = base / wu;
+        const uint32_t col0 = base - row0 * wu;
+        for (uint32_t u = 0; u < mf::kRectWindowUnits && base + u < total; ++u) {
+            uint32_t row = 0;
+            uint32_t col = 0;
+            mf::RectWindowRowCol(col0 + u, wu, p.magic[r], row, col);
+            std::memmove(reinterpret_cast<void *>(p.dst[r] + 16ull * (static_cast<uint64_t>(p.dpitchUnits[r]) * (row0 + row) + col)),
+                         reinterpret_cast<void *>(p.src[r] + 16ull * (static_cast<uint64_t>(p.spitchUnits[r]) * (row0 + row) + col)), 16);
+        }
+    }
+    return 0;
+}
+int mfk_copy2d_prelaunch(void *) { return 0; }
+
 uint64_t mfk_moe_workspace_bytes(uint32_t, uint32_t, uint32_t) { return 0; }
 int mfk_moe_dispatch(const void *, const void *, uint32_t, uint32_t, uint32_t, uint32_t, void *, void *, void *, void *, void *,
                      void *, void *) { return -1; }

@@ -24,6 +24,7 @@
 extern "C" uint64_t fake_rt_launches(void);
 extern "C" uint32_t fake_rt_last_hold(void);
 extern "C" uint32_t fake_rt_last_rect_mates(void);
+extern "C" uint32_t fake_rt_rect_windowed_launches(void);
 extern "C" int fake_rt_last_combine_paced(void);
 extern "C" uint64_t fake_rt_signals(void);
 extern "C" uint64_t fake_rt_stream_syncs(void);
@@ -910,6 +911,71 @@ static void TestUnorderedFanOut()
 }
 
 // Tables the engine cannot back with memory in a test: the launches are planned and checked, nothing is moved.
+// Rectangles of a launch that moves 512 MiB and more between device addresses take the windowed form: chunks of
+// 1024 units of the payload taken row-major.  Mates, rows narrower and wider than a chunk, a single column of units;
+// every row arrives, nothing lands between the rows.
+static void TestWindowedRectangles()
+{
+    CHECK(hybm_init(0, 0) == BM_OK);
+    CHECK(mf_xcopy_windows(6800000) == BM_OK);
+    const uint64_t rowsA = 57000;                      // 2 x 57000 rows of 4736 bytes: 540 MB
+    struct Shape { uint64_t width, height, spitch, dpitch; };
+    const Shape shapes[5] = {{4736, rowsA, 4736, 9472}, {4736, rowsA, 4736, 9472}, {48, 1000, 64, 80}, {40000, 50, 40016, 40032},
+                             {16, 3000, 16, 32}};
+    uint64_t srcBytes = 0;
+    uint64_t dstBytes = 0;
+    uint64_t srcAt[5];
+    uint64_t dstAt[5];
+    for (int i = 0; i < 5; ++i) {
+        srcAt[i] = srcBytes;
+        srcBytes += shapes[i].spitch * shapes[i].height;
+        if (i == 1) {
+            dstAt[i] = dstAt[0] + shapes[0].width;     // side by side with the first in the destination
+            continue;
+        }
+        dstAt[i] = dstBytes;
+        dstBytes += shapes[i].dpitch * shapes[i].height;
+    }
+    std::vector<unsigned char> src(srcBytes + 16);
+    std::vector<unsigned char> dst(dstBytes + 16, 0xEE);
+    for (uint64_t i = 0; i < srcBytes; i += 8) {
+        const uint64_t word = i * 0x9E3779B97F4A7C15ull + 1;
+        std::memcpy(&src[i], &word, 8);
+    }
+    const uint64_t s0 = (reinterpret_cast<uint64_t>(src.data()) + 15) & ~15ull;
+    const uint64_t d0 = (reinterpret_cast<uint64_t>(dst.data()) + 15) & ~15ull;
+    mf_copy2d_desc rects[5];
+    for (int i = 0; i < 5; ++i) {
+        rects[i] = {s0 + srcAt[i], d0 + dstAt[i], shapes[i].width, shapes[i].height, shapes[i].spitch, shapes[i].dpitch};
+    }
+    const uint32_t before = fake_rt_rect_windowed_launches();
+    CHECK(mf_xcopy_2d_batch(rects, 5, MF_ROUTE_HBM, nullptr) == BM_OK);
+    CHECK(fake_rt_rect_windowed_launches() == before + 1);
+    bool ok = true;
+    for (int i = 0; i < 5 && ok; ++i) {
+        const unsigned char *s = reinterpret_cast<const unsigned char *>(rects[i].src);
+        const unsigned char *d = reinterpret_cast<const unsigned char *>(rects[i].dst);
+        for (uint64_t r = 0; r < shapes[i].height && ok; ++r) {
+            ok = std::memcmp(d + r * shapes[i].dpitch, s + r * shapes[i].spitch, shapes[i].width) == 0;
+            // the gap behind a row (for the mates: behind the pair) is untouched
+            const uint64_t gapAt = i == 0 ? 2 * shapes[i].width : shapes[i].width;
+            if (i != 1 && gapAt < shapes[i].dpitch) {
+                ok = ok && d[r * shapes[i].dpitch + gapAt] == 0xEE && d[(r + 1) * shapes[i].dpitch - 1] == 0xEE;
+            }
+        }
+        CHECK(ok);
+    }
+    // the same call below the size takes the kernel of whole rows
+    rects[0].height = rects[1].height = 1000;
+    CHECK(mf_xcopy_2d_batch(rects, 5, MF_ROUTE_HBM, nullptr) == BM_OK);
+    CHECK(fake_rt_rect_windowed_launches() == before + 1);
+    // and so does a route over the host link
+    rects[0].height = rects[1].height = rowsA;
+    CHECK(mf_xcopy_2d_batch(rects, 5, MF_ROUTE_TO_HOST, nullptr) == BM_OK);
+    CHECK(fake_rt_rect_windowed_launches() == before + 1);
+    hybm_uninit();
+}
+
 static void TestLongSegments()
 {
     CHECK(hybm_init(0, 0) == BM_OK);
@@ -1414,6 +1480,7 @@ int main()
     TestHeldStores();
     TestWindows();
     TestLongSegments();
+    TestWindowedRectangles();
     TestCalibration();
     TestUnorderedFanOut();
     TestHostLaunchCosts();

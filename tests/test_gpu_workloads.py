@@ -98,6 +98,40 @@ def test_2d_batch_of_many_rectangles(gpu, oracle):
     assert np.array_equal(got, expect)
 
 
+def test_2d_batch_in_read_and_write_windows(gpu, oracle):
+    """A launch that moves more than 512 MiB between device addresses takes the windowed rectangle kernel (chunks of
+    1024 units of the payload taken row-major): two mates of the down_proj geometry, rows of one unit, rows narrower
+    and wider than a chunk, a row count that leaves a partial last chunk.  Compared with the oracle byte for byte,
+    gaps between the rows included."""
+    shapes = [(4736, 57001, 4736, 9472), (4736, 57001, 4736, 9472), (16, 3001, 32, 48), (48, 1000, 64, 80),
+              (40000, 51, 40016, 40032), (16384, 33, 16384, 16400), (16400, 7, 16416, 16400)]
+    src_at, dst_at, sbytes, dbytes = [], [], 0, 0
+    for i, (w, h, sp, dp) in enumerate(shapes):
+        src_at.append(sbytes)
+        sbytes += sp * h + 16
+        if i == 1:
+            dst_at.append(dst_at[0] + shapes[0][0])      # side by side with the first
+            continue
+        dst_at.append(dbytes)
+        dbytes += dp * h + 16
+    assert sum(w * h for w, h, _, _ in shapes) > 512 * MIB
+    src = _rand(oracle, sbytes, 77)
+    sbuf = gpu_util.DeviceBuffer(gpu, sbytes)
+    dbuf = gpu_util.DeviceBuffer(gpu, dbytes)
+    try:
+        sbuf.upload(src)
+        dbuf.fill(0x5C)
+        _copy2d(gpu, [(sbuf.ptr + src_at[i], dbuf.ptr + dst_at[i], w, h, sp, dp) for i, (w, h, sp, dp) in enumerate(shapes)])
+        got = dbuf.download()
+    finally:
+        sbuf.free()
+        dbuf.free()
+    expect = np.full(dbytes, 0x5C, dtype=np.uint8)
+    for i, (w, h, sp, dp) in enumerate(shapes):
+        oracle.orc_copy_2d(np_ptr(expect) + dst_at[i], dp, np_ptr(src) + src_at[i], sp, w, h)
+    assert np.array_equal(got, expect)
+
+
 def test_2d_argument_errors(gpu):
     d = (native.Copy2dDesc * 1)(native.Copy2dDesc(0x1000, 0x2000, 64, 4, 32, 64))
     assert gpu.mf_xcopy_2d_batch(d, 1, 0, None) == native.BM_INVALID_PARAM      # width > source pitch
