@@ -1313,10 +1313,11 @@ int XcopyEngine::SubmitOne(const uint64_t *src, const uint64_t *dst, const uint6
         queuedBytes = total;
         // A table of long segments between HBM addresses is cut into launches of kInlineSegs segments, each of which
         // then takes the form with read and write windows: the few extra launches cost microseconds, the windows
-        // gain 8 % (896 segments, 8.5 GB: 2.55 ms in seven launches against 2.78 ms in one).  The table kernel
-        // itself was measured under windows and is left without them: its chunk search lowers the rate it
-        // sustains (6.56 TB/s at a target of 6.6, erratic at 6.8), and 262 144 pages of 32 KiB at random
-        // places lose (5.1 against 5.4 TB/s).
+        // gain 8 % (896 segments, 8.5 GB: 2.55 ms in seven launches against 2.78 ms in one).  The table form
+        // itself was measured under windows twice, with the prefix search it once had and with the division and
+        // group map it has now, and is left without them: 262 144 pages of 32 KiB at random places lose 7 to 12 %
+        // (3.23 to 3.45 against 3.04 ms), 16 384 ragged segments 3 %, and the 896 long segments in one windowed
+        // table launch are no faster than in seven launches of the kernel-argument form.
         if (maySlice && n > kInlineSegs && route == MFRT_ROUTE_HBM && !unordered && tuning_.windowMBps != 0 && windowsAvailable_ &&
             tuning_.unitsOverride == 0 && total / n >= kWindowSliceMinSegmentBytes &&
             g_leasesOut.load(std::memory_order_relaxed) <= 1) {

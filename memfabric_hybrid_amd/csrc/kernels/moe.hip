@@ -509,13 +509,10 @@ __global__ __launch_bounds__(64) void MoePermuteLoopKernel(const u32x4 *__restri
 // wave, belongs to stream i % 8 (the dispatcher deals consecutive workgroups to the eight XCDs in turn);
 // stream s takes the steps s, s + 8, ... one after the other and walks a step's rows in list order, a row in
 // tiles of 128 units (2 KiB).  So an XCD writes runs of consecutive rows front to back, two stores per wave,
-// which is the only store pattern this part takes at more than 5.4 TB/s (6.1 in runs of 128 KiB, 6.6 in
-// eight sequential streams; waves that store 14 KiB each: 5.4 in any order), and the K reads of a token row
-// all come from the same XCD within the time it spends on the block: the first from HBM, the others from its
-// L2 (plain loads), which stores that are written through pass without evicting x (plain stores: 244 us).
-// 8192 x 7168, top-8, 256 experts: 163-166 us against 192 us for the token-ordered loop kernel; tiles of
-// 64 / 192 / 256 / 448 units 207 / 171 / 178 / 193 us, nontemporal stores that are not written through 166-172 us,
-// blocks of 2048 entries per stream step 165-171 us, streams that do not follow the XCDs 283 us.
+// the store pattern this part takes fastest, and the K reads of a token row all come from the same XCD within
+// the time it spends on the block: the first from HBM, the others from its L2 (plain loads), which stores that
+// are written through pass without evicting x.  8192 x 7168, top-8, 256 experts: 163-166 us against 192 us for
+// the token-ordered loop kernel; streams that do not follow the XCDs 283 us.
 constexpr uint32_t kTileUnits = 128;
 constexpr uint32_t kTileStreams = 8;
 
@@ -664,12 +661,10 @@ __global__ __launch_bounds__(kThreads) void MoeCombineKernel(const u32x4 *__rest
 // positions per lane) at its own offset of the part, reduces them when they have arrived and
 // keeps the result, 8 registers per item; in the write part it stores the kItems results at
 // its own offset of that part (top-6: six rows, twelve pieces).  The start of the first period is agreed through
-// AgreedStart(); after that every wave goes by the constant-rate clock alone.  Measured at top-8 on
-// 8192 tokens of 7168 elements: 164-168 us against 177-181 us for one workgroup per item, on
-// 16 384 tokens 323-330 against 359-365 us (read parts paced at 6.6-6.8 TB/s, write parts at
-// 6.0-6.5; reads at 7.0 make the waves fall behind now and then, and so did 6.8 with writes at
-// 6.5 on one machine when the launch ran for seven periods; the default is 6.8 and 6.2).  From
-// about six items per wave on it is the faster form.
+// AgreedStart(); after that every wave goes by the constant-rate clock alone.  8192 tokens of 7168
+// elements at top-8: 164-168 us against 177-181 us for one workgroup per item; from about six items per
+// wave on it is the faster form.  Read parts are paced at 6.8 TB/s, write parts at 6.2 (reads at 7.0
+// make the waves fall behind now and then).
 // Arithmetic and the rule for slots without a row are MoeCombineKernel's.
 constexpr uint32_t kCombineItems = 4;                  // 32 result registers, 116 in all: sixteen waves per CU
 constexpr uint32_t kCombineWavesPerCu = 16;
@@ -834,16 +829,10 @@ extern "C" int mfk_moe_dispatch(const void *x, const void *topk, uint32_t tokens
     const uint32_t upr = hidden / 8;
     // The output-ordered tile permute needs the token rows of one step (a block of kRankBlock entries, or a half, a
     // quarter ... down to one slice of 64 entries: stepEntries / topK tokens) to stay in an XCD's 4 MiB L2 while the
-    // step's rows are written, and enough steps for the eight streams.
-    // 8192 tokens, 256 experts, top-8, rows of 4096 / 7168 / 8192 elements (1.1 / 1.8 / 2.1 MB of x per block):
-    // 102 / 174 / 187 us against 125 / 208 / 249 us with the loop kernel; 12 288 / 16 384 elements in steps of half a
-    // block: 268 / 381 against 359 / 546 us.  512 / 64 / 8 experts at 7168 elements: 194 / 155 / 154 us (the fewer
-    // experts, the longer the runs).  16 384 tokens, top-2, 8 experts, 4096 / 6144 / 8192 elements: 67 / 94 / 126 against
-    // 70 / 123 / 170 us; top-4: 94 against 117 us (7168 elements, 64 experts), 72 against 82 us (5120, 128).
-    // Narrower rows (8192 tokens, top-8, 256 experts, 1024 / 2048 / 3072 elements): 44 / 62 / 91 against 49 / 75 / 108 us
-    // with one four-wave workgroup per token; 16 384 tokens of 2048 elements over 64 experts 102 against 136 us.
-    // Rows that are not whole cache lines (10 000 elements: 20 000 bytes) lose, 362 against 337 us, whatever the step:
-    // every tile then begins and ends inside a line; they keep the loop kernel.
+    // step's rows are written, and enough steps for the eight streams.  It wins on every shape of whole cache lines
+    // that was measured (8192 tokens, top-8, 256 experts, 7168 elements: 174 against 208 us with the loop kernel;
+    // 1024 elements: 44 against 49 us with one workgroup per token).  Rows that are not whole cache lines
+    // (10 000 elements) lose, whatever the step: every tile then begins and ends inside a line; they keep the loop kernel.
     uint32_t stepSlices = kRankSlices;
     while (stepSlices > 1 && static_cast<uint64_t>(stepSlices * 64 / topK + 1) * hidden * 2 > 2200000ull) {
         stepSlices /= 2;
@@ -892,15 +881,9 @@ extern "C" int mfk_moe_dispatch(const void *x, const void *topk, uint32_t tokens
                                tilesPerRow, static_cast<uint32_t>(steps), stepEntries, oo);
         } else if (upr >= 512) {
             // Wide rows: single-wave workgroups that hold up to 14 pieces per lane (a whole 7168-element
-            // row) and write them with plain stores.  Storing alone takes 177 us of the 200 us such a
-            // kernel needs when every wave reads its row first; with sixteen waves per CU that each
-            // take several tokens and fetch the next row while they store the current one
-            // the dispatch takes 207 us instead of 215.  Other shapes measured on these rows: two waves
-            // per row 221 us; four-wave workgroups with nontemporal stores 237 us; the row staged in LDS
-            // instead of registers 221 us (one wave) and 227 us (four waves); buffer-addressed
-            // stores at eight waves per SIMD 224 us; the destination-side form, one workgroup per output
-            // row reading x[srcOf[row]], 271 us: its eight reads of every token row are not absorbed by
-            // the caches.
+            // row) and write them with plain stores; sixteen waves per CU that each take several tokens and
+            // fetch the next row while they store the current one (207 us for 8192 x 7168 at top-8; staging in
+            // LDS, two waves per row, nontemporal stores and the destination-side form were all slower).
             // 123 vector registers per lane: four waves per SIMD, sixteen per CU, all resident at once
             const uint32_t wideParts = (upr + 64 * 14 - 1) / (64 * 14);
             const uint32_t items = tokens * wideParts;

@@ -1309,6 +1309,40 @@ extern "C" int mfk_xcopy_static_setup(void)
         g_staticDone[dev] = nullptr;   // calls then go unguarded, as documented for callers that overlap them
         (void)hipGetLastError();
     }
+    // The kernels of the device-table path once, on a table of no segments whose header lands in the array (what
+    // mfk_xcopy_prelaunch cannot do without device memory): a caller may then capture its very first call.
+    {
+        using namespace mf;
+        uint32_t *words = g_scratchOf[dev];
+        const uint64_t *none = reinterpret_cast<const uint64_t *>(words);
+        hipLaunchKernelGGL(XcopySignalKernel, dim3(1), dim3(64), 0, nullptr, reinterpret_cast<uint64_t *>(words + 2), 0u);   // the header's spare words
+        hipLaunchKernelGGL(XcopyPlanSumsKernel, dim3(1), dim3(kPlanThreads), 0, nullptr, none, 0u, kXcopyThreads, words, kStaticGroupCapacity);
+        hipLaunchKernelGGL(XcopyPlanKernel<1>, dim3(1), dim3(kPlanThreads), 0, nullptr, none, 0u, kXcopyThreads, words, kStaticGroupCapacity);
+        hipLaunchKernelGGL(XcopyPlanKernel<2>, dim3(1), dim3(kPlanThreads), 0, nullptr, none, 0u, kXcopyThreads, words, kStaticGroupCapacity);
+        hipLaunchKernelGGL(XcopyPlanKernel<4>, dim3(1), dim3(kPlanThreads), 0, nullptr, none, 0u, kXcopyThreads, words, kStaticGroupCapacity);
+        hipLaunchKernelGGL(XcopyPlanKernel<8>, dim3(1), dim3(kPlanThreads), 0, nullptr, none, 0u, kXcopyThreads, words, kStaticGroupCapacity);
+        const ScratchLayout at = ScratchLayoutFor(0, kStaticGroupCapacity);
+        TablePlan plan{};
+        plan.triples = none;
+        plan.first = words + at.first;
+        plan.group = words + at.group;
+        plan.header = reinterpret_cast<const TableHeader *>(words);   // the planner launches above left nchunk = 0 there
+        plan.units = kXcopyThreads;
+        for (int route = MFRT_ROUTE_HBM; route <= MFRT_ROUTE_FROM_HOST; ++route) {
+            (void)WithPolicy(PolicyOf(route), [&](auto ntLoad, auto store) {
+                hipLaunchKernelGGL((XcopyTableKernel<decltype(ntLoad)::value, decltype(store)::value, true>), dim3(1), dim3(64), 0,
+                                   nullptr, plan, 0u);
+                return 0;
+            });
+        }
+        err = hipGetLastError();
+        if (err == hipSuccess) {
+            err = hipStreamSynchronize(nullptr);
+        }
+        if (err != hipSuccess) {
+            return static_cast<int>(err);
+        }
+    }
     return 0;
 }
 
