@@ -136,6 +136,8 @@ def _held_case(rng, count, sizes, ragged):
     (100, (400000,), True),             # the same with heads, tails and last chunks that are not whole
     (488, (131072, 16384), False),      # 36 MB out of a table under a pattern, 16 KiB per wave
     (400, (150000, 40000, 98304), True),  # 38 MB, ragged: group map, 16 KiB per wave
+    (1, (16 << 20,), False),            # one segment of 16 MiB: 4096 chunks of 4 KiB, no table, stores of four loads held
+    (1, ((9 << 20) + 777,), True),      # the same with a head, a tail and a last chunk that is not whole
     (1, (48 << 20,), False),            # one segment of 48 MiB
     (1, ((40 << 20) + 12345,), True),
     (976, (131072, 16384), False),      # 72 MB: beyond what the waves hold at once, the usual form
