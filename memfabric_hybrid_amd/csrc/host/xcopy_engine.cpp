@@ -326,7 +326,9 @@ struct Submitter {
             std::unique_lock<std::mutex> guard(lock);
             asleep.store(true, std::memory_order_seq_cst);
             if (cell.seq.load(std::memory_order_seq_cst) != next + 1 && !stop.load(std::memory_order_acquire)) {
-                wake.wait_for(guard, std::chrono::milliseconds(50));   // the bound is a net under the handshake, not part of it
+                // the bound is a net under the handshake, not part of it (by the system clock: the wait on the steady
+                // clock is a call the thread sanitizer of this toolchain does not know, and it then misreads the mutex)
+                wake.wait_until(guard, std::chrono::system_clock::now() + std::chrono::milliseconds(50));
             }
             asleep.store(false, std::memory_order_release);
             idle = 0;

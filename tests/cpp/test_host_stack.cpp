@@ -651,8 +651,11 @@ static void TestMappedWindow()
             std::atomic<uint64_t> refused{0};
             std::atomic<uint64_t> other{0};
             std::thread hammer([&] {
-                hybm_copy_params p{base, base + page + 4096, 65536};
+                // copies that are declared independent must be: 32 destinations in turn, so that copies with the same
+                // destination always reach the same one of the two submit threads
+                uint64_t turn = 0;
                 while (phase.load() != 2) {
+                    hybm_copy_params p{base, base + page + 4096 + (turn++ % 32) * 65536, 65536};
                     const int ret = hybm_data_copy(e, &p, HYBM_GLOBAL_DEVICE_TO_GLOBAL_DEVICE, nullptr, ASYNC_COPY_FLAG | MF_COPY_UNORDERED_FLAG);
                     (ret == BM_OK ? done : (ret == BM_INVALID_PARAM ? refused : other)).fetch_add(1);
                     if (done.load() > 50) {

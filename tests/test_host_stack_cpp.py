@@ -13,7 +13,9 @@ SOURCES = ["mf_log.cpp", "xcopy_engine.cpp", "va_manager.cpp", "hip_data_op.cpp"
 def test_host_stack_over_fake_runtime(tmp_path):
     exe = str(tmp_path / "test_host_stack")
     cmd = ["g++", "-O1", "-std=c++17", "-pthread"]
-    if os.environ.get("MF_TEST_SANITIZE"):
+    if os.environ.get("MF_TEST_SANITIZE") == "thread":
+        cmd += ["-g", "-fsanitize=thread"]
+    elif os.environ.get("MF_TEST_SANITIZE"):
         cmd += ["-g", "-fsanitize=address,undefined"]
     cmd += ["-o", exe, os.path.join(ROOT, "tests", "cpp", "test_host_stack.cpp"),
             os.path.join(ROOT, "tests", "cpp", "fake_rt.cpp")] + [os.path.join(HOST, s) for s in SOURCES]
