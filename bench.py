@@ -318,7 +318,7 @@ def extras_block(lib, pool, dev, batches, tables, steps):
     # the same with the batches handed to submit threads of the library's (mf_xcopy_unordered_streams): one calling thread,
     # several streams
     fan = {}
-    for streams in (4, 6):
+    for streams in (3, 4, 6):
         assert lib.mf_xcopy_unordered_streams(streams) == 0
         walls = []
         for _ in range(5):
@@ -843,6 +843,11 @@ def main():
                    "note": "measured by hybm_init on this GPU (about 15 ms): the wait of the held stores is the fitted rule plus the offset "
                            "that was fastest here, the window rate the faster of two, either form off where it gains under 3 %"}
 
+    deck = (ctypes.c_uint32 * 16)()
+    stream_queues = {"hardware_queue_of_each_stream_in_hand_out_order": list(deck[:min(16, lib.mf_xcopy_stream_queues(deck, 16))]),
+                     "note": "hybm_init asks the GPU which of its first streams share a hardware queue (launches on such streams run one "
+                             "after the other) and hands out one stream of every queue before the second of any: the calling thread holds "
+                             "the first, threads and submit threads that come later the next ones"}
     wall, ms, rep_us = steady_state_headline(lib, pool.handle, batches, g2g, args.steps, args.warmup)
     per_launch_us = ms * 1e3 / args.steps
     value = payload * args.steps / wall / GB
@@ -876,6 +881,7 @@ def main():
             "payload_bytes": payload,
             "cu_count": lib.mfrt_cu_count(),
             "calibration": calibration,
+            "stream_queues": stream_queues,
             "submitting_thread": {"empty_launch_us_by_cpu": launch_us_by_cpu, "runs_on_cpus": near_cpus if kept > 0 else all_cpus,
                                   "note": "mf_pin_thread_near_gpu: the CPUs from which a launch with a full argument block is "
                                           "cheapest, measured at start; the threads of the concurrency extras inherit the set"},

@@ -38,10 +38,11 @@ extern "C" {
 /* Who launches unordered copies.  0 or 1 (the default): the calling thread, on its own stream, without a barrier.
  * 2 to 8: batches of up to 128 segments and 64 MiB between device addresses, submitted with MF_COPY_UNORDERED_FLAG and
  * no stream of the caller's, are planned by the caller and handed in turn to that many submit threads of the
- * library's, each with a stream of its own, which the GPU serves from different hardware queues: one calling
- * thread then gets the overlap several submitting threads get (the reference gives every thread one stream,
- * src/hybm/csrc/ts_engine/hybm_stream_manager.cpp:73-90): 9 MB batches take 4.4 / 4.1 / 3.9 / 4.0 us each with
- * 4 / 5 / 6 / 8 submit threads against 4.5 us without, and 1.2 us of the calling thread's time instead of 3.5.  One
+ * library's, each with a stream of its own on a hardware queue of its own as far as there are queues (four here; hybm_init
+ * asks the GPU which of its streams share one): one calling thread then gets the overlap several submitting threads get
+ * (the reference gives every thread one stream, src/hybm/csrc/ts_engine/hybm_stream_manager.cpp:73-90): 9 MB batches take
+ * 4.3 / 3.8 / 3.6 / 3.8 / 3.6-4.0 us each with 2 / 3 / 4 / 6 / 8 submit threads against 4.5 us without, and 1.2 us of the calling
+ * thread's time instead of 3.5.  Four is the number to use where the runtime has four hardware queues.  One
  * thread that launches on several streams itself does not: the launches then cost it more than on one stream.
  * The next copy WITHOUT the flag, smem_bm_wait / hybm_wait and every other call that uses the thread's stream first
  * make that stream wait for them.  What changes for the caller: a synchronisation of mf_xcopy_thread_stream() that it

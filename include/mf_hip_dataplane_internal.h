@@ -81,6 +81,12 @@ int64_t mf_xcopy_describe_plan(const uint64_t *src, const uint64_t *dst, const u
  * us per batch / per copy.  Returns 1 if the calibration ran, 0 if not.  mf_xcopy_hold_stores / mf_xcopy_windows still
  * override what it chose. */
 int32_t mf_xcopy_calibration(int32_t *holdEnabled, int32_t *holdDeltaNanos, uint32_t *windowMBps, float *micros);
+/* The streams hybm_init makes for calling threads and submit threads, in the order they are handed out (the calling
+ * thread of hybm_init holds the first): queues[i] is the hardware queue stream i sits on, numbered in order of
+ * appearance.  The library asks the GPU which of its streams share a queue (launches on such streams run one
+ * after the other) and hands out one stream of every queue before the second of any.  Returns the number of streams
+ * (at most `capacity` are written); all entries differ where the GPU gave no answer. */
+uint32_t mf_xcopy_stream_queues(uint32_t *queues, uint32_t capacity);
 /* Table launches.  stageUnordered: 1 (default) launches the upload of a ragged table's descriptors without a
  * barrier, so that it runs while the caller's earlier copies still do; 0 orders it behind them.
  * deviceTableWgPerCu: workgroups per CU of the launch that copies a table in device memory, whose chunk

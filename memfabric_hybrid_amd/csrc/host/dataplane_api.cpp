@@ -165,6 +165,11 @@ MF_EXPORT int32_t mf_xcopy_unordered_streams(uint32_t count)
     return BM_OK;
 }
 
+MF_EXPORT uint32_t mf_xcopy_stream_queues(uint32_t *queues, uint32_t capacity)
+{
+    return XcopyEngine::Instance().StreamQueues(queues, queues == nullptr ? 0 : capacity);
+}
+
 MF_EXPORT int32_t mf_xcopy_tune_table(uint32_t stageUnordered, uint32_t deviceTableWgPerCu)
 {
     XcopyTuning &t = XcopyEngine::Instance().Tuning();

@@ -124,13 +124,16 @@ public:
 
     // Whether an ordered launch that moves `bytes` on `route` takes the form with read and write windows.
     bool WindowsApply(uint64_t bytes, int route) const;
+    // Hardware queue (numbered in order of appearance) of each of the streams made at Start(), in the order they are handed out; returns their number.
+    uint32_t StreamQueues(uint32_t *queues, uint32_t capacity) const;
     // No second thread holds a stream of the library: kernels that pace themselves for the whole chip may be used.
     bool SingleSubmitter() const;
 
     // The calling thread's own stream (created on first use).  Unordered batches that were handed to the submit
     // threads are joined first: work queued on the returned stream afterwards waits for them.
     void *ThreadStream();
-    static constexpr uint32_t kFanStreams = 8;   // most submit threads for unordered batches (9 MB batches: 4 / 5 / 6 / 8 threads 4.40 / 4.07 / 3.87 / 4.00 us per batch)
+    static constexpr uint32_t kFanStreams = 8;   // most submit threads for unordered batches (9 MB batches: 2 / 3 / 4 / 6 / 8 threads 4.3 / 3.8 / 3.6 / 3.8 / 3.6-4.0 us per batch)
+    static constexpr uint32_t kDeckStreams = 8;   // streams made at Start() and dealt out so that consecutive takers sit on different hardware queues
     static constexpr uint64_t kFanMaxBytes = 64ull << 20;   // larger batches gain nothing from a second queue
     // Pinned, device-mapped staging memory of the calling thread, at least `bytes` long; it lives
     // until Stop().  NULL when it cannot be allocated.

@@ -193,6 +193,7 @@ _SIGNATURES = {
     "mf_xcopy_thread_stream": (vp, []),
     "mf_xcopy_tune": (i32, [u32, u32, u32]),
     "mf_xcopy_unordered_streams": (i32, [u32]),
+    "mf_xcopy_stream_queues": (u32, [ctypes.POINTER(u32), u32]),
     "mf_xcopy_tune_table": (i32, [u32, u32]),
     "mf_xcopy_tune_hold": (i32, [u32, i32, u32]),
     "mf_xcopy_calibration": (i32, [ctypes.POINTER(i32), ctypes.POINTER(i32), ctypes.POINTER(u32), ctypes.POINTER(ctypes.c_float)]),

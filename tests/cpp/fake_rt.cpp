@@ -31,6 +31,7 @@ bool g_skipCopies = false;       // launches count and check their plans but mov
 uint32_t g_lastTableShift = 0;   // group shift of the latest table launch that used a group map, 0 under a pattern
 uint64_t g_groupMapErrors = 0;
 uint32_t g_lastTableHold = 0;    // holdNanos of the latest table launch
+std::atomic<uint64_t> g_streamsMade{0};   // streams made since mfrt_init
 
 void *Track(uint64_t bytes, int kind)
 {
@@ -144,6 +145,7 @@ int mfrt_init(int device)
         return 101;
     }
     g_device = 0;
+    g_streamsMade = 0;
     return 0;
 }
 int mfrt_current_device(void) { return 0; }
@@ -200,7 +202,29 @@ int mfrt_pointer_kind(const void *p)
     --it;
     return a < it->first + it->second.first ? it->second.second : MFRT_PTR_PAGEABLE;
 }
-void *mfrt_stream_create(void) { return malloc(8); }
+// A stream remembers the how-manieth stream since mfrt_init it is: the stand-in for "which hardware queue the runtime
+// put it on" follows the pattern measured on the GPU (queues A B C C B A D C, then round robin).
+static int g_queueAnswers = 0;      // 0: by the pattern, 1: not known
+void fake_rt_queue_answers(int mode) { g_queueAnswers = mode; }
+void *mfrt_stream_create(void)
+{
+    uint64_t *token = static_cast<uint64_t *>(malloc(8));
+    *token = g_streamsMade.fetch_add(1);
+    return token;
+}
+static uint32_t FakeQueueOf(const void *stream)
+{
+    static const uint32_t first[8] = {0, 1, 2, 2, 1, 0, 3, 2};
+    const uint64_t index = *static_cast<const uint64_t *>(stream);
+    return index < 8 ? first[index] : static_cast<uint32_t>(index % 4);
+}
+int mfk_streams_share_queue(void *a, void *b)
+{
+    if (g_queueAnswers == 1) {
+        return -1;
+    }
+    return FakeQueueOf(a) == FakeQueueOf(b) ? 1 : 0;
+}
 int mfrt_stream_destroy(void *s) { Guard("mfrt_stream_destroy"); free(s); return 0; }
 uint64_t fake_rt_violations(void) { return g_violations; }
 uint64_t fake_rt_in_flight(void)

@@ -25,6 +25,7 @@ extern "C" uint64_t fake_rt_launches(void);
 extern "C" uint32_t fake_rt_last_hold(void);
 extern "C" uint32_t fake_rt_last_rect_mates(void);
 extern "C" uint32_t fake_rt_rect_windowed_launches(void);
+extern "C" void fake_rt_queue_answers(int mode);
 extern "C" int fake_rt_last_combine_paced(void);
 extern "C" uint64_t fake_rt_signals(void);
 extern "C" uint64_t fake_rt_stream_syncs(void);
@@ -979,6 +980,33 @@ static void TestWindowedRectangles()
     hybm_uninit();
 }
 
+// Streams are dealt out one per hardware queue before the second of any.  The stand-in runtime puts the first eight
+// streams of a process on queues A B C C B A D C, as the GPU did.
+static void TestStreamDeck()
+{
+    CHECK(hybm_init(0, 0) == BM_OK);
+    uint32_t queues[16] = {};
+    CHECK(mf_xcopy_stream_queues(queues, 16) == 8);
+    const uint32_t expect[8] = {0, 1, 2, 3, 0, 1, 2, 2};
+    for (int i = 0; i < 8; ++i) {
+        CHECK(queues[i] == expect[i]);
+    }
+    // the calling thread holds the first; four submit threads then sit on four different queues
+    void *mine = mf_xcopy_thread_stream();
+    CHECK(mine != nullptr);
+    CHECK(mf_xcopy_stream_queues(nullptr, 0) == 8);
+    hybm_uninit();
+    // no answer from the GPU: every stream a queue of its own, the order they were made in
+    fake_rt_queue_answers(1);
+    CHECK(hybm_init(0, 0) == BM_OK);
+    CHECK(mf_xcopy_stream_queues(queues, 16) == 8);
+    for (uint32_t i = 0; i < 8; ++i) {
+        CHECK(queues[i] == i);
+    }
+    hybm_uninit();
+    fake_rt_queue_answers(0);
+}
+
 static void TestLongSegments()
 {
     CHECK(hybm_init(0, 0) == BM_OK);
@@ -1483,6 +1511,7 @@ int main()
     TestHeldStores();
     TestWindows();
     TestLongSegments();
+    TestStreamDeck();
     TestWindowedRectangles();
     TestCalibration();
     TestUnorderedFanOut();

@@ -173,3 +173,57 @@ def test_table_batches_in_a_row_keep_their_descriptors(lib, oracle):
     finally:
         buf.free()
         lib.hybm_uninit()
+
+
+def test_streams_are_dealt_one_per_hardware_queue(lib):
+    """hybm_init classifies the streams it makes by hardware queue and hands out one of every queue before the second of
+    any.  Checked against a measurement of its own through the public calls: a long copy on one stream, a short one on
+    another, and whether the short one ends first."""
+    import ctypes
+    assert lib.hybm_init(0, 0) == 0, native.last_error()
+    try:
+        queues = (ctypes.c_uint32 * 16)()
+        count = lib.mf_xcopy_stream_queues(queues, 16)
+        assert count == 8
+        dealt = list(queues[:count])
+        kinds = len(set(dealt))
+        assert kinds >= 2, "the runtime of an MI355X spreads its streams over several hardware queues"
+        assert sorted(dealt[:kinds]) == list(range(kinds)), dealt      # the first round: one stream of every queue
+        # the calling thread holds the deck's first stream; a second thread gets the second, which must overlap with it
+        mine = lib.mf_xcopy_thread_stream()
+        other = []
+
+        def grab():
+            assert lib.mfrt_bind_thread() == 0
+            other.append(lib.mf_xcopy_thread_stream())
+
+        t = threading.Thread(target=grab)
+        t.start()
+        t.join()
+        assert other and other[0] and other[0] != mine
+        big = 256 * MIB
+        buf = gpu_util.DeviceBuffer(lib, 2 * big + 8192)
+        ea, eb = lib.mfrt_event_create(), lib.mfrt_event_create()
+        u64 = ctypes.c_uint64
+        try:
+            def copy(stream, src, dst, n):
+                assert lib.mf_xcopy_batch((u64 * 1)(src), (u64 * 1)(dst), (u64 * 1)(n), 1, native.ROUTE_HBM, stream) == 0
+            for s in (mine, other[0]):
+                copy(s, buf.ptr, buf.ptr + big, 4096)
+            assert lib.mfrt_device_sync() == 0
+            overlapped = 0
+            for _ in range(5):
+                copy(mine, buf.ptr, buf.ptr + big, big)                       # some 90 us
+                lib.mfrt_event_record(ea, mine)
+                copy(other[0], buf.ptr + 2 * big, buf.ptr + 2 * big + 4096, 4096)
+                lib.mfrt_event_record(eb, other[0])
+                assert lib.mfrt_event_sync(eb) == 0
+                overlapped += 0 if lib.mfrt_event_done(ea) else 1
+                assert lib.mfrt_event_sync(ea) == 0
+            assert overlapped >= 4, "the second thread's stream waits for the first thread's copies"
+        finally:
+            lib.mfrt_event_destroy(ea)
+            lib.mfrt_event_destroy(eb)
+            buf.free()
+    finally:
+        lib.hybm_uninit()
