@@ -127,7 +127,7 @@ struct ThreadLease {
 // evenly (of the first eight streams after the thread's own, the second and third shared a queue in every process
 // measured), and launches on streams that share a queue run one after the other: four submit threads whose streams
 // sat on two queues measured 4.3 us per 9 MB batch, on four queues 3.6 us.  So the deck asks
-// (mfk_streams_share_queue, 50 us per pair, all streams idle) which of its streams share, and deals one stream of
+// (mfrt_streams_share_queue, 50 us per pair, all streams idle) which of its streams share, and deals one stream of
 // every queue before the second of any.  Streams beyond the deck are made on demand and not classified.
 struct StreamDeck {
     std::mutex lock;
@@ -149,7 +149,7 @@ struct StreamDeck {
             }
             uint32_t q = static_cast<uint32_t>(firstOfQueue.size());   // a queue of its own unless it shares one
             for (uint32_t c = 0; known && c < firstOfQueue.size(); ++c) {
-                const int shared = mfk_streams_share_queue(firstOfQueue[c], stream);
+                const int shared = mfrt_streams_share_queue(firstOfQueue[c], stream);
                 if (shared < 0) {
                     known = false;      // no answer: from here on the streams keep the order they were made in
                     q = static_cast<uint32_t>(firstOfQueue.size());

@@ -14,8 +14,6 @@
 // device, the host link (1 byte per payload byte) when one side is pinned
 // host memory.  No LDS, no MFMA: nothing here is reused or contracted.
 #include <hip/hip_runtime.h>
-
-#include <chrono>
 #include <hip/hip_ext.h>
 #include <stdint.h>
 
@@ -1023,70 +1021,6 @@ extern "C" int mfk_xcopy_inline(const void *inlinePlan, int route, uint32_t grid
 extern "C" uint32_t mfk_xcopy_window_units(void)
 {
     return mf::kWindowUnits;
-}
-
-// Whether two streams share a hardware queue.  The runtime deals its streams out over a few hardware queues, and
-// launches on streams that share one run one after the other however independent they are.  A single lane that waits
-// 40 us by the clock is launched on `a`, an empty kernel on `b`; when the empty kernel has ended, either the wait
-// still runs (different queues: 0) or it has ended too (the empty kernel had to queue behind it: 1).  -1: not known
-// (no clock rate, or the host took so long between the two launches that the answer would mean nothing).  Both
-// streams must be idle.  About 50 us.
-namespace mf {
-namespace {
-__global__ void XcopyDelayKernel(uint32_t ticks)
-{
-    const uint64_t t0 = wall_clock64();
-    while (wall_clock64() - t0 < ticks) {
-        __builtin_amdgcn_s_sleep(8);
-    }
-}
-
-__global__ void XcopyNothingKernel() {}
-}  // namespace
-}  // namespace mf
-
-extern "C" int mfk_streams_share_queue(void *a, void *b)
-{
-    int dev = 0;
-    int khz = 0;
-    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&khz, hipDeviceAttributeWallClockRate, dev) != hipSuccess ||
-        khz <= 0) {
-        return -1;
-    }
-    hipEvent_t ea = nullptr;
-    hipEvent_t eb = nullptr;
-    if (hipEventCreateWithFlags(&ea, hipEventDisableTiming) != hipSuccess ||
-        hipEventCreateWithFlags(&eb, hipEventDisableTiming) != hipSuccess) {
-        if (ea != nullptr) {
-            (void)hipEventDestroy(ea);
-        }
-        (void)hipGetLastError();
-        return -1;
-    }
-    const uint32_t ticks = static_cast<uint32_t>(static_cast<uint64_t>(khz) * 40 / 1000);   // 40 us
-    int answer = -1;
-    for (int attempt = 0; attempt < 3 && answer < 0; ++attempt) {
-        const auto t0 = std::chrono::steady_clock::now();
-        hipLaunchKernelGGL(mf::XcopyDelayKernel, dim3(1), dim3(1), 0, static_cast<hipStream_t>(a), ticks);
-        (void)hipEventRecord(ea, static_cast<hipStream_t>(a));
-        hipLaunchKernelGGL(mf::XcopyNothingKernel, dim3(1), dim3(1), 0, static_cast<hipStream_t>(b));
-        (void)hipEventRecord(eb, static_cast<hipStream_t>(b));
-        const auto t1 = std::chrono::steady_clock::now();
-        if (hipGetLastError() != hipSuccess || hipEventSynchronize(eb) != hipSuccess) {
-            break;
-        }
-        const bool firstEnded = hipEventQuery(ea) == hipSuccess;
-        (void)hipGetLastError();   // hipErrorNotReady is the other answer, not a failure
-        if (hipEventSynchronize(ea) != hipSuccess) {
-            break;
-        }
-        if (std::chrono::duration<double, std::micro>(t1 - t0).count() < 20.0) {
-            answer = firstEnded ? 1 : 0;
-        }
-    }
-    (void)hipEventDestroy(ea);
-    (void)hipEventDestroy(eb);
-    return answer;
 }
 
 // 1 when the period of a windowed launch can be computed on the current device (its constant-rate clock is known).

@@ -61,7 +61,10 @@ void *mfrt_event_create(void);
 int mfrt_event_destroy(void *event);
 int mfrt_event_record(void *event, void *stream);
 int mfrt_event_sync(void *event);
-int mfrt_stream_wait_event(void *stream, void *event);   /* work queued on `stream` afterwards waits for the event */
+int mfrt_stream_wait_event(void *stream, void *event);
+/* 1: launches on the two (idle) streams run one after the other because the streams share a hardware queue; 0: they
+ * run side by side; -1: not known.  About 50 us. */
+int mfrt_streams_share_queue(void *a, void *b);   /* work queued on `stream` afterwards waits for the event */
 int mfrt_event_done(void *event);       /* 1 finished, 0 pending, <0 error */
 float mfrt_event_elapsed_ms(void *start, void *stop);
 
@@ -91,9 +94,6 @@ int mfk_xcopy_windowed(const void *inlinePlan, uint32_t windowMBps, void *mask, 
 int mfk_xcopy_table(const void *tablePlan, int route, uint32_t grid, void *mask, uint32_t maskValue, void *stream,
                     uint32_t holdNanos);
 /* Launches every copy kernel once on empty plans (a kernel's first launch is not capturable into a HIP graph). */
-/* 1: launches on the two (idle) streams run one after the other because the streams share a hardware queue; 0: they
- * run side by side; -1: not known.  About 50 us. */
-int mfk_streams_share_queue(void *a, void *b);
 int mfk_xcopy_prelaunch(void *stream);
 /* Times the calibration workloads on `stream` with HIP events, in 1 GiB of device memory it allocates and frees:
  * out[0 .. 3] = us per 2196-chunk batch without a hold and held for holdNanos[0 .. 2]; out[4 .. 6] = us per 512 MiB

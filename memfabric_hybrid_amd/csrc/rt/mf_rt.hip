@@ -6,6 +6,8 @@
 // stream is the submission queue, an event is the completion record.
 #include <hip/hip_runtime.h>
 
+#include <chrono>
+
 #include <atomic>
 #include <cstring>
 #include <mutex>
@@ -349,4 +351,66 @@ extern "C" int mfrt_memset(void *dst, int value, uint64_t bytes)
 extern "C" int mfrt_memcpy_async(void *dst, const void *src, uint64_t bytes, void *stream)
 {
     return Code(hipMemcpyAsync(dst, src, bytes, hipMemcpyDefault, static_cast<hipStream_t>(stream)));
+}
+
+// Whether two streams share a hardware queue.  The runtime deals its streams out over a few hardware queues, and
+// launches on streams that share one run one after the other however independent they are.  A single lane that waits
+// 40 us by the clock is launched on `a`, an empty kernel on `b`; when the empty kernel has ended, either the wait
+// still runs (different queues: 0) or it has ended too (the empty kernel had to queue behind it: 1).  -1: not known
+// (no clock rate, or the host took so long between the two launches that the answer would mean nothing).  Both
+// streams must be idle.  About 50 us.
+namespace {
+__global__ void DelayKernel(uint32_t ticks)
+{
+    const uint64_t t0 = wall_clock64();
+    while (wall_clock64() - t0 < ticks) {
+        __builtin_amdgcn_s_sleep(8);
+    }
+}
+
+__global__ void NothingKernel() {}
+}  // namespace
+
+extern "C" int mfrt_streams_share_queue(void *a, void *b)
+{
+    int dev = 0;
+    int khz = 0;
+    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&khz, hipDeviceAttributeWallClockRate, dev) != hipSuccess ||
+        khz <= 0) {
+        return -1;
+    }
+    hipEvent_t ea = nullptr;
+    hipEvent_t eb = nullptr;
+    if (hipEventCreateWithFlags(&ea, hipEventDisableTiming) != hipSuccess ||
+        hipEventCreateWithFlags(&eb, hipEventDisableTiming) != hipSuccess) {
+        if (ea != nullptr) {
+            (void)hipEventDestroy(ea);
+        }
+        (void)hipGetLastError();
+        return -1;
+    }
+    const uint32_t ticks = static_cast<uint32_t>(static_cast<uint64_t>(khz) * 40 / 1000);   // 40 us
+    int answer = -1;
+    for (int attempt = 0; attempt < 3 && answer < 0; ++attempt) {
+        const auto t0 = std::chrono::steady_clock::now();
+        hipLaunchKernelGGL(DelayKernel, dim3(1), dim3(1), 0, static_cast<hipStream_t>(a), ticks);
+        (void)hipEventRecord(ea, static_cast<hipStream_t>(a));
+        hipLaunchKernelGGL(NothingKernel, dim3(1), dim3(1), 0, static_cast<hipStream_t>(b));
+        (void)hipEventRecord(eb, static_cast<hipStream_t>(b));
+        const auto t1 = std::chrono::steady_clock::now();
+        if (hipGetLastError() != hipSuccess || hipEventSynchronize(eb) != hipSuccess) {
+            break;
+        }
+        const bool firstEnded = hipEventQuery(ea) == hipSuccess;
+        (void)hipGetLastError();   // hipErrorNotReady is the other answer, not a failure
+        if (hipEventSynchronize(ea) != hipSuccess) {
+            break;
+        }
+        if (std::chrono::duration<double, std::micro>(t1 - t0).count() < 20.0) {
+            answer = firstEnded ? 1 : 0;
+        }
+    }
+    (void)hipEventDestroy(ea);
+    (void)hipEventDestroy(eb);
+    return answer;
 }

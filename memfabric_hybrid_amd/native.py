@@ -231,6 +231,7 @@ _SIGNATURES = {
     "mfrt_event_record": (ctypes.c_int, [vp, vp]),
     "mfrt_event_sync": (ctypes.c_int, [vp]),
     "mfrt_stream_wait_event": (ctypes.c_int, [vp, vp]),
+    "mfrt_streams_share_queue": (ctypes.c_int, [vp, vp]),
     "mfrt_event_done": (ctypes.c_int, [vp]),
     "mfrt_event_elapsed_ms": (ctypes.c_float, [vp, vp]),
     "mfrt_memcpy": (ctypes.c_int, [vp, vp, u64]),

@@ -218,7 +218,7 @@ static uint32_t FakeQueueOf(const void *stream)
     const uint64_t index = *static_cast<const uint64_t *>(stream);
     return index < 8 ? first[index] : static_cast<uint32_t>(index % 4);
 }
-int mfk_streams_share_queue(void *a, void *b)
+int mfrt_streams_share_queue(void *a, void *b)
 {
     if (g_queueAnswers == 1) {
         return -1;

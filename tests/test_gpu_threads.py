@@ -221,6 +221,10 @@ def test_streams_are_dealt_one_per_hardware_queue(lib):
                 overlapped += 0 if lib.mfrt_event_done(ea) else 1
                 assert lib.mfrt_event_sync(ea) == 0
             assert overlapped >= 4, "the second thread's stream waits for the first thread's copies"
+            # the library's own probe says the same, and knows a stream shares a queue with itself
+            assert lib.mfrt_device_sync() == 0
+            assert lib.mfrt_streams_share_queue(mine, other[0]) == 0
+            assert lib.mfrt_streams_share_queue(mine, mine) == 1
         finally:
             lib.mfrt_event_destroy(ea)
             lib.mfrt_event_destroy(eb)
