@@ -92,7 +92,7 @@ __global__ __launch_bounds__(kRectThreads) void Copy2dKernel(const RectPlan p)
 // one chunk per period each; sixteen loads per lane at the wave's offset into the read half of the period, the
 // stores at the same offset into the write half.  plan.first counts these chunks (RectWindowChunks), a
 // rectangle holds fewer than 2^32 units, rowsPerChunk is not used.
-__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(4, 4))) void Copy2dWindowKernel(const RectPlan p, uint32_t period, uint32_t seq)
+__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(5))) void Copy2dWindowKernel(const RectPlan p, uint32_t period, uint32_t seq)
 {
     // Only what the search needs stays in vector registers; the rectangle a chunk belongs to is read from the
     // argument block by scalar loads once it is known (a period is microseconds long, their latency does not show).
@@ -127,54 +127,46 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(4, 4))) void
         const uint32_t col0 = base - row0 * rwu;
         const MF_GLOBAL u32x4 *s = reinterpret_cast<const MF_GLOBAL u32x4 *>(rs) + static_cast<uint64_t>(row0) * rsp;
         MF_GLOBAL u32x4 *d = reinterpret_cast<MF_GLOBAL u32x4 *>(rd) + static_cast<uint64_t>(row0) * rdp;
-        uint32_t row[kRectWindowDepth];   // the column follows from the row: kept in 16 registers, not 64 of offsets
-#pragma unroll
-        for (uint32_t j = 0; j < kRectWindowDepth; ++j) {
+        // Row and column of a unit are worked out where its address is needed, before the loads and again before the
+        // stores, from a lane offset the compiler cannot see through: kept across the waits (or worked out ahead of them,
+        // as it prefers) sixteen rows or thirty-two addresses beside the data take the kernel past the registers at which
+        // all kRectWindowWaves waves are resident together with room to spare, which the schedule needs.
+        uint32_t x0 = col0 + lane;
+        auto unitOffset = [&](uint32_t j, uint32_t pitch) -> uint64_t {
+            uint32_t row;
             uint32_t col;
-            RectWindowRowCol(col0 + j * 64 + lane, rwu, rmg, row[j], col);
-        }
-        const uint32_t x0 = col0 + lane;
+            RectWindowRowCol(x0 + j * 64, rwu, rmg, row, col);
+            return static_cast<uint64_t>(row) * pitch + col;
+        };
         u32x4 v[kRectWindowDepth];
         WaitForClock(slot);
-        // Addresses are worked out where they are used, from the sixteen row numbers: worked out ahead of the waits,
-        // as the compiler prefers, sixteen load and sixteen store addresses beside the data take the kernel past the
-        // 128 registers at which all kRectWindowWaves waves are resident together, which the schedule needs.
-#pragma unroll
-        for (uint32_t j = 0; j < kRectWindowDepth; ++j) {
-            asm volatile("" : "+v"(row[j]));
-        }
+        asm volatile("" : "+v"(x0));
         if (n == kRectWindowUnits) {
 #pragma unroll
             for (uint32_t j = 0; j < kRectWindowDepth; ++j) {
-                v[j] = __builtin_nontemporal_load(s + (static_cast<uint64_t>(row[j]) * rsp + (x0 + j * 64 - row[j] * rwu)));
+                v[j] = __builtin_nontemporal_load(s + unitOffset(j, rsp));
             }
             asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
             WaitForClock(slot + half);
+            asm volatile("" : "+v"(x0));
 #pragma unroll
             for (uint32_t j = 0; j < kRectWindowDepth; ++j) {
-                asm volatile("" : "+v"(row[j]));
-            }
-#pragma unroll
-            for (uint32_t j = 0; j < kRectWindowDepth; ++j) {
-                __builtin_nontemporal_store(v[j], d + (static_cast<uint64_t>(row[j]) * rdp + (x0 + j * 64 - row[j] * rwu)));
+                __builtin_nontemporal_store(v[j], d + unitOffset(j, rdp));
             }
         } else {
 #pragma unroll
             for (uint32_t j = 0; j < kRectWindowDepth; ++j) {
                 if (j * 64 + lane < n) {
-                    v[j] = __builtin_nontemporal_load(s + (static_cast<uint64_t>(row[j]) * rsp + (x0 + j * 64 - row[j] * rwu)));
+                    v[j] = __builtin_nontemporal_load(s + unitOffset(j, rsp));
                 }
             }
             asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
             WaitForClock(slot + half);
-#pragma unroll
-            for (uint32_t j = 0; j < kRectWindowDepth; ++j) {
-                asm volatile("" : "+v"(row[j]));
-            }
+            asm volatile("" : "+v"(x0));
 #pragma unroll
             for (uint32_t j = 0; j < kRectWindowDepth; ++j) {
                 if (j * 64 + lane < n) {
-                    __builtin_nontemporal_store(v[j], d + (static_cast<uint64_t>(row[j]) * rdp + (x0 + j * 64 - row[j] * rwu)));
+                    __builtin_nontemporal_store(v[j], d + unitOffset(j, rdp));
                 }
             }
         }
