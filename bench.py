@@ -788,8 +788,8 @@ def main():
         # a child process of its own, started before this one touches the GPU
         import subprocess
         exe = os.path.join(ROOT, "bench_phases", "mf_batch_phases")
-        if not os.path.exists(exe):   # not part of the product build: compiled on demand
-            subprocess.run(["make", "-C", os.path.join(ROOT, "bench_phases")], check=True, stdout=subprocess.DEVNULL)
+        # not part of the product build: compiled on demand, and again whenever the kernel sources it includes have changed
+        subprocess.run(["make", "-C", os.path.join(ROOT, "bench_phases")], check=True, stdout=subprocess.DEVNULL)
         done = subprocess.run([exe] + args.phase_args, stdout=subprocess.PIPE, text=True, timeout=600)
         sys.stdout.write(done.stdout)
         sys.exit(done.returncode)

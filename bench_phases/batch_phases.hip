@@ -151,6 +151,8 @@ struct Batch {
     TablePlan pinned;                   // triples in pinned host memory, owner by pattern
     TablePlan hbm;                      // triples in HBM, owner by pattern
     TablePlan grouped;                  // triples, prefix and group map in HBM, no pattern
+    TablePlan deepPinned;               // chunks of 16 KiB (what the library takes for 24 to 64 MiB), triples in pinned memory
+    TablePlan deepHbm;                  // the same with the triples in HBM
     uint32_t nchunk;
 };
 
@@ -310,6 +312,17 @@ std::vector<Batch> MakeBatches(char *pool, uint64_t poolBytes, int count, uint32
         const char *dev = devTables + b * tableBytes;
         plan.triples = reinterpret_cast<const uint64_t *>(dev);
         batch.hbm = plan;
+        {
+            TablePlan deep = batch.pinned;
+            deep.units = kDeepUnits;
+            deep.pattern.chunksPerPeriod = 9;      // 128 KiB: eight chunks of 16 KiB, 16 KiB: one
+            deep.pattern.start[1] = 8;
+            deep.pattern.start[2] = 9;
+            deep.nchunk = nseg / 2 * 9;
+            batch.deepPinned = deep;
+            deep.triples = reinterpret_cast<const uint64_t *>(dev);
+            batch.deepHbm = deep;
+        }
         plan.pattern = ChunkPattern{};
         plan.first = reinterpret_cast<const uint32_t *>(dev + tableWords64 * 8);
         plan.group = plan.first + nseg + 1;
@@ -351,9 +364,18 @@ void LaunchInlineProduct(const InlinePlan &plan, hipStream_t s, bool held, bool 
     }
 }
 
+// What the library launches for a batch of 24 to 64 MiB: 16 KiB per wave, sixteen loads per lane, stores held back
+// (1.6 us longer where every workgroup first fetches its descriptor over the link).
+void LaunchTableDeep(const TablePlan &plan, hipStream_t s, bool pinned)
+{
+    const uint32_t nanos = HoldNanosFor(plan.nchunk, plan.nchunk, plan.units, false);
+    const uint32_t ticks = HoldTicks(nanos != 0 && pinned ? nanos + 1600 : nanos);
+    hipLaunchKernelGGL((XcopyTableKernel<true, kStoreStream, false, kHoldDeep>), dim3(plan.nchunk), dim3(64), 0, s, plan, ticks);
+}
+
 void LaunchTableProduct(const TablePlan &plan, hipStream_t s)
 {
-    hipLaunchKernelGGL((XcopyTableKernel<true, kStoreStream, false>), dim3(plan.nchunk), dim3(64), 0, s, plan);
+    hipLaunchKernelGGL((XcopyTableKernel<true, kStoreStream, false>), dim3(plan.nchunk), dim3(64), 0, s, plan, 0u);
 }
 
 void Measure(uint32_t requests, char *pool, uint64_t poolBytes, hipStream_t s)
@@ -383,6 +405,10 @@ void Measure(uint32_t requests, char *pool, uint64_t poolBytes, hipStream_t s)
                         [](const Batch &b, hipStream_t st) { LaunchTableProduct(b.pinned, st); }, true});
         rows.push_back({"product_table_kernel_hbm_descriptors", [](const Batch &b, hipStream_t st) { LaunchTableProduct(b.hbm, st); }, true});
         rows.push_back({"product_table_kernel_group_map", [](const Batch &b, hipStream_t st) { LaunchTableProduct(b.grouped, st); }, true});
+        rows.push_back({"product_table_kernel_16KiB_chunks_held_pinned_descriptors",
+                        [](const Batch &b, hipStream_t st) { LaunchTableDeep(b.deepPinned, st, true); }, true});
+        rows.push_back({"product_table_kernel_16KiB_chunks_held_hbm_descriptors",
+                        [](const Batch &b, hipStream_t st) { LaunchTableDeep(b.deepHbm, st, false); }, true});
         rows.push_back({"inline_launches_first_ordered_rest_any_order", [](const Batch &b, hipStream_t st) {
                             for (size_t i = 0; i < b.slices.size(); ++i) {
                                 LaunchInlineProduct(b.slices[i], st, false, i != 0);
