@@ -187,7 +187,8 @@ MF_EXPORT int32_t mf_xcopy_tune_hold(uint32_t deepHold, int32_t pinnedExtraNanos
     return BM_OK;
 }
 
-MF_EXPORT int32_t mf_xcopy_calibration(int32_t *holdEnabled, int32_t *holdDeltaNanos, uint32_t *windowMBps, float *micros)
+MF_EXPORT int32_t mf_xcopy_calibration(int32_t *holdEnabled, int32_t *holdDeltaNanos, uint32_t *windowMBps, uint32_t *windowLongMBps,
+                                       float *micros)
 {
     const XcopyCalibration &c = XcopyEngine::Instance().Calibration();
     if (holdEnabled != nullptr) {
@@ -199,11 +200,14 @@ MF_EXPORT int32_t mf_xcopy_calibration(int32_t *holdEnabled, int32_t *holdDeltaN
     if (windowMBps != nullptr) {
         *windowMBps = XcopyEngine::Instance().Tuning().windowMBps;
     }
+    if (windowLongMBps != nullptr) {
+        *windowLongMBps = XcopyEngine::Instance().Tuning().windowLongMBps;
+    }
     if (micros != nullptr) {
         for (int i = 0; i < 4; ++i) {
             micros[i] = c.batchMicros[i];
         }
-        for (int i = 0; i < 3; ++i) {
+        for (int i = 0; i < 4; ++i) {
             micros[4 + i] = c.copyMicros[i];
         }
     }
@@ -225,6 +229,7 @@ MF_EXPORT int32_t mf_xcopy_windows(uint32_t megabytesPerSecond)
         MF_FAIL(BM_INVALID_PARAM, "windows: 0 (never) or a rate between 1 000 000 and 16 000 000 MB/s, got " << megabytesPerSecond);
     }
     XcopyEngine::Instance().Tuning().windowMBps = megabytesPerSecond;
+    XcopyEngine::Instance().Tuning().windowLongMBps = megabytesPerSecond;   // a rate set by hand holds for every windowed launch
     return BM_OK;
 }
 

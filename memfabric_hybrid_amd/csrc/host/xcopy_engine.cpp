@@ -953,14 +953,16 @@ uint64_t BuildTableDirect(const uint64_t *src, const uint64_t *dst, const uint64
     return run;
 }
 
-void ChooseCalibration(const float *batchMicros, const float *copyMicros, uint32_t defaultWindowMBps, XcopyCalibration &out)
+void ChooseCalibration(const float *batchMicros, const float *copyMicros, uint32_t defaultWindowMBps, uint32_t defaultLongMBps,
+                       XcopyCalibration &out)
 {
     out = XcopyCalibration{};
     out.windowMBps = defaultWindowMBps;
+    out.windowLongMBps = defaultLongMBps;
     for (int i = 0; i < 4; ++i) {
         out.batchMicros[i] = batchMicros[i];
     }
-    for (int i = 0; i < 3; ++i) {
+    for (int i = 0; i < 4; ++i) {
         out.copyMicros[i] = copyMicros[i];
     }
     const bool batchMeasured = batchMicros[0] > 0 && batchMicros[1] > 0 && batchMicros[2] > 0 && batchMicros[3] > 0;
@@ -983,6 +985,8 @@ void ChooseCalibration(const float *batchMicros, const float *copyMicros, uint32
         const uint32_t rate = slowerWins ? static_cast<uint32_t>(static_cast<uint64_t>(defaultWindowMBps) * kCalibrateSlowerWindowPercent / 100)
                                          : defaultWindowMBps;
         out.windowMBps = windowed <= copyMicros[0] * (1.0f - kCalibrateMinWindowGain) ? rate : 0u;
+        // the higher rate of long segments only where one long segment held it here: 2 % better than the rate just chosen
+        out.windowLongMBps = out.windowMBps != 0 && copyMicros[3] > 0 && copyMicros[3] < windowed * 0.98f ? defaultLongMBps : out.windowMBps;
         out.ran = true;
     }
 }
@@ -999,20 +1003,23 @@ int XcopyEngine::Calibrate()
     const uint32_t rule = HoldNanosFor(2196, 2196, kXcopyThreads, false);
     const uint32_t holds[3] = {rule - kCalibrateHoldStepNanos, rule, rule + kCalibrateHoldStepNanos};
     const uint32_t defaultRate = XcopyTuning{}.windowMBps;
-    const uint32_t rates[2] = {defaultRate, static_cast<uint32_t>(static_cast<uint64_t>(defaultRate) * kCalibrateSlowerWindowPercent / 100)};
-    float us[7] = {};
+    const uint32_t defaultLong = XcopyTuning{}.windowLongMBps;
+    const uint32_t rates[3] = {defaultRate, static_cast<uint32_t>(static_cast<uint64_t>(defaultRate) * kCalibrateSlowerWindowPercent / 100),
+                               defaultLong};
+    float us[8] = {};
     const int err = mfk_xcopy_calibrate(stream, holds, rates, us);
     if (err != 0) {
         calibration_ = XcopyCalibration{};
         MF_ERROR("calibration run failed (" << mfrt_error_string(err) << "): the fitted defaults stay");
         return BM_ERROR;
     }
-    ChooseCalibration(us, us + 4, defaultRate, calibration_);
+    ChooseCalibration(us, us + 4, defaultRate, defaultLong, calibration_);
     if (calibration_.ran) {
         tuning_.holdDeltaNanos = calibration_.holdDeltaNanos;
         tuning_.holdCalibratedOff = !calibration_.holdEnabled;
         if (windowsAvailable_) {
             tuning_.windowMBps = calibration_.windowMBps;
+            tuning_.windowLongMBps = calibration_.windowLongMBps;
             windowRateCalibrated_ = true;
         }
     }
@@ -1044,6 +1051,7 @@ int XcopyEngine::Start(int device)
     tuning_.holdCalibratedOff = false;
     if (windowRateCalibrated_) {   // what an earlier start of this process chose does not outlive it
         tuning_.windowMBps = XcopyTuning{}.windowMBps;
+        tuning_.windowLongMBps = XcopyTuning{}.windowLongMBps;
         windowRateCalibrated_ = false;
     }
     calibration_ = XcopyCalibration{};
@@ -1308,6 +1316,67 @@ int XcopyEngine::Submit(const uint64_t *src, const uint64_t *dst, const uint64_t
     return SubmitOne(src, dst, len, n, route, stream, mask, maskValue, unordered, true);
 }
 
+// A batch of up to kInlineSegs segments that moves twice kWindowMinBytes and more, submitted as consecutive runs of
+// kWindowMinBytes to twice that, one windowed launch each.  Runs end at segment ends where the segments are short and
+// inside a segment, at a multiple of 1 MiB from its start, where one is long.
+int XcopyEngine::SubmitInPieces(const uint64_t *src, const uint64_t *dst, const uint64_t *len, uint32_t n, uint64_t total, int route,
+                                void *stream, void *mask, uint32_t maskValue)
+{
+    const uint64_t pieces = total / kWindowMinBytes;
+    const uint64_t target = (total + pieces - 1) / pieces;
+    constexpr uint64_t kCutUnit = 1ull << 20;
+    std::vector<uint64_t> ps;
+    std::vector<uint64_t> pd;
+    std::vector<uint64_t> pl;
+    uint64_t inPiece = 0;
+    uint64_t left = total;
+    auto flush = [&](bool last) -> int {
+        if (ps.empty()) {
+            return BM_OK;
+        }
+        const int ret = SubmitOne(ps.data(), pd.data(), pl.data(), static_cast<uint32_t>(ps.size()), route, stream, last ? mask : nullptr,
+                                  maskValue, false, false);
+        ps.clear();
+        pd.clear();
+        pl.clear();
+        inPiece = 0;
+        return ret;
+    };
+    for (uint32_t i = 0; i < n; ++i) {
+        uint64_t at = 0;
+        while (at < len[i]) {
+            uint64_t take = len[i] - at;
+            const uint64_t room = target > inPiece ? target - inPiece : 0;
+            // what is left behind this piece must still make a launch of its own, else it stays with this one
+            if (take > room && left - room >= kWindowMinBytes) {
+                const uint64_t cut = room / kCutUnit * kCutUnit;
+                if (take >= 16 * kCutUnit && cut != 0 && take - cut >= kCutUnit) {
+                    take = cut;
+                } else if (inPiece != 0 && room < take / 2) {
+                    const int ret = flush(false);      // the segment starts the next piece whole
+                    if (ret != BM_OK) {
+                        return ret;
+                    }
+                    continue;
+                }
+            }
+            ps.push_back(src[i] + at);
+            pd.push_back(dst[i] + at);
+            pl.push_back(take);
+            at += take;
+            inPiece += take;
+            left -= take;
+            if (inPiece >= target && left >= kWindowMinBytes) {
+                const int ret = flush(false);
+                if (ret != BM_OK) {
+                    return ret;
+                }
+            }
+        }
+    }
+    return flush(true);
+}
+
 // maySlice: a table of long segments may be cut into launches of kInlineSegs segments; a slice is submitted
 // with false, so that one that cannot take the kernel-argument form (a segment of 4 GiB and more is cut into
 // pieces, which can carry it past kInlineSegs rows) goes to the table form instead of being sliced again.
@@ -1363,6 +1432,7 @@ int XcopyEngine::SubmitOne(const uint64_t *src, const uint64_t *dst, const uint6
     uint32_t units = 0;
     bool oversized = false;      // a run the 32-bit length of the inline table cannot hold is possible
     bool windowed = false;
+    uint32_t windowRate = tuning_.windowMBps;
     uint64_t queuedBytes = 0;
     if (n <= 4 * kInlineSegs) {  // small enough that a failed attempt costs next to nothing
         uint64_t total = 0;
@@ -1374,6 +1444,16 @@ int XcopyEngine::SubmitOne(const uint64_t *src, const uint64_t *dst, const uint6
         units = ChooseUnits(total, cu, route, tuning_);
         // Large HBM copies of one submitter: 16 KiB chunks for the kernel that alternates between read and write windows.
         windowed = !unordered && WindowsApply(total, route);
+        const bool longSegments = windowed && total / n >= kWindowLongSegmentBytes;
+        if (longSegments && maySlice && total >= 2 * kWindowMinBytes && n + total / kWindowMinBytes <= kInlineSegs) {
+            // A windowed launch that loses its schedule runs the rest of its bytes at the rate without windows, and the longer
+            // it runs the likelier that is: launches of kWindowMinBytes to twice that, each with a schedule of its own, hold
+            // a target the whole copy in one launch does not (2 GiB at 7.4 TB/s: 7.1 TB/s on average in four launches,
+            // 6.6 to 6.8 in one).  Only long segments are worth it: batches of segments of some 10 MB, which hold 6.6 TB/s
+            // in launches of 1.2 GB, measured 6.4 in launches of 540 MB at either rate.
+            return SubmitInPieces(src, dst, len, n, total, route, stream, mask, maskValue);
+        }
+        windowRate = longSegments && tuning_.windowLongMBps != 0 ? tuning_.windowLongMBps : tuning_.windowMBps;
         if (windowed) {
             units = mfk_xcopy_window_units();
         }
@@ -1390,7 +1470,7 @@ int XcopyEngine::SubmitOne(const uint64_t *src, const uint64_t *dst, const uint6
         inlined = BuildInlinePlan(ctx.segs, units, plan);
     }
     if (inlined && windowed) {
-        int err = mfk_xcopy_windowed(&plan, tuning_.windowMBps, mask, maskValue, stream);
+        int err = mfk_xcopy_windowed(&plan, windowRate, mask, maskValue, stream);
         if (err != 0) {
             MF_FAIL(BM_ERROR, "xcopy launch failed: " << mfrt_error_string(err));
         }
@@ -1436,7 +1516,7 @@ int XcopyEngine::SubmitOne(const uint64_t *src, const uint64_t *dst, const uint6
                 const uint32_t m = n - at < kInlineSegs ? n - at : kInlineSegs;
                 const bool last = at + m == n;
                 const int ret = SubmitOne(src + at, dst + at, len + at, m, route, stream, last ? mask : nullptr, maskValue, false,
-                                          false);
+                                          true);
                 if (ret != BM_OK) {
                     return ret;
                 }

@@ -1162,8 +1162,8 @@ extern "C" int mfk_xcopy_prelaunch(void *stream)
 
 // Calibration workloads, timed by events on `stream` (see XcopyEngine::Calibrate for what is chosen from them).
 // out[0 .. 3]: microseconds per batch of 122 segments (61 x 128 KiB and 16 KiB in turn, 2196 chunks, 32 tables in turn
-// inside 1 GiB of scratch) without a hold and held for holdNanos[0 .. 2]; out[4 .. 6]: microseconds per copy of 512 MiB by
-// the kernel without windows and in windows cut for windowMBps[0 .. 1].  The minimum of three rounds each.
+// inside 1 GiB of scratch) without a hold and held for holdNanos[0 .. 2]; out[4 .. 7]: microseconds per copy of 512 MiB by
+// the kernel without windows and in windows cut for windowMBps[0 .. 2].  The minimum of three rounds each.
 extern "C" int mfk_xcopy_calibrate(void *stream, const uint32_t *holdNanos, const uint32_t *windowMBps, float *out)
 {
     using namespace mf;
@@ -1250,7 +1250,7 @@ extern "C" int mfk_xcopy_calibrate(void *stream, const uint32_t *holdNanos, cons
         }
         return code != hipSuccess ? code : hipGetLastError();
     };
-    for (int i = 0; i < 7; ++i) {
+    for (int i = 0; i < 8; ++i) {
         out[i] = 0.0f;
     }
     for (int round = 0; round < 3; ++round) {
@@ -1264,7 +1264,7 @@ extern "C" int mfk_xcopy_calibrate(void *stream, const uint32_t *holdNanos, cons
         }
     }
     for (int round = 0; round < 3; ++round) {
-        for (int v = 0; v < 3; ++v) {
+        for (int v = 0; v < 4; ++v) {
             if (v == 0) {
                 big.units = kXcopyThreads;
                 big.nchunk = static_cast<uint32_t>(half / (kXcopyThreads * kUnitBytes));

@@ -96,8 +96,8 @@ int mfk_xcopy_table(const void *tablePlan, int route, uint32_t grid, void *mask,
 /* Launches every copy kernel once on empty plans (a kernel's first launch is not capturable into a HIP graph). */
 int mfk_xcopy_prelaunch(void *stream);
 /* Times the calibration workloads on `stream` with HIP events, in 1 GiB of device memory it allocates and frees:
- * out[0 .. 3] = us per 2196-chunk batch without a hold and held for holdNanos[0 .. 2]; out[4 .. 6] = us per 512 MiB
- * copy without windows and in windows cut for windowMBps[0 .. 1].  0, or a HIP error number. */
+ * out[0 .. 3] = us per 2196-chunk batch without a hold and held for holdNanos[0 .. 2]; out[4 .. 7] = us per 512 MiB
+ * copy without windows and in windows cut for windowMBps[0 .. 2].  0, or a HIP error number. */
 int mfk_xcopy_calibrate(void *stream, const uint32_t *holdNanos, const uint32_t *windowMBps, float *out);
 /* One lane stores `value` (as a 64-bit word, released at system scope) into `word` once everything queued on
  * `stream` before it has finished. */

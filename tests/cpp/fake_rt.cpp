@@ -287,7 +287,7 @@ int mfk_xcopy_inline(const void *inlinePlan, int, uint32_t, void *mask, uint32_t
 int mfk_xcopy_windows_available(void) { return 1; }
 int mfk_xcopy_prelaunch(void *) { return 0; }
 // The calibration "measures" what the test has put here (all zero: nothing measured, the defaults stay).
-static float g_calibration[7] = {};
+static float g_calibration[8] = {};
 static uint32_t g_calibrationHolds[3] = {};
 extern "C" void fake_rt_set_calibration(const float *us) { std::memcpy(g_calibration, us, sizeof(g_calibration)); }
 extern "C" const uint32_t *fake_rt_calibration_holds(void) { return g_calibrationHolds; }

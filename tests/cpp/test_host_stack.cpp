@@ -799,38 +799,46 @@ static void TestPlanners()
 static void TestCalibration()
 {
     const uint32_t rate = XcopyTuning{}.windowMBps;
+    const uint32_t longRate = XcopyTuning{}.windowLongMBps;
     XcopyCalibration c;
-    {   // the usual picture: the rule's wait is best, held stores gain 14 %, windows 7 %
+    {   // the usual picture: the rule's wait is best, held stores gain 14 %, windows 7 %, one long segment holds the higher rate
         const float batch[4] = {5.30f, 4.62f, 4.55f, 4.60f};
-        const float copy[3] = {172.0f, 160.0f, 163.0f};
-        ChooseCalibration(batch, copy, rate, c);
-        CHECK(c.ran && c.holdEnabled && c.holdDeltaNanos == 0 && c.windowMBps == rate);
+        const float copy[4] = {172.0f, 160.0f, 163.0f, 149.0f};
+        ChooseCalibration(batch, copy, rate, longRate, c);
+        CHECK(c.ran && c.holdEnabled && c.holdDeltaNanos == 0 && c.windowMBps == rate && c.windowLongMBps == longRate);
+    }
+    {   // the higher rate does not hold here (no better than the default by 2 %): long segments take the default too
+        const float batch[4] = {5.30f, 4.62f, 4.55f, 4.60f};
+        const float copy[4] = {172.0f, 160.0f, 163.0f, 158.5f};
+        ChooseCalibration(batch, copy, rate, longRate, c);
+        CHECK(c.windowMBps == rate && c.windowLongMBps == rate);
     }
     {   // a GPU whose loads land later: the longer wait wins clearly; windows only hold at the lower rate
         const float batch[4] = {5.30f, 4.95f, 4.80f, 4.60f};
-        const float copy[3] = {172.0f, 171.0f, 161.0f};
-        ChooseCalibration(batch, copy, rate, c);
-        CHECK(c.holdEnabled && c.holdDeltaNanos == kCalibrateHoldStepNanos && c.windowMBps == static_cast<uint32_t>(static_cast<uint64_t>(rate) * 94 / 100));
+        const float copy[4] = {172.0f, 171.0f, 161.0f, 176.0f};
+        ChooseCalibration(batch, copy, rate, longRate, c);
+        CHECK(c.holdEnabled && c.holdDeltaNanos == kCalibrateHoldStepNanos && c.windowMBps == static_cast<uint32_t>(static_cast<uint64_t>(rate) * 94 / 100) &&
+              c.windowLongMBps == c.windowMBps);
     }
     {   // a neighbour that is better by less than 1 % does not move the wait
         const float batch[4] = {5.30f, 4.53f, 4.55f, 4.60f};
-        const float copy[3] = {0.0f, 0.0f, 0.0f};
-        ChooseCalibration(batch, copy, rate, c);
-        CHECK(c.ran && c.holdDeltaNanos == 0 && c.windowMBps == rate);       // windows not measured: the default stays
+        const float copy[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+        ChooseCalibration(batch, copy, rate, longRate, c);
+        CHECK(c.ran && c.holdDeltaNanos == 0 && c.windowMBps == rate && c.windowLongMBps == longRate);   // windows not measured: the defaults stay
     }
     {   // a busy or capped chip: holding gains 2 %, windows lose: both off
         const float batch[4] = {5.30f, 5.25f, 5.20f, 5.28f};
-        const float copy[3] = {172.0f, 175.0f, 174.0f};
-        ChooseCalibration(batch, copy, rate, c);
-        CHECK(c.ran && !c.holdEnabled && c.windowMBps == 0);
+        const float copy[4] = {172.0f, 175.0f, 174.0f, 169.0f};
+        ChooseCalibration(batch, copy, rate, longRate, c);
+        CHECK(c.ran && !c.holdEnabled && c.windowMBps == 0 && c.windowLongMBps == 0);
     }
     {   // nothing measured
         const float none[4] = {0, 0, 0, 0};
-        ChooseCalibration(none, none, rate, c);
+        ChooseCalibration(none, none, rate, longRate, c);
         CHECK(!c.ran && c.holdEnabled && c.holdDeltaNanos == 0 && c.windowMBps == rate);
     }
     // through hybm_init: the engine applies what it chose, and mf_xcopy_hold_stores(-1) means the calibrated rule
-    const float shorter[7] = {5.30f, 4.40f, 4.60f, 4.70f, 172.0f, 160.0f, 163.0f};
+    const float shorter[8] = {5.30f, 4.40f, 4.60f, 4.70f, 172.0f, 160.0f, 163.0f, 150.0f};
     fake_rt_set_calibration(shorter);
     CHECK(hybm_init(0, 0) == BM_OK);
     const uint32_t rule = HoldNanosFor(2196, 2196, 256, false);
@@ -838,9 +846,10 @@ static void TestCalibration()
     int32_t enabled = -1;
     int32_t delta = 0;
     uint32_t mbps = 0;
-    float micros[7] = {};
-    CHECK(mf_xcopy_calibration(&enabled, &delta, &mbps, micros) == 1);
-    CHECK(enabled == 1 && delta == -200 && mbps == rate && micros[1] == 4.40f && micros[5] == 160.0f);
+    uint32_t longMbps = 0;
+    float micros[8] = {};
+    CHECK(mf_xcopy_calibration(&enabled, &delta, &mbps, &longMbps, micros) == 1);
+    CHECK(enabled == 1 && delta == -200 && mbps == rate && longMbps == longRate && micros[1] == 4.40f && micros[5] == 160.0f && micros[7] == 150.0f);
     {
         std::vector<uint8_t> from(12 << 20), to(12 << 20);
         const uint64_t fromBase = (reinterpret_cast<uint64_t>(from.data()) + 4095) & ~4095ull;
@@ -857,17 +866,18 @@ static void TestCalibration()
         CHECK(fake_rt_last_hold() == HoldNanosFor(2196, 2196, 256, false) - 200);
     }
     hybm_uninit();
-    const float lost[7] = {5.30f, 5.29f, 5.31f, 5.30f, 172.0f, 175.0f, 176.0f};
+    const float lost[8] = {5.30f, 5.29f, 5.31f, 5.30f, 172.0f, 175.0f, 176.0f, 177.0f};
     fake_rt_set_calibration(lost);
     CHECK(hybm_init(0, 0) == BM_OK);
-    CHECK(mf_xcopy_calibration(&enabled, &delta, &mbps, nullptr) == 1 && enabled == 0 && mbps == 0);
+    CHECK(mf_xcopy_calibration(&enabled, &delta, &mbps, &longMbps, nullptr) == 1 && enabled == 0 && mbps == 0 && longMbps == 0);
     hybm_uninit();
     setenv("MF_HIP_CALIBRATE", "0", 1);
     CHECK(hybm_init(0, 0) == BM_OK);
-    CHECK(mf_xcopy_calibration(&enabled, &delta, &mbps, nullptr) == 0 && enabled == 1 && delta == 0 && mbps == rate);
+    CHECK(mf_xcopy_calibration(&enabled, &delta, &mbps, &longMbps, nullptr) == 0 && enabled == 1 && delta == 0 && mbps == rate &&
+          longMbps == longRate);
     hybm_uninit();
     unsetenv("MF_HIP_CALIBRATE");
-    const float none[7] = {};
+    const float none[8] = {};
     fake_rt_set_calibration(none);
 }
 
@@ -1041,7 +1051,8 @@ static void TestLongSegments()
         CHECK(mf_xcopy_launch_count() - before == 1);          // a pattern of period 1: no upload
     }
     {
-        // 600 long segments are cut into slices of 128; the slice that holds a 5 GiB segment takes the table form, the others the windowed one
+        // 600 long segments are cut into slices of 128; the slice with the 5 GiB segment has more chunks than the kernel-argument
+        // form counts and goes through the table (upload + launch); everything in windows, the completion word behind the last launch
         const uint32_t n = 600;
         std::vector<uint64_t> src(n), dst(n), len(n, 8u << 20);
         for (uint32_t i = 0; i < n; ++i) {
@@ -1053,7 +1064,8 @@ static void TestLongSegments()
         const uint64_t before = mf_xcopy_launch_count();
         (void)fake_rt_last_window();
         CHECK(engine.Submit(src.data(), dst.data(), len.data(), n, MF_ROUTE_HBM, stream, &word, 32) == BM_OK);
-        CHECK(mf_xcopy_launch_count() - before == 6);          // 128 + 128 + (upload + table) + 128 + 88
+        // 128 + 128 + (upload + table) + 128 + 88
+        CHECK(mf_xcopy_launch_count() - before == 6);
         CHECK(word == 32);
         CHECK(fake_rt_last_window() != 0);
     }
@@ -1432,14 +1444,51 @@ static void TestWindows()
     uint64_t d1 = s1 + gib + 3;                    // an odd destination: head and tail bytes
     uint64_t l1 = gib;
     (void)fake_rt_last_window();
+    uint64_t launchesBefore = mf_xcopy_launch_count();
     CHECK(engine.Submit(&s1, &d1, &l1, 1, MF_ROUTE_HBM, stream, nullptr, 0) == BM_OK);
-    CHECK(fake_rt_last_window() == 6800000);
+    CHECK(fake_rt_last_window() == 7400000);
+    CHECK(mf_xcopy_launch_count() - launchesBefore == 2);      // twice the minimum: two launches of 512 MiB, a schedule each
     CHECK(engine.DrainThread() == BM_OK);
     bool ok = true;
     for (uint64_t i = 0; i < gib; i += 4093) {
         ok = ok && mem[gib + 3 + i] == static_cast<uint8_t>(i * 7 + 1);
     }
     CHECK(ok && mem[gib + 3 + gib - 1] == mem[gib - 1]);
+    {
+        // three segments, 600 + 24 + 400 MiB: the first piece ends inside the long segment, at a multiple of 1 MiB, the
+        // second takes its rest and the others; then 64 segments of 16 MiB: pieces end where segments end
+        const uint64_t mib = 1ull << 20;
+        std::memset(mem.data() + gib, 0, gib);
+        uint64_t src3[3] = {s1, s1 + 600 * mib, s1 + 624 * mib};
+        uint64_t dst3[3] = {s1 + gib, s1 + gib + 600 * mib, s1 + gib + 624 * mib};
+        uint64_t len3[3] = {600 * mib, 24 * mib, 400 * mib};
+        uint64_t word = 0;
+        launchesBefore = mf_xcopy_launch_count();
+        CHECK(engine.Submit(src3, dst3, len3, 3, MF_ROUTE_HBM, stream, &word, 32) == BM_OK);
+        CHECK(mf_xcopy_launch_count() - launchesBefore == 2 && word == 32);
+        CHECK(engine.DrainThread() == BM_OK);
+        bool same = true;
+        for (uint64_t i = 0; i < gib; i += 4093) {
+            same = same && mem[gib + i] == mem[i];
+        }
+        CHECK(same && mem[2 * gib - 1] == mem[gib - 1]);
+        std::memset(mem.data() + gib, 0, gib);
+        std::vector<uint64_t> src64(64), dst64(64), len64(64, 16 * mib - 4096);
+        for (uint32_t i = 0; i < 64; ++i) {
+            src64[i] = s1 + i * 16 * mib;
+            dst64[i] = s1 + gib + ((i * 5) % 64) * 16 * mib + 7;
+        }
+        launchesBefore = mf_xcopy_launch_count();
+        CHECK(engine.Submit(src64.data(), dst64.data(), len64.data(), 64, MF_ROUTE_HBM, stream, nullptr, 0) == BM_OK);
+        CHECK(mf_xcopy_launch_count() - launchesBefore == 1);      // 1023.75 MiB: below twice the minimum, one launch
+        CHECK(engine.DrainThread() == BM_OK);
+        same = true;
+        for (uint32_t i = 0; i < 64 && same; ++i) {
+            same = std::memcmp(reinterpret_cast<void *>(dst64[i]), reinterpret_cast<void *>(src64[i]), len64[i]) == 0;
+        }
+        CHECK(same);
+        CHECK(fake_rt_last_window() == 6800000);       // segments of 16 MiB are not long ones: the general rate
+    }
     l1 = (gib >> 1) - 1;                           // one byte below the limit: the ordinary form
     CHECK(engine.Submit(&s1, &d1, &l1, 1, MF_ROUTE_HBM, stream, nullptr, 0) == BM_OK);
     CHECK(fake_rt_last_window() == 0);
