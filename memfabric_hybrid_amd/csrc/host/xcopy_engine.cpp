@@ -1445,7 +1445,7 @@ int XcopyEngine::SubmitOne(const uint64_t *src, const uint64_t *dst, const uint6
         // Large HBM copies of one submitter: 16 KiB chunks for the kernel that alternates between read and write windows.
         windowed = !unordered && WindowsApply(total, route);
         const bool longSegments = windowed && total / n >= kWindowLongSegmentBytes;
-        if (longSegments && maySlice && total >= 2 * kWindowMinBytes && n + total / kWindowMinBytes <= kInlineSegs) {
+        if (longSegments && maySlice && total >= 2 * kWindowMinBytes) {
             // A windowed launch that loses its schedule runs the rest of its bytes at the rate without windows, and the longer
             // it runs the likelier that is: launches of kWindowMinBytes to twice that, each with a schedule of its own, hold
             // a target the whole copy in one launch does not (2 GiB at 7.4 TB/s: 7.1 TB/s on average in four launches,

@@ -1048,7 +1048,12 @@ static void TestLongSegments()
         uint64_t len = 129 * gib + 5;
         const uint64_t before = mf_xcopy_launch_count();
         CHECK(engine.Submit(&src, &dst, &len, 1, MF_ROUTE_HBM, stream, nullptr, 0) == BM_OK);
-        CHECK(mf_xcopy_launch_count() - before == 1);          // a pattern of period 1: no upload
+        CHECK(mf_xcopy_launch_count() - before == 258);        // windowed launches of 512 MiB, however long the segment
+        CHECK(fake_rt_last_window() != 0);
+        // declared independent of what is in flight it takes no windows: one launch of the table form, a pattern of period 1, no upload
+        const uint64_t again = mf_xcopy_launch_count();
+        CHECK(engine.Submit(&src, &dst, &len, 1, MF_ROUTE_HBM, stream, nullptr, 0, true) == BM_OK);
+        CHECK(mf_xcopy_launch_count() - again == 1);
     }
     {
         // 600 long segments are cut into slices of 128; the slice with the 5 GiB segment has more chunks than the kernel-argument

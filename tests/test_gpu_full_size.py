@@ -4,6 +4,8 @@ copies host -> device -> device -> host through smem_bm_copy, and the paged KV g
 40 GiB pool.  Sources are built from one random block XORed with a per-block constant, so every
 64 MiB of a large buffer differs and a piece that lands at a wrong offset cannot go unnoticed."""
 
+import ctypes
+
 import numpy as np
 import pytest
 
@@ -127,6 +129,58 @@ def test_ragged_batch_above_one_gib_in_read_and_write_windows(pool, lib, oracle,
         assert np.array_equal(got[d_off - lo:d_off - lo + n], host_all[s_off:s_off + n]), d_off
         cursor = d_off + n
     assert np.all(got[cursor - lo:] == 0x5A)
+
+
+def test_one_segment_beyond_four_gib_goes_out_in_windowed_launches(lib, oracle):
+    """One device-to-device segment of 5 GiB + 4 MiB + 777 bytes (its length does not fit 32 bits) from an odd source
+    address to an odd destination address: the engine cuts it into windowed launches of about 512 MiB.  Every byte
+    arrives (each 64 MiB of the source differs from the others, so a piece at a wrong offset shows), and the bytes
+    in front of and behind the destination stay as they were."""
+    assert lib.hybm_init(0, 0) == 0, native.last_error()
+    nbytes = 5 * GIB + 4 * MIB + 777
+    room = nbytes + 2 * GUARD
+    src = lib.mfrt_alloc_device(room)
+    dst = lib.mfrt_alloc_device(room)
+    if not src or not dst:
+        for p in (src, dst):
+            if p:
+                lib.mfrt_free_device(p)
+        lib.hybm_uninit()
+        pytest.skip("two device allocations of 5 GiB are not available on this GPU right now")
+    try:
+        block = _pattern_block(oracle)
+        s_at, d_at = src + GUARD + 5, dst + GUARD + 3
+        piece = np.empty(len(block), dtype=np.uint8)
+        for i in range(0, nbytes, len(block)):
+            m = min(len(block), nbytes - i)
+            np.bitwise_xor(block[:m], np.uint8((i // len(block) * 29 + 3) & 0xFF), out=piece[:m])
+            assert lib.mfrt_memcpy(s_at + i, np_ptr(piece), m) == 0
+        assert lib.mfrt_memset(dst, 0x5A, room) == 0
+        assert lib.mfrt_device_sync() == 0
+        before = lib.mf_xcopy_launch_count()
+        gpu_util.xcopy(lib, [s_at], [d_at], [nbytes], native.ROUTE_HBM)
+        launches = lib.mf_xcopy_launch_count() - before
+        if _window_rate(lib) != 0:      # the start-up check may have found that windows gain nothing on this GPU
+            assert launches == nbytes // (512 * MIB), launches
+        for i in range(0, nbytes, len(block)):
+            m = min(len(block), nbytes - i)
+            assert lib.mfrt_memcpy(np_ptr(piece), d_at + i, m) == 0
+            assert np.array_equal(piece[:m], block[:m] ^ np.uint8((i // len(block) * 29 + 3) & 0xFF)), i
+        edge = np.empty(GUARD + 3, dtype=np.uint8)
+        assert lib.mfrt_memcpy(np_ptr(edge), dst, GUARD + 3) == 0
+        assert np.all(edge == 0x5A)
+        assert lib.mfrt_memcpy(np_ptr(edge), d_at + nbytes, GUARD - 3) == 0
+        assert np.all(edge[:GUARD - 3] == 0x5A)
+    finally:
+        lib.mfrt_free_device(src)
+        lib.mfrt_free_device(dst)
+        lib.hybm_uninit()
+
+
+def _window_rate(lib):
+    rate = ctypes.c_uint32(0)
+    lib.mf_xcopy_calibration(None, None, ctypes.byref(rate), None, None)
+    return rate.value
 
 
 def test_paged_gather_and_scatter_on_a_40_gib_pool(lib, oracle):
