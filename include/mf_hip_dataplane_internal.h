@@ -81,10 +81,10 @@ int64_t mf_xcopy_describe_plan(const uint64_t *src, const uint64_t *dst, const u
  * (holdDeltaNanos), and holding is switched off where it does not beat the plain launch by 3 % (holdEnabled 0).  A copy
  * of 512 MiB is timed without windows, at the default rate, at 94 % of it and at the higher rate that launches of few long
  * segments take: windowMBps receives the rate in force (0: windows did not beat the plain kernel and are off),
- * windowLongMBps the one for long segments (the higher rate where it was 2 % faster here, else the same).  micros (8 floats,
+ * windowAlignedMBps the one for long segments (the higher rate where it was 2 % faster here, else the same).  micros (8 floats,
  * may be NULL): the eight times in that order, us per batch / per copy.  Returns 1 if the calibration ran, 0 if not.
  * mf_xcopy_hold_stores / mf_xcopy_windows still override what it chose (a rate set by hand holds for both). */
-int32_t mf_xcopy_calibration(int32_t *holdEnabled, int32_t *holdDeltaNanos, uint32_t *windowMBps, uint32_t *windowLongMBps,
+int32_t mf_xcopy_calibration(int32_t *holdEnabled, int32_t *holdDeltaNanos, uint32_t *windowMBps, uint32_t *windowAlignedMBps,
                              float *micros);
 /* The streams hybm_init makes for calling threads and submit threads, in the order they are handed out (the calling
  * thread of hybm_init holds the first): queues[i] is the hardware queue stream i sits on, numbered in order of

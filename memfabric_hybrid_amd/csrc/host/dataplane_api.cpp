@@ -187,7 +187,7 @@ MF_EXPORT int32_t mf_xcopy_tune_hold(uint32_t deepHold, int32_t pinnedExtraNanos
     return BM_OK;
 }
 
-MF_EXPORT int32_t mf_xcopy_calibration(int32_t *holdEnabled, int32_t *holdDeltaNanos, uint32_t *windowMBps, uint32_t *windowLongMBps,
+MF_EXPORT int32_t mf_xcopy_calibration(int32_t *holdEnabled, int32_t *holdDeltaNanos, uint32_t *windowMBps, uint32_t *windowAlignedMBps,
                                        float *micros)
 {
     const XcopyCalibration &c = XcopyEngine::Instance().Calibration();
@@ -200,8 +200,8 @@ MF_EXPORT int32_t mf_xcopy_calibration(int32_t *holdEnabled, int32_t *holdDeltaN
     if (windowMBps != nullptr) {
         *windowMBps = XcopyEngine::Instance().Tuning().windowMBps;
     }
-    if (windowLongMBps != nullptr) {
-        *windowLongMBps = XcopyEngine::Instance().Tuning().windowLongMBps;
+    if (windowAlignedMBps != nullptr) {
+        *windowAlignedMBps = XcopyEngine::Instance().Tuning().windowAlignedMBps;
     }
     if (micros != nullptr) {
         for (int i = 0; i < 4; ++i) {
@@ -229,7 +229,7 @@ MF_EXPORT int32_t mf_xcopy_windows(uint32_t megabytesPerSecond)
         MF_FAIL(BM_INVALID_PARAM, "windows: 0 (never) or a rate between 1 000 000 and 16 000 000 MB/s, got " << megabytesPerSecond);
     }
     XcopyEngine::Instance().Tuning().windowMBps = megabytesPerSecond;
-    XcopyEngine::Instance().Tuning().windowLongMBps = megabytesPerSecond;   // a rate set by hand holds for every windowed launch
+    XcopyEngine::Instance().Tuning().windowAlignedMBps = megabytesPerSecond;   // a rate set by hand holds for every windowed launch
     return BM_OK;
 }
 

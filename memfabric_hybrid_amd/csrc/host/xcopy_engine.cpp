@@ -953,12 +953,12 @@ uint64_t BuildTableDirect(const uint64_t *src, const uint64_t *dst, const uint64
     return run;
 }
 
-void ChooseCalibration(const float *batchMicros, const float *copyMicros, uint32_t defaultWindowMBps, uint32_t defaultLongMBps,
+void ChooseCalibration(const float *batchMicros, const float *copyMicros, uint32_t defaultWindowMBps, uint32_t defaultAlignedMBps,
                        XcopyCalibration &out)
 {
     out = XcopyCalibration{};
     out.windowMBps = defaultWindowMBps;
-    out.windowLongMBps = defaultLongMBps;
+    out.windowAlignedMBps = defaultAlignedMBps;
     for (int i = 0; i < 4; ++i) {
         out.batchMicros[i] = batchMicros[i];
     }
@@ -985,8 +985,8 @@ void ChooseCalibration(const float *batchMicros, const float *copyMicros, uint32
         const uint32_t rate = slowerWins ? static_cast<uint32_t>(static_cast<uint64_t>(defaultWindowMBps) * kCalibrateSlowerWindowPercent / 100)
                                          : defaultWindowMBps;
         out.windowMBps = windowed <= copyMicros[0] * (1.0f - kCalibrateMinWindowGain) ? rate : 0u;
-        // the higher rate of long segments only where one long segment held it here: 2 % better than the rate just chosen
-        out.windowLongMBps = out.windowMBps != 0 && copyMicros[3] > 0 && copyMicros[3] < windowed * 0.98f ? defaultLongMBps : out.windowMBps;
+        // the higher rate of aligned segments only where an aligned copy held it here: 2 % better than the rate just chosen
+        out.windowAlignedMBps = out.windowMBps != 0 && copyMicros[3] > 0 && copyMicros[3] < windowed * 0.98f ? defaultAlignedMBps : out.windowMBps;
         out.ran = true;
     }
 }
@@ -1003,7 +1003,7 @@ int XcopyEngine::Calibrate()
     const uint32_t rule = HoldNanosFor(2196, 2196, kXcopyThreads, false);
     const uint32_t holds[3] = {rule - kCalibrateHoldStepNanos, rule, rule + kCalibrateHoldStepNanos};
     const uint32_t defaultRate = XcopyTuning{}.windowMBps;
-    const uint32_t defaultLong = XcopyTuning{}.windowLongMBps;
+    const uint32_t defaultLong = XcopyTuning{}.windowAlignedMBps;
     const uint32_t rates[3] = {defaultRate, static_cast<uint32_t>(static_cast<uint64_t>(defaultRate) * kCalibrateSlowerWindowPercent / 100),
                                defaultLong};
     float us[8] = {};
@@ -1019,7 +1019,7 @@ int XcopyEngine::Calibrate()
         tuning_.holdCalibratedOff = !calibration_.holdEnabled;
         if (windowsAvailable_) {
             tuning_.windowMBps = calibration_.windowMBps;
-            tuning_.windowLongMBps = calibration_.windowLongMBps;
+            tuning_.windowAlignedMBps = calibration_.windowAlignedMBps;
             windowRateCalibrated_ = true;
         }
     }
@@ -1051,7 +1051,7 @@ int XcopyEngine::Start(int device)
     tuning_.holdCalibratedOff = false;
     if (windowRateCalibrated_) {   // what an earlier start of this process chose does not outlive it
         tuning_.windowMBps = XcopyTuning{}.windowMBps;
-        tuning_.windowLongMBps = XcopyTuning{}.windowLongMBps;
+        tuning_.windowAlignedMBps = XcopyTuning{}.windowAlignedMBps;
         windowRateCalibrated_ = false;
     }
     calibration_ = XcopyCalibration{};
@@ -1436,14 +1436,26 @@ int XcopyEngine::SubmitOne(const uint64_t *src, const uint64_t *dst, const uint6
     uint64_t queuedBytes = 0;
     if (n <= 4 * kInlineSegs) {  // small enough that a failed attempt costs next to nothing
         uint64_t total = 0;
+        uint64_t addressBits = 0;      // low bits any source or destination address has set
+        uint64_t apartBits = 0;        // low bits in which a source differs from its destination
         for (uint32_t i = 0; i < n; ++i) {
             total += len[i];
+            addressBits |= src[i] | dst[i];
+            apartBits |= src[i] ^ dst[i];
         }
         queuedBytes = total;
         oversized = total > 0xFFFFFFFFull;
         units = ChooseUnits(total, cu, route, tuning_);
         // Large HBM copies of one submitter: 16 KiB chunks for the kernel that alternates between read and write windows.
-        windowed = !unordered && WindowsApply(total, route);
+        // Not where a source and its destination differ modulo 16: the kernels align their 128-bit units on the destination,
+        // the loads then straddle units, cost twice the issue slots, and the waves keep no schedule at any rate that pays
+        // (100 segments of 10 MB: 5.35 TB/s in windows cut for 6.8, 5.26 for 7.4, 5.51 to 5.56 without windows).
+        windowed = !unordered && (apartBits & (kUnitBytes - 1)) == 0 && WindowsApply(total, route);
+        // Segments that all start on cache lines, in source and destination, hold the higher rate (back to back, 6.8 against
+        // 7.4 TB/s: 100 x 10 MB 6.41 to 6.47 against 6.72 to 6.87 TB/s, 32 x 16 MiB 6.56 against 6.94 to 7.03, 3 x 700 MB 6.30 to
+        // 6.35 against 6.78).  Where they start elsewhere every wave's kilobyte straddles a line it shares with its
+        // neighbour; such launches hold 6.8 (6.24 to 6.27 against 5.65 to 5.80 TB/s without windows) and fall apart at 7.4 (5.36 to 5.48).
+        const bool aligned = (addressBits & (kWindowAlignBytes - 1)) == 0;
         const bool longSegments = windowed && total / n >= kWindowLongSegmentBytes;
         if (longSegments && maySlice && total >= 2 * kWindowMinBytes) {
             // A windowed launch that loses its schedule runs the rest of its bytes at the rate without windows, and the longer
@@ -1453,7 +1465,7 @@ int XcopyEngine::SubmitOne(const uint64_t *src, const uint64_t *dst, const uint6
             // in launches of 1.2 GB, measured 6.4 in launches of 540 MB at either rate.
             return SubmitInPieces(src, dst, len, n, total, route, stream, mask, maskValue);
         }
-        windowRate = longSegments && tuning_.windowLongMBps != 0 ? tuning_.windowLongMBps : tuning_.windowMBps;
+        windowRate = aligned && tuning_.windowAlignedMBps != 0 ? tuning_.windowAlignedMBps : tuning_.windowMBps;
         if (windowed) {
             units = mfk_xcopy_window_units();
         }

@@ -56,13 +56,14 @@ struct XcopyTuning {
     bool stageUnordered = true;  // the upload of a ragged table's descriptors is launched without a barrier
     uint32_t deviceTableWgPerCu = 0;   // grid of a device-resident table in workgroups per CU, 0 = eight per segment between 32 and 4096 per CU
     uint32_t windowMBps = 6800000;   // HBM copies of kWindowMinBytes and more alternate between read and write windows cut for this rate; 0 = never
-    uint32_t windowLongMBps = 7400000;   // the same for launches of few long segments (kWindowLongSegmentBytes on average), which hold more; 0 = the rate above
+    uint32_t windowAlignedMBps = 7400000;   // the same for launches of segments that all start at multiples of kWindowAlignBytes in source and destination, which hold more; 0 = the rate above
 };
 
 // From this total on a batch of up to 128 segments between HBM addresses is copied in read and write windows
 // (XcopyWindowKernel has the measurements; 512 MiB gains 2 %, 256 MiB nothing).
 constexpr uint64_t kWindowMinBytes = 512ull << 20;
-constexpr uint64_t kWindowLongSegmentBytes = 64ull << 20;     // launches whose segments average this much take the higher rate and go out in pieces
+constexpr uint64_t kWindowLongSegmentBytes = 64ull << 20;     // launches whose segments average this much go out in pieces of kWindowMinBytes and more
+constexpr uint64_t kWindowAlignBytes = 128;                   // a cache line: segments that start on one are read and written in whole lines by every wave
 constexpr uint64_t kWindowSliceMinSegmentBytes = 4ull << 20;   // tables of segments this long on average are cut into windowed launches
 
 // What Start() measured on the GPU it runs on and chose from it (XcopyEngine::Calibrate).
@@ -71,16 +72,16 @@ struct XcopyCalibration {
     bool holdEnabled = true;        // the held stores beat the launch that stores at once by kCalibrateMinGain
     int32_t holdDeltaNanos = 0;     // added to every wait HoldNanosFor gives
     uint32_t windowMBps = 0;        // rate the read and write windows are cut for; 0: the form lost against the plain kernel
-    uint32_t windowLongMBps = 0;    // rate for launches of few long segments: the higher one where it beat the rate above, else that rate
+    uint32_t windowAlignedMBps = 0;    // rate for launches of segments on cache-line boundaries: the higher one where it beat the rate above, else that rate
     float batchMicros[4] = {};      // 2196-chunk batch: not held, rule - step, rule, rule + step
-    float copyMicros[4] = {};       // 512 MiB copy: no windows, default rate, reduced rate, the higher rate of long segments
+    float copyMicros[4] = {};       // 512 MiB copy: no windows, default rate, reduced rate, the higher rate of aligned segments
 };
 constexpr int32_t kCalibrateHoldStepNanos = 200;
 constexpr float kCalibrateMinGain = 0.03f;          // held stores that do not gain this much over the plain launch are switched off
 constexpr float kCalibrateMinWindowGain = 0.005f;   // windows stay unless they lose: on the 512 MiB that is measured they gain least (2 to 5 %, 8 % on 1 GiB)
 constexpr uint32_t kCalibrateSlowerWindowPercent = 94;   // the second window rate tried, in percent of the default
 // The choice, from the measured times alone (microseconds; a time of 0 means "not measured" and leaves the default).
-void ChooseCalibration(const float *batchMicros, const float *copyMicros, uint32_t defaultWindowMBps, uint32_t defaultLongMBps,
+void ChooseCalibration(const float *batchMicros, const float *copyMicros, uint32_t defaultWindowMBps, uint32_t defaultAlignedMBps,
                        XcopyCalibration &out);
 
 uint32_t ChooseUnits(uint64_t totalBytes, uint32_t cuCount, int route, const XcopyTuning &tuning);

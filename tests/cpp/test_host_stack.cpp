@@ -799,42 +799,42 @@ static void TestPlanners()
 static void TestCalibration()
 {
     const uint32_t rate = XcopyTuning{}.windowMBps;
-    const uint32_t longRate = XcopyTuning{}.windowLongMBps;
+    const uint32_t alignedRate = XcopyTuning{}.windowAlignedMBps;
     XcopyCalibration c;
     {   // the usual picture: the rule's wait is best, held stores gain 14 %, windows 7 %, one long segment holds the higher rate
         const float batch[4] = {5.30f, 4.62f, 4.55f, 4.60f};
         const float copy[4] = {172.0f, 160.0f, 163.0f, 149.0f};
-        ChooseCalibration(batch, copy, rate, longRate, c);
-        CHECK(c.ran && c.holdEnabled && c.holdDeltaNanos == 0 && c.windowMBps == rate && c.windowLongMBps == longRate);
+        ChooseCalibration(batch, copy, rate, alignedRate, c);
+        CHECK(c.ran && c.holdEnabled && c.holdDeltaNanos == 0 && c.windowMBps == rate && c.windowAlignedMBps == alignedRate);
     }
     {   // the higher rate does not hold here (no better than the default by 2 %): long segments take the default too
         const float batch[4] = {5.30f, 4.62f, 4.55f, 4.60f};
         const float copy[4] = {172.0f, 160.0f, 163.0f, 158.5f};
-        ChooseCalibration(batch, copy, rate, longRate, c);
-        CHECK(c.windowMBps == rate && c.windowLongMBps == rate);
+        ChooseCalibration(batch, copy, rate, alignedRate, c);
+        CHECK(c.windowMBps == rate && c.windowAlignedMBps == rate);
     }
     {   // a GPU whose loads land later: the longer wait wins clearly; windows only hold at the lower rate
         const float batch[4] = {5.30f, 4.95f, 4.80f, 4.60f};
         const float copy[4] = {172.0f, 171.0f, 161.0f, 176.0f};
-        ChooseCalibration(batch, copy, rate, longRate, c);
+        ChooseCalibration(batch, copy, rate, alignedRate, c);
         CHECK(c.holdEnabled && c.holdDeltaNanos == kCalibrateHoldStepNanos && c.windowMBps == static_cast<uint32_t>(static_cast<uint64_t>(rate) * 94 / 100) &&
-              c.windowLongMBps == c.windowMBps);
+              c.windowAlignedMBps == c.windowMBps);
     }
     {   // a neighbour that is better by less than 1 % does not move the wait
         const float batch[4] = {5.30f, 4.53f, 4.55f, 4.60f};
         const float copy[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-        ChooseCalibration(batch, copy, rate, longRate, c);
-        CHECK(c.ran && c.holdDeltaNanos == 0 && c.windowMBps == rate && c.windowLongMBps == longRate);   // windows not measured: the defaults stay
+        ChooseCalibration(batch, copy, rate, alignedRate, c);
+        CHECK(c.ran && c.holdDeltaNanos == 0 && c.windowMBps == rate && c.windowAlignedMBps == alignedRate);   // windows not measured: the defaults stay
     }
     {   // a busy or capped chip: holding gains 2 %, windows lose: both off
         const float batch[4] = {5.30f, 5.25f, 5.20f, 5.28f};
         const float copy[4] = {172.0f, 175.0f, 174.0f, 169.0f};
-        ChooseCalibration(batch, copy, rate, longRate, c);
-        CHECK(c.ran && !c.holdEnabled && c.windowMBps == 0 && c.windowLongMBps == 0);
+        ChooseCalibration(batch, copy, rate, alignedRate, c);
+        CHECK(c.ran && !c.holdEnabled && c.windowMBps == 0 && c.windowAlignedMBps == 0);
     }
     {   // nothing measured
         const float none[4] = {0, 0, 0, 0};
-        ChooseCalibration(none, none, rate, longRate, c);
+        ChooseCalibration(none, none, rate, alignedRate, c);
         CHECK(!c.ran && c.holdEnabled && c.holdDeltaNanos == 0 && c.windowMBps == rate);
     }
     // through hybm_init: the engine applies what it chose, and mf_xcopy_hold_stores(-1) means the calibrated rule
@@ -846,10 +846,10 @@ static void TestCalibration()
     int32_t enabled = -1;
     int32_t delta = 0;
     uint32_t mbps = 0;
-    uint32_t longMbps = 0;
+    uint32_t alignedMbps = 0;
     float micros[8] = {};
-    CHECK(mf_xcopy_calibration(&enabled, &delta, &mbps, &longMbps, micros) == 1);
-    CHECK(enabled == 1 && delta == -200 && mbps == rate && longMbps == longRate && micros[1] == 4.40f && micros[5] == 160.0f && micros[7] == 150.0f);
+    CHECK(mf_xcopy_calibration(&enabled, &delta, &mbps, &alignedMbps, micros) == 1);
+    CHECK(enabled == 1 && delta == -200 && mbps == rate && alignedMbps == alignedRate && micros[1] == 4.40f && micros[5] == 160.0f && micros[7] == 150.0f);
     {
         std::vector<uint8_t> from(12 << 20), to(12 << 20);
         const uint64_t fromBase = (reinterpret_cast<uint64_t>(from.data()) + 4095) & ~4095ull;
@@ -869,12 +869,12 @@ static void TestCalibration()
     const float lost[8] = {5.30f, 5.29f, 5.31f, 5.30f, 172.0f, 175.0f, 176.0f, 177.0f};
     fake_rt_set_calibration(lost);
     CHECK(hybm_init(0, 0) == BM_OK);
-    CHECK(mf_xcopy_calibration(&enabled, &delta, &mbps, &longMbps, nullptr) == 1 && enabled == 0 && mbps == 0 && longMbps == 0);
+    CHECK(mf_xcopy_calibration(&enabled, &delta, &mbps, &alignedMbps, nullptr) == 1 && enabled == 0 && mbps == 0 && alignedMbps == 0);
     hybm_uninit();
     setenv("MF_HIP_CALIBRATE", "0", 1);
     CHECK(hybm_init(0, 0) == BM_OK);
-    CHECK(mf_xcopy_calibration(&enabled, &delta, &mbps, &longMbps, nullptr) == 0 && enabled == 1 && delta == 0 && mbps == rate &&
-          longMbps == longRate);
+    CHECK(mf_xcopy_calibration(&enabled, &delta, &mbps, &alignedMbps, nullptr) == 0 && enabled == 1 && delta == 0 && mbps == rate &&
+          alignedMbps == alignedRate);
     hybm_uninit();
     unsetenv("MF_HIP_CALIBRATE");
     const float none[8] = {};
@@ -1044,7 +1044,7 @@ static void TestLongSegments()
     {
         // one segment beyond what 128 pieces of 1 GiB hold
         uint64_t src = base;
-        uint64_t dst = base + 4096 * gib + 3;
+        uint64_t dst = base + 4096 * gib + 384;
         uint64_t len = 129 * gib + 5;
         const uint64_t before = mf_xcopy_launch_count();
         CHECK(engine.Submit(&src, &dst, &len, 1, MF_ROUTE_HBM, stream, nullptr, 0) == BM_OK);
@@ -1062,7 +1062,7 @@ static void TestLongSegments()
         std::vector<uint64_t> src(n), dst(n), len(n, 8u << 20);
         for (uint32_t i = 0; i < n; ++i) {
             src[i] = base + i * 16 * gib;
-            dst[i] = base + (2048 + i) * 16 * gib + 9;
+            dst[i] = base + (2048 + i) * 16 * gib + 512;
         }
         len[300] = 5 * gib;
         uint64_t word = 0;
@@ -1439,31 +1439,54 @@ static void TestWindows()
     }
     CHECK(hybm_init(0, 0) == BM_OK);
     const uint64_t gib = 1ull << 30;
-    std::vector<uint8_t> mem(2 * gib + 64);
+    std::vector<uint8_t> mem(2 * gib + 1024);
+    uint64_t s1 = (reinterpret_cast<uint64_t>(mem.data()) + 127) & ~127ull;      // on a cache line
+    uint8_t *from = reinterpret_cast<uint8_t *>(s1);
     for (uint64_t i = 0; i < gib; i += 4093) {
-        mem[i] = static_cast<uint8_t>(i * 7 + 1);
+        from[i] = static_cast<uint8_t>(i * 7 + 1);
     }
     XcopyEngine &engine = XcopyEngine::Instance();
     void *stream = mf_xcopy_thread_stream();
-    uint64_t s1 = reinterpret_cast<uint64_t>(mem.data());
-    uint64_t d1 = s1 + gib + 3;                    // an odd destination: head and tail bytes
+    uint64_t d1 = s1 + gib + 256;
     uint64_t l1 = gib;
     (void)fake_rt_last_window();
     uint64_t launchesBefore = mf_xcopy_launch_count();
     CHECK(engine.Submit(&s1, &d1, &l1, 1, MF_ROUTE_HBM, stream, nullptr, 0) == BM_OK);
-    CHECK(fake_rt_last_window() == 7400000);
+    CHECK(fake_rt_last_window() == 7400000);                   // source and destination on cache lines: the higher rate
     CHECK(mf_xcopy_launch_count() - launchesBefore == 2);      // twice the minimum: two launches of 512 MiB, a schedule each
     CHECK(engine.DrainThread() == BM_OK);
     bool ok = true;
     for (uint64_t i = 0; i < gib; i += 4093) {
-        ok = ok && mem[gib + 3 + i] == static_cast<uint8_t>(i * 7 + 1);
+        ok = ok && from[gib + 256 + i] == static_cast<uint8_t>(i * 7 + 1);
     }
-    CHECK(ok && mem[gib + 3 + gib - 1] == mem[gib - 1]);
+    CHECK(ok && from[gib + 256 + gib - 1] == from[gib - 1]);
+    {
+        // odd addresses that agree modulo 16 (head and tail bytes): windows at the general rate;
+        // addresses that differ modulo 16: no windows, one launch
+        uint64_t so = s1 + 3;
+        uint64_t dO = s1 + gib + 256 + 19;
+        uint64_t lo = gib - 64;
+        std::memset(from + gib, 0, gib + 512);
+        launchesBefore = mf_xcopy_launch_count();
+        CHECK(engine.Submit(&so, &dO, &lo, 1, MF_ROUTE_HBM, stream, nullptr, 0) == BM_OK);
+        CHECK(fake_rt_last_window() == 6800000);
+        CHECK(mf_xcopy_launch_count() - launchesBefore == 1);      // 64 bytes short of twice the minimum
+        CHECK(engine.DrainThread() == BM_OK);
+        CHECK(std::memcmp(from + gib + 256 + 19, from + 3, lo) == 0 && from[gib + 256 + 18] == 0 && from[gib + 256 + 19 + lo] == 0);
+        dO = s1 + gib + 256 + 5;
+        std::memset(from + gib, 0, gib + 512);
+        launchesBefore = mf_xcopy_launch_count();
+        CHECK(engine.Submit(&so, &dO, &lo, 1, MF_ROUTE_HBM, stream, nullptr, 0) == BM_OK);
+        CHECK(fake_rt_last_window() == 0);
+        CHECK(mf_xcopy_launch_count() - launchesBefore == 1);
+        CHECK(engine.DrainThread() == BM_OK);
+        CHECK(std::memcmp(from + gib + 256 + 5, from + 3, lo) == 0 && from[gib + 256 + 4] == 0 && from[gib + 256 + 5 + lo] == 0);
+    }
     {
         // three segments, 600 + 24 + 400 MiB: the first piece ends inside the long segment, at a multiple of 1 MiB, the
         // second takes its rest and the others; then 64 segments of 16 MiB: pieces end where segments end
         const uint64_t mib = 1ull << 20;
-        std::memset(mem.data() + gib, 0, gib);
+        std::memset(from + gib, 0, gib);
         uint64_t src3[3] = {s1, s1 + 600 * mib, s1 + 624 * mib};
         uint64_t dst3[3] = {s1 + gib, s1 + gib + 600 * mib, s1 + gib + 624 * mib};
         uint64_t len3[3] = {600 * mib, 24 * mib, 400 * mib};
@@ -1474,14 +1497,14 @@ static void TestWindows()
         CHECK(engine.DrainThread() == BM_OK);
         bool same = true;
         for (uint64_t i = 0; i < gib; i += 4093) {
-            same = same && mem[gib + i] == mem[i];
+            same = same && from[gib + i] == from[i];
         }
-        CHECK(same && mem[2 * gib - 1] == mem[gib - 1]);
-        std::memset(mem.data() + gib, 0, gib);
+        CHECK(same && from[2 * gib - 1] == from[gib - 1]);
+        std::memset(from + gib, 0, gib);
         std::vector<uint64_t> src64(64), dst64(64), len64(64, 16 * mib - 4096);
         for (uint32_t i = 0; i < 64; ++i) {
             src64[i] = s1 + i * 16 * mib;
-            dst64[i] = s1 + gib + ((i * 5) % 64) * 16 * mib + 7;
+            dst64[i] = s1 + gib + ((i * 5) % 64) * 16 * mib + 48;     // as the sources modulo 16, not on cache lines
         }
         launchesBefore = mf_xcopy_launch_count();
         CHECK(engine.Submit(src64.data(), dst64.data(), len64.data(), 64, MF_ROUTE_HBM, stream, nullptr, 0) == BM_OK);
@@ -1492,7 +1515,7 @@ static void TestWindows()
             same = std::memcmp(reinterpret_cast<void *>(dst64[i]), reinterpret_cast<void *>(src64[i]), len64[i]) == 0;
         }
         CHECK(same);
-        CHECK(fake_rt_last_window() == 6800000);       // segments of 16 MiB are not long ones: the general rate
+        CHECK(fake_rt_last_window() == 6800000);       // destinations between cache lines: the general rate
     }
     l1 = (gib >> 1) - 1;                           // one byte below the limit: the ordinary form
     CHECK(engine.Submit(&s1, &d1, &l1, 1, MF_ROUTE_HBM, stream, nullptr, 0) == BM_OK);
@@ -1531,8 +1554,8 @@ static void TestWindows()
         const uint64_t seg = 4ull << 20;
         std::vector<uint64_t> src(count), dst(count), len(count, seg);
         for (uint32_t i = 0; i < count; ++i) {
-            src[i] = reinterpret_cast<uint64_t>(mem.data()) + (i % 200) * seg + i;     // not adjacent: no merging
-            dst[i] = reinterpret_cast<uint64_t>(mem.data()) + gib + ((i * 7) % 200) * seg + 2 * i;
+            src[i] = s1 + (i % 200) * seg + 128 * i;     // not adjacent: no merging
+            dst[i] = s1 + gib + ((i * 7) % 200) * seg + 256 * i;
         }
         const uint64_t before = mf_xcopy_launch_count();
         (void)fake_rt_last_window();

@@ -82,16 +82,18 @@ def test_single_copies_at_full_size_host_device_device_host(pool, lib, oracle, n
     assert _same_as_pattern(host_all[back_off:back_off + nbytes], block)
 
 
+@pytest.mark.parametrize("agree", [True, False], ids=["same-modulo-16", "apart-modulo-16"])
 @pytest.mark.parametrize("pieces", [7, 200], ids=["7-pieces", "200-pieces"])
 @pytest.mark.parametrize("rate", [-1, 7400000, 0], ids=["default-windows", "short-periods", "no-windows"])
-def test_ragged_batch_above_one_gib_in_read_and_write_windows(pool, lib, oracle, rate, pieces):
+def test_ragged_batch_above_one_gib_in_read_and_write_windows(pool, lib, oracle, rate, pieces, agree):
     """A device-to-device batch of 1 GiB and more goes through the kernel that alternates between read and
     write windows.  Seven pieces of about 170 MB, or 200 of about 6 MB (a table that the engine cuts into
     launches of 128 segments), with odd lengths at odd source and destination addresses (partial first and
     last chunks, head and tail bytes), with the default period, with a period too short for the waves to
     keep up (they then proceed late; the result must not depend on timing) and with the form switched off:
     what comes back equals the same slices cut on the CPU, and the bytes between and round the destinations
-    are untouched."""
+    are untouched.  Sources and destinations either agree modulo 16 (the batch then takes the windows) or do not
+    (the engine then leaves the windows out, whatever the rate)."""
     dev = pool.peer_rank_ptr(0, bm.BmMemType.DEVICE)
     host = pool.peer_rank_ptr(0, bm.BmMemType.HOST)
     span = 2 * GIB + GUARD
@@ -107,7 +109,12 @@ def test_ragged_batch_above_one_gib_in_read_and_write_windows(pool, lib, oracle,
     lens = rng.integers(each - each // 20, each + each // 25, pieces) | 1  # odd lengths
     gaps = rng.integers(1, 4096, pieces) | 1
     src = GUARD + np.cumsum(lens + gaps) - lens                            # odd addresses
-    dst = span + GUARD + np.cumsum(lens + 2 * gaps + 1) - lens
+    dst = span + GUARD + np.cumsum(lens + 2 * gaps + 17) - lens
+    if agree:
+        dst = dst + ((src - dst) % 16)
+    else:
+        dst = dst + ((src - dst) % 16 == 0)
+    assert bool(np.all((src - dst) % 16 == 0)) == agree and bool(np.any((src - dst) % 16 == 0)) == agree
     assert int(lens.sum()) >= GIB and int(src[-1] + lens[-1]) <= GUARD + total
     assert int(dst[-1] + lens[-1]) + GUARD <= 2 * span + GUARD
     try:
@@ -149,7 +156,7 @@ def test_one_segment_beyond_four_gib_goes_out_in_windowed_launches(lib, oracle):
         pytest.skip("two device allocations of 5 GiB are not available on this GPU right now")
     try:
         block = _pattern_block(oracle)
-        s_at, d_at = src + GUARD + 5, dst + GUARD + 3
+        s_at, d_at = src + GUARD + 5, dst + GUARD + 21        # the same modulo 16: the copy takes the windows
         piece = np.empty(len(block), dtype=np.uint8)
         for i in range(0, nbytes, len(block)):
             m = min(len(block), nbytes - i)
@@ -166,11 +173,11 @@ def test_one_segment_beyond_four_gib_goes_out_in_windowed_launches(lib, oracle):
             m = min(len(block), nbytes - i)
             assert lib.mfrt_memcpy(np_ptr(piece), d_at + i, m) == 0
             assert np.array_equal(piece[:m], block[:m] ^ np.uint8((i // len(block) * 29 + 3) & 0xFF)), i
-        edge = np.empty(GUARD + 3, dtype=np.uint8)
-        assert lib.mfrt_memcpy(np_ptr(edge), dst, GUARD + 3) == 0
+        edge = np.empty(GUARD + 21, dtype=np.uint8)
+        assert lib.mfrt_memcpy(np_ptr(edge), dst, GUARD + 21) == 0
         assert np.all(edge == 0x5A)
-        assert lib.mfrt_memcpy(np_ptr(edge), d_at + nbytes, GUARD - 3) == 0
-        assert np.all(edge[:GUARD - 3] == 0x5A)
+        assert lib.mfrt_memcpy(np_ptr(edge), d_at + nbytes, GUARD - 21) == 0
+        assert np.all(edge[:GUARD - 21] == 0x5A)
     finally:
         lib.mfrt_free_device(src)
         lib.mfrt_free_device(dst)
