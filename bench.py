@@ -839,9 +839,9 @@ def main():
     calibration = {"ran": bool(cal_ran), "held_stores": bool(cal_on.value), "hold_delta_ns": cal_delta.value,
                    "window_MBps": cal_rate.value, "window_MBps_aligned_segments": cal_aligned.value,
                    "us_per_2196_chunk_batch_not_held_and_held_rule_minus_200_rule_plus_200": [round(v, 2) for v in cal_us[:4]],
-                   "us_per_512MiB_copy_plain_windows_default_windows_94_percent_windows_long_segment_rate": [round(v, 1) for v in cal_us[4:]],
+                   "us_per_512MiB_copy_plain_windows_default_windows_94_percent_windows_aligned_segment_rate": [round(v, 1) for v in cal_us[4:]],
                    "note": "measured by hybm_init on this GPU (about 15 ms): the wait of the held stores is the fitted rule plus the offset "
-                           "that was fastest here, the window rate the faster of two (the higher rate for launches of few long segments where one such copy "
+                           "that was fastest here, the window rate the faster of two (the higher rate for segments on cache lines where one such copy "
                            "held it), either form off where it does not gain"}
 
     deck = (ctypes.c_uint32 * 16)()

@@ -1461,8 +1461,8 @@ int XcopyEngine::SubmitOne(const uint64_t *src, const uint64_t *dst, const uint6
             // A windowed launch that loses its schedule runs the rest of its bytes at the rate without windows, and the longer
             // it runs the likelier that is: launches of kWindowMinBytes to twice that, each with a schedule of its own, hold
             // a target the whole copy in one launch does not (2 GiB at 7.4 TB/s: 7.1 TB/s on average in four launches,
-            // 6.6 to 6.8 in one).  Only long segments are worth it: batches of segments of some 10 MB, which hold 6.6 TB/s
-            // in launches of 1.2 GB, measured 6.4 in launches of 540 MB at either rate.
+            // 6.6 to 6.8 in one).  Only long segments are worth it: 896 segments of some 10 MB in launches of 64 or 96
+            // segments (600 to 900 MB) were no faster than in launches of 128.
             return SubmitInPieces(src, dst, len, n, total, route, stream, mask, maskValue);
         }
         windowRate = aligned && tuning_.windowAlignedMBps != 0 ? tuning_.windowAlignedMBps : tuning_.windowMBps;
