@@ -398,12 +398,12 @@ def extras_block(lib, pool, dev, batches, tables, steps):
         src_off = np.arange(32, dtype=np.uint64) * block
         dst_off = (POOL_BYTES // 2) + np.arange(32, dtype=np.uint64) * block
         b = Batch(dev + src_off, dev + dst_off, np.full(32, block, dtype=np.uint64))
-        for _ in range(5):
+        for _ in range(20):     # the first calls after a different workload take 2 us longer
             lib.smem_bm_copy_batch(handle, b.ref, g2g, 0)
         t0 = time.perf_counter()
-        for _ in range(30):
+        for _ in range(100):
             lib.smem_bm_copy_batch(handle, b.ref, g2g, 0)
-        per_call = (time.perf_counter() - t0) / 30
+        per_call = (time.perf_counter() - t0) / 100
         grid.append({"block_KiB": block >> 10, "us_per_call": round(per_call * 1e6, 1),
                      "payload_GBps": round(32 * block / per_call / GB, 1)})
     out["batch32_blocking_calls_d2d"] = grid
