@@ -173,7 +173,7 @@ int mfrt_event_sync(void *event);
 int mfrt_stream_wait_event(void *stream, void *event);
 /* Whether two idle streams share a hardware queue: 1 (launches on them run one after the other however independent
  * they are), 0 (they run side by side), -1 (not known).  The runtime spreads the streams of a process over a few hardware
- * queues, not evenly; the library's own streams are handed out one per queue (see INTEGRATION.md), a caller that brings
+ * queues, not evenly; the library's own streams are handed out one per queue, a caller that brings
  * streams of its own can ask here.  Takes about 50 us (a lane waits 40 us by the clock on `a`, an empty kernel on `b`). */
 int mfrt_streams_share_queue(void *a, void *b);
 int mfrt_event_done(void *event);
