@@ -834,14 +834,15 @@ def main():
     near_cpus = sorted(os.sched_getaffinity(0))
 
     cal_on, cal_delta, cal_rate, cal_aligned = ctypes.c_int32(0), ctypes.c_int32(0), ctypes.c_uint32(0), ctypes.c_uint32(0)
+    cal_long = ctypes.c_uint32(0)
     cal_us = (ctypes.c_float * 8)()
-    cal_ran = lib.mf_xcopy_calibration(ctypes.byref(cal_on), ctypes.byref(cal_delta), ctypes.byref(cal_rate), ctypes.byref(cal_aligned), cal_us)
+    cal_ran = lib.mf_xcopy_calibration(ctypes.byref(cal_on), ctypes.byref(cal_delta), ctypes.byref(cal_rate), ctypes.byref(cal_aligned), ctypes.byref(cal_long), cal_us)
     calibration = {"ran": bool(cal_ran), "held_stores": bool(cal_on.value), "hold_delta_ns": cal_delta.value,
-                   "window_MBps": cal_rate.value, "window_MBps_aligned_segments": cal_aligned.value,
+                   "window_MBps": cal_rate.value, "window_MBps_aligned_segments": cal_aligned.value, "window_MBps_long_aligned_segments": cal_long.value,
                    "us_per_2196_chunk_batch_not_held_and_held_rule_minus_200_rule_plus_200": [round(v, 2) for v in cal_us[:4]],
-                   "us_per_512MiB_copy_plain_windows_default_windows_94_percent_windows_aligned_segment_rate": [round(v, 1) for v in cal_us[4:]],
+                   "us_per_512MiB_copy_plain_windows_default_windows_94_percent_windows_long_segment_rate": [round(v, 1) for v in cal_us[4:]],
                    "note": "measured by hybm_init on this GPU (about 15 ms): the wait of the held stores is the fitted rule plus the offset "
-                           "that was fastest here, the window rate the faster of two (the higher rate for segments on cache lines where one such copy "
+                           "that was fastest here, the window rate the faster of two (higher rates for segments on cache lines where a long one "
                            "held it), either form off where it does not gain"}
 
     deck = (ctypes.c_uint32 * 16)()

@@ -59,12 +59,15 @@ int32_t mf_xcopy_hold_stores(int32_t nanos);
  * period is cut for a rate of HBM traffic (read + written) in MB/s, 6 800 000 by default; at 7 000 000 the waves
  * of a 2 GiB copy now and then no longer keep up, the windows dissolve and the copy runs at about the rate it
  * has without them; at 7 200 000 and above most launches do.  That holds for segments that start between
- * cache lines.  Segments whose sources and destinations all start on 128-byte lines are paced for 7 400 000
- * (32 x 16 MiB back to back: 6.9-7.0 instead of 6.6 TB/s), and a batch of 1 GiB and more whose segments are
- * 64 MiB and longer on average is cut into launches of about 512 MiB, which hold their schedule more often
- * than longer ones (1 GiB: 7.1 instead of 6.7 TB/s).  Segments whose source and destination differ modulo 16
- * take no windows.  The call sets both rates; 0 switches the form off.  While several threads submit on
- * streams of their own it is not used. */
+ * cache lines.  Segments whose sources and destinations all start on 128-byte lines take windows from 128 MiB
+ * on and are paced for 7 100 000 (32 x 16 MiB back to back: 6.95 instead of 6.65 TB/s), those of 64 MiB and
+ * more on average for 7 400 000, and a batch of 1 GiB and more of such long segments is cut into launches of
+ * about 512 MiB, which hold their schedule more often than longer ones (1 GiB: 7.1-7.2 instead of 6.7 TB/s).
+ * Segments whose source and destination differ modulo 16 take no windows.  The call sets all three rates; 0
+ * switches the form off, MF_XCOPY_WINDOWS_OWN_CHOICE brings back the rates the library chose itself (what
+ * hybm_init measured, else the defaults above).  While several threads submit on streams of their own the
+ * form is not used. */
+#define MF_XCOPY_WINDOWS_OWN_CHOICE 1u
 int32_t mf_xcopy_windows(uint32_t megabytesPerSecond);
 uint32_t mf_xcopy_choose_units(uint64_t totalBytes, uint32_t cuCount, int32_t route);
 uint64_t mf_xcopy_launch_count(void);
@@ -81,13 +84,14 @@ int64_t mf_xcopy_describe_plan(const uint64_t *src, const uint64_t *dst, const u
  * MF_HIP_CALIBRATE=0 skips it and keeps the fitted defaults).  A batch of 2196 chunks is timed with its stores not held
  * and held for the rule's wait and 200 ns either side: the best of the three becomes the process's offset to every wait
  * (holdDeltaNanos), and holding is switched off where it does not beat the plain launch by 3 % (holdEnabled 0).  A copy
- * of 512 MiB is timed without windows, at the default rate, at 94 % of it and at the higher rate that segments on
+ * of 512 MiB is timed without windows, at the default rate, at 94 % of it and at the highest rate, the one long segments on
  * cache lines take: windowMBps receives the rate in force (0: windows did not beat the plain kernel and are off),
- * windowAlignedMBps the one for segments on cache lines (the higher rate where it was 2 % faster here, else the same).  micros (8 floats,
+ * windowAlignedMBps and windowLongMBps the ones for segments on cache lines and for long ones among them (the higher
+ * rates where the highest was 2 % faster here, else the same as windowMBps).  micros (8 floats,
  * may be NULL): the eight times in that order, us per batch / per copy.  Returns 1 if the calibration ran, 0 if not.
  * mf_xcopy_hold_stores / mf_xcopy_windows still override what it chose (a rate set by hand holds for both). */
 int32_t mf_xcopy_calibration(int32_t *holdEnabled, int32_t *holdDeltaNanos, uint32_t *windowMBps, uint32_t *windowAlignedMBps,
-                             float *micros);
+                             uint32_t *windowLongMBps, float *micros);
 /* The streams hybm_init makes for calling threads and submit threads, in the order they are handed out (the calling
  * thread of hybm_init holds the first): queues[i] is the hardware queue stream i sits on, numbered in order of
  * appearance.  The library asks the GPU which of its streams share a queue (launches on such streams run one

@@ -188,7 +188,7 @@ MF_EXPORT int32_t mf_xcopy_tune_hold(uint32_t deepHold, int32_t pinnedExtraNanos
 }
 
 MF_EXPORT int32_t mf_xcopy_calibration(int32_t *holdEnabled, int32_t *holdDeltaNanos, uint32_t *windowMBps, uint32_t *windowAlignedMBps,
-                                       float *micros)
+                                       uint32_t *windowLongMBps, float *micros)
 {
     const XcopyCalibration &c = XcopyEngine::Instance().Calibration();
     if (holdEnabled != nullptr) {
@@ -202,6 +202,9 @@ MF_EXPORT int32_t mf_xcopy_calibration(int32_t *holdEnabled, int32_t *holdDeltaN
     }
     if (windowAlignedMBps != nullptr) {
         *windowAlignedMBps = XcopyEngine::Instance().Tuning().windowAlignedMBps;
+    }
+    if (windowLongMBps != nullptr) {
+        *windowLongMBps = XcopyEngine::Instance().Tuning().windowLongMBps;
     }
     if (micros != nullptr) {
         for (int i = 0; i < 4; ++i) {
@@ -225,11 +228,23 @@ MF_EXPORT int32_t mf_xcopy_hold_stores(int32_t nanos)
 
 MF_EXPORT int32_t mf_xcopy_windows(uint32_t megabytesPerSecond)
 {
+    if (megabytesPerSecond == MF_XCOPY_WINDOWS_OWN_CHOICE) {
+        // back to what the library chose: what hybm_init measured on this GPU, else the fitted defaults
+        const XcopyCalibration &c = XcopyEngine::Instance().Calibration();
+        const XcopyTuning fitted;
+        XcopyTuning &t = XcopyEngine::Instance().Tuning();
+        t.windowMBps = c.ran ? c.windowMBps : fitted.windowMBps;
+        t.windowAlignedMBps = c.ran ? c.windowAlignedMBps : fitted.windowAlignedMBps;
+        t.windowLongMBps = c.ran ? c.windowLongMBps : fitted.windowLongMBps;
+        return BM_OK;
+    }
     if (megabytesPerSecond != 0 && (megabytesPerSecond < 1000000 || megabytesPerSecond > 16000000)) {
-        MF_FAIL(BM_INVALID_PARAM, "windows: 0 (never) or a rate between 1 000 000 and 16 000 000 MB/s, got " << megabytesPerSecond);
+        MF_FAIL(BM_INVALID_PARAM, "windows: 0 (never), 1 (the library's own choice) or a rate between 1 000 000 and 16 000 000 MB/s, got "
+                                      << megabytesPerSecond);
     }
     XcopyEngine::Instance().Tuning().windowMBps = megabytesPerSecond;
     XcopyEngine::Instance().Tuning().windowAlignedMBps = megabytesPerSecond;   // a rate set by hand holds for every windowed launch
+    XcopyEngine::Instance().Tuning().windowLongMBps = megabytesPerSecond;
     return BM_OK;
 }
 

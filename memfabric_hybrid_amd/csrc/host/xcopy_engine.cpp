@@ -954,11 +954,12 @@ uint64_t BuildTableDirect(const uint64_t *src, const uint64_t *dst, const uint64
 }
 
 void ChooseCalibration(const float *batchMicros, const float *copyMicros, uint32_t defaultWindowMBps, uint32_t defaultAlignedMBps,
-                       XcopyCalibration &out)
+                       uint32_t defaultLongMBps, XcopyCalibration &out)
 {
     out = XcopyCalibration{};
     out.windowMBps = defaultWindowMBps;
     out.windowAlignedMBps = defaultAlignedMBps;
+    out.windowLongMBps = defaultLongMBps;
     for (int i = 0; i < 4; ++i) {
         out.batchMicros[i] = batchMicros[i];
     }
@@ -986,7 +987,10 @@ void ChooseCalibration(const float *batchMicros, const float *copyMicros, uint32
                                          : defaultWindowMBps;
         out.windowMBps = windowed <= copyMicros[0] * (1.0f - kCalibrateMinWindowGain) ? rate : 0u;
         // the higher rate of aligned segments only where an aligned copy held it here: 2 % better than the rate just chosen
-        out.windowAlignedMBps = out.windowMBps != 0 && copyMicros[3] > 0 && copyMicros[3] < windowed * 0.98f ? defaultAlignedMBps : out.windowMBps;
+        // (the rate between the two, for shorter segments on cache lines, goes with it: a GPU that holds the highest holds that one)
+        const bool higherHolds = out.windowMBps != 0 && copyMicros[3] > 0 && copyMicros[3] < windowed * 0.98f;
+        out.windowLongMBps = higherHolds ? defaultLongMBps : out.windowMBps;
+        out.windowAlignedMBps = higherHolds ? defaultAlignedMBps : out.windowMBps;
         out.ran = true;
     }
 }
@@ -1003,7 +1007,7 @@ int XcopyEngine::Calibrate()
     const uint32_t rule = HoldNanosFor(2196, 2196, kXcopyThreads, false);
     const uint32_t holds[3] = {rule - kCalibrateHoldStepNanos, rule, rule + kCalibrateHoldStepNanos};
     const uint32_t defaultRate = XcopyTuning{}.windowMBps;
-    const uint32_t defaultLong = XcopyTuning{}.windowAlignedMBps;
+    const uint32_t defaultLong = XcopyTuning{}.windowLongMBps;
     const uint32_t rates[3] = {defaultRate, static_cast<uint32_t>(static_cast<uint64_t>(defaultRate) * kCalibrateSlowerWindowPercent / 100),
                                defaultLong};
     float us[8] = {};
@@ -1013,13 +1017,14 @@ int XcopyEngine::Calibrate()
         MF_ERROR("calibration run failed (" << mfrt_error_string(err) << "): the fitted defaults stay");
         return BM_ERROR;
     }
-    ChooseCalibration(us, us + 4, defaultRate, defaultLong, calibration_);
+    ChooseCalibration(us, us + 4, defaultRate, XcopyTuning{}.windowAlignedMBps, defaultLong, calibration_);
     if (calibration_.ran) {
         tuning_.holdDeltaNanos = calibration_.holdDeltaNanos;
         tuning_.holdCalibratedOff = !calibration_.holdEnabled;
         if (windowsAvailable_) {
             tuning_.windowMBps = calibration_.windowMBps;
             tuning_.windowAlignedMBps = calibration_.windowAlignedMBps;
+            tuning_.windowLongMBps = calibration_.windowLongMBps;
             windowRateCalibrated_ = true;
         }
     }
@@ -1052,6 +1057,7 @@ int XcopyEngine::Start(int device)
     if (windowRateCalibrated_) {   // what an earlier start of this process chose does not outlive it
         tuning_.windowMBps = XcopyTuning{}.windowMBps;
         tuning_.windowAlignedMBps = XcopyTuning{}.windowAlignedMBps;
+        tuning_.windowLongMBps = XcopyTuning{}.windowLongMBps;
         windowRateCalibrated_ = false;
     }
     calibration_ = XcopyCalibration{};
@@ -1297,11 +1303,11 @@ bool XcopyEngine::DeepHoldApplies(uint64_t bytes, uint32_t n, int route, bool un
            g_leasesOut.load(std::memory_order_relaxed) <= 1;
 }
 
-bool XcopyEngine::WindowsApply(uint64_t bytes, int route) const
+bool XcopyEngine::WindowsApply(uint64_t bytes, int route, uint64_t minBytes) const
 {
     // Two such launches at a time would each cut their periods for the whole chip's rate, so a second thread with a
     // stream of its own switches the form off, as it does for the largest held launches.
-    return route == MFRT_ROUTE_HBM && bytes >= kWindowMinBytes && tuning_.windowMBps != 0 && tuning_.unitsOverride == 0 &&
+    return route == MFRT_ROUTE_HBM && bytes >= minBytes && tuning_.windowMBps != 0 && tuning_.unitsOverride == 0 &&
            windowsAvailable_ && g_leasesOut.load(std::memory_order_relaxed) <= 1;
 }
 
@@ -1316,13 +1322,13 @@ int XcopyEngine::Submit(const uint64_t *src, const uint64_t *dst, const uint64_t
     return SubmitOne(src, dst, len, n, route, stream, mask, maskValue, unordered, true);
 }
 
-// A batch of up to kInlineSegs segments that moves twice kWindowMinBytes and more, submitted as consecutive runs of
-// kWindowMinBytes to twice that, one windowed launch each.  Runs end at segment ends where the segments are short and
+// A batch of up to kInlineSegs segments that moves twice kWindowPieceBytes and more, submitted as consecutive runs of
+// kWindowPieceBytes to twice that, one windowed launch each.  Runs end at segment ends where the segments are short and
 // inside a segment, at a multiple of 1 MiB from its start, where one is long.
 int XcopyEngine::SubmitInPieces(const uint64_t *src, const uint64_t *dst, const uint64_t *len, uint32_t n, uint64_t total, int route,
                                 void *stream, void *mask, uint32_t maskValue)
 {
-    const uint64_t pieces = total / kWindowMinBytes;
+    const uint64_t pieces = total / kWindowPieceBytes;
     const uint64_t target = (total + pieces - 1) / pieces;
     constexpr uint64_t kCutUnit = 1ull << 20;
     std::vector<uint64_t> ps;
@@ -1348,7 +1354,7 @@ int XcopyEngine::SubmitInPieces(const uint64_t *src, const uint64_t *dst, const 
             uint64_t take = len[i] - at;
             const uint64_t room = target > inPiece ? target - inPiece : 0;
             // what is left behind this piece must still make a launch of its own, else it stays with this one
-            if (take > room && left - room >= kWindowMinBytes) {
+            if (take > room && left - room >= kWindowPieceBytes) {
                 const uint64_t cut = room / kCutUnit * kCutUnit;
                 if (take >= 16 * kCutUnit && cut != 0 && take - cut >= kCutUnit) {
                     take = cut;
@@ -1366,7 +1372,7 @@ int XcopyEngine::SubmitInPieces(const uint64_t *src, const uint64_t *dst, const 
             at += take;
             inPiece += take;
             left -= take;
-            if (inPiece >= target && left >= kWindowMinBytes) {
+            if (inPiece >= target && left >= kWindowPieceBytes) {
                 const int ret = flush(false);
                 if (ret != BM_OK) {
                     return ret;
@@ -1450,22 +1456,31 @@ int XcopyEngine::SubmitOne(const uint64_t *src, const uint64_t *dst, const uint6
         // Not where a source and its destination differ modulo 16: the kernels align their 128-bit units on the destination,
         // the loads then straddle units, cost twice the issue slots, and the waves keep no schedule at any rate that pays
         // (100 segments of 10 MB: 5.35 TB/s in windows cut for 6.8, 5.26 for 7.4, 5.51 to 5.56 without windows).
-        windowed = !unordered && (apartBits & (kUnitBytes - 1)) == 0 && WindowsApply(total, route);
-        // Segments that all start on cache lines, in source and destination, hold the higher rate (back to back, 6.8 against
-        // 7.4 TB/s: 100 x 10 MB 6.41 to 6.47 against 6.72 to 6.87 TB/s, 32 x 16 MiB 6.56 against 6.94 to 7.03, 3 x 700 MB 6.30 to
-        // 6.35 against 6.78).  Where they start elsewhere every wave's kilobyte straddles a line it shares with its
-        // neighbour; such launches hold 6.8 (6.24 to 6.27 against 5.65 to 5.80 TB/s without windows) and fall apart at 7.4 (5.36 to 5.48).
         const bool aligned = (addressBits & (kWindowAlignBytes - 1)) == 0;
+        windowed = !unordered && (apartBits & (kUnitBytes - 1)) == 0 &&
+                   WindowsApply(total, route, aligned && tuning_.windowAlignedMBps != 0 ? kWindowMinBytes : kWindowGeneralMinBytes);
+        // Segments that all start on cache lines, in source and destination, hold a higher rate.  Back to back at 6.8 / 7.1 /
+        // 7.4 TB/s, the same in four processes: 2 GiB in one segment 6.65 / 6.95 / 7.02 to 7.27, 32 x 16 MiB 6.65 / 6.95 / 7.05 to
+        // 7.26, 128 x 9 MiB 6.65 / 6.95 / 6.76 to 7.32.  The reshard's launches of 128 segments of 0.4 to 17 MB from eight
+        // places hold 7.1 in every process (6.87 to 7.00) and 7.4 only in some (7.0 to 7.2 in one, 5.8 to 6.1 in three others):
+        // long segments take the highest rate, other aligned ones the one between.  Where segments start between cache lines
+        // every wave's kilobyte straddles a line it shares with its neighbour; such launches hold 6.8 (6.24 to 6.27 against 5.65
+        // to 5.80 TB/s without windows) and fall apart at 7.4 (5.36 to 5.48).
         const bool longSegments = windowed && total / n >= kWindowLongSegmentBytes;
-        if (longSegments && maySlice && total >= 2 * kWindowMinBytes) {
+        if (longSegments && maySlice && total >= 2 * kWindowPieceBytes) {
             // A windowed launch that loses its schedule runs the rest of its bytes at the rate without windows, and the longer
-            // it runs the likelier that is: launches of kWindowMinBytes to twice that, each with a schedule of its own, hold
+            // it runs the likelier that is: launches of kWindowPieceBytes to twice that, each with a schedule of its own, hold
             // a target the whole copy in one launch does not (2 GiB at 7.4 TB/s: 7.1 TB/s on average in four launches,
             // 6.6 to 6.8 in one).  Only long segments are worth it: 896 segments of some 10 MB in launches of 64 or 96
             // segments (600 to 900 MB) were no faster than in launches of 128.
             return SubmitInPieces(src, dst, len, n, total, route, stream, mask, maskValue);
         }
-        windowRate = aligned && tuning_.windowAlignedMBps != 0 ? tuning_.windowAlignedMBps : tuning_.windowMBps;
+        windowRate = tuning_.windowMBps;
+        if (aligned && longSegments && tuning_.windowLongMBps != 0) {
+            windowRate = tuning_.windowLongMBps;
+        } else if (aligned && tuning_.windowAlignedMBps != 0) {
+            windowRate = tuning_.windowAlignedMBps;
+        }
         if (windowed) {
             units = mfk_xcopy_window_units();
         }
@@ -1509,20 +1524,26 @@ int XcopyEngine::SubmitOne(const uint64_t *src, const uint64_t *dst, const uint6
     {
         uint64_t total = 0;
         uint64_t longest = 0;
+        uint64_t addressBits = 0;
         for (uint32_t i = 0; i < n; ++i) {
             total += len[i];
             longest = len[i] > longest ? len[i] : longest;
+            addressBits |= src[i] | dst[i];
         }
         queuedBytes = total;
         // A table of long segments between HBM addresses is cut into launches of kInlineSegs segments, each of which
         // then takes the form with read and write windows: the few extra launches cost microseconds, the windows
-        // gain 8 % (896 segments, 8.5 GB: 2.55 ms in seven launches against 2.78 ms in one).  The table form
+        // gain 8 % (896 segments, 8.5 GB: 2.55 ms in seven launches against 2.78 ms in one).  Segments on cache lines
+        // are worth it from 1 MiB each, 128 MiB a launch (1024 x 1 MiB 327 against 361 us, 1024 x 2 MiB 658 against
+        // 753 to 772 us, 512 x 3 MiB 458 against 588 us; 1024 x 512 KiB, 64 MiB a launch, the same either way).  The table form
         // itself was measured under windows twice, with the prefix search it once had and with the division and
         // group map it has now, and is left without them: 262 144 pages of 32 KiB at random places lose 7 to 12 %
         // (3.23 to 3.45 against 3.04 ms), 16 384 ragged segments 3 %, and the 896 long segments in one windowed
         // table launch are no faster than in seven launches of the kernel-argument form.
         if (maySlice && n > kInlineSegs && route == MFRT_ROUTE_HBM && !unordered && tuning_.windowMBps != 0 && windowsAvailable_ &&
-            tuning_.unitsOverride == 0 && total / n >= kWindowSliceMinSegmentBytes &&
+            tuning_.unitsOverride == 0 &&
+            total / n >= ((addressBits & (kWindowAlignBytes - 1)) == 0 && tuning_.windowAlignedMBps != 0 ? kWindowSliceMinAlignedSegmentBytes
+                                                                                                         : kWindowSliceMinSegmentBytes) &&
             g_leasesOut.load(std::memory_order_relaxed) <= 1) {
             for (uint32_t at = 0; at < n; at += kInlineSegs) {
                 const uint32_t m = n - at < kInlineSegs ? n - at : kInlineSegs;

@@ -55,16 +55,24 @@ struct XcopyTuning {
     int32_t holdPinnedExtraNanos = 1600;   // added to the rule for table launches, whose descriptors come from pinned host memory: a link round trip before the loads
     bool stageUnordered = true;  // the upload of a ragged table's descriptors is launched without a barrier
     uint32_t deviceTableWgPerCu = 0;   // grid of a device-resident table in workgroups per CU, 0 = eight per segment between 32 and 4096 per CU
-    uint32_t windowMBps = 6800000;   // HBM copies of kWindowMinBytes and more alternate between read and write windows cut for this rate; 0 = never
-    uint32_t windowAlignedMBps = 7400000;   // the same for launches of segments that all start at multiples of kWindowAlignBytes in source and destination, which hold more; 0 = the rate above
+    uint32_t windowMBps = 6800000;   // HBM copies of kWindowGeneralMinBytes and more alternate between read and write windows cut for this rate; 0 = never
+    uint32_t windowAlignedMBps = 7100000;   // the same for launches of segments that all start at multiples of kWindowAlignBytes in source and destination, which hold more; 0 = the rate above
+    uint32_t windowLongMBps = 7400000;      // and for those of them whose segments are kWindowLongSegmentBytes and longer on average, which hold more still; 0 = the rate above
 };
 
-// From this total on a batch of up to 128 segments between HBM addresses is copied in read and write windows
-// (XcopyWindowKernel has the measurements; 512 MiB gains 2 %, 256 MiB nothing).
-constexpr uint64_t kWindowMinBytes = 512ull << 20;
-constexpr uint64_t kWindowLongSegmentBytes = 64ull << 20;     // launches whose segments average this much go out in pieces of kWindowMinBytes and more
+// From this total on a batch of up to 128 segments between HBM addresses is copied in read and write windows.
+// Segments on cache lines, paced for windowAlignedMBps, gain from where the held stores of 16 KiB per wave end:
+// back to back, 32 segments, windows against none: 66 MiB 6.37 against 5.71 TB/s, 80 MiB 6.57 against 5.76, 130 MiB
+// 6.94 against 6.14, 256 MiB 7.14 against 6.37, 600 MiB 7.20 against 6.31 (at 64 MiB and below the held stores are
+// as fast).  A launch on its own gains less and less steadily below 128 MiB (80 MiB: 32.4 against 31.9 us), hence
+// the limit.  Other segments, paced for windowMBps, and rectangles were measured from 512 MiB on (2 % there).
+constexpr uint64_t kWindowMinBytes = 128ull << 20;
+constexpr uint64_t kWindowGeneralMinBytes = 512ull << 20;
+constexpr uint64_t kWindowPieceBytes = 512ull << 20;          // launches into which long segments are cut
+constexpr uint64_t kWindowLongSegmentBytes = 64ull << 20;     // launches whose segments average this much go out in pieces of kWindowPieceBytes and more
 constexpr uint64_t kWindowAlignBytes = 128;                   // a cache line: segments that start on one are read and written in whole lines by every wave
 constexpr uint64_t kWindowSliceMinSegmentBytes = 4ull << 20;   // tables of segments this long on average are cut into windowed launches
+constexpr uint64_t kWindowSliceMinAlignedSegmentBytes = 1ull << 20;   // the same for segments on cache lines: kInlineSegs of them reach kWindowMinBytes
 
 // What Start() measured on the GPU it runs on and chose from it (XcopyEngine::Calibrate).
 struct XcopyCalibration {
@@ -72,16 +80,17 @@ struct XcopyCalibration {
     bool holdEnabled = true;        // the held stores beat the launch that stores at once by kCalibrateMinGain
     int32_t holdDeltaNanos = 0;     // added to every wait HoldNanosFor gives
     uint32_t windowMBps = 0;        // rate the read and write windows are cut for; 0: the form lost against the plain kernel
-    uint32_t windowAlignedMBps = 0;    // rate for launches of segments on cache-line boundaries: the higher one where it beat the rate above, else that rate
+    uint32_t windowAlignedMBps = 0;    // rate for launches of segments on cache-line boundaries
+    uint32_t windowLongMBps = 0;       // rate for launches of long segments on cache-line boundaries; both the higher ones where a long copy held the highest, else the rate above
     float batchMicros[4] = {};      // 2196-chunk batch: not held, rule - step, rule, rule + step
-    float copyMicros[4] = {};       // 512 MiB copy: no windows, default rate, reduced rate, the higher rate of aligned segments
+    float copyMicros[4] = {};       // 512 MiB copy: no windows, default rate, reduced rate, the rate of long segments on cache lines
 };
 constexpr int32_t kCalibrateHoldStepNanos = 200;
 constexpr float kCalibrateMinGain = 0.03f;          // held stores that do not gain this much over the plain launch are switched off
 constexpr float kCalibrateMinWindowGain = 0.005f;   // windows stay unless they lose: on the 512 MiB that is measured they gain least (2 to 5 %, 8 % on 1 GiB)
 constexpr uint32_t kCalibrateSlowerWindowPercent = 94;   // the second window rate tried, in percent of the default
 // The choice, from the measured times alone (microseconds; a time of 0 means "not measured" and leaves the default).
-void ChooseCalibration(const float *batchMicros, const float *copyMicros, uint32_t defaultWindowMBps, uint32_t defaultAlignedMBps,
+void ChooseCalibration(const float *batchMicros, const float *copyMicros, uint32_t defaultWindowMBps, uint32_t defaultAlignedMBps, uint32_t defaultLongMBps,
                        XcopyCalibration &out);
 
 uint32_t ChooseUnits(uint64_t totalBytes, uint32_t cuCount, int route, const XcopyTuning &tuning);
@@ -128,7 +137,7 @@ public:
     int Calibrate();
 
     // Whether an ordered launch that moves `bytes` on `route` takes the form with read and write windows.
-    bool WindowsApply(uint64_t bytes, int route) const;
+    bool WindowsApply(uint64_t bytes, int route, uint64_t minBytes = kWindowGeneralMinBytes) const;
     // Hardware queue (numbered in order of appearance) of each of the streams made at Start(), in the order they are handed out; returns their number.
     uint32_t StreamQueues(uint32_t *queues, uint32_t capacity) const;
     // No second thread holds a stream of the library: kernels that pace themselves for the whole chip may be used.

@@ -183,7 +183,7 @@ extern "C" int mfk_copy2d_windowed(const void *rectPlan, uint32_t windowMBps, vo
     if (plan.nchunk == 0) {
         return 0;
     }
-    const uint32_t grid = plan.nchunk < mf::kRectWindowWaves ? plan.nchunk : mf::kRectWindowWaves;
+    const uint32_t grid = mf::WindowGrid(plan.nchunk, mf::kRectWindowWaves);
     const uint32_t ticks = mf::WindowPeriodTicks(2ull * grid * mf::kRectWindowUnits * 16u, windowMBps);
     if (ticks == 0) {
         return static_cast<int>(hipErrorInvalidValue);

@@ -77,6 +77,18 @@ inline uint32_t WindowPeriodTicks(uint64_t bytes, uint32_t windowMBps)
     return ticks < 16 || ticks > 1000000 ? 0 : static_cast<uint32_t>(ticks);
 }
 
+// Waves of a windowed launch of nchunk chunks, at most maxWaves: the chunks are shared out evenly over the fewest
+// periods that many waves need, so that the last period is as full as the others (the period is cut for the
+// waves there are; 18.2 periods' worth of chunks on maxWaves waves would pay for 19).
+inline uint32_t WindowGrid(uint32_t nchunk, uint32_t maxWaves)
+{
+    if (nchunk <= maxWaves) {
+        return nchunk;
+    }
+    const uint32_t periods = (nchunk + maxWaves - 1) / maxWaves;
+    return (nchunk + periods - 1) / periods;
+}
+
 // Sequence number of a windowed launch: the 24 bits the kernels compare are never 0, which is what an untouched slot holds.
 inline uint32_t NextWindowSeq()
 {

@@ -1057,7 +1057,7 @@ extern "C" int mfk_xcopy_windowed(const void *inlinePlan, uint32_t windowMBps, v
     if (plan.units != mf::kWindowUnits || plan.nchunk == 0 || windowMBps == 0) {
         return -1;
     }
-    const uint32_t grid = plan.nchunk < mf::kWindowWaves ? plan.nchunk : mf::kWindowWaves;
+    const uint32_t grid = mf::WindowGrid(plan.nchunk, mf::kWindowWaves);
     const int err = mf::WithPolicy(mf::PolicyOf(MFRT_ROUTE_HBM), [&](auto ntLoad, auto store) {
         return mf::LaunchWindowed<decltype(ntLoad)::value, decltype(store)::value>(plan, grid, windowMBps, s);
     });

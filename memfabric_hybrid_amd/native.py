@@ -197,7 +197,7 @@ _SIGNATURES = {
     "mf_xcopy_tune_table": (i32, [u32, u32]),
     "mf_xcopy_tune_hold": (i32, [u32, i32, u32]),
     "mf_xcopy_calibration": (i32, [ctypes.POINTER(i32), ctypes.POINTER(i32), ctypes.POINTER(u32), ctypes.POINTER(u32),
-                                 ctypes.POINTER(ctypes.c_float)]),
+                                 ctypes.POINTER(u32), ctypes.POINTER(ctypes.c_float)]),
     "mf_xcopy_hold_stores": (i32, [i32]),
     "mf_xcopy_windows": (i32, [u32]),
     "mf_xcopy_choose_units": (u32, [u64, u32, i32]),

@@ -800,41 +800,42 @@ static void TestCalibration()
 {
     const uint32_t rate = XcopyTuning{}.windowMBps;
     const uint32_t alignedRate = XcopyTuning{}.windowAlignedMBps;
+    const uint32_t longRate = XcopyTuning{}.windowLongMBps;
     XcopyCalibration c;
     {   // the usual picture: the rule's wait is best, held stores gain 14 %, windows 7 %, one long segment holds the higher rate
         const float batch[4] = {5.30f, 4.62f, 4.55f, 4.60f};
         const float copy[4] = {172.0f, 160.0f, 163.0f, 149.0f};
-        ChooseCalibration(batch, copy, rate, alignedRate, c);
-        CHECK(c.ran && c.holdEnabled && c.holdDeltaNanos == 0 && c.windowMBps == rate && c.windowAlignedMBps == alignedRate);
+        ChooseCalibration(batch, copy, rate, alignedRate, longRate, c);
+        CHECK(c.ran && c.holdEnabled && c.holdDeltaNanos == 0 && c.windowMBps == rate && c.windowAlignedMBps == alignedRate && c.windowLongMBps == longRate);
     }
     {   // the higher rate does not hold here (no better than the default by 2 %): long segments take the default too
         const float batch[4] = {5.30f, 4.62f, 4.55f, 4.60f};
         const float copy[4] = {172.0f, 160.0f, 163.0f, 158.5f};
-        ChooseCalibration(batch, copy, rate, alignedRate, c);
-        CHECK(c.windowMBps == rate && c.windowAlignedMBps == rate);
+        ChooseCalibration(batch, copy, rate, alignedRate, longRate, c);
+        CHECK(c.windowMBps == rate && c.windowAlignedMBps == rate && c.windowLongMBps == rate);
     }
     {   // a GPU whose loads land later: the longer wait wins clearly; windows only hold at the lower rate
         const float batch[4] = {5.30f, 4.95f, 4.80f, 4.60f};
         const float copy[4] = {172.0f, 171.0f, 161.0f, 176.0f};
-        ChooseCalibration(batch, copy, rate, alignedRate, c);
+        ChooseCalibration(batch, copy, rate, alignedRate, longRate, c);
         CHECK(c.holdEnabled && c.holdDeltaNanos == kCalibrateHoldStepNanos && c.windowMBps == static_cast<uint32_t>(static_cast<uint64_t>(rate) * 94 / 100) &&
-              c.windowAlignedMBps == c.windowMBps);
+              c.windowAlignedMBps == c.windowMBps && c.windowLongMBps == c.windowMBps);
     }
     {   // a neighbour that is better by less than 1 % does not move the wait
         const float batch[4] = {5.30f, 4.53f, 4.55f, 4.60f};
         const float copy[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-        ChooseCalibration(batch, copy, rate, alignedRate, c);
-        CHECK(c.ran && c.holdDeltaNanos == 0 && c.windowMBps == rate && c.windowAlignedMBps == alignedRate);   // windows not measured: the defaults stay
+        ChooseCalibration(batch, copy, rate, alignedRate, longRate, c);
+        CHECK(c.ran && c.holdDeltaNanos == 0 && c.windowMBps == rate && c.windowAlignedMBps == alignedRate && c.windowLongMBps == longRate);   // windows not measured: the defaults stay
     }
     {   // a busy or capped chip: holding gains 2 %, windows lose: both off
         const float batch[4] = {5.30f, 5.25f, 5.20f, 5.28f};
         const float copy[4] = {172.0f, 175.0f, 174.0f, 169.0f};
-        ChooseCalibration(batch, copy, rate, alignedRate, c);
-        CHECK(c.ran && !c.holdEnabled && c.windowMBps == 0 && c.windowAlignedMBps == 0);
+        ChooseCalibration(batch, copy, rate, alignedRate, longRate, c);
+        CHECK(c.ran && !c.holdEnabled && c.windowMBps == 0 && c.windowAlignedMBps == 0 && c.windowLongMBps == 0);
     }
     {   // nothing measured
         const float none[4] = {0, 0, 0, 0};
-        ChooseCalibration(none, none, rate, alignedRate, c);
+        ChooseCalibration(none, none, rate, alignedRate, longRate, c);
         CHECK(!c.ran && c.holdEnabled && c.holdDeltaNanos == 0 && c.windowMBps == rate);
     }
     // through hybm_init: the engine applies what it chose, and mf_xcopy_hold_stores(-1) means the calibrated rule
@@ -847,9 +848,10 @@ static void TestCalibration()
     int32_t delta = 0;
     uint32_t mbps = 0;
     uint32_t alignedMbps = 0;
+    uint32_t longMbps = 0;
     float micros[8] = {};
-    CHECK(mf_xcopy_calibration(&enabled, &delta, &mbps, &alignedMbps, micros) == 1);
-    CHECK(enabled == 1 && delta == -200 && mbps == rate && alignedMbps == alignedRate && micros[1] == 4.40f && micros[5] == 160.0f && micros[7] == 150.0f);
+    CHECK(mf_xcopy_calibration(&enabled, &delta, &mbps, &alignedMbps, &longMbps, micros) == 1);
+    CHECK(enabled == 1 && delta == -200 && mbps == rate && alignedMbps == alignedRate && longMbps == longRate && micros[1] == 4.40f && micros[5] == 160.0f && micros[7] == 150.0f);
     {
         std::vector<uint8_t> from(12 << 20), to(12 << 20);
         const uint64_t fromBase = (reinterpret_cast<uint64_t>(from.data()) + 4095) & ~4095ull;
@@ -869,12 +871,12 @@ static void TestCalibration()
     const float lost[8] = {5.30f, 5.29f, 5.31f, 5.30f, 172.0f, 175.0f, 176.0f, 177.0f};
     fake_rt_set_calibration(lost);
     CHECK(hybm_init(0, 0) == BM_OK);
-    CHECK(mf_xcopy_calibration(&enabled, &delta, &mbps, &alignedMbps, nullptr) == 1 && enabled == 0 && mbps == 0 && alignedMbps == 0);
+    CHECK(mf_xcopy_calibration(&enabled, &delta, &mbps, &alignedMbps, &longMbps, nullptr) == 1 && enabled == 0 && mbps == 0 && alignedMbps == 0 && longMbps == 0);
     hybm_uninit();
     setenv("MF_HIP_CALIBRATE", "0", 1);
     CHECK(hybm_init(0, 0) == BM_OK);
-    CHECK(mf_xcopy_calibration(&enabled, &delta, &mbps, &alignedMbps, nullptr) == 0 && enabled == 1 && delta == 0 && mbps == rate &&
-          alignedMbps == alignedRate);
+    CHECK(mf_xcopy_calibration(&enabled, &delta, &mbps, &alignedMbps, &longMbps, nullptr) == 0 && enabled == 1 && delta == 0 && mbps == rate &&
+          alignedMbps == alignedRate && longMbps == longRate);
     hybm_uninit();
     unsetenv("MF_HIP_CALIBRATE");
     const float none[8] = {};
@@ -1516,10 +1518,30 @@ static void TestWindows()
         }
         CHECK(same);
         CHECK(fake_rt_last_window() == 6800000);       // destinations between cache lines: the general rate
+        for (uint32_t i = 0; i < 64; ++i) {
+            dst64[i] += 128 - 48;
+        }
+        CHECK(engine.Submit(src64.data(), dst64.data(), len64.data(), 64, MF_ROUTE_HBM, stream, nullptr, 0) == BM_OK);
+        CHECK(fake_rt_last_window() == 7100000);       // on cache lines, 16 MiB each: the rate between
+        CHECK(engine.DrainThread() == BM_OK);
     }
-    l1 = (gib >> 1) - 1;                           // one byte below the limit: the ordinary form
+    l1 = (gib >> 3) - 1;                           // one byte below the limit of segments on cache lines: the ordinary form
     CHECK(engine.Submit(&s1, &d1, &l1, 1, MF_ROUTE_HBM, stream, nullptr, 0) == BM_OK);
     CHECK(fake_rt_last_window() == 0);
+    l1 = gib >> 3;
+    CHECK(engine.Submit(&s1, &d1, &l1, 1, MF_ROUTE_HBM, stream, nullptr, 0) == BM_OK);
+    CHECK(fake_rt_last_window() == 7400000);
+    {
+        // between cache lines the limit is 512 MiB
+        uint64_t so = s1 + 16;
+        uint64_t dO = d1 + 48;
+        uint64_t lo = (gib >> 1) - 1;
+        CHECK(engine.Submit(&so, &dO, &lo, 1, MF_ROUTE_HBM, stream, nullptr, 0) == BM_OK);
+        CHECK(fake_rt_last_window() == 0);
+        lo = gib >> 1;
+        CHECK(engine.Submit(&so, &dO, &lo, 1, MF_ROUTE_HBM, stream, nullptr, 0) == BM_OK);
+        CHECK(fake_rt_last_window() == 6800000);
+    }
     l1 = gib;
     CHECK(engine.Submit(&s1, &d1, &l1, 1, MF_ROUTE_HBM, stream, nullptr, 0, true) == BM_OK);
     CHECK(fake_rt_last_window() == 0);             // unordered launches overlap on purpose
@@ -1562,10 +1584,44 @@ static void TestWindows()
         uint64_t word = 0;
         CHECK(engine.Submit(src.data(), dst.data(), len.data(), count, MF_ROUTE_HBM, stream, &word, 32) == BM_OK);
         CHECK(mf_xcopy_launch_count() - before == 3);
-        CHECK(fake_rt_last_window() == 6800000);   // the two full slices (512 MiB each) went in windows; the last one (176 MiB) is below the limit
+        CHECK(fake_rt_last_window() == 6800000);   // all three slices in windows (512, 512 and 176 MiB of segments on cache lines)
         CHECK(word == 32);
         CHECK(engine.DrainThread() == BM_OK);
     }
+    {
+        // segments on cache lines are worth slicing from 1 MiB each (128 MiB a launch); between cache lines only from 4 MiB
+        const uint32_t count = 300;
+        const uint64_t seg = 1ull << 20;
+        std::vector<uint64_t> src(count), dst(count), len(count, seg);
+        for (uint32_t i = 0; i < count; ++i) {
+            src[i] = s1 + (i % 200) * 2 * seg + 128 * i;
+            dst[i] = s1 + gib + ((i * 7) % 300) * 2 * seg + 256 * i;        // 300 places of 2 MiB, none shared
+        }
+        uint64_t before = mf_xcopy_launch_count();
+        (void)fake_rt_last_window();
+        CHECK(engine.Submit(src.data(), dst.data(), len.data(), count, MF_ROUTE_HBM, stream, nullptr, 0) == BM_OK);
+        CHECK(mf_xcopy_launch_count() - before == 3);      // 128 + 128 + 44 segments; the last launch (44 MiB) without windows
+        CHECK(engine.DrainThread() == BM_OK);
+        bool same = true;
+        for (uint32_t i = 0; i < count && same; i += 7) {
+            same = std::memcmp(reinterpret_cast<void *>(dst[i]), reinterpret_cast<void *>(src[i]), seg) == 0;
+        }
+        CHECK(same);
+        for (uint32_t i = 0; i < count; ++i) {
+            src[i] += 16;
+            dst[i] += 48;
+        }
+        before = mf_xcopy_launch_count();
+        (void)fake_rt_last_window();
+        CHECK(engine.Submit(src.data(), dst.data(), len.data(), count, MF_ROUTE_HBM, stream, nullptr, 0) == BM_OK);
+        CHECK(mf_xcopy_launch_count() - before <= 2 && fake_rt_last_window() == 0);     // one table launch (and its upload)
+        CHECK(engine.DrainThread() == BM_OK);
+    }
+    CHECK(mf_xcopy_windows(MF_XCOPY_WINDOWS_OWN_CHOICE) == BM_OK);      // from the rate set by hand back to the library's three
+    l1 = gib;
+    CHECK(engine.Submit(&s1, &d1, &l1, 1, MF_ROUTE_HBM, stream, nullptr, 0) == BM_OK);
+    CHECK(fake_rt_last_window() == XcopyTuning{}.windowLongMBps);
+    CHECK(engine.DrainThread() == BM_OK);
     hybm_uninit();
 }
 
