@@ -1536,10 +1536,11 @@ int XcopyEngine::SubmitOne(const uint64_t *src, const uint64_t *dst, const uint6
         // gain 8 % (896 segments, 8.5 GB: 2.55 ms in seven launches against 2.78 ms in one).  Segments on cache lines
         // are worth it from 1 MiB each, 128 MiB a launch (1024 x 1 MiB 327 against 361 us, 1024 x 2 MiB 658 against
         // 753 to 772 us, 512 x 3 MiB 458 against 588 us; 1024 x 512 KiB, 64 MiB a launch, the same either way).  The table form
-        // itself was measured under windows twice, with the prefix search it once had and with the division and
-        // group map it has now, and is left without them: 262 144 pages of 32 KiB at random places lose 7 to 12 %
-        // (3.23 to 3.45 against 3.04 ms), 16 384 ragged segments 3 %, and the 896 long segments in one windowed
-        // table launch are no faster than in seven launches of the kernel-argument form.
+        // itself was measured under windows three times, with the prefix search it once had, with the division and
+        // group map it has now, and with full periods at rates from 6.0 to 7.1 TB/s, and is left without them: 262 144
+        // pages of 32 KiB at random places lose 7 to 12 % (3.23 to 3.45 against 3.04 ms; the third time 2.93 to 3.38
+        // against 2.89 to 3.06), 4096 pages take 58 to 60 instead of 46.5 to 49 us, 16 384 ragged segments lose 3 %, and
+        // the 896 long segments in one windowed table launch are no faster than in seven launches of the kernel-argument form.
         if (maySlice && n > kInlineSegs && route == MFRT_ROUTE_HBM && !unordered && tuning_.windowMBps != 0 && windowsAvailable_ &&
             tuning_.unitsOverride == 0 &&
             total / n >= ((addressBits & (kWindowAlignBytes - 1)) == 0 && tuning_.windowAlignedMBps != 0 ? kWindowSliceMinAlignedSegmentBytes
