@@ -59,8 +59,8 @@ int32_t mf_xcopy_hold_stores(int32_t nanos);
  * period is cut for a rate of HBM traffic (read + written) in MB/s, 6 800 000 by default; at 7 000 000 the waves
  * of a 2 GiB copy now and then no longer keep up, the windows dissolve and the copy runs at about the rate it
  * has without them; at 7 200 000 and above most launches do.  That holds for segments that start between
- * cache lines.  Segments whose sources and destinations all start on 128-byte lines take windows from 128 MiB
- * on and are paced for 7 100 000 (32 x 16 MiB back to back: 6.95 instead of 6.65 TB/s), those of 64 MiB and
+ * cache lines.  Segments whose sources and destinations all start on 128-byte lines are paced for
+ * 7 100 000 (32 x 16 MiB back to back: 6.95 instead of 6.65 TB/s), those of 64 MiB and
  * more on average for 7 400 000, and a batch of 1 GiB and more of such long segments is cut into launches of
  * about 512 MiB, which hold their schedule more often than longer ones (1 GiB: 7.1-7.2 instead of 6.7 TB/s).
  * Segments whose source and destination differ modulo 16 take no windows.  The call sets all three rates; 0

@@ -73,7 +73,7 @@ MF_EXPORT int32_t mf_xcopy_2d_batch(const mf_copy2d_desc *descs, uint32_t n, int
     RectPlan plan;
     uint32_t used = 0;
     uint64_t run = 0;
-    // the same launch in the chunks of the windowed form (RectWindowChunks), which a launch of kWindowGeneralMinBytes and
+    // the same launch in the chunks of the windowed form (RectWindowChunks), which a launch of kWindowRectMinBytes and
     // more between device addresses takes where the segment path would
     uint32_t firstWindowed[kRectInline];
     uint64_t runWindowed = 0;

@@ -1457,8 +1457,7 @@ int XcopyEngine::SubmitOne(const uint64_t *src, const uint64_t *dst, const uint6
         // the loads then straddle units, cost twice the issue slots, and the waves keep no schedule at any rate that pays
         // (100 segments of 10 MB: 5.35 TB/s in windows cut for 6.8, 5.26 for 7.4, 5.51 to 5.56 without windows).
         const bool aligned = (addressBits & (kWindowAlignBytes - 1)) == 0;
-        windowed = !unordered && (apartBits & (kUnitBytes - 1)) == 0 &&
-                   WindowsApply(total, route, aligned && tuning_.windowAlignedMBps != 0 ? kWindowMinBytes : kWindowGeneralMinBytes);
+        windowed = !unordered && (apartBits & (kUnitBytes - 1)) == 0 && WindowsApply(total, route, kWindowMinBytes);
         // Segments that all start on cache lines, in source and destination, hold a higher rate.  Back to back at 6.8 / 7.1 /
         // 7.4 TB/s, the same in four processes: 2 GiB in one segment 6.65 / 6.95 / 7.02 to 7.27, 32 x 16 MiB 6.65 / 6.95 / 7.05 to
         // 7.26, 128 x 9 MiB 6.65 / 6.95 / 6.76 to 7.32.  The reshard's launches of 128 segments of 0.4 to 17 MB from eight

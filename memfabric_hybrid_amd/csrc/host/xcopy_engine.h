@@ -55,7 +55,7 @@ struct XcopyTuning {
     int32_t holdPinnedExtraNanos = 1600;   // added to the rule for table launches, whose descriptors come from pinned host memory: a link round trip before the loads
     bool stageUnordered = true;  // the upload of a ragged table's descriptors is launched without a barrier
     uint32_t deviceTableWgPerCu = 0;   // grid of a device-resident table in workgroups per CU, 0 = eight per segment between 32 and 4096 per CU
-    uint32_t windowMBps = 6800000;   // HBM copies of kWindowGeneralMinBytes and more alternate between read and write windows cut for this rate; 0 = never
+    uint32_t windowMBps = 6800000;   // HBM copies of kWindowRectMinBytes and more alternate between read and write windows cut for this rate; 0 = never
     uint32_t windowAlignedMBps = 7100000;   // the same for launches of segments that all start at multiples of kWindowAlignBytes in source and destination, which hold more; 0 = the rate above
     uint32_t windowLongMBps = 7400000;      // and for those of them whose segments are kWindowLongSegmentBytes and longer on average, which hold more still; 0 = the rate above
 };
@@ -65,9 +65,11 @@ struct XcopyTuning {
 // back to back, 32 segments, windows against none: 66 MiB 6.37 against 5.71 TB/s, 80 MiB 6.57 against 5.76, 130 MiB
 // 6.94 against 6.14, 256 MiB 7.14 against 6.37, 600 MiB 7.20 against 6.31 (at 64 MiB and below the held stores are
 // as fast).  A launch on its own gains less and less steadily below 128 MiB (80 MiB: 32.4 against 31.9 us), hence
-// the limit.  Other segments, paced for windowMBps, and rectangles were measured from 512 MiB on (2 % there).
+// the limit.  Segments between cache lines, paced for windowMBps, gain 5 to 7 % from there on (136 MB 43.7 against
+// 46.8 us, 272 MB 85 against 91.5, 407 MB 129.5 against 137).  Rectangles do not below 512 MiB (136 MB 45 against
+// 47 us, but 407 MB 141 against 136): they keep the limit they were measured at.
 constexpr uint64_t kWindowMinBytes = 128ull << 20;
-constexpr uint64_t kWindowGeneralMinBytes = 512ull << 20;
+constexpr uint64_t kWindowRectMinBytes = 512ull << 20;
 constexpr uint64_t kWindowPieceBytes = 512ull << 20;          // launches into which long segments are cut
 constexpr uint64_t kWindowLongSegmentBytes = 64ull << 20;     // launches whose segments average this much go out in pieces of kWindowPieceBytes and more
 constexpr uint64_t kWindowAlignBytes = 128;                   // a cache line: segments that start on one are read and written in whole lines by every wave
@@ -137,7 +139,7 @@ public:
     int Calibrate();
 
     // Whether an ordered launch that moves `bytes` on `route` takes the form with read and write windows.
-    bool WindowsApply(uint64_t bytes, int route, uint64_t minBytes = kWindowGeneralMinBytes) const;
+    bool WindowsApply(uint64_t bytes, int route, uint64_t minBytes = kWindowRectMinBytes) const;
     // Hardware queue (numbered in order of appearance) of each of the streams made at Start(), in the order they are handed out; returns their number.
     uint32_t StreamQueues(uint32_t *queues, uint32_t capacity) const;
     // No second thread holds a stream of the library: kernels that pace themselves for the whole chip may be used.

@@ -1532,13 +1532,13 @@ static void TestWindows()
     CHECK(engine.Submit(&s1, &d1, &l1, 1, MF_ROUTE_HBM, stream, nullptr, 0) == BM_OK);
     CHECK(fake_rt_last_window() == 7400000);
     {
-        // between cache lines the limit is 512 MiB
+        // between cache lines the same limit, at the general rate
         uint64_t so = s1 + 16;
         uint64_t dO = d1 + 48;
-        uint64_t lo = (gib >> 1) - 1;
+        uint64_t lo = (gib >> 3) - 1;
         CHECK(engine.Submit(&so, &dO, &lo, 1, MF_ROUTE_HBM, stream, nullptr, 0) == BM_OK);
         CHECK(fake_rt_last_window() == 0);
-        lo = gib >> 1;
+        lo = gib >> 3;
         CHECK(engine.Submit(&so, &dO, &lo, 1, MF_ROUTE_HBM, stream, nullptr, 0) == BM_OK);
         CHECK(fake_rt_last_window() == 6800000);
     }

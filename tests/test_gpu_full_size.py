@@ -138,6 +138,55 @@ def test_ragged_batch_above_one_gib_in_read_and_write_windows(pool, lib, oracle,
     assert np.all(got[cursor - lo:] == 0x5A)
 
 
+@pytest.mark.parametrize("layout", ["on-cache-lines", "between-cache-lines", "apart-modulo-16"])
+@pytest.mark.parametrize("total_mib", [130, 200, 300], ids=["130MiB", "200MiB", "300MiB"])
+def test_batches_of_some_hundred_mib_in_windows_whose_last_period_is_full(pool, lib, oracle, total_mib, layout):
+    """Device-to-device batches of 130 to 300 MiB in 37 ragged segments: sizes whose chunks do not fill a whole number
+    of periods on 4096 waves, so the launch runs on fewer waves with every period full.  Segments on cache lines
+    (the higher window rate), between cache lines (the general rate) and with sources apart from their destinations
+    modulo 16 (no windows): what arrives equals the same slices cut on the CPU, the gaps between destinations stay."""
+    dev = pool.peer_rank_ptr(0, bm.BmMemType.DEVICE)
+    host = pool.peer_rank_ptr(0, bm.BmMemType.HOST)
+    span = 2 * GIB + GUARD
+    host_all = gpu_util.host_view(host, 2 * span + GUARD)
+    block = _pattern_block(oracle)
+    total = total_mib * MIB
+    room = total + 64 * MIB
+    _fill_pattern(host_all[GUARD:GUARD + room], block)
+    g2g = bm.BmCopyType.G2G
+    assert pool.copy_data(host + GUARD, dev + GUARD, room, g2g) == 0, native.last_error()
+    assert lib.mfrt_memset(dev + span, 0x5A, room + 2 * GUARD) == 0
+    rng = np.random.default_rng(total_mib)
+    pieces = 37
+    each = total // pieces
+    unit = 128 if layout == "on-cache-lines" else 16
+    lens = rng.integers(each - each // 10, each + each // 10, pieces)
+    lens = lens // unit * unit if layout == "on-cache-lines" else (lens | 1)
+    gaps = rng.integers(1, 64, pieces) * unit
+    src = GUARD + np.cumsum(lens + gaps) - lens
+    src = (src + unit - 1) // unit * unit
+    dst = span + GUARD + np.cumsum(lens + 3 * gaps) - lens
+    dst = (dst + unit - 1) // unit * unit
+    if layout == "between-cache-lines":
+        src, dst = src + 16, dst + 48
+    elif layout == "apart-modulo-16":
+        src, dst = src + 5, dst + 9
+    assert int(src[-1] + lens[-1]) <= GUARD + room and int(dst[-1] + lens[-1]) + GUARD <= span + 2 * GUARD + room
+    assert np.all(src[1:] >= src[:-1] + lens[:-1]) and np.all(dst[1:] >= dst[:-1] + lens[:-1])
+    assert pool.copy_data_batch((dev + src).tolist(), (dev + dst).tolist(), lens.tolist(), len(lens), g2g, 0) == 0, \
+        native.last_error()
+    lo, hi = int(dst[0]) - GUARD, int(dst[-1] + lens[-1]) + GUARD
+    back = span + GUARD
+    assert pool.copy_data(dev + lo, host + back, hi - lo, g2g) == 0, native.last_error()
+    got = host_all[back:back + hi - lo]
+    cursor = lo
+    for s_off, d_off, n in zip(src.tolist(), dst.tolist(), lens.tolist()):
+        assert np.all(got[cursor - lo:d_off - lo] == 0x5A), d_off
+        assert np.array_equal(got[d_off - lo:d_off - lo + n], host_all[s_off:s_off + n]), d_off
+        cursor = d_off + n
+    assert np.all(got[cursor - lo:] == 0x5A)
+
+
 def test_one_segment_beyond_four_gib_goes_out_in_windowed_launches(lib, oracle):
     """One device-to-device segment of 5 GiB + 4 MiB + 777 bytes (its length does not fit 32 bits) from an odd source
     address to an odd destination address: the engine cuts it into windowed launches of about 512 MiB.  Every byte
