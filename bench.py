@@ -386,6 +386,26 @@ def extras_block(lib, pool, dev, batches, tables, steps):
     entry.update({"payload_bytes": blocks[0].payload, "hbm_GBps": round(2 * blocks[0].payload / entry["us_per_call"] / 1e3, 1),
                   "frac_of_hbm_peak": frac(2 * blocks[0].payload / entry["us_per_call"] / 1e3, HBM_PEAK_GBPS)})
     multi["32_x_1MiB"] = entry
+    # ragged tables (no repeating chunk counts: descriptors, prefix and group map are uploaded, the owner of a chunk is looked up)
+    for count, lo, hi in ((400, 30000, 70000), (300, 60000, 180000)):
+        group = []
+        for b in range(16):
+            rng = np.random.default_rng(0xE1 + count + b)
+            lens = (rng.integers(lo, hi, count) // 128 * 128).astype(np.uint64)
+            slot = np.uint64((hi + 4095) // 4096 * 4096)
+            src = rng.permutation(2 * count)[:count].astype(np.uint64) * slot
+            dst = np.uint64(POOL_BYTES // 2) + rng.permutation(2 * count)[:count].astype(np.uint64) * slot
+            group.append(Batch(dev + src, dev + dst, lens))
+        entry = {}
+        for name, hold in (("us_per_call", -1), ("us_per_call_stores_not_held", 0)):
+            assert lib.mf_xcopy_hold_stores(hold) == 0
+            reps = sorted(timed_steps(lib, handle, group, g2g, 300, 30, native.ASYNC_COPY_FLAG)[1] * 1e3 / 300 for _ in range(5))
+            entry[name] = round(reps[2], 2)
+        assert lib.mf_xcopy_hold_stores(-1) == 0
+        entry.update({"segments": count, "payload_bytes": group[0].payload,
+                      "hbm_GBps": round(2 * group[0].payload / entry["us_per_call"] / 1e3, 1),
+                      "frac_of_hbm_peak": frac(2 * group[0].payload / entry["us_per_call"] / 1e3, HBM_PEAK_GBPS)})
+        multi[f"ragged_{count}_segments_{lo // 1000}_to_{hi // 1000}_KB"] = entry
     multi["note"] = ("asynchronous smem_bm_copy_batch calls back to back on one stream, 16 tables in turn, HIP events, median of 5 runs; more than "
                      "128 segments take the table form (descriptors read from the pinned staging slot), up to 24 MiB in 4 KiB chunks and up "
                      "to 64 MiB in 16 KiB chunks with the stores held back until the loads of the launch are out")

@@ -365,11 +365,11 @@ void LaunchInlineProduct(const InlinePlan &plan, hipStream_t s, bool held, bool 
 }
 
 // What the library launches for a batch of 24 to 64 MiB: 16 KiB per wave, sixteen loads per lane, stores held back
-// (1.6 us longer where every workgroup first fetches its descriptor over the link).
+// (2.4 us longer where every workgroup first fetches its descriptor over the link).
 void LaunchTableDeep(const TablePlan &plan, hipStream_t s, bool pinned)
 {
     const uint32_t nanos = HoldNanosFor(plan.nchunk, plan.nchunk, plan.units, false);
-    const uint32_t ticks = HoldTicks(nanos != 0 && pinned ? nanos + 1600 : nanos);
+    const uint32_t ticks = HoldTicks(nanos != 0 && pinned ? nanos + 2400 : nanos);
     hipLaunchKernelGGL((XcopyTableKernel<true, kStoreStream, false, kHoldDeep>), dim3(plan.nchunk), dim3(64), 0, s, plan, ticks);
 }
 

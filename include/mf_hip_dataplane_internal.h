@@ -108,7 +108,8 @@ int32_t mf_xcopy_tune_table(uint32_t stageUnordered, uint32_t deviceTableWgPerCu
  * average 32 KiB and more be copied in 16 KiB chunks, one single wave each with sixteen loads per lane in flight,
  * stores held like those of the smaller batches; 0 keeps them on 4 KiB chunks that store at once.
  * pinnedExtraNanos: added to the wait of launches of more than 128 segments, whose descriptors come out of pinned
- * host memory rather than out of the kernel arguments (default 1600: a wave's loads start a link round trip later).
+ * host memory rather than out of the kernel arguments (default 1600: a wave's loads start a link round trip later;
+ * launches on 16 KiB chunks wait 800 ns more than that).
  * holdOnSideStreams: 1 lets batches launched by the submit threads (mf_xcopy_unordered_streams) hold their stores too;
  * 0 (default): they overlap one another on purpose and store at once. */
 int32_t mf_xcopy_tune_hold(uint32_t deepHold, int32_t pinnedExtraNanos, uint32_t holdOnSideStreams);

@@ -1272,9 +1272,10 @@ uint32_t XcopyEngine::HoldFor(const InlinePlan &plan, uint32_t grid, int route, 
     return with > 0 ? static_cast<uint32_t>(with) : 0;
 }
 
-// Hold of a table launch under a pattern: its waves fetch their descriptors across the host link and issue their
-// loads that much later than those of a launch whose descriptors are kernel arguments.
-uint32_t XcopyEngine::HoldForTable(uint32_t nchunk, uint32_t grid, uint32_t units, int route, bool unordered) const
+// Hold of a table launch.  Under a pattern (pinned) its waves fetch their descriptors across the host link and issue
+// their loads that much later than those of a launch whose descriptors are kernel arguments; without one they find them
+// through the group map in device memory, two dependent loads.
+uint32_t XcopyEngine::HoldForTable(uint32_t nchunk, uint32_t grid, uint32_t units, int route, bool unordered, bool pinned) const
 {
     if (route != MFRT_ROUTE_HBM || unordered || tuning_.holdNanos == 0) {
         return 0;
@@ -1292,7 +1293,16 @@ uint32_t XcopyEngine::HoldForTable(uint32_t nchunk, uint32_t grid, uint32_t unit
     if (tuning_.holdCalibratedOff) {
         return 0;
     }
-    const int64_t with = static_cast<int64_t>(rule) + tuning_.holdPinnedExtraNanos + tuning_.holdDeltaNanos;
+    // The 16 KiB form wants its wait another 800 ns longer than the link round trip explains (sixteen loads per lane take
+    // longer to leave than four): K and V blocks of 3 / 4 / 5 / 6 requests, 27 to 54 MB, with 1600 / 2000 / 2400 / 2800 ns on
+    // top of the rule: 13.3 / 12.7 / 13.0 / 13.4 us, 17.2 / 16.5 / 16.1 / 16.4, 20.3 / 19.8 / 19.1 / 19.3, 24.3 / 23.8 / 23.5 / 23.5;
+    // two requests on 4 KiB chunks 9.3 / 9.7 / 10.1 / 10.5 (and 9.3 with 1200).
+    // Ragged tables, whose descriptors were uploaded: 36 / 40 / 58 MB on 16 KiB chunks 18.4 / 20.0 / 26.2 us with 500 ns on top
+    // of the rule (19.0 / 20.5 / 27.0 with none, 18.7 / 20.4 / 26.0 with 1000) against 20.5 / 22.6 / 28.7 us not held; 12 / 13 /
+    // 20 / 19 MB on 4 KiB chunks 10.9 / 11.6 / 13.8 / 13.9 us with 800 ns against 11.3 / 12.3 / 14.8 / 14.7 (6 MB: 9.3 either way).
+    const int32_t extra = pinned ? tuning_.holdPinnedExtraNanos + (units == kDeepUnits ? kHoldPinnedDeepExtraNanos : 0)
+                                 : (units == kDeepUnits ? kHoldLookupDeepExtraNanos : kHoldLookupExtraNanos);
+    const int64_t with = static_cast<int64_t>(rule) + extra + tuning_.holdDeltaNanos;
     return with > 0 ? static_cast<uint32_t>(with) : 0;
 }
 
@@ -1626,7 +1636,7 @@ int XcopyEngine::SubmitOne(const uint64_t *src, const uint64_t *dst, const uint6
     // stream 2 us whether it overlaps or not, more than the fetch from HBM saves: 36 MB of K and V blocks 20.5
     // against 18.4 us per call.)
     if (pattern.period != 0) {
-        const uint32_t hold = HoldForTable(static_cast<uint32_t>(nchunk), grid, units, route, unordered);
+        const uint32_t hold = HoldForTable(static_cast<uint32_t>(nchunk), grid, units, route, unordered, true);
         table.triples = triples;
         table.pattern = pattern;
         err = mfk_xcopy_table(&table, route, grid, mask, maskValue, stream, hold);
@@ -1660,7 +1670,8 @@ int XcopyEngine::SubmitOne(const uint64_t *src, const uint64_t *dst, const uint6
         table.triples = reinterpret_cast<const uint64_t *>(devBase);
         table.first = reinterpret_cast<const uint32_t *>(devBase + tripleBytes);
         table.group = reinterpret_cast<const uint32_t *>(devBase + tripleBytes + prefixBytes);
-        err = mfk_xcopy_table(&table, route, grid, mask, maskValue, stream, 0);
+        err = mfk_xcopy_table(&table, route, grid, mask, maskValue, stream,
+                              HoldForTable(static_cast<uint32_t>(nchunk), grid, units, route, unordered, false));
         g_launches.fetch_add(2, std::memory_order_relaxed);
     }
     if (err != 0) {

@@ -72,6 +72,9 @@ constexpr uint64_t kWindowMinBytes = 128ull << 20;
 constexpr uint64_t kWindowRectMinBytes = 512ull << 20;
 constexpr uint64_t kWindowPieceBytes = 512ull << 20;          // launches into which long segments are cut
 constexpr uint64_t kWindowLongSegmentBytes = 64ull << 20;     // launches whose segments average this much go out in pieces of kWindowPieceBytes and more
+constexpr int32_t kHoldLookupExtraNanos = 800;                // on top of the rule where a table launch finds its descriptors through the group map
+constexpr int32_t kHoldLookupDeepExtraNanos = 500;            // the same on 16 KiB chunks
+constexpr int32_t kHoldPinnedDeepExtraNanos = 800;            // on top of holdPinnedExtraNanos where a table launch works on 16 KiB chunks
 constexpr uint64_t kWindowAlignBytes = 128;                   // a cache line: segments that start on one are read and written in whole lines by every wave
 constexpr uint64_t kWindowSliceMinSegmentBytes = 4ull << 20;   // tables of segments this long on average are cut into windowed launches
 constexpr uint64_t kWindowSliceMinAlignedSegmentBytes = 1ull << 20;   // the same for segments on cache lines: kInlineSegs of them reach kWindowMinBytes
@@ -195,7 +198,7 @@ private:
     XcopyEngine() = default;
 
     uint32_t HoldFor(const InlinePlan &plan, uint32_t grid, int route, bool unordered) const;
-    uint32_t HoldForTable(uint32_t nchunk, uint32_t grid, uint32_t units, int route, bool unordered) const;
+    uint32_t HoldForTable(uint32_t nchunk, uint32_t grid, uint32_t units, int route, bool unordered, bool pinned) const;
     // Whether a batch of `bytes` in n segments is planned in chunks of kDeepUnits units, to hold the stores of 16 KiB per wave.
     bool DeepHoldApplies(uint64_t bytes, uint32_t n, int route, bool unordered) const;
     int SubmitInPieces(const uint64_t *src, const uint64_t *dst, const uint64_t *len, uint32_t n, uint64_t total, int route,

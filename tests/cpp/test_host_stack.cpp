@@ -39,6 +39,7 @@ extern "C" uint64_t fake_rt_stream_waits(void);
 extern "C" void fake_rt_set_calibration(const float *us);
 extern "C" const uint32_t *fake_rt_calibration_holds(void);
 extern "C" uint32_t fake_rt_last_table_shift(void);
+extern "C" uint32_t fake_rt_last_table_hold(void);
 extern "C" uint64_t fake_rt_group_map_errors(void);
 extern "C" uint64_t fake_rt_in_flight(void);
 
@@ -1419,6 +1420,48 @@ static void TestHeldStores()
         ok = ok && std::memcmp(to.data() + (count - 1 - i) * seg, from.data() + i * seg, seg) == 0;
     }
     CHECK(ok);
+    {
+        // Tables (more than 128 segments) hold their stores too, a little longer than the kernel-argument form: K and V blocks in
+        // turn (a pattern: descriptors out of the pinned slot) and ragged segments (descriptors through the group map), on 4 KiB
+        // chunks below 24 MiB and on 16 KiB chunks from there to 64 MiB.
+        const uint64_t k = 128u << 10;
+        const uint64_t v = 16u << 10;
+        std::vector<uint8_t> a(80u << 20), b(80u << 20);
+        const uint64_t sa = (reinterpret_cast<uint64_t>(a.data()) + 4095) & ~4095ull;
+        const uint64_t sb = (reinterpret_cast<uint64_t>(b.data()) + 4095) & ~4095ull;
+        auto submit = [&](uint32_t n, bool ragged) {
+            std::vector<uint64_t> s(n), d(n), l(n);
+            uint64_t at = 0;
+            for (uint32_t i = 0; i < n; ++i) {
+                l[i] = ragged ? 4096u * (1 + (i * 2654435761u >> 27)) + 4096u * (i % 3) : (i % 2 == 0 ? k : v);
+                s[i] = sa + at;
+                d[i] = sb + at + 4096;
+                at += l[i] + 8192;
+            }
+            CHECK(at + 8192 < (76u << 20));
+            CHECK(engine.Submit(s.data(), d.data(), l.data(), n, MF_ROUTE_HBM, stream, nullptr, 0) == BM_OK);
+            CHECK(engine.DrainThread() == BM_OK);
+            uint64_t chunks4 = 0;
+            uint64_t chunks16 = 0;
+            uint64_t total = 0;
+            for (uint32_t i = 0; i < n; ++i) {
+                chunks4 += (l[i] + 4095) / 4096;
+                chunks16 += (l[i] + 16383) / 16384;
+                total += l[i];
+            }
+            const bool deep = total > (24u << 20);
+            const uint32_t chunks = static_cast<uint32_t>(deep ? chunks16 : chunks4);
+            return HoldNanosFor(chunks, chunks, deep ? 1024 : 256, false);
+        };
+        uint32_t rule = submit(244, false);                 // 17.6 MB: 4 KiB chunks
+        CHECK(rule != 0 && fake_rt_last_table_hold() == rule + 1600);
+        rule = submit(488, false);                          // 35 MB: 16 KiB chunks
+        CHECK(rule != 0 && fake_rt_last_table_hold() == rule + 1600 + kHoldPinnedDeepExtraNanos);
+        rule = submit(300, true);                           // ragged, some 20 MB
+        CHECK(rule != 0 && fake_rt_last_table_hold() == rule + kHoldLookupExtraNanos);
+        rule = submit(600, true);                           // ragged, some 40 MB
+        CHECK(rule != 0 && fake_rt_last_table_hold() == rule + kHoldLookupDeepExtraNanos);
+    }
     hybm_uninit();
 }
 
