@@ -187,6 +187,43 @@ def test_batches_of_some_hundred_mib_in_windows_whose_last_period_is_full(pool, 
     assert np.all(got[cursor - lo:] == 0x5A)
 
 
+def test_table_of_segments_on_cache_lines_is_cut_into_windowed_launches(pool, lib, oracle):
+    """300 segments of about 1.5 MiB on cache lines, shuffled: more than the kernel-argument form holds, so the engine cuts
+    the table into launches of 128 segments (192 MiB each, in read and write windows; the last 44 segments without).  Every
+    segment arrives, the gaps between destinations stay, and mf_xcopy_windows(1) has brought the library's own rates back."""
+    dev = pool.peer_rank_ptr(0, bm.BmMemType.DEVICE)
+    host = pool.peer_rank_ptr(0, bm.BmMemType.HOST)
+    span = 2 * GIB + GUARD
+    host_all = gpu_util.host_view(host, 2 * span + GUARD)
+    block = _pattern_block(oracle)
+    count, slot = 300, 2 * MIB
+    room = count * slot
+    _fill_pattern(host_all[GUARD:GUARD + room], block)
+    g2g = bm.BmCopyType.G2G
+    assert pool.copy_data(host + GUARD, dev + GUARD, room, g2g) == 0, native.last_error()
+    assert lib.mfrt_memset(dev + span, 0x5A, room + 2 * GUARD) == 0
+    rng = np.random.default_rng(300)
+    lens = (rng.integers(MIB + MIB // 4, 2 * MIB - 4096, count) // 128 * 128).astype(np.int64)
+    order = rng.permutation(count)
+    src = GUARD + order * slot + rng.integers(0, 16, count) * 128
+    dst = span + GUARD + np.arange(count) * slot + rng.integers(0, 16, count) * 128
+    assert lib.mf_xcopy_windows(1) == 0
+    before = lib.mf_xcopy_launch_count()
+    assert pool.copy_data_batch((dev + src).tolist(), (dev + dst).tolist(), lens.tolist(), count, g2g, 0) == 0, native.last_error()
+    if _window_rate(lib) != 0:
+        assert lib.mf_xcopy_launch_count() - before == 3
+    lo, hi = int(dst[0]) - GUARD, int(dst[-1] + lens[-1]) + GUARD
+    back = span + GUARD
+    assert pool.copy_data(dev + lo, host + back, hi - lo, g2g) == 0, native.last_error()
+    got = host_all[back:back + hi - lo]
+    cursor = lo
+    for s_off, d_off, n in zip(src.tolist(), dst.tolist(), lens.tolist()):
+        assert np.all(got[cursor - lo:d_off - lo] == 0x5A), d_off
+        assert np.array_equal(got[d_off - lo:d_off - lo + n], host_all[s_off:s_off + n]), d_off
+        cursor = d_off + n
+    assert np.all(got[cursor - lo:] == 0x5A)
+
+
 def test_one_segment_beyond_four_gib_goes_out_in_windowed_launches(lib, oracle):
     """One device-to-device segment of 5 GiB + 4 MiB + 777 bytes (its length does not fit 32 bits) from an odd source
     address to an odd destination address: the engine cuts it into windowed launches of about 512 MiB.  Every byte
