@@ -1163,7 +1163,8 @@ extern "C" int mfk_xcopy_prelaunch(void *stream)
 // Calibration workloads, timed by events on `stream` (see XcopyEngine::Calibrate for what is chosen from them).
 // out[0 .. 3]: microseconds per batch of 122 segments (61 x 128 KiB and 16 KiB in turn, 2196 chunks, 32 tables in turn
 // inside 1 GiB of scratch) without a hold and held for holdNanos[0 .. 2]; out[4 .. 7]: microseconds per copy of 512 MiB by
-// the kernel without windows and in windows cut for windowMBps[0 .. 2].  The minimum of three rounds each.
+// the kernel without windows and in windows cut for windowMBps[0 .. 2].  Batches: the fastest of three rounds of 128
+// launches; copies: the fastest of six, each timed on its own.
 extern "C" int mfk_xcopy_calibrate(void *stream, const uint32_t *holdNanos, const uint32_t *windowMBps, float *out)
 {
     using namespace mf;
