@@ -279,7 +279,9 @@ MF_EXPORT int32_t hybm_data_batch_copy(hybm_entity_t e, hybm_batch_copy_params *
     if (bad == n && MustCheckSource(direction)) {
         bad = entity->FirstOutside(params->sources, params->dataSizes, n);
     }
-    if (bad == n) {   // sides that are not checked against the pool must at least not be null
+    if (bad == n && MustCheckDestination(direction) && MustCheckSource(direction)) {
+        // both sides lie in the pool, and no pool address is null
+    } else if (bad == n) {   // sides that are not checked against the pool must at least not be null
         for (uint32_t i = 0; i < n; ++i) {
             if (params->sources[i] == nullptr || params->destinations[i] == nullptr) {
                 MF_FAIL(BM_INVALID_PARAM, "batch element " << i << " has a null address");

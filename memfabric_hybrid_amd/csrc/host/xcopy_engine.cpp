@@ -797,6 +797,40 @@ bool BuildInlineDirect(const uint64_t *src, const uint64_t *dst, const uint64_t 
 {
     const bool pow2 = (units & (units - 1)) == 0;
     const uint32_t shift = pow2 ? static_cast<uint32_t>(__builtin_ctz(units)) : 0;
+    // The usual batch (blocks scattered over a pool) has nothing to merge, nothing empty and nothing of 4 GiB: one pass
+    // without branches says so, and the plan is then filled by a straight-line loop (the general loop below merges as it
+    // goes and tests every step).
+    if (n != 0 && n <= kInlineSegs && pow2) {
+        uint64_t special = (len[n - 1] == 0 ? 1u : 0u) | (len[n - 1] >> 32);
+        for (uint32_t i = 0; i + 1 < n; ++i) {
+            const uint64_t l = len[i];
+            special |= (l == 0 ? 1u : 0u) | (l >> 32) |
+                       ((src[i] + l == src[i + 1] ? 1u : 0u) & (dst[i] + l == dst[i + 1] ? 1u : 0u));
+        }
+        if (special == 0) {
+            uint32_t run32 = 0;
+            for (uint32_t i = 0; i < n; ++i) {
+                const uint64_t l = len[i];
+                uint64_t head = (0 - dst[i]) & (kUnitBytes - 1);
+                head = head > l ? l : head;
+                const uint64_t chunks = ((l - head) / kUnitBytes + units - 1) >> shift;
+                plan.src[i] = src[i];
+                plan.dst[i] = dst[i];
+                plan.len[i] = static_cast<uint32_t>(l);
+                plan.first[i] = run32;
+                run32 += static_cast<uint32_t>(chunks == 0 ? 1 : chunks);      // n * 2^32 / 4096 chunks at most: no overflow
+            }
+            for (uint32_t i = n; i < kInlineSegs; ++i) {
+                plan.src[i] = 0;
+                plan.dst[i] = 0;
+                plan.len[i] = 0;
+                plan.first[i] = kNoChunk;
+            }
+            plan.nchunk = run32;
+            plan.units = units;
+            return run32 < kNoChunk;
+        }
+    }
     uint32_t used = 0;
     uint64_t run = 0;
     uint64_t curSrc = 0;
